@@ -1,0 +1,214 @@
+/*
+ * nnhip - C ABI of the MI355X (gfx950) GGUF block-quantized linear library, libnnhip.so.
+ *
+ * This is the native boundary that replaces, for the quantized-linear path only, what NNtrain's managed
+ * operator objects reach through ArcExecutionLane + embedded OpenCL kernels.  Every entry point cites the
+ * reference interface it stands in for (paths relative to the NNtrain tree).
+ *
+ * Conventions (taken from the reference's own native boundary, NNtrain.Cuda/Interop/CudaNativeGateway.cs):
+ *   - extern "C", cdecl, default visibility; blittable arguments only (pointers, sizes, ints).
+ *   - every entry returns int status, 0 = success (CudaNativeGateway.cs:275-283); details of the most recent
+ *     failure are fetched with nnhip_last_error (CudaNativeGateway.cs:1360-1371 record layout).
+ *   - packed ABI version (major << 16) | minor, major must match (CudaNativeGateway.cs:7-50).
+ *   - device pointers, lanes, events and graphs are opaque handles (void*).
+ *   - a lane owns one in-order HIP stream (ArcExecutionLane.cs:156); compute entries enqueue and return,
+ *     only transfers and nnhip_synchronize block (ArcExecutionLane.cs:447-474,658).  Calls on one lane must be
+ *     serialised by the caller (the managed lane takes lock(_sync), ArcExecutionLane.cs:28).
+ *   - weights are raw GGUF blocks, uploaded unchanged; matrix row o is in_w/block_elems consecutive blocks
+ *     (NNtrain.Arc/Kernels/qwen.cl:372-373).
+ */
+#ifndef NNHIP_H
+#define NNHIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#if defined(NNHIP_BUILD)
+#define NNHIP_API __attribute__((visibility("default")))
+#else
+#define NNHIP_API
+#endif
+
+#define NNHIP_ABI_MAJOR 1u
+#define NNHIP_ABI_MINOR 0u
+
+/* GGML tensor type ids accepted as `ggml_type` (Qwen2Gguf.cs:8-12, Qwen35Gguf.cs:6-7, Gemma3LocalModel.cs:80). */
+enum {
+    NNHIP_TYPE_Q8_0 = 8,
+    NNHIP_TYPE_Q4_K = 12,
+    NNHIP_TYPE_Q5_K = 13,
+    NNHIP_TYPE_Q6_K = 14,
+    NNHIP_TYPE_IQ2_S = 22
+};
+
+/* Status codes.  Positive values below 1000 are this library's own; HIP runtime errors are reported as
+ * NNHIP_ERR_HIP with the hipError_t in nnhip_error_info.reserved. */
+enum {
+    NNHIP_OK = 0,
+    NNHIP_ERR_INVALID_ARGUMENT = 1,   /* null pointer, non-positive width, rows < 1 ...                */
+    NNHIP_ERR_UNSUPPORTED_TYPE = 2,   /* ggml_type is not one of the five above                         */
+    NNHIP_ERR_INCOMPLETE_BLOCKS = 3,  /* in_w (or elements) is not a whole number of blocks             */
+    NNHIP_ERR_OUT_OF_MEMORY = 4,
+    NNHIP_ERR_HIP = 5,                /* a HIP call failed                                               */
+    NNHIP_ERR_NO_DEVICE = 6,
+    NNHIP_ERR_BAD_HANDLE = 7,         /* lane / event / graph handle not created by this library        */
+    NNHIP_ERR_TOO_LARGE = 8           /* a size exceeds what one launch or the fixed workspace can hold  */
+};
+
+/* Operation ids recorded with a failure (nnhip_error_info.operation). */
+enum {
+    NNHIP_OP_NONE = 0, NNHIP_OP_LANE_CREATE, NNHIP_OP_LANE_DESTROY, NNHIP_OP_ALLOC, NNHIP_OP_FREE,
+    NNHIP_OP_UPLOAD, NNHIP_OP_DOWNLOAD, NNHIP_OP_COPY, NNHIP_OP_SYNCHRONIZE, NNHIP_OP_DEQUANTIZE,
+    NNHIP_OP_MATVEC, NNHIP_OP_MATVEC_BATCH, NNHIP_OP_MATMUL_BF16, NNHIP_OP_EVENT, NNHIP_OP_GRAPH,
+    NNHIP_OP_DEVICE_QUERY, NNHIP_OP_FILL
+};
+
+/* Same field order as the reference's NativeErrorInfo (CudaNativeGateway.cs:1360-1371). */
+typedef struct nnhip_error_info {
+    uint32_t struct_size;
+    uint32_t abi_version;
+    uint64_t sequence;      /* increments with every recorded failure */
+    int32_t status;
+    int32_t device_index;
+    uint32_t operation;
+    uint32_t reserved;      /* hipError_t when status == NNHIP_ERR_HIP */
+} nnhip_error_info;
+
+/* Lane byte counters, the quantities ArcExecutionLane exposes (ArcExecutionLane.cs:71-91). */
+typedef struct nnhip_lane_counters {
+    uint32_t struct_size;
+    uint32_t reserved;
+    uint64_t h2d_bytes;
+    uint64_t d2h_bytes;
+    uint64_t allocated_bytes;
+    uint64_t peak_allocated_bytes;
+    uint64_t kernel_launches;
+} nnhip_lane_counters;
+
+/* One quantized mat-vec of a batch (nnhip_quant_matvec_batch).  Same meaning as the arguments of
+ * nnhip_quant_matvec; 48 bytes, no padding. */
+typedef struct nnhip_matvec_desc {
+    const float* x;         /* device, f32 [rows, in_w]       */
+    const void* w;          /* device, raw blocks             */
+    const float* bias;      /* device, f32 [out_w], nullable  */
+    float* y;               /* device, f32 [rows, out_w]      */
+    uint32_t ggml_type;
+    int32_t rows;
+    int32_t in_w;
+    int32_t out_w;
+} nnhip_matvec_desc;
+
+/* --- library ---------------------------------------------------------------------------------------------- */
+
+/* Packed ABI version.  Replaces nntrain_abi_version (NNtrain.Cuda/native/cuda_runtime_bridge.cu:1436-1438). */
+NNHIP_API uint32_t nnhip_abi_version(void);
+
+/* Copies the most recent failure record; returns NNHIP_OK, or NNHIP_ERR_INVALID_ARGUMENT when out is null or
+ * out_size < sizeof(nnhip_error_info).  Replaces nntrain_last_error (cuda_runtime_bridge.cu:1440-1481). */
+NNHIP_API int nnhip_last_error(nnhip_error_info* out, size_t out_size);
+
+/* Human-readable text of the most recent failure (NUL terminated, truncated to cap).  The managed side turns
+ * it into the exception message, as OpenClNative.Check does (NNtrain.Arc/OpenClNative.cs:37-41). */
+NNHIP_API int nnhip_last_error_message(char* buf, int cap);
+
+/* Device enumeration.  Replaces ArcDevices.Enumerate (NNtrain.Arc/ArcDevices.cs:18). */
+NNHIP_API int nnhip_device_count(int* count);
+NNHIP_API int nnhip_device_name(int device, char* buf, int cap);
+/* Compute units and bytes of device memory, for reporting. */
+NNHIP_API int nnhip_device_info(int device, int* compute_units, uint64_t* total_memory_bytes);
+
+/* Block geometry of a type: elements per block and bytes per block (Qwen35Gguf.cs:15-34). */
+NNHIP_API int nnhip_type_block(uint32_t ggml_type, int* block_elems, int* block_bytes);
+/* Payload bytes of an [out_w, in_w] matrix, with the same validation as ArcQuantizedMatrix's constructor
+ * (NNtrain.Core/Serialization/ArcQuantizedMatrix.cs:20-32). */
+NNHIP_API int nnhip_matrix_bytes(uint32_t ggml_type, int in_w, int out_w, uint64_t* bytes);
+
+/* --- lane: one device, one in-order stream ------------------------------------------------------------------ */
+
+/* Replaces ArcExecutionLane construction (ArcExecutionLane.cs:120-209) and Dispose (:872-915).
+ * Destroy synchronises, then frees every buffer the lane still owns. */
+NNHIP_API int nnhip_lane_create(int device, void** lane);
+NNHIP_API int nnhip_lane_destroy(void* lane);
+
+/* Replaces ArcExecutionLane.Allocate / AllocateBytes (:241,:271) and ArcBuffer.Dispose (:917-931).
+ * Memory is not cleared. */
+NNHIP_API int nnhip_alloc(void* lane, size_t bytes, void** dptr);
+NNHIP_API int nnhip_free(void* lane, void* dptr);
+
+/* Blocking raw transfers.  Replace UploadRaw (:322-327) and Read / ReadRaw (:277,:334).  The bytes are not
+ * interpreted: GGUF blocks go up exactly as they sit in the file. */
+NNHIP_API int nnhip_upload(void* lane, void* dptr, size_t offset, const void* host, size_t bytes);
+NNHIP_API int nnhip_download(void* lane, const void* dptr, size_t offset, void* host, size_t bytes);
+/* Device-to-device copy on the lane's stream (asynchronous).  Replaces the lane's CopyBuffer used for KV
+ * growth and staging (Qwen35QuantizedModel.cs:1037-1061). */
+NNHIP_API int nnhip_copy(void* lane, void* dst, size_t dst_offset, const void* src, size_t src_offset, size_t bytes);
+/* Fill `count` 32-bit words with `value` on the lane's stream (asynchronous); used for zero bias and NaN guards. */
+NNHIP_API int nnhip_fill_u32(void* lane, void* dptr, size_t offset, uint32_t value, size_t count);
+
+/* Replaces ArcExecutionLane.Synchronize (:658). */
+NNHIP_API int nnhip_synchronize(void* lane);
+
+/* Replaces the H2DBytes / D2HBytes / AllocatedBytes / PeakAllocatedBytes properties (:71-91). */
+NNHIP_API int nnhip_lane_get_counters(void* lane, nnhip_lane_counters* out, size_t out_size);
+
+/* The lane's hipStream_t, for callers that interoperate with other HIP code. */
+NNHIP_API int nnhip_lane_stream(void* lane, void** stream);
+
+/* --- compute ------------------------------------------------------------------------------------------------ */
+
+/* out[i] = decoded weight i, FP32, bit-identical to the managed decoders GgufQ4K.Dequantize / GgufQ6K.Dequantize
+ * (NNtrain.Core/Serialization/GgufQ4K.cs:9-60, GgufQ6K.cs:9-54) and to native ggml for Q5_K / IQ2_S / Q8_0
+ * (NNtrain.Arc/Kernels/qwen35_iq.cl:398-419).  Also the embedding-row lookup of
+ * Matrix.Embedding (Qwen35QuantizedModel.cs:1497-1521) when w points at one row.  `elements` must be a whole
+ * number of blocks.  Asynchronous. */
+NNHIP_API int nnhip_dequantize(void* lane, uint32_t ggml_type, const void* w, float* out, int64_t elements);
+
+/* y[r, o] = bias[o] + sum_k x[r, k] * w[o, k], FP32 accumulate, dequantization fused.  Argument order is the
+ * kernel signature used throughout the reference, (x, weight, bias, y, rows, input_width, output_width)
+ * (NNtrain.Arc/Kernels/qwen.cl:374-377; call site Qwen35QuantizedModel.cs:1355-1358).  Replaces the launch made
+ * by Qwen35QuantizedModel.Matrix.Forward (Qwen35QuantizedModel.cs:1210-1369) and Tensor.ArcQwenQuantizedLinear
+ * (NNtrain.Core/Tensors/Tensor.QwenQuantized.cs:29-96) for decode (rows == 1) and small row counts.  Each
+ * output row of y is computed with the same operation order whatever `rows` is, so rows > 1 equals stacked
+ * rows == 1 calls bit for bit (Qwen35InferencePrefillLinearTests.cs:64-77).  bias may be null (zero).
+ * Asynchronous. */
+NNHIP_API int nnhip_quant_matvec(void* lane, uint32_t ggml_type, const float* x, const void* w, const float* bias,
+                                 float* y, int rows, int in_w, int out_w);
+
+/* `count` independent mat-vecs enqueued as one unit of work (a single launch per group of equal type), for the
+ * per-token projection sets that ForwardTokenDevice issues back to back (Qwen35QuantizedModel.cs:451-513).
+ * `descs` is a host array.  Results are identical to `count` nnhip_quant_matvec calls.  Asynchronous. */
+NNHIP_API int nnhip_quant_matvec_batch(void* lane, const nnhip_matvec_desc* descs, int count);
+
+/* Prefill: y[r, o] = bias[o] + sum_k x[r, k] * w[o, k] with x given as bfloat16 bit patterns [rows, in_w];
+ * weight tiles are dequantized to bfloat16 in LDS and contracted on MFMA with FP32 accumulators.  Replaces the
+ * XMX prefill launch of Matrix.Forward for rows >= 16 (Qwen35QuantizedModel.cs:1249-1317, kernel
+ * NNtrain.Arc/Kernels/qwen35_prefill_xmx.cl:112-184).  Asynchronous. */
+NNHIP_API int nnhip_quant_matmul_bf16(void* lane, uint32_t ggml_type, const uint16_t* x_bf16, const void* w,
+                                      const float* bias, float* y, int rows, int in_w, int out_w);
+
+/* --- timing and replay --------------------------------------------------------------------------------------- */
+
+/* Device events on the lane's stream.  Replace the per-kernel OpenCL event timing of
+ * ArcExecutionLane.RecordKernelTime (ArcExecutionLane.cs:727-742). */
+NNHIP_API int nnhip_event_create(void* lane, void** event);
+NNHIP_API int nnhip_event_destroy(void* lane, void* event);
+NNHIP_API int nnhip_event_record(void* lane, void* event);
+/* Blocks until `stop` has completed, then returns the milliseconds between the two events. */
+NNHIP_API int nnhip_event_elapsed_ms(void* lane, void* start, void* stop, float* ms);
+
+/* Capture the work enqueued on the lane between begin and end into a replayable HIP graph, for launch-bound
+ * decode loops (the reference batches dispatches instead: ArcExecutionOptions.BatchDispatch,
+ * ArcExecutionLane.cs:318,642).  No allocation, transfer or synchronise call is allowed while capturing. */
+NNHIP_API int nnhip_graph_begin(void* lane);
+NNHIP_API int nnhip_graph_end(void* lane, void** graph);
+NNHIP_API int nnhip_graph_launch(void* lane, void* graph);
+NNHIP_API int nnhip_graph_destroy(void* lane, void* graph);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NNHIP_H */

@@ -1,0 +1,518 @@
+// C ABI of libnnhip.so: lanes, device memory, transfers, error record, and validated dispatch to the kernels.
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <new>
+
+#include "nnhip_internal.h"
+
+namespace nnhip {
+
+namespace {
+
+std::mutex g_error_mutex;
+nnhip_error_info g_last_error{sizeof(nnhip_error_info), (NNHIP_ABI_MAJOR << 16) | NNHIP_ABI_MINOR, 0, 0, -1, 0, 0};
+char g_last_message[256] = "";
+
+Lane* as_lane(void* h)
+{
+    Lane* l = static_cast<Lane*>(h);
+    return (l && l->magic == kLaneMagic) ? l : nullptr;
+}
+
+int hip_fail(hipError_t e, uint32_t op, int device, const char* what)
+{
+    return fail(NNHIP_ERR_HIP, op, device, static_cast<uint32_t>(e), "%s failed: %s (%d)", what, hipGetErrorString(e),
+                static_cast<int>(e));
+}
+
+#define NNHIP_LANE(handle, op)                                                                     \
+    Lane* lane = as_lane(handle);                                                                  \
+    if (!lane) return fail(NNHIP_ERR_BAD_HANDLE, op, -1, 0, "lane handle is null or not a lane");   \
+    {                                                                                              \
+        hipError_t e_ = hipSetDevice(lane->device);                                                \
+        if (e_ != hipSuccess) return hip_fail(e_, op, lane->device, "hipSetDevice");               \
+    }
+
+// Shape checks shared by the compute entries; mirror ArcQuantizedMatrix's constructor and Forward
+// (NNtrain.Core/Serialization/ArcQuantizedMatrix.cs:20-32,49-54).
+int check_linear(uint32_t op, Lane* lane, uint32_t type, const void* x, const void* w, const void* y, int rows, int in_w,
+                 int out_w)
+{
+    int elems = 0, bytes = 0;
+    if (!type_block(type, &elems, &bytes))
+        return fail(NNHIP_ERR_UNSUPPORTED_TYPE, op, lane->device, 0, "GGML type %u is not a supported quantized matrix type", type);
+    if (!x || !w || !y) return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0, "x, w and y must be non-null");
+    if (rows < 1 || in_w < 1 || out_w < 1)
+        return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0, "rows, in_w and out_w must be positive (got %d, %d, %d)", rows, in_w, out_w);
+    if (in_w % elems != 0)
+        return fail(NNHIP_ERR_INCOMPLETE_BLOCKS, op, lane->device, 0, "quantized rows must contain complete %d-value blocks (in_w = %d)", elems, in_w);
+    if ((reinterpret_cast<uintptr_t>(x) & 15u) || (reinterpret_cast<uintptr_t>(y) & 3u))
+        return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0, "x must be 16-byte aligned and y 4-byte aligned");
+    const uintptr_t wa = (type == NNHIP_TYPE_Q4_K || type == NNHIP_TYPE_Q5_K) ? 15u : 3u;
+    if (reinterpret_cast<uintptr_t>(w) & wa)
+        return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0, "weight pointer must be %u-byte aligned", static_cast<unsigned>(wa + 1));
+    return NNHIP_OK;
+}
+
+}  // namespace
+
+bool type_block(uint32_t type, int* elems, int* bytes)
+{
+    int e = 0, b = 0;
+    switch (type) {
+    case NNHIP_TYPE_Q8_0: e = 32; b = 34; break;
+    case NNHIP_TYPE_Q4_K: e = 256; b = 144; break;
+    case NNHIP_TYPE_Q5_K: e = 256; b = 176; break;
+    case NNHIP_TYPE_Q6_K: e = 256; b = 210; break;
+    case NNHIP_TYPE_IQ2_S: e = 256; b = 82; break;
+    default: return false;
+    }
+    if (elems) *elems = e;
+    if (bytes) *bytes = b;
+    return true;
+}
+
+int fail(int status, uint32_t op, int device, uint32_t hip_error, const char* fmt, ...)
+{
+    std::lock_guard<std::mutex> guard(g_error_mutex);
+    g_last_error.sequence += 1;
+    g_last_error.status = status;
+    g_last_error.device_index = device;
+    g_last_error.operation = op;
+    g_last_error.reserved = hip_error;
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_last_message, sizeof(g_last_message), fmt, ap);
+    va_end(ap);
+    return status;
+}
+
+}  // namespace nnhip
+
+using namespace nnhip;
+
+extern "C" {
+
+uint32_t nnhip_abi_version(void) { return (NNHIP_ABI_MAJOR << 16) | NNHIP_ABI_MINOR; }
+
+int nnhip_last_error(nnhip_error_info* out, size_t out_size)
+{
+    if (!out || out_size < sizeof(nnhip_error_info)) return NNHIP_ERR_INVALID_ARGUMENT;
+    std::lock_guard<std::mutex> guard(g_error_mutex);
+    *out = g_last_error;
+    return NNHIP_OK;
+}
+
+int nnhip_last_error_message(char* buf, int cap)
+{
+    if (!buf || cap < 1) return NNHIP_ERR_INVALID_ARGUMENT;
+    std::lock_guard<std::mutex> guard(g_error_mutex);
+    snprintf(buf, static_cast<size_t>(cap), "%s", g_last_message);
+    return NNHIP_OK;
+}
+
+int nnhip_device_count(int* count)
+{
+    if (!count) return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_DEVICE_QUERY, -1, 0, "count is null");
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e == hipErrorNoDevice) {
+        *count = 0;
+        return NNHIP_OK;
+    }
+    if (e != hipSuccess) return hip_fail(e, NNHIP_OP_DEVICE_QUERY, -1, "hipGetDeviceCount");
+    *count = n;
+    return NNHIP_OK;
+}
+
+int nnhip_device_name(int device, char* buf, int cap)
+{
+    if (!buf || cap < 1) return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_DEVICE_QUERY, device, 0, "buffer is null or empty");
+    hipDeviceProp_t prop;
+    hipError_t e = hipGetDeviceProperties(&prop, device);
+    if (e != hipSuccess) return hip_fail(e, NNHIP_OP_DEVICE_QUERY, device, "hipGetDeviceProperties");
+    snprintf(buf, static_cast<size_t>(cap), "%s (%s)", prop.name, prop.gcnArchName);
+    return NNHIP_OK;
+}
+
+int nnhip_device_info(int device, int* compute_units, uint64_t* total_memory_bytes)
+{
+    hipDeviceProp_t prop;
+    hipError_t e = hipGetDeviceProperties(&prop, device);
+    if (e != hipSuccess) return hip_fail(e, NNHIP_OP_DEVICE_QUERY, device, "hipGetDeviceProperties");
+    if (compute_units) *compute_units = prop.multiProcessorCount;
+    if (total_memory_bytes) *total_memory_bytes = prop.totalGlobalMem;
+    return NNHIP_OK;
+}
+
+int nnhip_type_block(uint32_t ggml_type, int* block_elems, int* block_bytes)
+{
+    if (!type_block(ggml_type, block_elems, block_bytes))
+        return fail(NNHIP_ERR_UNSUPPORTED_TYPE, NNHIP_OP_NONE, -1, 0, "GGML type %u is not a supported quantized matrix type", ggml_type);
+    return NNHIP_OK;
+}
+
+int nnhip_matrix_bytes(uint32_t ggml_type, int in_w, int out_w, uint64_t* bytes)
+{
+    int elems = 0, bb = 0;
+    if (!type_block(ggml_type, &elems, &bb))
+        return fail(NNHIP_ERR_UNSUPPORTED_TYPE, NNHIP_OP_NONE, -1, 0, "GGML type %u is not a supported quantized matrix type", ggml_type);
+    if (!bytes || in_w < 1 || out_w < 1)
+        return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_NONE, -1, 0, "widths must be positive and bytes non-null");
+    if (in_w % elems != 0)
+        return fail(NNHIP_ERR_INCOMPLETE_BLOCKS, NNHIP_OP_NONE, -1, 0, "quantized rows must contain complete %d-value blocks", elems);
+    *bytes = static_cast<uint64_t>(out_w) * static_cast<uint64_t>(in_w / elems) * static_cast<uint64_t>(bb);
+    return NNHIP_OK;
+}
+
+int nnhip_lane_create(int device, void** out)
+{
+    if (!out) return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_LANE_CREATE, device, 0, "lane output pointer is null");
+    *out = nullptr;
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess || n == 0) return fail(NNHIP_ERR_NO_DEVICE, NNHIP_OP_LANE_CREATE, device, static_cast<uint32_t>(e), "no HIP device is available");
+    if (device < 0 || device >= n)
+        return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_LANE_CREATE, device, 0, "device index %d is outside 0..%d", device, n - 1);
+    e = hipSetDevice(device);
+    if (e != hipSuccess) return hip_fail(e, NNHIP_OP_LANE_CREATE, device, "hipSetDevice");
+    hipDeviceProp_t prop;
+    e = hipGetDeviceProperties(&prop, device);
+    if (e != hipSuccess) return hip_fail(e, NNHIP_OP_LANE_CREATE, device, "hipGetDeviceProperties");
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return fail(NNHIP_ERR_NO_DEVICE, NNHIP_OP_LANE_CREATE, device, 0, "device %d is %s; this library is built for gfx950 only", device, prop.gcnArchName);
+    Lane* lane = new (std::nothrow) Lane();
+    if (!lane) return fail(NNHIP_ERR_OUT_OF_MEMORY, NNHIP_OP_LANE_CREATE, device, 0, "host allocation failed");
+    lane->device = device;
+    lane->compute_units = prop.multiProcessorCount;
+    lane->counters.struct_size = sizeof(nnhip_lane_counters);
+    e = hipStreamCreateWithFlags(&lane->stream, hipStreamNonBlocking);
+    if (e != hipSuccess) {
+        delete lane;
+        return hip_fail(e, NNHIP_OP_LANE_CREATE, device, "hipStreamCreateWithFlags");
+    }
+    *out = lane;
+    return NNHIP_OK;
+}
+
+int nnhip_lane_destroy(void* handle)
+{
+    NNHIP_LANE(handle, NNHIP_OP_LANE_DESTROY)
+    hipError_t first = hipStreamSynchronize(lane->stream);
+    for (auto& kv : lane->buffers) {
+        hipError_t e = hipFree(kv.first);
+        if (first == hipSuccess) first = e;
+    }
+    lane->buffers.clear();
+    if (lane->batch_table) (void)hipFree(lane->batch_table);
+    if (lane->batch_table_host) (void)hipHostFree(lane->batch_table_host);
+    hipError_t e = hipStreamDestroy(lane->stream);
+    if (first == hipSuccess) first = e;
+    const int device = lane->device;
+    lane->magic = 0;
+    delete lane;
+    if (first != hipSuccess) return hip_fail(first, NNHIP_OP_LANE_DESTROY, device, "lane teardown");
+    return NNHIP_OK;
+}
+
+int nnhip_alloc(void* handle, size_t bytes, void** dptr)
+{
+    NNHIP_LANE(handle, NNHIP_OP_ALLOC)
+    if (!dptr || bytes == 0) return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_ALLOC, lane->device, 0, "allocation size must be positive and dptr non-null");
+    if (lane->capturing) return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_ALLOC, lane->device, 0, "no allocation while a graph is being captured");
+    void* p = nullptr;
+    hipError_t e = hipMalloc(&p, bytes);
+    if (e == hipErrorOutOfMemory) {
+        (void)hipGetLastError();
+        return fail(NNHIP_ERR_OUT_OF_MEMORY, NNHIP_OP_ALLOC, lane->device, static_cast<uint32_t>(e), "device allocation of %zu bytes failed", bytes);
+    }
+    if (e != hipSuccess) return hip_fail(e, NNHIP_OP_ALLOC, lane->device, "hipMalloc");
+    std::lock_guard<std::mutex> guard(lane->mutex);
+    lane->buffers.emplace(p, bytes);
+    lane->counters.allocated_bytes += bytes;
+    if (lane->counters.allocated_bytes > lane->counters.peak_allocated_bytes)
+        lane->counters.peak_allocated_bytes = lane->counters.allocated_bytes;
+    *dptr = p;
+    return NNHIP_OK;
+}
+
+int nnhip_free(void* handle, void* dptr)
+{
+    NNHIP_LANE(handle, NNHIP_OP_FREE)
+    if (!dptr) return NNHIP_OK;
+    if (lane->capturing) return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_FREE, lane->device, 0, "no free while a graph is being captured");
+    {
+        std::lock_guard<std::mutex> guard(lane->mutex);
+        auto it = lane->buffers.find(dptr);
+        if (it == lane->buffers.end())
+            return fail(NNHIP_ERR_BAD_HANDLE, NNHIP_OP_FREE, lane->device, 0, "pointer was not allocated by this lane");
+        lane->counters.allocated_bytes -= it->second;
+        lane->buffers.erase(it);
+    }
+    // Work already enqueued may still read the buffer: drain the lane's stream first (hipFree itself only waits for
+    // the null stream, which a non-blocking stream does not join).
+    hipError_t e = hipStreamSynchronize(lane->stream);
+    if (e != hipSuccess) return hip_fail(e, NNHIP_OP_FREE, lane->device, "hipStreamSynchronize");
+    e = hipFree(dptr);
+    if (e != hipSuccess) return hip_fail(e, NNHIP_OP_FREE, lane->device, "hipFree");
+    return NNHIP_OK;
+}
+
+int nnhip_upload(void* handle, void* dptr, size_t offset, const void* host, size_t bytes)
+{
+    NNHIP_LANE(handle, NNHIP_OP_UPLOAD)
+    if (bytes == 0) return NNHIP_OK;
+    if (!dptr || !host) return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_UPLOAD, lane->device, 0, "null pointer");
+    if (lane->capturing) return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_UPLOAD, lane->device, 0, "no transfer while a graph is being captured");
+    hipError_t e = hipMemcpyAsync(static_cast<char*>(dptr) + offset, host, bytes, hipMemcpyHostToDevice, lane->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(lane->stream);
+    if (e != hipSuccess) return hip_fail(e, NNHIP_OP_UPLOAD, lane->device, "host-to-device copy");
+    std::lock_guard<std::mutex> guard(lane->mutex);
+    lane->counters.h2d_bytes += bytes;
+    return NNHIP_OK;
+}
+
+int nnhip_download(void* handle, const void* dptr, size_t offset, void* host, size_t bytes)
+{
+    NNHIP_LANE(handle, NNHIP_OP_DOWNLOAD)
+    if (bytes == 0) return NNHIP_OK;
+    if (!dptr || !host) return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_DOWNLOAD, lane->device, 0, "null pointer");
+    if (lane->capturing) return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_DOWNLOAD, lane->device, 0, "no transfer while a graph is being captured");
+    hipError_t e = hipMemcpyAsync(host, static_cast<const char*>(dptr) + offset, bytes, hipMemcpyDeviceToHost, lane->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(lane->stream);
+    if (e != hipSuccess) return hip_fail(e, NNHIP_OP_DOWNLOAD, lane->device, "device-to-host copy");
+    std::lock_guard<std::mutex> guard(lane->mutex);
+    lane->counters.d2h_bytes += bytes;
+    return NNHIP_OK;
+}
+
+int nnhip_copy(void* handle, void* dst, size_t dst_offset, const void* src, size_t src_offset, size_t bytes)
+{
+    NNHIP_LANE(handle, NNHIP_OP_COPY)
+    if (bytes == 0) return NNHIP_OK;
+    if (!dst || !src) return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_COPY, lane->device, 0, "null pointer");
+    hipError_t e = hipMemcpyAsync(static_cast<char*>(dst) + dst_offset, static_cast<const char*>(src) + src_offset, bytes,
+                                  hipMemcpyDeviceToDevice, lane->stream);
+    if (e != hipSuccess) return hip_fail(e, NNHIP_OP_COPY, lane->device, "device-to-device copy");
+    return NNHIP_OK;
+}
+
+int nnhip_fill_u32(void* handle, void* dptr, size_t offset, uint32_t value, size_t count)
+{
+    NNHIP_LANE(handle, NNHIP_OP_FILL)
+    if (!dptr || (offset & 3u)) return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_FILL, lane->device, 0, "null pointer or offset not a multiple of 4");
+    hipError_t e = launch_fill_u32(lane, reinterpret_cast<uint32_t*>(static_cast<char*>(dptr) + offset), value, count);
+    if (e != hipSuccess) return hip_fail(e, NNHIP_OP_FILL, lane->device, "fill launch");
+    return NNHIP_OK;
+}
+
+int nnhip_synchronize(void* handle)
+{
+    NNHIP_LANE(handle, NNHIP_OP_SYNCHRONIZE)
+    if (lane->capturing) return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_SYNCHRONIZE, lane->device, 0, "no synchronise while a graph is being captured");
+    hipError_t e = hipStreamSynchronize(lane->stream);
+    if (e != hipSuccess) return hip_fail(e, NNHIP_OP_SYNCHRONIZE, lane->device, "hipStreamSynchronize");
+    return NNHIP_OK;
+}
+
+int nnhip_lane_get_counters(void* handle, nnhip_lane_counters* out, size_t out_size)
+{
+    Lane* lane = as_lane(handle);
+    if (!lane) return fail(NNHIP_ERR_BAD_HANDLE, NNHIP_OP_NONE, -1, 0, "lane handle is null or not a lane");
+    if (!out || out_size < sizeof(nnhip_lane_counters)) return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_NONE, lane->device, 0, "counter buffer too small");
+    std::lock_guard<std::mutex> guard(lane->mutex);
+    *out = lane->counters;
+    return NNHIP_OK;
+}
+
+int nnhip_lane_stream(void* handle, void** stream)
+{
+    Lane* lane = as_lane(handle);
+    if (!lane || !stream) return fail(NNHIP_ERR_BAD_HANDLE, NNHIP_OP_NONE, -1, 0, "lane handle is null or not a lane");
+    *stream = lane->stream;
+    return NNHIP_OK;
+}
+
+int nnhip_dequantize(void* handle, uint32_t ggml_type, const void* w, float* out, int64_t elements)
+{
+    NNHIP_LANE(handle, NNHIP_OP_DEQUANTIZE)
+    int elems = 0, bytes = 0;
+    if (!type_block(ggml_type, &elems, &bytes))
+        return fail(NNHIP_ERR_UNSUPPORTED_TYPE, NNHIP_OP_DEQUANTIZE, lane->device, 0, "GGML type %u is not a supported quantized matrix type", ggml_type);
+    if (elements < 0) return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_DEQUANTIZE, lane->device, 0, "element count must be non-negative");
+    if (elements % elems != 0)
+        return fail(NNHIP_ERR_INCOMPLETE_BLOCKS, NNHIP_OP_DEQUANTIZE, lane->device, 0, "element count must be a multiple of %d", elems);
+    if (elements == 0) return NNHIP_OK;
+    if (!w || !out) return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_DEQUANTIZE, lane->device, 0, "null pointer");
+    const uintptr_t wa = (ggml_type == NNHIP_TYPE_Q4_K || ggml_type == NNHIP_TYPE_Q5_K) ? 3u : 1u;
+    if ((reinterpret_cast<uintptr_t>(out) & 15u) || (reinterpret_cast<uintptr_t>(w) & wa))
+        return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_DEQUANTIZE, lane->device, 0, "out must be 16-byte aligned and w %u-byte aligned", static_cast<unsigned>(wa + 1));
+    hipError_t e = launch_dequantize(lane, ggml_type, w, out, elements);
+    if (e != hipSuccess) return hip_fail(e, NNHIP_OP_DEQUANTIZE, lane->device, "dequantize launch");
+    lane->counters.kernel_launches += 1;
+    return NNHIP_OK;
+}
+
+int nnhip_quant_matvec(void* handle, uint32_t ggml_type, const float* x, const void* w, const float* bias, float* y,
+                       int rows, int in_w, int out_w)
+{
+    NNHIP_LANE(handle, NNHIP_OP_MATVEC)
+    int rc = check_linear(NNHIP_OP_MATVEC, lane, ggml_type, x, w, y, rows, in_w, out_w);
+    if (rc != NNHIP_OK) return rc;
+    if (in_w > matvec_max_in_w(ggml_type))
+        return fail(NNHIP_ERR_TOO_LARGE, NNHIP_OP_MATVEC, lane->device, 0, "in_w %d exceeds the %d values one workgroup can stage", in_w, matvec_max_in_w(ggml_type));
+    if (rows > 65535) return fail(NNHIP_ERR_TOO_LARGE, NNHIP_OP_MATVEC, lane->device, 0, "rows %d exceeds 65535", rows);
+    hipError_t e = launch_matvec(lane, ggml_type, x, w, bias, y, rows, in_w, out_w);
+    if (e != hipSuccess) return hip_fail(e, NNHIP_OP_MATVEC, lane->device, "mat-vec launch");
+    lane->counters.kernel_launches += 1;
+    return NNHIP_OK;
+}
+
+int nnhip_quant_matvec_batch(void* handle, const nnhip_matvec_desc* descs, int count)
+{
+    NNHIP_LANE(handle, NNHIP_OP_MATVEC_BATCH)
+    if (count < 0 || (count > 0 && !descs))
+        return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_MATVEC_BATCH, lane->device, 0, "descriptor array is null or count negative");
+    for (int i = 0; i < count; ++i) {
+        const nnhip_matvec_desc& d = descs[i];
+        int rc = check_linear(NNHIP_OP_MATVEC_BATCH, lane, d.ggml_type, d.x, d.w, d.y, d.rows, d.in_w, d.out_w);
+        if (rc != NNHIP_OK) return rc;
+        if (d.in_w > matvec_max_in_w(d.ggml_type))
+            return fail(NNHIP_ERR_TOO_LARGE, NNHIP_OP_MATVEC_BATCH, lane->device, 0, "descriptor %d: in_w %d exceeds the %d values one workgroup can stage", i, d.in_w, matvec_max_in_w(d.ggml_type));
+    }
+    if (count == 0) return NNHIP_OK;
+    hipError_t e = launch_matvec_batch(lane, descs, count);
+    if (e != hipSuccess) return hip_fail(e, NNHIP_OP_MATVEC_BATCH, lane->device, "batched mat-vec launch");
+    return NNHIP_OK;
+}
+
+int nnhip_quant_matmul_bf16(void* handle, uint32_t ggml_type, const uint16_t* x_bf16, const void* w, const float* bias,
+                            float* y, int rows, int in_w, int out_w)
+{
+    NNHIP_LANE(handle, NNHIP_OP_MATMUL_BF16)
+    int rc = check_linear(NNHIP_OP_MATMUL_BF16, lane, ggml_type, x_bf16, w, y, rows, in_w, out_w);
+    if (rc != NNHIP_OK) return rc;
+    hipError_t e = launch_matmul_bf16(lane, ggml_type, x_bf16, w, bias, y, rows, in_w, out_w);
+    if (e == hipErrorNotSupported)
+        return fail(NNHIP_ERR_UNSUPPORTED_TYPE, NNHIP_OP_MATMUL_BF16, lane->device, 0, "bf16 prefill mat-mul does not support GGML type %u", ggml_type);
+    if (e != hipSuccess) return hip_fail(e, NNHIP_OP_MATMUL_BF16, lane->device, "mat-mul launch");
+    lane->counters.kernel_launches += 1;
+    return NNHIP_OK;
+}
+
+int nnhip_event_create(void* handle, void** event)
+{
+    NNHIP_LANE(handle, NNHIP_OP_EVENT)
+    if (!event) return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_EVENT, lane->device, 0, "event output pointer is null");
+    Event* ev = new (std::nothrow) Event();
+    if (!ev) return fail(NNHIP_ERR_OUT_OF_MEMORY, NNHIP_OP_EVENT, lane->device, 0, "host allocation failed");
+    hipError_t e = hipEventCreate(&ev->event);
+    if (e != hipSuccess) {
+        delete ev;
+        return hip_fail(e, NNHIP_OP_EVENT, lane->device, "hipEventCreate");
+    }
+    *event = ev;
+    return NNHIP_OK;
+}
+
+int nnhip_event_destroy(void* handle, void* event)
+{
+    NNHIP_LANE(handle, NNHIP_OP_EVENT)
+    Event* ev = static_cast<Event*>(event);
+    if (!ev || ev->magic != kEventMagic) return fail(NNHIP_ERR_BAD_HANDLE, NNHIP_OP_EVENT, lane->device, 0, "not an event handle");
+    hipError_t e = hipEventDestroy(ev->event);
+    ev->magic = 0;
+    delete ev;
+    if (e != hipSuccess) return hip_fail(e, NNHIP_OP_EVENT, lane->device, "hipEventDestroy");
+    return NNHIP_OK;
+}
+
+int nnhip_event_record(void* handle, void* event)
+{
+    NNHIP_LANE(handle, NNHIP_OP_EVENT)
+    Event* ev = static_cast<Event*>(event);
+    if (!ev || ev->magic != kEventMagic) return fail(NNHIP_ERR_BAD_HANDLE, NNHIP_OP_EVENT, lane->device, 0, "not an event handle");
+    hipError_t e = hipEventRecord(ev->event, lane->stream);
+    if (e != hipSuccess) return hip_fail(e, NNHIP_OP_EVENT, lane->device, "hipEventRecord");
+    return NNHIP_OK;
+}
+
+int nnhip_event_elapsed_ms(void* handle, void* start, void* stop, float* ms)
+{
+    NNHIP_LANE(handle, NNHIP_OP_EVENT)
+    Event* a = static_cast<Event*>(start);
+    Event* b = static_cast<Event*>(stop);
+    if (!a || !b || a->magic != kEventMagic || b->magic != kEventMagic || !ms)
+        return fail(NNHIP_ERR_BAD_HANDLE, NNHIP_OP_EVENT, lane->device, 0, "not an event handle, or ms is null");
+    hipError_t e = hipEventSynchronize(b->event);
+    if (e == hipSuccess) e = hipEventElapsedTime(ms, a->event, b->event);
+    if (e != hipSuccess) return hip_fail(e, NNHIP_OP_EVENT, lane->device, "hipEventElapsedTime");
+    return NNHIP_OK;
+}
+
+int nnhip_graph_begin(void* handle)
+{
+    NNHIP_LANE(handle, NNHIP_OP_GRAPH)
+    if (lane->capturing) return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_GRAPH, lane->device, 0, "a capture is already in progress");
+    hipError_t e = hipStreamBeginCapture(lane->stream, hipStreamCaptureModeThreadLocal);
+    if (e != hipSuccess) return hip_fail(e, NNHIP_OP_GRAPH, lane->device, "hipStreamBeginCapture");
+    lane->capturing = true;
+    return NNHIP_OK;
+}
+
+int nnhip_graph_end(void* handle, void** graph)
+{
+    NNHIP_LANE(handle, NNHIP_OP_GRAPH)
+    if (!lane->capturing) return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_GRAPH, lane->device, 0, "no capture in progress");
+    lane->capturing = false;
+    hipGraph_t g = nullptr;
+    hipError_t e = hipStreamEndCapture(lane->stream, &g);
+    if (e != hipSuccess) return hip_fail(e, NNHIP_OP_GRAPH, lane->device, "hipStreamEndCapture");
+    if (!graph) {
+        (void)hipGraphDestroy(g);
+        return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_GRAPH, lane->device, 0, "graph output pointer is null");
+    }
+    Graph* gr = new (std::nothrow) Graph();
+    if (!gr) {
+        (void)hipGraphDestroy(g);
+        return fail(NNHIP_ERR_OUT_OF_MEMORY, NNHIP_OP_GRAPH, lane->device, 0, "host allocation failed");
+    }
+    gr->graph = g;
+    e = hipGraphInstantiate(&gr->exec, g, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+        (void)hipGraphDestroy(g);
+        delete gr;
+        return hip_fail(e, NNHIP_OP_GRAPH, lane->device, "hipGraphInstantiate");
+    }
+    *graph = gr;
+    return NNHIP_OK;
+}
+
+int nnhip_graph_launch(void* handle, void* graph)
+{
+    NNHIP_LANE(handle, NNHIP_OP_GRAPH)
+    Graph* gr = static_cast<Graph*>(graph);
+    if (!gr || gr->magic != kGraphMagic) return fail(NNHIP_ERR_BAD_HANDLE, NNHIP_OP_GRAPH, lane->device, 0, "not a graph handle");
+    hipError_t e = hipGraphLaunch(gr->exec, lane->stream);
+    if (e != hipSuccess) return hip_fail(e, NNHIP_OP_GRAPH, lane->device, "hipGraphLaunch");
+    return NNHIP_OK;
+}
+
+int nnhip_graph_destroy(void* handle, void* graph)
+{
+    NNHIP_LANE(handle, NNHIP_OP_GRAPH)
+    Graph* gr = static_cast<Graph*>(graph);
+    if (!gr || gr->magic != kGraphMagic) return fail(NNHIP_ERR_BAD_HANDLE, NNHIP_OP_GRAPH, lane->device, 0, "not a graph handle");
+    hipError_t e = hipStreamSynchronize(lane->stream);
+    hipError_t e2 = hipGraphExecDestroy(gr->exec);
+    hipError_t e3 = hipGraphDestroy(gr->graph);
+    gr->magic = 0;
+    delete gr;
+    if (e == hipSuccess) e = e2;
+    if (e == hipSuccess) e = e3;
+    if (e != hipSuccess) return hip_fail(e, NNHIP_OP_GRAPH, lane->device, "graph teardown");
+    return NNHIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,182 @@
+"""HipExecutionLane: one device, one in-order HIP stream, and the buffers it owns.
+
+Mirrors the part of ArcExecutionLane the quantized operator uses (NNtrain.Arc/ArcExecutionLane.cs): UploadRaw :322,
+Allocate :241, AllocateBytes :271, Read :334, Synchronize :658, the byte counters :71-91 and ArcBuffer :917-931.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import byref, c_float, c_int, c_uint64, c_void_p
+
+import numpy as np
+
+from . import native
+from .native import check
+
+
+class HipBuffer:
+    """Device allocation owned by a lane (the reference's ArcBuffer).  Dispose frees it; the lane frees leaks."""
+
+    def __init__(self, lane: "HipExecutionLane", ptr: int, nbytes: int):
+        self.lane = lane
+        self.ptr = ptr
+        self.nbytes = nbytes
+
+    @property
+    def disposed(self) -> bool:
+        return self.ptr == 0
+
+    def dispose(self) -> None:
+        if self.ptr and not self.lane.disposed:
+            check(self.lane._lib.nnhip_free(self.lane._handle, c_void_p(self.ptr)), "free")
+        self.ptr = 0
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.dispose()
+
+    def _require(self) -> int:
+        if not self.ptr:
+            raise ValueError("buffer has been disposed")
+        return self.ptr
+
+
+class HipEvent:
+    def __init__(self, lane: "HipExecutionLane"):
+        self.lane = lane
+        h = c_void_p()
+        check(lane._lib.nnhip_event_create(lane._handle, byref(h)), "event_create")
+        self.handle = h
+
+    def record(self) -> "HipEvent":
+        check(self.lane._lib.nnhip_event_record(self.lane._handle, self.handle), "event_record")
+        return self
+
+    def dispose(self) -> None:
+        if self.handle:
+            check(self.lane._lib.nnhip_event_destroy(self.lane._handle, self.handle), "event_destroy")
+            self.handle = None
+
+
+class HipExecutionLane:
+    def __init__(self, device: int = 0):
+        self._lib = native.load_library()
+        h = c_void_p()
+        check(self._lib.nnhip_lane_create(device, byref(h)), "lane_create")
+        self._handle = h
+        self.device = device
+        cu, mem = c_int(), c_uint64()
+        check(self._lib.nnhip_device_info(device, byref(cu), byref(mem)), "device_info")
+        self.compute_units = cu.value
+        self.total_memory_bytes = mem.value
+
+    # ---- enumeration (ArcDevices.Enumerate) ----
+    @staticmethod
+    def device_count() -> int:
+        lib = native.load_library()
+        n = c_int()
+        check(lib.nnhip_device_count(byref(n)), "device_count")
+        return n.value
+
+    @staticmethod
+    def device_name(device: int = 0) -> str:
+        lib = native.load_library()
+        buf = ctypes.create_string_buffer(256)
+        check(lib.nnhip_device_name(device, buf, len(buf)), "device_name")
+        return buf.value.decode()
+
+    @property
+    def disposed(self) -> bool:
+        return self._handle is None
+
+    def dispose(self) -> None:
+        if self._handle is not None:
+            h, self._handle = self._handle, None
+            check(self._lib.nnhip_lane_destroy(h), "lane_destroy")
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.dispose()
+
+    # ---- memory ----
+    def allocate_bytes(self, nbytes: int) -> HipBuffer:
+        p = c_void_p()
+        check(self._lib.nnhip_alloc(self._handle, nbytes, byref(p)), "alloc")
+        return HipBuffer(self, p.value, nbytes)
+
+    def allocate(self, elements: int) -> HipBuffer:
+        """FP32 elements, as ArcExecutionLane.Allocate."""
+        return self.allocate_bytes(4 * elements)
+
+    def upload_raw(self, values) -> HipBuffer:
+        """Upload a host array byte for byte (ArcExecutionLane.UploadRaw)."""
+        a = np.ascontiguousarray(values)
+        buf = self.allocate_bytes(max(a.nbytes, 4))
+        self.write(buf, a)
+        return buf
+
+    def write(self, buf: HipBuffer, values, offset: int = 0) -> None:
+        a = np.ascontiguousarray(values)
+        if offset + a.nbytes > buf.nbytes:
+            raise ValueError("write exceeds the buffer")
+        check(self._lib.nnhip_upload(self._handle, c_void_p(buf._require()), offset, a.ctypes.data_as(c_void_p), a.nbytes),
+              "upload")
+
+    def read(self, buf: HipBuffer, dtype=np.float32, count: int | None = None, offset: int = 0) -> np.ndarray:
+        itemsize = np.dtype(dtype).itemsize
+        if count is None:
+            count = (buf.nbytes - offset) // itemsize
+        out = np.empty(count, dtype=dtype)
+        if offset + out.nbytes > buf.nbytes:
+            raise ValueError("read exceeds the buffer")
+        check(self._lib.nnhip_download(self._handle, c_void_p(buf._require()), offset, out.ctypes.data_as(c_void_p),
+                                       out.nbytes), "download")
+        return out
+
+    def copy(self, dst: HipBuffer, src: HipBuffer, nbytes: int, dst_offset: int = 0, src_offset: int = 0) -> None:
+        if dst_offset + nbytes > dst.nbytes or src_offset + nbytes > src.nbytes:
+            raise ValueError("copy exceeds a buffer")
+        check(self._lib.nnhip_copy(self._handle, c_void_p(dst._require()), dst_offset, c_void_p(src._require()), src_offset,
+                                   nbytes), "copy")
+
+    def fill_u32(self, buf: HipBuffer, value: int, count: int, offset: int = 0) -> None:
+        if offset + 4 * count > buf.nbytes:
+            raise ValueError("fill exceeds the buffer")
+        check(self._lib.nnhip_fill_u32(self._handle, c_void_p(buf._require()), offset, value & 0xFFFFFFFF, count), "fill")
+
+    def synchronize(self) -> None:
+        check(self._lib.nnhip_synchronize(self._handle), "synchronize")
+
+    # ---- counters (ArcExecutionLane.H2DBytes etc.) ----
+    def counters(self) -> dict:
+        c = native.LaneCounters()
+        check(self._lib.nnhip_lane_get_counters(self._handle, byref(c), ctypes.sizeof(c)), "counters")
+        return {"h2d_bytes": c.h2d_bytes, "d2h_bytes": c.d2h_bytes, "allocated_bytes": c.allocated_bytes,
+                "peak_allocated_bytes": c.peak_allocated_bytes, "kernel_launches": c.kernel_launches}
+
+    # ---- timing / replay ----
+    def event(self) -> HipEvent:
+        return HipEvent(self)
+
+    def elapsed_ms(self, start: HipEvent, stop: HipEvent) -> float:
+        ms = c_float()
+        check(self._lib.nnhip_event_elapsed_ms(self._handle, start.handle, stop.handle, byref(ms)), "event_elapsed")
+        return ms.value
+
+    def graph_begin(self) -> None:
+        check(self._lib.nnhip_graph_begin(self._handle), "graph_begin")
+
+    def graph_end(self):
+        g = c_void_p()
+        check(self._lib.nnhip_graph_end(self._handle, byref(g)), "graph_end")
+        return g
+
+    def graph_launch(self, graph) -> None:
+        check(self._lib.nnhip_graph_launch(self._handle, graph), "graph_launch")
+
+    def graph_destroy(self, graph) -> None:
+        check(self._lib.nnhip_graph_destroy(self._handle, graph), "graph_destroy")

@@ -1,0 +1,131 @@
+"""HipQuantizedMatrix: an immutable GGUF block-quantized matrix that stays encoded in HBM.
+
+Constructor checks, error kinds and `forward` semantics follow ArcQuantizedMatrix
+(NNtrain.Core/Serialization/ArcQuantizedMatrix.cs:16-60) and Qwen35QuantizedModel.Matrix.Forward
+(NNtrain.Core/Modules/Qwen35QuantizedModel.cs:1210-1369), extended from Q4_K/Q6_K to the five types of this path.
+Exceptions map as: NotSupportedException -> NotImplementedError, ArgumentOutOfRangeException/ArgumentException ->
+ValueError, InvalidDataException -> ValueError("... payload ...").
+"""
+from __future__ import annotations
+
+from ctypes import c_void_p
+
+import numpy as np
+
+from . import native
+from .lane import HipBuffer, HipExecutionLane
+from .native import check
+
+GGML_Q8_0, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_IQ2_S = 8, 12, 13, 14, 22
+BLOCK_ELEMS = {GGML_Q8_0: 32, GGML_Q4_K: 256, GGML_Q5_K: 256, GGML_Q6_K: 256, GGML_IQ2_S: 256}
+BLOCK_BYTES = {GGML_Q8_0: 34, GGML_Q4_K: 144, GGML_Q5_K: 176, GGML_Q6_K: 210, GGML_IQ2_S: 82}
+
+# rows at or above which forward() uses the bf16 MFMA mat-mul when asked to (Qwen35QuantizedModel.cs:1249: rows >= 16)
+PREFILL_MIN_ROWS = 16
+
+
+class HipQuantizedMatrix:
+    def __init__(self, payload, ggml_type: int, output_width: int, input_width: int):
+        if payload is None:
+            raise TypeError("payload is null")
+        if ggml_type not in BLOCK_ELEMS:
+            raise NotImplementedError(f"GGML type {ggml_type} is not a supported quantized matrix type.")
+        if output_width <= 0 or input_width <= 0:
+            raise ValueError("outputWidth and inputWidth must be positive.")
+        elems = BLOCK_ELEMS[ggml_type]
+        if input_width % elems != 0:
+            raise NotImplementedError(f"Quantized rows must contain complete {elems}-value blocks.")
+        data = np.ascontiguousarray(np.frombuffer(payload, dtype=np.uint8) if isinstance(payload, (bytes, bytearray, memoryview))
+                                    else payload)
+        if data.dtype != np.uint8:
+            raise TypeError("payload must be raw bytes")
+        expected = output_width * (input_width // elems) * BLOCK_BYTES[ggml_type]
+        if data.size != expected:
+            raise ValueError(f"Quantized matrix payload has {data.size} bytes; expected {expected}.")
+        self._payload = data
+        self.ggml_type = ggml_type
+        self.output_width = output_width
+        self.input_width = input_width
+        self._lane: HipExecutionLane | None = None
+        self._device_payload: HipBuffer | None = None
+
+    @property
+    def storage_bytes(self) -> int:
+        return int(self._payload.size) if self._payload is not None else self._storage_bytes
+
+    def device_payload(self, lane: HipExecutionLane) -> HipBuffer:
+        """Lazy one-time upload of the raw blocks (ArcQuantizedMatrix.DevicePayload, :80-88)."""
+        if self._device_payload is not None and self._lane is lane:
+            return self._device_payload
+        if self._payload is None:
+            raise ValueError("host payload was dropped; the matrix is bound to its first lane")
+        if self._device_payload is not None:
+            self._device_payload.dispose()
+        self._device_payload = lane.upload_raw(self._payload)
+        self._lane = lane
+        return self._device_payload
+
+    def drop_host_payload(self) -> None:
+        """Keep only the device copy, as Qwen35QuantizedModel.LoadTensor does (Qwen35QuantizedModel.cs:239-241)."""
+        if self._device_payload is None:
+            raise ValueError("upload first")
+        self._storage_bytes = int(self._payload.size)
+        self._payload = None
+
+    def forward(self, lane: HipExecutionLane, x: HipBuffer, bias: HipBuffer | None, rows: int = 1,
+                out: HipBuffer | None = None) -> HipBuffer:
+        """y[rows, out] = bias + x[rows, in] . W^T on the device; x is FP32.  The caller disposes the result."""
+        if rows < 1:
+            raise ValueError("rows must be positive.")
+        if x.nbytes < 4 * rows * self.input_width:
+            raise ValueError("Quantized linear input width mismatch.")
+        if bias is not None and bias.nbytes < 4 * self.output_width:
+            raise ValueError("Quantized linear bias width mismatch.")
+        w = self.device_payload(lane)
+        y = out if out is not None else lane.allocate(rows * self.output_width)
+        if y.nbytes < 4 * rows * self.output_width:
+            raise ValueError("output buffer too small")
+        check(lane._lib.nnhip_quant_matvec(lane._handle, self.ggml_type, c_void_p(x._require()), c_void_p(w._require()),
+                                           c_void_p(bias._require()) if bias is not None else None,
+                                           c_void_p(y._require()), rows, self.input_width, self.output_width), "quant_matvec")
+        return y
+
+    def forward_bf16(self, lane: HipExecutionLane, x_bf16: HipBuffer, bias: HipBuffer | None, rows: int,
+                     out: HipBuffer | None = None) -> HipBuffer:
+        """Prefill: x holds bfloat16 bit patterns [rows, in]; bf16 MFMA with FP32 accumulation."""
+        if rows < 1:
+            raise ValueError("rows must be positive.")
+        if x_bf16.nbytes < 2 * rows * self.input_width:
+            raise ValueError("Quantized linear input width mismatch.")
+        if bias is not None and bias.nbytes < 4 * self.output_width:
+            raise ValueError("Quantized linear bias width mismatch.")
+        w = self.device_payload(lane)
+        y = out if out is not None else lane.allocate(rows * self.output_width)
+        check(lane._lib.nnhip_quant_matmul_bf16(lane._handle, self.ggml_type, c_void_p(x_bf16._require()),
+                                                c_void_p(w._require()),
+                                                c_void_p(bias._require()) if bias is not None else None,
+                                                c_void_p(y._require()), rows, self.input_width, self.output_width),
+              "quant_matmul_bf16")
+        return y
+
+    def dequantize(self, lane: HipExecutionLane, row: int | None = None) -> HipBuffer:
+        """Decode the whole matrix, or one row (the embedding lookup of Matrix.Embedding,
+        Qwen35QuantizedModel.cs:1497-1521), to FP32 on the device."""
+        w = self.device_payload(lane)
+        row_bytes = self.input_width // BLOCK_ELEMS[self.ggml_type] * BLOCK_BYTES[self.ggml_type]
+        if row is None:
+            elements, offset = self.output_width * self.input_width, 0
+        else:
+            if not 0 <= row < self.output_width:
+                raise IndexError(f"Embedding index {row} is outside the vocabulary.")
+            elements, offset = self.input_width, row * row_bytes
+        out = lane.allocate(elements)
+        check(lane._lib.nnhip_dequantize(lane._handle, self.ggml_type, c_void_p(w._require() + offset),
+                                         c_void_p(out._require()), elements), "dequantize")
+        return out
+
+    def dispose(self) -> None:
+        if self._device_payload is not None:
+            self._device_payload.dispose()
+        self._device_payload = None
+        self._lane = None

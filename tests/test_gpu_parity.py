@@ -1,0 +1,265 @@
+"""GPU parity: the HIP path (through the C ABI) against the CPU oracle and the reference's golden vectors.
+
+Bars: dequantized weights bit-exact (+0/-0 equal); mat-vec relative L2 <= 1e-5 against the float64 oracle, plus the
+reference's per-element bound 2e-6 + 3e-6 * sum|x*w| (NNtrain.Core.Tests/Qwen35GpuLinearTests.cs:66-84).
+"""
+import base64
+import json
+
+import numpy as np
+import pytest
+
+import oracle
+from nntrain_amd import (BLOCK_BYTES, BLOCK_ELEMS, GGML_IQ2_S, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_Q8_0, GgufReader,
+                         HipExecutionLane, HipQuantizedMatrix, NnHipError, synth)
+
+pytestmark = pytest.mark.gpu
+
+ALL_TYPES = [GGML_Q8_0, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_IQ2_S]
+NAN_BITS = 0x7FC00000
+REL_L2_BAR = 1e-5
+
+
+@pytest.fixture(scope="module")
+def lane():
+    with HipExecutionLane(0) as ln:
+        yield ln
+
+
+def _bits(a):
+    return np.ascontiguousarray(a, dtype=np.float32).view(np.uint32)
+
+
+def _same_mod_zero(a, b):
+    return bool(np.all((_bits(a) == _bits(b)) | ((a == 0) & (b == 0))))
+
+
+def _random_payload(typ, out_w, in_w, seed):
+    if typ == GGML_Q8_0:
+        rng = np.random.default_rng(seed)
+        w = rng.standard_normal((out_w, in_w), dtype=np.float32) * np.float32(0.02)
+        return synth.quantize_q8_0(w)
+    return synth.k_quant_matrix(typ, out_w, in_w, seed)
+
+
+def _run_matvec(lane, typ, payload, x, bias, rows, in_w, out_w):
+    """Returns y[rows, out_w]; checks NaN guards past the output and that the launch moved no bytes."""
+    mat = HipQuantizedMatrix(payload, typ, out_w, in_w)
+    mat.device_payload(lane)
+    xb = lane.upload_raw(np.ascontiguousarray(x, np.float32))
+    bb = lane.upload_raw(np.ascontiguousarray(bias, np.float32)) if bias is not None else None
+    yb = lane.allocate(rows * out_w + 2)
+    lane.fill_u32(yb, NAN_BITS, rows * out_w + 2)
+    lane.synchronize()
+    before = lane.counters()
+    mat.forward(lane, xb, bb, rows, out=yb)
+    lane.synchronize()
+    after = lane.counters()
+    assert after["h2d_bytes"] == before["h2d_bytes"] and after["d2h_bytes"] == before["d2h_bytes"]
+    assert after["allocated_bytes"] == before["allocated_bytes"]
+    y = lane.read(yb)
+    assert np.isnan(y[-1]) and np.isnan(y[-2]), "guard elements past the output were overwritten"
+    for b in (xb, bb, yb):
+        if b is not None:
+            b.dispose()
+    mat.dispose()
+    assert np.all(np.isfinite(y[:-2]))
+    return y[:-2].reshape(rows, out_w)
+
+
+def _check_against_f64(y, ref, asum):
+    assert oracle.rel_l2(y, ref) <= REL_L2_BAR
+    assert np.all(np.abs(y.astype(np.float64) - ref) <= 2e-6 + 3e-6 * asum)
+
+
+# ----------------------------------------------------------------------------------------------- dequantize
+
+def test_dequantize_q4k_q6k_bit_exact_vs_gguf_py(lane, golden_dir):
+    expected = json.loads((golden_dir / "qwen_gguf_expected.json").read_text())
+    with GgufReader(str(golden_dir / "qwen_gguf_reference.gguf")) as reader:
+        seen = 0
+        for t in expected["tensors"]:
+            if t["type"] not in (GGML_Q4_K, GGML_Q6_K):
+                continue
+            info = reader.get_tensor(t["name"])
+            in_w, out_w = reader.matrix_dims(info)
+            mat = HipQuantizedMatrix(reader.read_tensor_bytes(info), info.type, out_w, in_w)
+            got = lane.read(mat.dequantize(lane))
+            want = np.frombuffer(base64.b64decode(t["decodedFloat32Base64"]), "<f4")
+            assert np.array_equal(_bits(got), _bits(want)), t["name"]
+            row = lane.read(mat.dequantize(lane, row=out_w - 1))
+            assert np.array_equal(_bits(row), _bits(want[-in_w:]))
+            mat.dispose()
+            seen += 1
+        assert seen == 4
+
+
+@pytest.mark.parametrize("typ", [GGML_Q5_K, GGML_IQ2_S])
+def test_dequantize_bit_exact_vs_native_ggml_blocks(lane, golden_dir, typ):
+    cases = [c for c in json.loads((golden_dir / "iq_quant_blocks.json").read_text())["cases"] if c["type"] == typ]
+    assert len(cases) == {GGML_Q5_K: 25, GGML_IQ2_S: 69}[typ]
+    raw = np.concatenate([np.frombuffer(base64.b64decode(c["encoded"]), np.uint8) for c in cases])
+    want = np.concatenate([np.frombuffer(base64.b64decode(c["decodedFloat32Base64"]), "<f4") for c in cases])
+    mat = HipQuantizedMatrix(raw, typ, len(cases), 256)
+    got = lane.read(mat.dequantize(lane))
+    mat.dispose()
+    for i, c in enumerate(cases):
+        assert _same_mod_zero(got[256 * i:256 * i + 256], want[256 * i:256 * i + 256]), c["id"]
+
+
+@pytest.mark.parametrize("typ", ALL_TYPES)
+def test_dequantize_bit_exact_vs_oracle_random_blocks(lane, typ):
+    rng = np.random.default_rng(500 + typ)
+    n_blocks = 4096 + 7
+    raw = rng.integers(0, 256, size=(n_blocks, BLOCK_BYTES[typ]), dtype=np.uint8)
+    for off in ((0, 2) if typ in (GGML_Q4_K, GGML_Q5_K) else (208,) if typ == GGML_Q6_K else (0,)):
+        raw[:, off + 1] &= 0x7B          # keep fp16 scales finite (any sign, normal and subnormal)
+    raw[:64, 0 if typ != GGML_Q6_K else 208] = rng.integers(0, 256, 64)
+    raw[:64, 1 if typ != GGML_Q6_K else 209] &= 0x83  # subnormal-only scales in the first blocks
+    mat = HipQuantizedMatrix(raw.reshape(-1), typ, n_blocks, BLOCK_ELEMS[typ])
+    got = lane.read(mat.dequantize(lane))
+    mat.dispose()
+    want = oracle.dequantize(typ, raw.reshape(-1))
+    assert np.array_equal(_bits(got), _bits(want))
+
+
+def test_dequantize_rejects_bad_arguments(lane):
+    buf = lane.allocate(256)
+    from ctypes import c_void_p
+    lib, h = lane._lib, lane._handle
+    assert lib.nnhip_dequantize(h, 99, c_void_p(buf.ptr), c_void_p(buf.ptr), 256) == 2     # unsupported type
+    assert lib.nnhip_dequantize(h, GGML_Q4_K, c_void_p(buf.ptr), c_void_p(buf.ptr), 255) == 3  # incomplete block
+    assert lib.nnhip_dequantize(h, GGML_Q4_K, None, c_void_p(buf.ptr), 256) == 1
+    assert lib.nnhip_dequantize(h, GGML_Q4_K, c_void_p(buf.ptr), c_void_p(buf.ptr), 0) == 0
+    buf.dispose()
+
+
+# ----------------------------------------------------------------------------------------------- mat-vec
+
+def test_matvec_reference_float64_vectors(lane, golden_dir):
+    """Rows 1/3/5, K=512, N=7, with bias; tolerance of QwenGgufIndependentReferenceTests.cs:76-97."""
+    expected = json.loads((golden_dir / "qwen_gguf_expected.json").read_text())
+    K, N = expected["inputWidth"], expected["outputWidth"]
+    x_all = np.frombuffer(base64.b64decode(expected["inputFloat32Base64"]), "<f4").reshape(expected["inputRows"], K)
+    with GgufReader(str(golden_dir / "qwen_gguf_reference.gguf")) as reader:
+        for t in expected["tensors"]:
+            if t["type"] not in (GGML_Q4_K, GGML_Q6_K):
+                continue
+            payload = np.frombuffer(reader.read_tensor_bytes(reader.get_tensor(t["name"])), np.uint8)
+            bias = np.frombuffer(base64.b64decode(t["biasFloat32Base64"]), "<f4")
+            want = np.frombuffer(base64.b64decode(t["linearFloat64Base64"]), "<f8").reshape(-1, N)
+            rows = want.shape[0]
+            for r in (1, 3, rows):
+                y = _run_matvec(lane, t["type"], payload, x_all[:r], bias, r, K, N)
+                bound = np.max(np.abs(want[:r])) * 5e-6 + 1e-9
+                assert np.max(np.abs(y - want[:r])) <= bound, (t["name"], r)
+
+
+@pytest.mark.parametrize("typ", ALL_TYPES)
+@pytest.mark.parametrize("in_w,out_w", [(256, 1), (512, 7), (1024, 67), (5120, 131), (17408, 33)])
+def test_matvec_vs_oracle_shapes(lane, typ, in_w, out_w):
+    payload = _random_payload(typ, out_w, in_w, seed=1000 * typ + in_w + out_w)
+    x = synth.activations(1, in_w, seed=7 + in_w)
+    bias = np.random.default_rng(3).standard_normal(out_w).astype(np.float32)
+    y = _run_matvec(lane, typ, payload, x, bias, 1, in_w, out_w)
+    ref, asum = oracle.linear_f64(typ, payload, x, bias, 1, in_w, out_w)
+    _check_against_f64(y, ref, asum)
+    # FP32 sequential CPU statement of the operator agrees to the same bar
+    assert oracle.rel_l2(oracle.cpu_linear(typ, payload, x, bias, 1, in_w, out_w), y) <= REL_L2_BAR
+
+
+@pytest.mark.parametrize("typ", ALL_TYPES)
+def test_matvec_rows_equal_stacked_single_rows_bitwise(lane, typ):
+    in_w, out_w, rows = 1024, 45, 5
+    payload = _random_payload(typ, out_w, in_w, seed=42 + typ)
+    x = synth.activations(rows, in_w, seed=9)
+    y = _run_matvec(lane, typ, payload, x, None, rows, in_w, out_w)
+    for r in range(rows):
+        y1 = _run_matvec(lane, typ, payload, x[r:r + 1], None, 1, in_w, out_w)
+        assert np.array_equal(_bits(y[r]), _bits(y1[0]))
+    ref, asum = oracle.linear_f64(typ, payload, x, None, rows, in_w, out_w)
+    _check_against_f64(y, ref, asum)
+
+
+def test_matvec_q8_0_odd_block_count_rows(lane):
+    in_w, out_w = 32 * 5, 19
+    payload = _random_payload(GGML_Q8_0, out_w, in_w, seed=77)
+    x = synth.activations(2, in_w, seed=78)
+    y = _run_matvec(lane, GGML_Q8_0, payload, x, None, 2, in_w, out_w)
+    ref, asum = oracle.linear_f64(GGML_Q8_0, payload, x, None, 2, in_w, out_w)
+    _check_against_f64(y, ref, asum)
+
+
+@pytest.mark.parametrize("typ", [GGML_Q4_K, GGML_Q6_K])
+def test_matvec_subnormal_only_scales_zero_bias(lane, typ):
+    """All fp16 scales subnormal (QwenQuantizedLinearFastTests.cs:99-123): lost subnormals would zero the output."""
+    in_w, out_w = 512, 9
+    rng = np.random.default_rng(typ)
+    raw = rng.integers(0, 256, size=(out_w * 2, BLOCK_BYTES[typ]), dtype=np.uint8)
+    for off in ((0, 2) if typ == GGML_Q4_K else (208,)):
+        raw[:, off + 1] &= 0x03
+        raw[:, off] |= 0x01
+    x = synth.activations(1, in_w, seed=5)
+    y = _run_matvec(lane, typ, raw.reshape(-1), x, None, 1, in_w, out_w)
+    ref, asum = oracle.linear_f64(typ, raw.reshape(-1), x, None, 1, in_w, out_w)
+    assert np.all(ref != 0)
+    _check_against_f64(y, ref, asum)
+
+
+def test_matvec_linearity_and_one_hot(lane):
+    typ, in_w, out_w = GGML_Q5_K, 768, 21
+    payload = _random_payload(typ, out_w, in_w, seed=8)
+    e = np.zeros((1, in_w), np.float32)
+    e[0, 517] = 1.0
+    y = _run_matvec(lane, typ, payload, e, None, 1, in_w, out_w)
+    w = oracle.dequantize(typ, payload).reshape(out_w, in_w)
+    assert np.array_equal(_bits(y[0]), _bits(w[:, 517]))     # a one-hot activation reads one weight column exactly
+    x = synth.activations(1, in_w, seed=1)
+    y1 = _run_matvec(lane, typ, payload, x, None, 1, in_w, out_w)
+    y2 = _run_matvec(lane, typ, payload, 2 * x, None, 1, in_w, out_w)
+    assert np.array_equal(_bits(2 * y1), _bits(y2))           # scaling by 2 is exact in binary FP
+
+
+def test_operator_argument_errors(lane):
+    with pytest.raises(NotImplementedError):
+        HipQuantizedMatrix(np.zeros(144, np.uint8), 2, 1, 256)
+    with pytest.raises(NotImplementedError):
+        HipQuantizedMatrix(np.zeros(144, np.uint8), GGML_Q4_K, 1, 255)
+    with pytest.raises(ValueError):
+        HipQuantizedMatrix(np.zeros(143, np.uint8), GGML_Q4_K, 1, 256)
+    mat = HipQuantizedMatrix(np.zeros(144, np.uint8), GGML_Q4_K, 1, 256)
+    x = lane.allocate(128)
+    with pytest.raises(ValueError):
+        mat.forward(lane, x, None)
+    x.dispose()
+    from ctypes import c_void_p
+    buf = lane.allocate(1024)
+    rc = lane._lib.nnhip_quant_matvec(lane._handle, GGML_Q4_K, c_void_p(buf.ptr), c_void_p(buf.ptr), None, c_void_p(buf.ptr),
+                                      0, 256, 1)
+    assert rc == 1
+    with pytest.raises(NnHipError):
+        from nntrain_amd.native import check
+        check(rc, "quant_matvec")
+    buf.dispose()
+    mat.dispose()
+
+
+# ----------------------------------------------------------------------------------------------- full-size configs
+
+FULL = [
+    ("cfg1_q8_0", GGML_Q8_0, 5376, 21504, 1001, 1002),
+    ("cfg2_q4_k", GGML_Q4_K, 5120, 17408, 2001, 2000),
+    ("cfg2_q5_k", GGML_Q5_K, 5120, 17408, 2002, 2000),
+    ("cfg2_q6_k", GGML_Q6_K, 5120, 17408, 2003, 2000),
+    ("cfg5_iq2_s", GGML_IQ2_S, 17408, 5120, 5001, 5002),
+]
+
+
+@pytest.mark.parametrize("name,typ,in_w,out_w,wseed,xseed", FULL, ids=[f[0] for f in FULL])
+def test_matvec_full_size_configs(lane, name, typ, in_w, out_w, wseed, xseed):
+    payload = synth.matrix(typ, out_w, in_w, wseed)
+    x = synth.activations(1, in_w, xseed)
+    y = _run_matvec(lane, typ, payload, x, None, 1, in_w, out_w)
+    ref, asum = oracle.linear_f64(typ, payload, x, None, 1, in_w, out_w)
+    _check_against_f64(y, ref, asum)
+    print(f"{name}: rel_l2 vs f64 = {oracle.rel_l2(y, ref):.3e}")
