@@ -3,17 +3,19 @@
 // y[r, o] = bias[o] + sum_k x[r, k] * w[o, k]     (NNtrain.Arc/Kernels/qwen.cl:374-406 defines the operator)
 //
 // Work decomposition (the same for every block format):
-//   * a row of the matrix is cut into "units" of 64 consecutive weights (two Q8_0 blocks, a quarter of a
-//     256-weight super-block); a unit is the work of one lane: it loads the unit's bytes with 128-bit loads,
-//     unpacks scales / nibbles in registers and produces one FP32 partial dot product;
-//   * a workgroup owns a contiguous range of output rows and walks the (row, unit) pairs of that range as ONE flat
-//     index space, 1024 lanes at a time, so consecutive lanes read consecutive memory across row ends and no lane
-//     idles when units-per-row is not a multiple of 64;
-//   * the activation vector is staged once per workgroup in LDS as float4 pieces, transposed so that the 64 lanes of
-//     a wave read 64 consecutive pieces with every ds_read_b128 (piece k/4 lives at [(k/4)%16][k/64]);
-//   * unit partials go to LDS as part[row][unit]; after one barrier each row is summed in a fixed order
-//     (lane-strided, then a DPP butterfly).  The order depends only on in_w, never on the launch geometry, so the
-//     result for a row is bit-identical for any `rows`, out_w or batch composition.
+//   * a row of the matrix is cut into "units" of 64 weights (two Q8_0 blocks, a quarter of a 256-weight
+//     super-block); a unit is the work of one lane: it loads the unit's bytes with 128-bit loads, unpacks scales and
+//     nibbles in registers and produces one FP32 partial dot product;
+//   * a workgroup of T lanes walks the matrix in "row steps" of RS = floor(T / units_per_row) whole rows: lane t always
+//     owns unit t % units_per_row of row t / units_per_row of the step.  Because every step starts on a row boundary
+//     a lane meets the same 64 activations in every step, so it loads them ONCE into registers (with their block
+//     sums; staged through LDS so the workgroup fetches the vector once) and never recomputes an index for them;
+//   * consecutive steps of a workgroup are gridDim.x steps apart (grid-stride), so at any moment all workgroups read
+//     one contiguous window of the weight stream, and consecutive lanes read consecutive memory across row ends;
+//   * the weight loads of the next DEPTH-1 steps are in flight while a step is reduced (rotating register sets);
+//   * unit partials go to LDS (one float per lane, double buffered); after the step's barrier one wave per row adds
+//     the row's partials in a fixed order (lane-strided, then a DPP butterfly) and stores y.  The order depends only
+//     on in_w, never on the launch geometry, so a row's result is bit-identical for any `rows`, out_w or batching.
 #include "nnhip_internal.h"
 #include "quant_device.h"
 
@@ -25,9 +27,9 @@ namespace {
 
 __device__ const uint64_t g_iq2s_grid[1024] = { NNHIP_IQ2S_GRID_VALUES };
 
-constexpr int kWG = 1024;          // lanes per workgroup (16 waves: 4 per SIMD)
+constexpr int kMaxWG = 1024;       // lanes per workgroup (16 waves: 4 per SIMD)
 constexpr int kUnitW = 64;         // weights per lane-unit
-constexpr int kMaxLds = 160 * 1024;
+constexpr int kMaxDynamicLds = 140 * 1024;   // staged activations; 16 KB of the 160 KB stay for the static arrays
 
 struct MatvecArgs {
     const float* x;
@@ -37,21 +39,11 @@ struct MatvecArgs {
     int in_w;
     int out_w;
     int units_per_row;     // in_w / 64
-    int cpad;              // odd stride (in float4 pieces) between the 16 piece-planes of the staged x
-    int rows_per_wg;
+    int rows_per_step;     // RS
+    int steps;             // ceil(out_w / RS)
     uint32_t row_bytes;
-    uint32_t magic;        // ceil(2^32 / units_per_row): u / units_per_row == umulhi(u, magic) for u < 2^32 / upr
+    uint32_t magic;        // ceil(2^32 / units_per_row): t / units_per_row == umulhi(t, magic) for t < 2^32 / upr
 };
-
-// LDS view shared by the unit functions.
-struct Staged {
-    const float4* xp;      // transposed activation pieces
-    const float* xs;       // per-type block sums of x (32-wide for Q4_K/Q5_K, 16-wide for Q6_K), or nullptr
-    const uint64_t* grid;  // IQ2_S codebook copy, or nullptr
-    int cpad;
-};
-
-__device__ __forceinline__ float4 xpiece(const Staged& s, int chunk, int q) { return s.xp[q * s.cpad + chunk]; }
 
 __device__ __forceinline__ float dot4s(uint32_t v, const float4 x, float acc)  // 4 signed bytes . x
 {
@@ -71,67 +63,122 @@ __device__ __forceinline__ float dot4u(uint32_t v, const float4 x, float acc)  /
     return acc;
 }
 
+__device__ __forceinline__ float sum4(const float4 v) { return (v.x + v.y) + (v.z + v.w); }
+
+// 64 consecutive activations of unit c, as 16 float4 pieces.
+struct XChunk {
+    float4 p[16];
+};
+
+// The staged activation vector: float4 pieces in natural order with one padding piece after every 16 (a 64-value
+// chunk occupies 272 bytes), so lanes that read consecutive chunks hit different LDS banks.
+constexpr int kChunkPieces = 17;
+
+__device__ __forceinline__ XChunk load_chunk(const float4* xs, int c)
+{
+    XChunk r;
+    const float4* src = xs + c * kChunkPieces;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) r.p[i] = src[i];
+    return r;
+}
+
 // ---------------------------------------------------------------------------------------------------- Q8_0
 // Unit = two consecutive 34-byte blocks (68 bytes, 4-byte aligned because a row holds an even number of blocks).
 struct Q8_0Unit {
-    static constexpr int kXsWidth = 0;
     static constexpr bool kGrid = false;
-    static constexpr int kUnitBytes = 68;
+    struct X { XChunk c; };
+    struct Regs { u32x4 a, b, c, d; uint32_t e; };
 
-    static __device__ __forceinline__ float dot(const uint8_t* row, int unit, const Staged& s)
+    static __device__ __forceinline__ X load_x(const float4* x, int unit)
+    {
+        X r;
+        r.c = load_chunk(x, unit);
+        return r;
+    }
+
+    static __device__ __forceinline__ Regs load(const uint8_t* row, int unit)
     {
         const uint8_t* p = row + static_cast<uint32_t>(unit) * 68u;
-        const u32x4 a = ld128(p), b = ld128(p + 16), c = ld128(p + 32), d = ld128(p + 48);
-        const uint32_t e = ld32(p + 64);
-        const uint32_t w[17] = {a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3], c[0], c[1], c[2], c[3],
-                                d[0], d[1], d[2], d[3], e};
+        Regs r;
+        r.a = ld128(p); r.b = ld128(p + 16); r.c = ld128(p + 32); r.d = ld128(p + 48);
+        r.e = ld32(p + 64);
+        return r;
+    }
+
+    static __device__ __forceinline__ float dot(const Regs& r, const X& x, int, const uint64_t*)
+    {
+        const uint32_t w[17] = {r.a[0], r.a[1], r.a[2], r.a[3], r.b[0], r.b[1], r.b[2], r.b[3], r.c[0], r.c[1], r.c[2],
+                                r.c[3], r.d[0], r.d[1], r.d[2], r.d[3], r.e};
         const float d0 = half_bits_to_float(w[0]);
         const float d1 = half_bits_to_float(w[8] >> 16);
         float acc0 = 0.0f, acc1 = 0.0f;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const uint32_t q = __builtin_amdgcn_alignbyte(w[i + 1], w[i], 2);  // quants of block 0 start at byte 2
-            acc0 = dot4s(q, xpiece(s, unit, i), acc0);
+            acc0 = dot4s(q, x.c.p[i], acc0);
         }
 #pragma unroll
-        for (int i = 0; i < 8; ++i) acc1 = dot4s(w[9 + i], xpiece(s, unit, 8 + i), acc1);
+        for (int i = 0; i < 8; ++i) acc1 = dot4s(w[9 + i], x.c.p[8 + i], acc1);
         return fmaf(d1, acc1, d0 * acc0);
     }
 };
 
 // ---------------------------------------------------------------------------------------------------- Q4_K
 // Unit j of a super-block = sub-blocks 2j (low nibbles) and 2j+1 (high nibbles) of qs[32j .. 32j+31].
-// sum_k x (s*q - m) = s * sum(q x) - m * sum(x); the 32-wide sums of x are staged once per workgroup.
+// sum_k x (s*q - m) = s * sum(q x) - m * sum(x); the two 32-wide sums of x are taken once per lane.
 struct Q4KUnit {
-    static constexpr int kXsWidth = 32;
     static constexpr bool kGrid = false;
+    struct X { XChunk c; float xs_lo, xs_hi; };
+    struct Regs { u32x4 h, qa, qb; };
 
-    static __device__ __forceinline__ float dot(const uint8_t* row, int unit, const Staged& s)
+    static __device__ __forceinline__ X load_x(const float4* x, int unit)
+    {
+        X r;
+        r.c = load_chunk(x, unit);
+        float lo = 0.0f, hi = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            lo += sum4(r.c.p[i]);
+            hi += sum4(r.c.p[8 + i]);
+        }
+        r.xs_lo = lo;
+        r.xs_hi = hi;
+        return r;
+    }
+
+    static __device__ __forceinline__ Regs load(const uint8_t* row, int unit)
     {
         const int sb = unit >> 2, j = unit & 3;
         const uint8_t* blk = row + static_cast<uint32_t>(sb) * 144u;
-        const u32x4 h = *reinterpret_cast<const u32x4*>(blk);
-        const u32x4 qa = *reinterpret_cast<const u32x4*>(blk + 16 + 32 * j);
-        const u32x4 qb = *reinterpret_cast<const u32x4*>(blk + 32 + 32 * j);
-        const float d = half_bits_to_float(h[0]), dmin = half_bits_to_float(h[0] >> 16);
+        Regs r;
+        r.h = *reinterpret_cast<const u32x4*>(blk);
+        r.qa = *reinterpret_cast<const u32x4*>(blk + 16 + 32 * j);
+        r.qb = *reinterpret_cast<const u32x4*>(blk + 32 + 32 * j);
+        return r;
+    }
+
+    static __device__ __forceinline__ float dot(const Regs& r, const X& x, int unit, const uint64_t*)
+    {
+        const int j = unit & 3;
+        const float d = half_bits_to_float(r.h[0]), dmin = half_bits_to_float(r.h[0] >> 16);
         uint32_t sc, mn;
-        k4_scale_pair(h[1], h[2], h[3], j, sc, mn);
-        const uint32_t q[8] = {qa[0], qa[1], qa[2], qa[3], qb[0], qb[1], qb[2], qb[3]};
+        k4_scale_pair(r.h[1], r.h[2], r.h[3], j, sc, mn);
+        const uint32_t q[8] = {r.qa[0], r.qa[1], r.qa[2], r.qa[3], r.qb[0], r.qb[1], r.qb[2], r.qb[3]};
         float lo = 0.0f, hi = 0.0f;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const uint32_t l4 = opaque(q[i] & 0x0f0f0f0fu);
             const uint32_t h4 = opaque(q[i] & 0xf0f0f0f0u);   // 16 * high nibble; the 1/16 is folded into the scale
-            lo = dot4u(l4, xpiece(s, unit, i), lo);
-            hi = dot4u(h4, xpiece(s, unit, 8 + i), hi);
+            lo = dot4u(l4, x.c.p[i], lo);
+            hi = dot4u(h4, x.c.p[8 + i], hi);
         }
         const float s_lo = d * ubyte0(sc), s_hi = d * ubyte1(sc) * 0.0625f;
         const float m_lo = dmin * ubyte0(mn), m_hi = dmin * ubyte1(mn);
-        const float xs_lo = s.xs[2 * unit], xs_hi = s.xs[2 * unit + 1];
         float acc = s_lo * lo;
         acc = fmaf(s_hi, hi, acc);
-        acc = fmaf(-m_lo, xs_lo, acc);
-        acc = fmaf(-m_hi, xs_hi, acc);
+        acc = fmaf(-m_lo, x.xs_lo, acc);
+        acc = fmaf(-m_hi, x.xs_hi, acc);
         return acc;
     }
 };
@@ -139,39 +186,48 @@ struct Q4KUnit {
 // ---------------------------------------------------------------------------------------------------- Q5_K
 // As Q4_K plus one high bit per weight: bit g of qh[i] belongs to element i of sub-block g.
 struct Q5KUnit {
-    static constexpr int kXsWidth = 32;
     static constexpr bool kGrid = false;
+    using X = Q4KUnit::X;
+    struct Regs { u32x4 h, ha, hb, qa, qb; };
 
-    static __device__ __forceinline__ float dot(const uint8_t* row, int unit, const Staged& s)
+    static __device__ __forceinline__ X load_x(const float4* x, int unit) { return Q4KUnit::load_x(x, unit); }
+
+    static __device__ __forceinline__ Regs load(const uint8_t* row, int unit)
     {
         const int sb = unit >> 2, j = unit & 3;
         const uint8_t* blk = row + static_cast<uint32_t>(sb) * 176u;
-        const u32x4 h = *reinterpret_cast<const u32x4*>(blk);
-        const u32x4 ha = *reinterpret_cast<const u32x4*>(blk + 16);
-        const u32x4 hb = *reinterpret_cast<const u32x4*>(blk + 32);
-        const u32x4 qa = *reinterpret_cast<const u32x4*>(blk + 48 + 32 * j);
-        const u32x4 qb = *reinterpret_cast<const u32x4*>(blk + 64 + 32 * j);
-        const float d = half_bits_to_float(h[0]), dmin = half_bits_to_float(h[0] >> 16);
+        Regs r;
+        r.h = *reinterpret_cast<const u32x4*>(blk);
+        r.ha = *reinterpret_cast<const u32x4*>(blk + 16);
+        r.hb = *reinterpret_cast<const u32x4*>(blk + 32);
+        r.qa = *reinterpret_cast<const u32x4*>(blk + 48 + 32 * j);
+        r.qb = *reinterpret_cast<const u32x4*>(blk + 64 + 32 * j);
+        return r;
+    }
+
+    static __device__ __forceinline__ float dot(const Regs& r, const X& x, int unit, const uint64_t*)
+    {
+        const int j = unit & 3;
+        const float d = half_bits_to_float(r.h[0]), dmin = half_bits_to_float(r.h[0] >> 16);
         uint32_t sc, mn;
-        k4_scale_pair(h[1], h[2], h[3], j, sc, mn);
-        const uint32_t q[8] = {qa[0], qa[1], qa[2], qa[3], qb[0], qb[1], qb[2], qb[3]};
-        const uint32_t hq[8] = {ha[0], ha[1], ha[2], ha[3], hb[0], hb[1], hb[2], hb[3]};
+        k4_scale_pair(r.h[1], r.h[2], r.h[3], j, sc, mn);
+        const uint32_t q[8] = {r.qa[0], r.qa[1], r.qa[2], r.qa[3], r.qb[0], r.qb[1], r.qb[2], r.qb[3]};
+        const uint32_t hq[8] = {r.ha[0], r.ha[1], r.ha[2], r.ha[3], r.hb[0], r.hb[1], r.hb[2], r.hb[3]};
         float lo = 0.0f, hi = 0.0f;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const uint32_t hb2 = hq[i] >> (2 * j);                       // bit 0: sub-block 2j, bit 1: sub-block 2j+1
             const uint32_t l5 = opaque((q[i] & 0x0f0f0f0fu) | ((hb2 << 4) & 0x10101010u));
             const uint32_t h5 = opaque(((q[i] >> 4) & 0x0f0f0f0fu) | ((hb2 << 3) & 0x10101010u));
-            lo = dot4u(l5, xpiece(s, unit, i), lo);
-            hi = dot4u(h5, xpiece(s, unit, 8 + i), hi);
+            lo = dot4u(l5, x.c.p[i], lo);
+            hi = dot4u(h5, x.c.p[8 + i], hi);
         }
         const float s_lo = d * ubyte0(sc), s_hi = d * ubyte1(sc);
         const float m_lo = dmin * ubyte0(mn), m_hi = dmin * ubyte1(mn);
-        const float xs_lo = s.xs[2 * unit], xs_hi = s.xs[2 * unit + 1];
         float acc = s_lo * lo;
         acc = fmaf(s_hi, hi, acc);
-        acc = fmaf(-m_lo, xs_lo, acc);
-        acc = fmaf(-m_hi, xs_hi, acc);
+        acc = fmaf(-m_lo, x.xs_lo, acc);
+        acc = fmaf(-m_hi, x.xs_hi, acc);
         return acc;
     }
 };
@@ -180,40 +236,66 @@ struct Q5KUnit {
 // Unit (sb, half h, part p): elements 128h + 32e + 16p + i, i < 16, e < 4 - the four 16-runs that share
 // ql[64h+16p ..], ql[64h+32+16p ..] and qh[32h+16p ..].  w = d*scale*(q - 32): sum(q x) - 32 sum16(x).
 struct Q6KUnit {
-    static constexpr int kXsWidth = 16;
     static constexpr bool kGrid = false;
+    struct X { float4 p[4][4]; float xs[4]; };   // [run e][piece]
+    struct Regs { u32x4 la, lb, hh; u32x2 scw; uint32_t d; };
 
-    static __device__ __forceinline__ float dot(const uint8_t* row, int unit, const Staged& s)
+    static __device__ __forceinline__ X load_x(const float4* x, int unit)
+    {
+        const int sb = unit >> 2, h = (unit >> 1) & 1, p = unit & 1;
+        X r;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            // run e covers pieces 8e + 4p .. +3 of half h: chunk 4 sb + 2 h + (e >> 1), piece 8 (e & 1) + 4 p + i
+            const float4* src = x + (4 * sb + 2 * h + (e >> 1)) * kChunkPieces + 8 * (e & 1) + 4 * p;
+            float t = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                r.p[e][i] = src[i];
+                t += sum4(r.p[e][i]);
+            }
+            r.xs[e] = t;
+        }
+        return r;
+    }
+
+    static __device__ __forceinline__ Regs load(const uint8_t* row, int unit)
     {
         const int sb = unit >> 2, h = (unit >> 1) & 1, p = unit & 1;
         const uint8_t* blk = row + static_cast<uint32_t>(sb) * 210u;
-        const u32x4 la = ld128(blk + 64 * h + 16 * p);
-        const u32x4 lb = ld128(blk + 64 * h + 32 + 16 * p);
-        const u32x4 hh = ld128(blk + 128 + 32 * h + 16 * p);
-        const u32x2 scw = ld64(blk + 192 + 8 * h);
-        const float d = half_bits_to_float(ld16(blk + 208));
+        Regs r;
+        r.la = ld128(blk + 64 * h + 16 * p);
+        r.lb = ld128(blk + 64 * h + 32 + 16 * p);
+        r.hh = ld128(blk + 128 + 32 * h + 16 * p);
+        r.scw = ld64(blk + 192 + 8 * h);
+        r.d = ld16(blk + 208);
+        return r;
+    }
+
+    static __device__ __forceinline__ float dot(const Regs& r, const X& x, int unit, const uint64_t*)
+    {
+        const int p = unit & 1;
+        const float d = half_bits_to_float(r.d);
         float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
-        const int c0 = 4 * sb + 2 * h;       // 64-chunk holding e = 0,1; e = 2,3 are in chunk c0 + 1
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const uint32_t a = la[i], b = lb[i], q2 = hh[i];
+            const uint32_t a = r.la[i], b = r.lb[i], q2 = r.hh[i];
             const uint32_t q1 = opaque((a & 0x0f0f0f0fu) | ((q2 << 4) & 0x30303030u));
             const uint32_t q2v = opaque((b & 0x0f0f0f0fu) | ((q2 << 2) & 0x30303030u));
             const uint32_t q3 = opaque(((a >> 4) & 0x0f0f0f0fu) | (q2 & 0x30303030u));
             const uint32_t q4 = opaque(((b >> 4) & 0x0f0f0f0fu) | ((q2 >> 2) & 0x30303030u));
-            a0 = dot4u(q1, xpiece(s, c0, 4 * p + i), a0);
-            a1 = dot4u(q2v, xpiece(s, c0, 8 + 4 * p + i), a1);
-            a2 = dot4u(q3, xpiece(s, c0 + 1, 4 * p + i), a2);
-            a3 = dot4u(q4, xpiece(s, c0 + 1, 8 + 4 * p + i), a3);
+            a0 = dot4u(q1, x.p[0][i], a0);
+            a1 = dot4u(q2v, x.p[1][i], a1);
+            a2 = dot4u(q3, x.p[2][i], a2);
+            a3 = dot4u(q4, x.p[3][i], a3);
         }
-        // int8 sub-scales 8h + 2e + p; 16-wide sums of x at run index 16 sb + 8 h + 2 e + p
-        const uint32_t s01 = scw[0] >> (8 * p), s23 = scw[1] >> (8 * p);
+        // int8 sub-scales 8h + 2e + p live in byte 2e + p of the 8 bytes loaded for half h
+        const uint32_t s01 = r.scw[0] >> (8 * p), s23 = r.scw[1] >> (8 * p);
         const float sc0 = sbyte0(s01), sc1 = sbyte2(s01), sc2 = sbyte0(s23), sc3 = sbyte2(s23);
-        const float* xs = s.xs + 16 * sb + 8 * h + p;
-        float acc = (d * sc0) * fmaf(-32.0f, xs[0], a0);
-        acc = fmaf(d * sc1, fmaf(-32.0f, xs[2], a1), acc);
-        acc = fmaf(d * sc2, fmaf(-32.0f, xs[4], a2), acc);
-        acc = fmaf(d * sc3, fmaf(-32.0f, xs[6], a3), acc);
+        float acc = (d * sc0) * fmaf(-32.0f, x.xs[0], a0);
+        acc = fmaf(d * sc1, fmaf(-32.0f, x.xs[1], a1), acc);
+        acc = fmaf(d * sc2, fmaf(-32.0f, x.xs[2], a2), acc);
+        acc = fmaf(d * sc3, fmaf(-32.0f, x.xs[3], a3), acc);
         return acc;
     }
 };
@@ -222,8 +304,29 @@ struct Q6KUnit {
 // Unit gp of a super-block = 32-groups 2gp and 2gp+1.  Each octet: 10-bit index into the 1024-entry codebook held
 // in LDS (8 magnitude bytes), 8 sign bits, 4-bit sub-scale shared by two octets.
 struct IQ2SUnit {
-    static constexpr int kXsWidth = 0;
     static constexpr bool kGrid = true;
+    struct X { XChunk c; };
+    struct Regs { u32x2 qs, sg; uint32_t qh, scl, d; };
+
+    static __device__ __forceinline__ X load_x(const float4* x, int unit)
+    {
+        X r;
+        r.c = load_chunk(x, unit);
+        return r;
+    }
+
+    static __device__ __forceinline__ Regs load(const uint8_t* row, int unit)
+    {
+        const int sb = unit >> 2, gp = unit & 3;
+        const uint8_t* blk = row + static_cast<uint32_t>(sb) * 82u;
+        Regs r;
+        r.qs = ld64(blk + 2 + 8 * gp);
+        r.sg = ld64(blk + 34 + 8 * gp);
+        r.qh = ld16(blk + 66 + 2 * gp);
+        r.scl = ld16(blk + 74 + 2 * gp);
+        r.d = ld16(blk);
+        return r;
+    }
 
     static __device__ __forceinline__ float signed_mag(float mag, uint32_t signs, int t)
     {
@@ -231,28 +334,22 @@ struct IQ2SUnit {
         return __uint_as_float(__float_as_uint(mag) | sign);
     }
 
-    static __device__ __forceinline__ float dot(const uint8_t* row, int unit, const Staged& s)
+    static __device__ __forceinline__ float dot(const Regs& r, const X& x, int, const uint64_t* grid)
     {
-        const int sb = unit >> 2, gp = unit & 3;
-        const uint8_t* blk = row + static_cast<uint32_t>(sb) * 82u;
-        const u32x2 qs = ld64(blk + 2 + 8 * gp);
-        const u32x2 sg = ld64(blk + 34 + 8 * gp);
-        const uint32_t qh = ld16(blk + 66 + 2 * gp);
-        const uint32_t scl = ld16(blk + 74 + 2 * gp);
-        const float d = half_bits_to_float(ld16(blk));
+        const float d = half_bits_to_float(r.d);
         float acc = 0.0f;
 #pragma unroll
         for (int g = 0; g < 2; ++g) {
-            const uint32_t q4 = qs[g], s4 = sg[g];
-            const uint32_t hbits = (qh >> (8 * g)) & 0xffu;
-            const uint32_t sc = (scl >> (8 * g)) & 0xffu;
+            const uint32_t q4 = r.qs[g], s4 = r.sg[g];
+            const uint32_t hbits = (r.qh >> (8 * g)) & 0xffu;
+            const uint32_t sc = (r.scl >> (8 * g)) & 0xffu;
 #pragma unroll
             for (int o = 0; o < 4; ++o) {
                 const uint32_t idx = ((q4 >> (8 * o)) & 0xffu) | (((hbits >> (2 * o)) & 3u) << 8);
-                const uint64_t gv = s.grid[idx];
+                const uint64_t gv = grid[idx];
                 const uint32_t glo = static_cast<uint32_t>(gv), ghi = static_cast<uint32_t>(gv >> 32);
                 const uint32_t signs = (s4 >> (8 * o)) & 0xffu;
-                const float4 xa = xpiece(s, unit, 8 * g + 2 * o), xb = xpiece(s, unit, 8 * g + 2 * o + 1);
+                const float4 xa = x.c.p[8 * g + 2 * o], xb = x.c.p[8 * g + 2 * o + 1];
                 float t = 0.0f;
                 t = fmaf(signed_mag(ubyte0(glo), signs, 0), xa.x, t);
                 t = fmaf(signed_mag(ubyte1(glo), signs, 1), xa.y, t);
@@ -272,61 +369,94 @@ struct IQ2SUnit {
 };
 
 // ---------------------------------------------------------------------------------------------- the kernel
-// grid.x = row groups, grid.y = input rows.  Dynamic LDS: [16 * cpad float4][xs floats][grid 8 KB][part floats].
+// Launch shape of one block format: lanes per workgroup, waves per SIMD the register budget is sized for, and the
+// number of weight register sets that rotate (DEPTH - 1 row steps are in flight while one is reduced).
+template <class Q> struct Shape;
+template <> struct Shape<Q8_0Unit> { static constexpr int kMaxT = 768, kWavesPerEu = 3, kDepth = 3; };
+template <> struct Shape<Q4KUnit> { static constexpr int kMaxT = 1024, kWavesPerEu = 4, kDepth = 3; };
+template <> struct Shape<Q5KUnit> { static constexpr int kMaxT = 768, kWavesPerEu = 3, kDepth = 3; };
+template <> struct Shape<Q6KUnit> { static constexpr int kMaxT = 768, kWavesPerEu = 3, kDepth = 4; };
+template <> struct Shape<IQ2SUnit> { static constexpr int kMaxT = 1024, kWavesPerEu = 4, kDepth = 4; };
+
+// grid.x = workgroups striding over row steps, grid.y = input rows, blockDim.x = T (a multiple of 64).
 template <class Q>
-__global__ __launch_bounds__(kWG) void matvec_flat_kernel(MatvecArgs a)
+__global__ __launch_bounds__(Shape<Q>::kMaxT) __attribute__((amdgpu_waves_per_eu(Shape<Q>::kWavesPerEu, Shape<Q>::kWavesPerEu)))
+void matvec_rowstep_kernel(MatvecArgs a, const float* __restrict__ bias)
 {
-    extern __shared__ float4 lds[];
-    float4* xp = lds;
-    float* xs = reinterpret_cast<float*>(xp + 16 * a.cpad);
-    constexpr int kXsDiv = Q::kXsWidth ? Q::kXsWidth : 1;
-    const int n_xs = Q::kXsWidth ? a.in_w / kXsDiv : 0;
-    uint64_t* grid = reinterpret_cast<uint64_t*>(xs + ((n_xs + 3) & ~3));
-    float* part = reinterpret_cast<float*>(grid + (Q::kGrid ? 1024 : 0));
+    constexpr int kDepth = Shape<Q>::kDepth;
+    __shared__ float part[2][kMaxWG];
+    __shared__ uint64_t grid[Q::kGrid ? 1024 : 1];
 
     const int tid = threadIdx.x;
-    const int m = blockIdx.y;
-    const int row0 = blockIdx.x * a.rows_per_wg;
-    const int nrows = min(a.rows_per_wg, a.out_w - row0);
-    const float4* xg = reinterpret_cast<const float4*>(a.x + static_cast<size_t>(m) * a.in_w);
+    const int upr = a.units_per_row, rs = a.rows_per_step;
+    const int rl = upr == 1 ? tid : static_cast<int>(__umulhi(static_cast<uint32_t>(tid), a.magic));  // row within a step
+    const int c = tid - rl * upr;                                                                    // unit within the row
+    const bool owner = rl < rs;
+    const float* x = a.x + static_cast<size_t>(blockIdx.y) * a.in_w;
+    float* y = a.y + static_cast<size_t>(blockIdx.y) * a.out_w;
+    const int last_row = a.out_w - 1;
 
-    // stage x (and its block sums, and the codebook)
+    // Loads are unconditional: rows past the end re-read the last row, spare lanes re-read row 0 (both stay in L2),
+    // and their products are dropped.  That keeps the stream free of branches between loads.
+    auto fetch = [&](int step) {
+        const int row = owner ? min(step * rs + rl, last_row) : 0;
+        return Q::load(a.w + static_cast<size_t>(row) * a.row_bytes, c);
+    };
+
+    // The activations are requested first (they come from L2 and return ahead of the weight stream), staged through
+    // LDS so that the workgroup reads them from memory once, and then kept in registers: 64 per lane.
+    extern __shared__ float4 xstage[];
     const int pieces = a.in_w >> 2;
-    for (int L = tid; L < pieces; L += kWG) {
-        const float4 v = xg[L];
-        xp[(L & 15) * a.cpad + (L >> 4)] = v;
-        if (Q::kXsWidth == 32) {
-            const float t = oct_sum((v.x + v.y) + (v.z + v.w));
-            if ((L & 7) == 0) xs[L >> 3] = t;
-        } else if (Q::kXsWidth == 16) {
-            float t = (v.x + v.y) + (v.z + v.w);
-            t += dpp_mov<0xB1>(t);
-            t += dpp_mov<0x4E>(t);
-            if ((L & 3) == 0) xs[L >> 2] = t;
+    const float4* xg = reinterpret_cast<const float4*>(x);
+    const int T = blockDim.x;
+    float4 xv0 = tid < pieces ? xg[tid] : make_float4(0.f, 0.f, 0.f, 0.f);
+    float4 xv1 = tid + T < pieces ? xg[tid + T] : make_float4(0.f, 0.f, 0.f, 0.f);
+    // The compute unit returns vector-memory data in the order the requests were queued, across waves.  This barrier
+    // (no memory wait, just a rendezvous) puts every wave's activation requests ahead of every wave's weight
+    // requests, so staging does not wait for the first weight rows to come back from HBM.
+    __syncthreads();
+
+    const int stride = gridDim.x;
+    int step = blockIdx.x;
+    typename Q::Regs regs[kDepth];
+#pragma unroll
+    for (int d = 0; d < kDepth - 1; ++d) regs[d] = fetch(step + d * stride);
+
+    if (tid < pieces) xstage[tid + (tid >> 4)] = xv0;
+    if (tid + T < pieces) xstage[tid + T + ((tid + T) >> 4)] = xv1;
+    for (int L = tid + 2 * T; L < pieces; L += T) xstage[L + (L >> 4)] = xg[L];
+    if (Q::kGrid)
+        for (int i = tid; i < 1024; i += T) grid[i] = g_iq2s_grid[i];
+    __syncthreads();
+    typename Q::X xr = Q::load_x(xstage, owner ? c : 0);
+
+    const int wave = tid >> 6, lane = tid & 63, waves = T >> 6;
+    int buf = 0;
+    auto finish = [&](const typename Q::Regs& r, int st) {
+        part[buf][tid] = Q::dot(r, xr, c, grid);
+        __syncthreads();
+        for (int rr = wave; rr < rs; rr += waves) {
+            const int row = st * rs + rr;
+            if (row < a.out_w) {
+                float t = 0.0f;
+                for (int u = lane; u < upr; u += 64) t += part[buf][rr * upr + u];
+                t = wave_sum(t);
+                // the row index is wave-uniform: the bias comes through the scalar cache and does not wait on the
+                // vector-memory counter that the prefetched weights are tracked by
+                const int urow = __builtin_amdgcn_readfirstlane(row);
+                if (lane == 0) y[urow] = (bias ? bias[urow] : 0.0f) + t;
+            }
         }
-    }
-    if (Q::kGrid) grid[tid] = g_iq2s_grid[tid];
-    __syncthreads();
+        buf ^= 1;
+    };
 
-    Staged s{xp, xs, grid, a.cpad};
-    const int upr = a.units_per_row;
-    const int units = nrows * upr;
-    for (int u = tid; u < units; u += kWG) {
-        const int r = upr == 1 ? u : static_cast<int>(__umulhi(static_cast<uint32_t>(u), a.magic));
-        const int c = u - r * upr;
-        const uint8_t* row = a.w + static_cast<size_t>(row0 + r) * a.row_bytes;
-        part[u] = Q::dot(row, c, s);
-    }
-    __syncthreads();
-
-    const int wave = tid >> 6, lane = tid & 63;
-    for (int r = wave; r < nrows; r += kWG / 64) {
-        float t = 0.0f;
-        for (int c = lane; c < upr; c += 64) t += part[r * upr + c];
-        t = wave_sum(t);
-        if (lane == 0) {
-            const int o = row0 + r;
-            a.y[static_cast<size_t>(m) * a.out_w + o] = (a.bias ? a.bias[o] : 0.0f) + t;
+    while (step < a.steps) {
+#pragma unroll
+        for (int d = 0; d < kDepth; ++d) {
+            regs[(d + kDepth - 1) % kDepth] = fetch(step + (kDepth - 1) * stride);
+            finish(regs[d], step);
+            step += stride;
+            if (step >= a.steps) break;
         }
     }
 }
@@ -355,58 +485,66 @@ __global__ __launch_bounds__(256) void matvec_q8_0_oddrow_kernel(MatvecArgs a)
 }
 
 struct Geometry {
-    int cpad;
-    int rows_per_wg;
+    int threads;        // T
+    int rows_per_step;  // RS
+    int steps;
     int groups;
-    size_t lds_bytes;
 };
 
-// Picks rows per workgroup so that one workgroup per compute unit covers the matrix, within the LDS budget.
-bool plan(uint32_t type, int in_w, int out_w, int compute_units, Geometry* g)
+// Picks RS (whole rows per step) and from it the workgroup size.  Every workgroup runs ceil(steps / groups) rounds of
+// RS rows, so the launch lasts about rounds * RS row-times.  The largest RS that fits max_t lanes keeps the most
+// bytes in flight; a smaller one is taken only if it saves at least 2 % of rounds * RS.
+bool plan(int in_w, int out_w, int compute_units, int max_t, Geometry* g)
 {
     const int upr = in_w / kUnitW;
-    const int cpad = upr | 1;
-    int xs_width = (type == NNHIP_TYPE_Q4_K || type == NNHIP_TYPE_Q5_K) ? 32 : type == NNHIP_TYPE_Q6_K ? 16 : 0;
-    size_t fixed = static_cast<size_t>(16) * cpad * sizeof(float4);
-    if (xs_width) fixed += static_cast<size_t>(((in_w / xs_width) + 3) & ~3) * sizeof(float);
-    if (type == NNHIP_TYPE_IQ2_S) fixed += 1024 * sizeof(uint64_t);
-    if (fixed + static_cast<size_t>(upr) * sizeof(float) > static_cast<size_t>(kMaxLds)) return false;
-    const int max_rows = static_cast<int>((kMaxLds - fixed) / (static_cast<size_t>(upr) * sizeof(float)));
-    int rpw = (out_w + compute_units - 1) / compute_units;
-    if (rpw > max_rows) rpw = max_rows;
-    if (rpw < 1) rpw = 1;
-    g->cpad = cpad;
-    g->rows_per_wg = rpw;
-    g->groups = (out_w + rpw - 1) / rpw;
-    g->lds_bytes = fixed + static_cast<size_t>(rpw) * upr * sizeof(float);
+    if (upr < 1 || upr > max_t) return false;
+    const int rs_max = max_t / upr;
+    const int rs_min = (3 * rs_max + 3) / 4;     // never give up more than a quarter of the lanes
+    int best_rs = 0;
+    long best_cost = 0;
+    for (int rs = rs_max; rs >= rs_min && rs >= 1; --rs) {
+        const int steps = (out_w + rs - 1) / rs;
+        const int rounds = (steps + compute_units - 1) / compute_units;
+        const long cost = static_cast<long>(rounds) * rs;
+        if (!best_rs || cost * 100 < best_cost * 98) {   // a smaller step must save at least 2 %
+            best_rs = rs;
+            best_cost = cost;
+        }
+    }
+    if (best_rs > out_w) best_rs = out_w;   // tiny matrices: shrink to the rows there are
+    g->rows_per_step = best_rs;
+    g->threads = (best_rs * upr + 63) / 64 * 64;
+    g->steps = (out_w + best_rs - 1) / best_rs;
+    g->groups = g->steps < compute_units ? g->steps : compute_units;
     return true;
 }
 
 template <class Q>
-hipError_t launch_flat(Lane* lane, const MatvecArgs& args, const Geometry& g, int rows)
+hipError_t launch_rowstep(Lane* lane, MatvecArgs args, int rows)
 {
-    static size_t configured = 0;  // largest dynamic LDS size this kernel has been enabled for
-    if (g.lds_bytes > 64 * 1024 && g.lds_bytes > configured) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&matvec_flat_kernel<Q>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds);
+    Geometry g;
+    if (!plan(args.in_w, args.out_w, lane->compute_units, Shape<Q>::kMaxT, &g)) return hipErrorInvalidValue;
+    args.rows_per_step = g.rows_per_step;
+    args.steps = g.steps;
+    const size_t lds = static_cast<size_t>(kChunkPieces) * args.units_per_row * sizeof(float4);
+    static bool big_lds_enabled = false;
+    if (lds > 48 * 1024 && !big_lds_enabled) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&matvec_rowstep_kernel<Q>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, kMaxDynamicLds);
         if (e != hipSuccess) return e;
-        configured = kMaxLds;
+        big_lds_enabled = true;
     }
-    hipLaunchKernelGGL(matvec_flat_kernel<Q>, dim3(g.groups, rows), dim3(kWG), g.lds_bytes, lane->stream, args);
+    hipLaunchKernelGGL(matvec_rowstep_kernel<Q>, dim3(g.groups, rows), dim3(g.threads), lds, lane->stream, args, args.bias);
     return hipGetLastError();
 }
 
 }  // namespace
 
-int matvec_max_in_w(uint32_t type)
+int matvec_max_in_w(uint32_t)
 {
-    // 16 planes of (in_w/64 | 1) float4 pieces plus side tables must leave room for at least one row of partials.
-    int best = 0;
-    for (int k = 256; k <= 65536; k += 256) {
-        Geometry g;
-        if (plan(type, k, 1, 1, &g)) best = k;
-    }
-    return best;
+    const int by_lds = kMaxDynamicLds / (kChunkPieces * static_cast<int>(sizeof(float4))) * kUnitW;
+    const int by_lanes = 768 * kUnitW;   // the narrowest workgroup shape must still hold one row
+    return by_lds < by_lanes ? by_lds : by_lanes;
 }
 
 hipError_t launch_matvec(Lane* lane, uint32_t type, const float* x, const void* w, const float* bias, float* y,
@@ -428,18 +566,14 @@ hipError_t launch_matvec(Lane* lane, uint32_t type, const float* x, const void* 
         return hipGetLastError();
     }
 
-    Geometry g;
-    if (!plan(type, in_w, out_w, lane->compute_units, &g)) return hipErrorInvalidValue;
     a.units_per_row = in_w / kUnitW;
-    a.cpad = g.cpad;
-    a.rows_per_wg = g.rows_per_wg;
     a.magic = static_cast<uint32_t>((0x100000000ull + a.units_per_row - 1) / a.units_per_row);
     switch (type) {
-    case NNHIP_TYPE_Q8_0: return launch_flat<Q8_0Unit>(lane, a, g, rows);
-    case NNHIP_TYPE_Q4_K: return launch_flat<Q4KUnit>(lane, a, g, rows);
-    case NNHIP_TYPE_Q5_K: return launch_flat<Q5KUnit>(lane, a, g, rows);
-    case NNHIP_TYPE_Q6_K: return launch_flat<Q6KUnit>(lane, a, g, rows);
-    case NNHIP_TYPE_IQ2_S: return launch_flat<IQ2SUnit>(lane, a, g, rows);
+    case NNHIP_TYPE_Q8_0: return launch_rowstep<Q8_0Unit>(lane, a, rows);
+    case NNHIP_TYPE_Q4_K: return launch_rowstep<Q4KUnit>(lane, a, rows);
+    case NNHIP_TYPE_Q5_K: return launch_rowstep<Q5KUnit>(lane, a, rows);
+    case NNHIP_TYPE_Q6_K: return launch_rowstep<Q6KUnit>(lane, a, rows);
+    case NNHIP_TYPE_IQ2_S: return launch_rowstep<IQ2SUnit>(lane, a, rows);
     default: return hipErrorInvalidValue;
     }
 }

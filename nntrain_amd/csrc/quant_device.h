@@ -35,7 +35,7 @@ __device__ __forceinline__ float half_bits_to_float(uint32_t h)
 // folded back into one bit-field extract per byte.
 __device__ __forceinline__ uint32_t opaque(uint32_t v)
 {
-    asm volatile("" : "+v"(v));
+    asm("" : "+v"(v));
     return v;
 }
 
