@@ -1,0 +1,374 @@
+#!/usr/bin/env python3
+"""Benchmark of the GGUF block-quantized linear path on one MI355X.
+
+Default workload (`decode27b`): the full per-token mat-vec set of a Gemma-3-27B-shaped stack, all weights Q8_0 and
+random-init, resident in HBM (62 layers x {q,k,v,o,gate,up,down} + lm_head = 435 mat-vecs, 28,695,625,728 weight bytes
+per token).  A "step" is one token: every mat-vec of the set once, fresh N(0,1) FP32 activations, batch 1.
+`value` is tokens/s; `roofline` is the Q8_0 mat-vec kernel's achieved HBM rate over the same timed region.
+
+Other workloads (`--workload gemv|prefill|all`) time the single-matrix configurations and are reported under "also".
+
+One JSON line on stdout; progress on stderr.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+from ctypes import c_void_p
+from pathlib import Path
+
+import numpy as np
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+BF16_PEAK_TFLOPS = 2500.0      # MI355X dense bf16 MFMA, published
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def decode27b_tensors():
+    """(name, out_w, in_w) of every mat-vec of one token: Gemma-3-27B shapes (hidden 5376, 32 q heads, 16 kv heads,
+    head_dim 128, ffn 21504, vocab 262144)."""
+    hidden, q_out, kv_out, ffn, vocab, layers = 5376, 32 * 128, 16 * 128, 21504, 262144, 62
+    per_layer = [("attn_q", q_out, hidden), ("attn_k", kv_out, hidden), ("attn_v", kv_out, hidden),
+                 ("attn_o", hidden, q_out), ("ffn_gate", ffn, hidden), ("ffn_up", ffn, hidden),
+                 ("ffn_down", hidden, ffn)]
+    out = []
+    for layer in range(layers):
+        out += [(f"blk.{layer}.{n}", o, i) for n, o, i in per_layer]
+    out.append(("output", vocab, hidden))
+    return out
+
+
+def q8_bytes(out_w, in_w):
+    return out_w * (in_w // 32) * 34
+
+
+class Synth:
+    def __init__(self):
+        path = ROOT / "nntrain_amd" / "csrc" / "libnnhip_synth.so"
+        if not path.exists():
+            raise FileNotFoundError(f"{path} is missing: run __graft_entry__.build()")
+        self.lib = ctypes.CDLL(str(path))
+        self.lib.nnhip_synth_q8_0.argtypes = [c_void_p, c_void_p, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_float]
+        self.lib.nnhip_synth_normal_f32.argtypes = [c_void_p, c_void_p, ctypes.c_uint64, ctypes.c_uint64]
+
+    def q8_0(self, lane, buf, blocks, seed, sigma=0.02):
+        s = c_void_p()
+        lane._lib.nnhip_lane_stream(lane._handle, ctypes.byref(s))
+        rc = self.lib.nnhip_synth_q8_0(s, c_void_p(buf.ptr), blocks, seed, sigma)
+        if rc:
+            raise RuntimeError(f"nnhip_synth_q8_0 failed ({rc})")
+
+    def normal(self, lane, buf, count, seed):
+        s = c_void_p()
+        lane._lib.nnhip_lane_stream(lane._handle, ctypes.byref(s))
+        rc = self.lib.nnhip_synth_normal_f32(s, c_void_p(buf.ptr), count, seed)
+        if rc:
+            raise RuntimeError(f"nnhip_synth_normal_f32 failed ({rc})")
+
+
+def timed(lane, fn, reps):
+    """Device time of `reps` calls of fn on the lane's stream (HIP events), plus host wall time around a sync."""
+    e0, e1 = lane.event(), lane.event()
+    lane.synchronize()
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(reps):
+        fn()
+    e1.record()
+    ms = lane.elapsed_ms(e0, e1)
+    lane.synchronize()
+    wall = (time.perf_counter() - t0) * 1e3
+    e0.dispose()
+    e1.dispose()
+    return ms, wall
+
+
+def run_decode27b(args, lane, nn, oracle):
+    from nntrain_amd.native import MatvecDesc
+    tensors = decode27b_tensors()
+    total_bytes = sum(q8_bytes(o, i) for _, o, i in tensors)
+    assert total_bytes == 28_695_625_728, total_bytes
+    synth = Synth()
+    log(f"[decode27b] generating {len(tensors)} Q8_0 tensors, {total_bytes / 1e9:.2f} GB, on the device")
+    weights, xs, ys = [], [], []
+    for t, (name, out_w, in_w) in enumerate(tensors):
+        w = lane.allocate_bytes(q8_bytes(out_w, in_w))
+        synth.q8_0(lane, w, out_w * (in_w // 32), 3000 + t)
+        x = lane.allocate(in_w)
+        synth.normal(lane, x, in_w, 3999_000 + t)
+        y = lane.allocate(out_w)
+        weights.append(w)
+        xs.append(x)
+        ys.append(y)
+    lane.synchronize()
+    lib, h = lane._lib, lane._handle
+
+    descs = (MatvecDesc * len(tensors))()
+    for t, (name, out_w, in_w) in enumerate(tensors):
+        descs[t] = MatvecDesc(xs[t].ptr, weights[t].ptr, None, ys[t].ptr, nn.GGML_Q8_0, 1, in_w, out_w)
+
+    def token_forward():
+        for t, (name, out_w, in_w) in enumerate(tensors):
+            rc = lib.nnhip_quant_matvec(h, nn.GGML_Q8_0, c_void_p(xs[t].ptr), c_void_p(weights[t].ptr), None,
+                                        c_void_p(ys[t].ptr), 1, in_w, out_w)
+            if rc:
+                nn.native.check(rc, "quant_matvec")
+
+    def token_batch():
+        nn.native.check(lib.nnhip_quant_matvec_batch(h, descs, len(tensors)), "quant_matvec_batch")
+
+    graph = None
+    if args.mode == "graph":
+        lane.graph_begin()
+        token_forward()
+        graph = lane.graph_end()
+
+    def token():
+        if args.mode == "forward":
+            token_forward()
+        elif args.mode == "batch":
+            token_batch()
+        else:
+            lane.graph_launch(graph)
+
+    def verify(tag):
+        """Sampled parity against the float64 oracle on the bytes that are actually in HBM."""
+        worst = 0.0
+        for t in (0, 3, 6, len(tensors) - 1):
+            name, out_w, in_w = tensors[t]
+            rows = min(out_w, 256)
+            row_bytes = (in_w // 32) * 34
+            x = lane.read(xs[t], np.float32)
+            y = lane.read(ys[t], np.float32)
+            for r0 in (0, out_w - rows):
+                raw = lane.read(weights[t], np.uint8, rows * row_bytes, r0 * row_bytes)
+                ref, _ = oracle.linear_f64(nn.GGML_Q8_0, raw, x, None, 1, in_w, rows)
+                worst = max(worst, oracle.rel_l2(y[r0:r0 + rows], ref[0]))
+        log(f"[decode27b] parity {tag}: worst sampled rel-L2 vs float64 oracle = {worst:.3e}")
+        if not worst <= 1e-5:
+            raise SystemExit(f"parity failure ({tag}): rel-L2 {worst:.3e} > 1e-5")
+        return worst
+
+    for _ in range(max(args.warmup, 1)):
+        token()
+    lane.synchronize()
+    rel = verify("before timing")
+    ms, wall = timed(lane, token, args.steps)
+    rel = max(rel, verify("after timing"))
+    ms_per_step = ms / args.steps
+    tok_s = 1e3 / ms_per_step
+    gbs = total_bytes / (ms_per_step * 1e-3) / 1e9
+    log(f"[decode27b] {ms_per_step:.3f} ms/token (device events), wall {wall / args.steps:.3f} ms/token, "
+        f"{tok_s:.1f} tok/s, {gbs:.0f} GB/s")
+
+    cpu = None
+    if not args.no_cpu_baseline:
+        cpu = cpu_baseline_decode(lane, nn, oracle, tensors, weights, xs)
+    if graph is not None:
+        lane.graph_destroy(graph)
+    for b in weights + xs + ys:
+        b.dispose()
+    n_launch = len(tensors) if args.mode != "batch" else 1
+    return {
+        "metric": "27B-shape Q8_0 decode tokens/sec", "value": round(tok_s, 2), "unit": "tokens/s",
+        "ms_per_step": round(ms_per_step, 4),
+        "config": {"workload": "decode27b: 435 Q8_0 mat-vecs of a Gemma-3-27B-shaped stack (BASELINE configs[2]), "
+                               "28,695,625,728 weight bytes/token resident in HBM, batch 1, fp32 activations",
+                   "launch": args.mode, "launches_per_token": n_launch},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "matvec_rowstep_kernel<Q8_0Unit>",
+                     "bytes_per_launch": total_bytes // n_launch},
+        "cpu_baseline": cpu,
+        "parity": {"rel_l2_vs_f64_oracle_sampled": rel, "bar": 1e-5},
+    }
+
+
+def cpu_baseline_decode(lane, nn, oracle, tensors, weights, xs):
+    """The CPU restatement of the reference's operator (dequantize row + sequential FP32 FMA) on one layer's seven
+    matrices, all host threads; the token rate is extrapolated by bytes to the whole set."""
+    threads = oracle.max_threads()
+    sample = list(range(7))
+    host = []
+    for t in sample:
+        name, out_w, in_w = tensors[t]
+        host.append((lane.read(weights[t], np.uint8), lane.read(xs[t], np.float32), in_w, out_w))
+    sample_bytes = sum(w.size for w, _, _, _ in host)
+    total_bytes = sum(q8_bytes(o, i) for _, o, i in tensors)
+    reps, spent = 0, 0.0
+    t_begin = time.perf_counter()
+    while spent < 10.0 or reps < 2:
+        for w, x, in_w, out_w in host:
+            oracle.cpu_linear(nn.GGML_Q8_0, w, x, None, 1, in_w, out_w, threads)
+        reps += 1
+        spent = time.perf_counter() - t_begin
+    per_layer = spent / reps
+    tok_s = 1.0 / (per_layer * total_bytes / sample_bytes)
+    log(f"[cpu_baseline] {threads} threads: layer sample {per_layer * 1e3:.1f} ms ({sample_bytes / per_layer / 1e9:.1f} GB/s)"
+        f" -> {tok_s:.3f} tok/s extrapolated")
+    return {"value": round(tok_s, 4), "unit": "tokens/s", "cores": threads, "kind": "port",
+            "sample": f"layer 0's seven Q8_0 matrices ({sample_bytes} bytes) x {reps} passes, {spent:.1f} s; token rate "
+                      f"extrapolated by weight bytes to the 435-matrix set",
+            "gb_per_s": round(sample_bytes / per_layer / 1e9, 2)}
+
+
+GEMV_CONFIGS = [
+    ("cfg1 Q8_0 21504x5376", "GGML_Q8_0", 5376, 21504, 1001, 1002),
+    ("cfg2 Q4_K 17408x5120", "GGML_Q4_K", 5120, 17408, 2001, 2000),
+    ("cfg2 Q5_K 17408x5120", "GGML_Q5_K", 5120, 17408, 2002, 2000),
+    ("cfg2 Q6_K 17408x5120", "GGML_Q6_K", 5120, 17408, 2003, 2000),
+    ("cfg5 IQ2_S 5120x17408", "GGML_IQ2_S", 17408, 5120, 5001, 5002),
+]
+
+
+def run_gemv(args, lane, nn, oracle):
+    """Single-matrix decode mat-vecs.  Weights rotate through copies totalling >= 1 GB so every launch streams from
+    HBM rather than from the 256 MB Infinity Cache; the cache-resident figure is reported beside it."""
+    from nntrain_amd import synth
+    out = {}
+    lib, h = lane._lib, lane._handle
+    for name, tname, in_w, out_w, wseed, xseed in GEMV_CONFIGS:
+        typ = getattr(nn, tname)
+        payload = synth.matrix(typ, out_w, in_w, wseed)
+        x_host = synth.activations(1, in_w, xseed)
+        nbytes = payload.size
+        copies = max(2, int(np.ceil(1.0e9 / nbytes)))
+        w0 = lane.upload_raw(payload)
+        ring = [w0]
+        for _ in range(copies - 1):
+            b = lane.allocate_bytes(nbytes)
+            lane.copy(b, w0, nbytes)
+            ring.append(b)
+        x = lane.upload_raw(x_host)
+        y = lane.allocate(out_w)
+
+        def launch(w):
+            rc = lib.nnhip_quant_matvec(h, typ, c_void_p(x.ptr), c_void_p(w.ptr), None, c_void_p(y.ptr), 1, in_w, out_w)
+            if rc:
+                nn.native.check(rc, "quant_matvec")
+
+        for w in ring:
+            launch(w)
+        lane.synchronize()
+        ref, _ = oracle.linear_f64(typ, payload, x_host, None, 1, in_w, out_w)
+        rel = oracle.rel_l2(lane.read(y, np.float32), ref[0])
+        if not rel <= 1e-5:
+            raise SystemExit(f"{name}: parity failure, rel-L2 {rel:.3e}")
+        samples_ring, samples_same = [], []
+        for _ in range(9):
+            ms, _ = timed(lane, lambda: [launch(w) for w in ring], 1)
+            samples_ring.append(ms * 1e3 / len(ring))
+            ms, _ = timed(lane, lambda: [launch(w0) for _ in ring], 1)
+            samples_same.append(ms * 1e3 / len(ring))
+        us_ring, us_same = float(np.median(samples_ring)), float(np.median(samples_same))
+        algo = nbytes + 4 * in_w + 4 * out_w
+        out[name] = {"us_per_launch_hbm": round(us_ring, 2), "gb_per_s_hbm": round(algo / us_ring / 1e3, 1),
+                     "frac_of_8TBs": round(algo / us_ring / 1e3 / HBM_PEAK_GBS, 4),
+                     "us_per_launch_cache_resident": round(us_same, 2), "algorithmic_bytes": algo,
+                     "rel_l2_vs_f64_oracle": rel, "weight_copies_rotated": len(ring)}
+        log(f"[gemv] {name}: {us_ring:.2f} us ({algo / us_ring / 1e3:.0f} GB/s, {100 * algo / us_ring / 1e3 / HBM_PEAK_GBS:.1f}% "
+            f"of 8 TB/s) HBM; {us_same:.2f} us cache-resident; rel-L2 {rel:.2e}")
+        for b in ring + [x, y]:
+            b.dispose()
+    return out
+
+
+def run_prefill(args, lane, nn, oracle):
+    """Q4_K 17408x5120 bf16-MFMA prefill mat-mul at M = 128, 256, 512, 2048 (BASELINE configs[3])."""
+    from nntrain_amd import synth
+    typ, in_w, out_w = nn.GGML_Q4_K, 5120, 17408
+    payload = synth.matrix(typ, out_w, in_w, 2001)
+    mat = nn.HipQuantizedMatrix(payload, typ, out_w, in_w)
+    mat.device_payload(lane)
+    out = {}
+    for m in (128, 256, 512, 2048):
+        xb = synth.to_bf16_bits(synth.activations(m, in_w, 4000))
+        x = lane.upload_raw(xb)
+        y = lane.allocate(m * out_w)
+        try:
+            mat.forward_bf16(lane, x, None, m, out=y)
+        except nn.NnHipError as e:
+            log(f"[prefill] unavailable: {e}")
+            x.dispose()
+            y.dispose()
+            mat.dispose()
+            return None
+        lane.synchronize()
+        rows = min(m, 16)
+        got = lane.read(y, np.float32, rows * out_w)
+        ref, _ = oracle.linear_f64(typ, payload, xb[:rows], None, rows, in_w, out_w, x_is_bf16=True)
+        rel = oracle.rel_l2(got, ref)
+        if not rel <= 2e-3:
+            raise SystemExit(f"prefill M={m}: parity failure, rel-L2 {rel:.3e} > 2e-3")
+        samples = []
+        for _ in range(7):
+            ms, _ = timed(lane, lambda: mat.forward_bf16(lane, x, None, m, out=y), 3)
+            samples.append(ms / 3)
+        ms = float(np.median(samples))
+        flops = 2.0 * m * in_w * out_w
+        out[f"M={m}"] = {"ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 1),
+                         "mfma_util_vs_2500_TFLOPs_bf16": round(flops / ms / 1e9 / BF16_PEAK_TFLOPS, 4),
+                         "rel_l2_vs_f64_oracle": rel}
+        log(f"[prefill] M={m}: {ms:.3f} ms, {flops / ms / 1e9:.0f} TFLOP/s, rel-L2 {rel:.2e}")
+        x.dispose()
+        y.dispose()
+    mat.dispose()
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", choices=["decode27b", "gemv", "prefill", "all"], default="all")
+    ap.add_argument("--mode", choices=["forward", "graph", "batch"], default="batch",
+                    help="decode27b: one launch per matrix, the same captured in a HIP graph, or the batched entry point")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("this build measures one GPU: the quantized linear path has no collectives and every box has a "
+                         "single MI355X; run with --gpus 1")
+
+    import nntrain_amd as nn
+    import oracle
+    lane = nn.HipExecutionLane(0)
+    log(f"device: {lane.device_name()}, {lane.compute_units} CUs, {lane.total_memory_bytes / 2**30:.0f} GiB")
+
+    also = {}
+    if args.workload in ("gemv", "all"):
+        also["gemv_single_matrix"] = run_gemv(args, lane, nn, oracle)
+    if args.workload in ("prefill", "all"):
+        also["prefill_q4k_bf16_mfma"] = run_prefill(args, lane, nn, oracle)
+    if args.workload in ("decode27b", "all"):
+        res = run_decode27b(args, lane, nn, oracle)
+    else:
+        res = {"metric": "quant GEMV GB/s", "value": None, "unit": "GB/s", "ms_per_step": None,
+               "config": {"workload": args.workload}, "roofline": None, "cpu_baseline": None}
+    lane.dispose()
+
+    line = {
+        "metric": res["metric"], "value": res["value"], "unit": res["unit"], "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": res["ms_per_step"], "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic", "config": res["config"],
+        "roofline": res["roofline"], "cpu_baseline": res["cpu_baseline"],
+    }
+    if "parity" in res:
+        line["parity"] = res["parity"]
+    if also:
+        line["also"] = also
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,169 @@
+"""CPU-side tests: the C ABI loads and exports what include/nnhip.h declares, host-layer validation, GGUF reader."""
+import ctypes
+import json
+import re
+import struct
+from ctypes import byref, c_int, c_uint64, c_void_p
+
+import numpy as np
+import pytest
+
+import nntrain_amd as nn
+from nntrain_amd import native
+from nntrain_amd.gguf import GgufReader, GgufReadLimits, InvalidDataError
+
+
+def test_library_exports_every_declared_symbol():
+    header = (native.library_path().parent.parent.parent / "include" / "nnhip.h").read_text()
+    declared = set(re.findall(r"NNHIP_API\s+[\w\s\*]+?\b(nnhip_\w+)\s*\(", header))
+    assert len(declared) >= 30
+    lib = ctypes.CDLL(str(native.library_path()))
+    for name in declared:
+        assert hasattr(lib, name), f"{name} declared in nnhip.h but not exported"
+    assert declared == set(native.PROTOTYPES), declared ^ set(native.PROTOTYPES)
+
+
+def test_abi_version_and_struct_layouts():
+    assert native.abi_version() == (1, 0)
+    assert ctypes.sizeof(native.ErrorInfo) == 32      # the reference's NativeErrorInfo layout
+    assert ctypes.sizeof(native.MatvecDesc) == 48
+    assert ctypes.sizeof(native.LaneCounters) == 48
+
+
+def test_geometry_queries_without_a_gpu():
+    lib = native.load_library()
+    e, b = c_int(), c_int()
+    for typ, (elems, nbytes) in {8: (32, 34), 12: (256, 144), 13: (256, 176), 14: (256, 210), 22: (256, 82)}.items():
+        assert lib.nnhip_type_block(typ, byref(e), byref(b)) == 0
+        assert (e.value, b.value) == (elems, nbytes)
+    assert lib.nnhip_type_block(2, byref(e), byref(b)) == 2
+    n = c_uint64()
+    assert lib.nnhip_matrix_bytes(8, 5376, 21504, byref(n)) == 0 and n.value == 122_830_848
+    assert lib.nnhip_matrix_bytes(12, 5120, 17408, byref(n)) == 0 and n.value == 50_135_040
+    assert lib.nnhip_matrix_bytes(13, 5120, 17408, byref(n)) == 0 and n.value == 61_276_160
+    assert lib.nnhip_matrix_bytes(14, 5120, 17408, byref(n)) == 0 and n.value == 73_113_600
+    assert lib.nnhip_matrix_bytes(22, 17408, 5120, byref(n)) == 0 and n.value == 28_549_120
+    assert lib.nnhip_matrix_bytes(12, 5000, 10, byref(n)) == 3
+    info, msg = native.last_error()
+    assert info.status == 3 and "256" in msg and info.struct_size == 32
+
+
+def test_bad_handles_are_reported_not_dereferenced():
+    lib = native.load_library()
+    assert lib.nnhip_synchronize(None) == 7
+    p = c_void_p()
+    assert lib.nnhip_alloc(None, 16, byref(p)) == 7
+    assert lib.nnhip_quant_matvec(None, 8, None, None, None, None, 1, 32, 1) == 7
+
+
+def test_quantized_matrix_constructor_validation():
+    """Mirrors ArcQuantizedMatrix's constructor checks (NNtrain.Core/Serialization/ArcQuantizedMatrix.cs:20-32)."""
+    with pytest.raises(TypeError):
+        nn.HipQuantizedMatrix(None, nn.GGML_Q4_K, 1, 256)
+    with pytest.raises(NotImplementedError):
+        nn.HipQuantizedMatrix(b"\0" * 144, 0, 1, 256)              # F32 is not a quantized matrix type
+    with pytest.raises(ValueError):
+        nn.HipQuantizedMatrix(b"\0" * 144, nn.GGML_Q4_K, 0, 256)
+    with pytest.raises(NotImplementedError):
+        nn.HipQuantizedMatrix(b"\0" * 144, nn.GGML_Q4_K, 1, 128)   # incomplete 256-value block
+    with pytest.raises(ValueError, match="expected 144"):
+        nn.HipQuantizedMatrix(b"\0" * 145, nn.GGML_Q4_K, 1, 256)
+    m = nn.HipQuantizedMatrix(b"\0" * (34 * 4), nn.GGML_Q8_0, 2, 64)
+    assert (m.ggml_type, m.output_width, m.input_width, m.storage_bytes) == (8, 2, 64, 136)
+    for typ in (8, 12, 13, 14, 22):
+        nn.HipQuantizedMatrix(np.zeros(nn.BLOCK_BYTES[typ] * 3, np.uint8), typ, 3, nn.BLOCK_ELEMS[typ])
+
+
+# ------------------------------------------------------------------------------------------------ GGUF reader
+
+def test_gguf_reader_reference_fixture(golden_dir):
+    expected = json.loads((golden_dir / "qwen_gguf_expected.json").read_text())
+    with GgufReader(str(golden_dir / "qwen_gguf_reference.gguf")) as r:
+        assert r.version == 3 and r.data_offset == 480
+        assert r.metadata["general.architecture"] == "qwen2"
+        assert [t.name for t in r.tensors] == [t["name"] for t in expected["tensors"]]
+        for want in expected["tensors"]:
+            info = r.get_tensor(want["name"])
+            assert info.type == want["type"] and list(info.shape) == list(want["shape"])
+            assert info.byte_count() == want["payloadBytes"]
+            assert len(r.read_tensor_bytes(info)) == want["payloadBytes"]
+        q = r.get_tensor("q4_k_mixed.weight")
+        assert r.matrix_dims(q) == (512, 7)           # GGUF shape is [input_width, output_width]
+        with pytest.raises(KeyError):
+            r.get_tensor("missing")
+        with pytest.raises(EOFError):
+            r.read_tensor_bytes(r.tensors[-1], 10_000)
+
+
+def _gguf(tmp_path, *, magic=0x46554747, version=3, kvs=(), tensors=(), name="t.gguf", tail=b""):
+    def s(x):
+        b = x.encode()
+        return struct.pack("<Q", len(b)) + b
+    blob = struct.pack("<IIQQ", magic, version, len(tensors), len(kvs))
+    for k, t, v in kvs:
+        blob += s(k) + struct.pack("<I", t) + v
+    for n, shape, typ, off in tensors:
+        blob += s(n) + struct.pack("<I", len(shape)) + b"".join(struct.pack("<Q", d) for d in shape)
+        blob += struct.pack("<IQ", typ, off)
+    p = tmp_path / name
+    p.write_bytes(blob + tail)
+    return str(p)
+
+
+def test_gguf_reader_rejects_what_the_reference_rejects(tmp_path):
+    with pytest.raises(InvalidDataError, match="Not a GGUF"):
+        GgufReader(_gguf(tmp_path, magic=0x12345678))
+    with pytest.raises(NotImplementedError, match="version 4"):
+        GgufReader(_gguf(tmp_path, version=4))
+    with pytest.raises(NotImplementedError, match="version 1"):
+        GgufReader(_gguf(tmp_path, version=1))
+    with pytest.raises(InvalidDataError, match="rank"):
+        GgufReader(_gguf(tmp_path, tensors=[("w", (), 12, 0)], tail=b"\0" * 64))
+    with pytest.raises(InvalidDataError, match="rank"):
+        GgufReader(_gguf(tmp_path, tensors=[("w", (1, 2, 3, 4, 5), 12, 0)], tail=b"\0" * 64))
+    with pytest.raises(InvalidDataError, match="alignment"):
+        GgufReader(_gguf(tmp_path, kvs=[("general.alignment", 4, struct.pack("<I", 24))]))
+    with pytest.raises(InvalidDataError, match="bool"):
+        GgufReader(_gguf(tmp_path, kvs=[("flag", 7, b"\x02")]))
+    with pytest.raises(NotImplementedError, match="metadata type"):
+        GgufReader(_gguf(tmp_path, kvs=[("k", 13, b"\0" * 8)]))
+    with pytest.raises(EOFError):
+        GgufReader(_gguf(tmp_path, kvs=[("k", 8, struct.pack("<Q", 1000) + b"abc")]))
+    with pytest.raises(EOFError):                      # the table cannot fit in the bytes that remain
+        GgufReader(_gguf(tmp_path, tensors=[("w", (), 12, 0)]))
+    with pytest.raises(InvalidDataError, match="too large"):
+        GgufReader(_gguf(tmp_path, kvs=[("k", 9, struct.pack("<IQ", 4, 5) + b"\0" * 20)]),
+                   GgufReadLimits(maximum_array_elements=4))
+    with pytest.raises(InvalidDataError, match="table"):
+        GgufReader(_gguf(tmp_path, tensors=[("a", (256,), 12, 0), ("b", (256,), 12, 0)]), GgufReadLimits(maximum_tensors=1))
+
+
+def test_gguf_reader_alignment_metadata_and_payload(tmp_path):
+    kvs = [("general.alignment", 4, struct.pack("<I", 64)), ("x.count", 10, struct.pack("<Q", 7)),
+           ("x.names", 9, struct.pack("<IQ", 8, 2) + struct.pack("<Q", 1) + b"a" + struct.pack("<Q", 2) + b"bc"),
+           ("x.f", 6, struct.pack("<f", 1.5)), ("x.ok", 7, b"\x01")]
+    path = _gguf(tmp_path, version=2, kvs=kvs, tensors=[("w", (256, 3), 12, 64)], tail=b"\0" * 64 + bytes(range(256)) * 4)
+    with GgufReader(path) as r:
+        assert r.version == 2 and r.data_offset % 64 == 0
+        assert r.metadata["x.count"] == 7 and r.metadata["x.names"] == ["a", "bc"] and r.metadata["x.ok"] is True
+        t = r.get_tensor("w")
+        assert t.byte_count() == 3 * 144 and r.matrix_dims(t) == (256, 3)
+        with pytest.raises(InvalidDataError):
+            nn.GgufTensorInfo("bad", (100, 3), 12, 0).byte_count()
+
+
+def test_synthetic_payload_generators():
+    from nntrain_amd import synth
+    import oracle
+    w = np.random.default_rng(0).standard_normal((4, 64)).astype(np.float32) * 0.02
+    raw = synth.quantize_q8_0(w)
+    assert raw.size == 4 * 2 * 34
+    back = oracle.dequantize(8, raw).reshape(4, 64)
+    d = raw.reshape(-1, 34)[:, :2].copy().view(np.float16).astype(np.float32).reshape(4, 2)
+    # half a quantisation step, plus up to 127 steps of the fp16 rounding of the scale (2^-11 relative)
+    assert np.all(np.abs(back - w).reshape(4, 2, 32) <= 0.57 * d[:, :, None] + 1e-9)
+    for typ in (12, 13, 14, 22):
+        p = synth.k_quant_matrix(typ, 5, 512, 3)
+        assert p.size == 5 * 2 * nn.BLOCK_BYTES[typ]
+        assert np.all(np.isfinite(oracle.dequantize(typ, p)))
+    assert np.array_equal(synth.to_bf16_bits(np.array([1.0, -2.0], np.float32)), np.array([0x3F80, 0xC000], np.uint16))
