@@ -16,6 +16,9 @@
 //   * unit partials go to LDS (one float per lane, double buffered); after the step's barrier one wave per row adds
 //     the row's partials in a fixed order (lane-strided, then a DPP butterfly) and stores y.  The order depends only
 //     on in_w, never on the launch geometry, so a row's result is bit-identical for any `rows`, out_w or batching.
+#include <cstring>
+#include <vector>
+
 #include "nnhip_internal.h"
 #include "quant_device.h"
 
@@ -461,6 +464,192 @@ void matvec_rowstep_kernel(MatvecArgs a, const float* __restrict__ bias)
     }
 }
 
+// ------------------------------------------------------------------------------------------- batched kernel
+// One entry of the device table of a batched launch (see matvec_batch_kernel for the chunk sequence).
+// Pointers read from a table are generic ("flat") to the device compiler; flat loads tick the LDS counter as well as
+// the vector-memory one.  The device pass therefore declares them as global-address-space pointers.
+#if defined(__HIP_DEVICE_COMPILE__)
+#define NNHIP_GLOBAL_PTR __attribute__((address_space(1)))
+#else
+#define NNHIP_GLOBAL_PTR
+#endif
+struct BatchEntry {
+    const NNHIP_GLOBAL_PTR float* x;
+    const NNHIP_GLOBAL_PTR uint8_t* w;
+    const NNHIP_GLOBAL_PTR float* bias;
+    NNHIP_GLOBAL_PTR float* y;
+    int in_w;
+    int out_w;
+    int upr;          // units per row
+    int rs;           // rows per step
+    int steps;
+    uint32_t row_bytes;
+    uint32_t magic;
+    int first_chunk;  // offset of the matrix in the global chunk sequence
+    int chunks;       // ceil(steps / DEPTH)
+    int pad_[2];
+};
+
+// Persistent form of matvec_rowstep_kernel: the weight prefetch runs ahead across matrix boundaries, so the stream
+// from HBM never drains between the mat-vecs of a batch.
+//
+// The steps of a matrix are grouped in chunks of DEPTH consecutive steps (the last chunk of a matrix may be short);
+// the chunks of all matrices form one global sequence and chunk j goes to workgroup j % G.  A chunk is exactly one turn
+// of the rotating register sets, so a workgroup can only change matrix at the top of a turn, and it stays with a
+// matrix for DEPTH steps even when the matrix has few rows (small matrices of a batch are worked on side by side by
+// different workgroups).
+//
+// On entering a matrix a lane re-derives its (row, unit) slot and swaps in that matrix' activations.  Those are
+// pumped ahead of time: once the staging area in LDS has been read by everyone, each step requests two float4 per lane
+// of the NEXT matrix' vector into a holding register pair and the following step moves them to LDS, so the vector is
+// usually complete when the reduction reaches that matrix and the switch costs one barrier and 16 LDS reads.  What the
+// pump did not get to is fetched at the switch (the stream stalls once).
+template <class Q>
+__global__ __launch_bounds__(Shape<Q>::kMaxT) __attribute__((amdgpu_waves_per_eu(Shape<Q>::kWavesPerEu, Shape<Q>::kWavesPerEu)))
+void matvec_batch_kernel(const BatchEntry* __restrict__ table, int total_chunks)
+{
+    constexpr int kDepth = Shape<Q>::kDepth;
+    __shared__ float part[2][kMaxWG];
+    __shared__ uint64_t grid[Q::kGrid ? 1024 : 1];
+    extern __shared__ float4 xstage[];
+
+    const int tid = threadIdx.x, T = blockDim.x, G = gridDim.x;
+    const int wave = tid >> 6, lane = tid & 63, waves = T >> 6;
+    if (Q::kGrid)
+        for (int i = tid; i < 1024; i += T) grid[i] = g_iq2s_grid[i];
+
+    auto uni = [](int v) { return __builtin_amdgcn_readfirstlane(v); };   // pins workgroup-uniform state to SGPRs
+    auto slot = [&](const BatchEntry& e, int& rl, int& c, bool& owner) {
+        rl = e.upr == 1 ? tid : static_cast<int>(__umulhi(static_cast<uint32_t>(tid), e.magic));
+        c = tid - rl * e.upr;
+        owner = rl < e.rs;
+    };
+    auto find = [&](int m, int chunk) {       // index of the entry that holds global chunk `chunk`, searching from m
+        while (chunk >= table[m].first_chunk + table[m].chunks) ++m;
+        return uni(m);
+    };
+
+    // ---- weight prefetch side: entry `fe`, this lane's slot in it, the chunk being fetched
+    int f_m = -1, f_rl = 0, f_c = 0, f_chunk = blockIdx.x;
+    bool f_owner = false;
+    BatchEntry fe{};
+    auto fetch_enter = [&]() {                 // called when f_chunk has moved to a new chunk
+        if (f_chunk < total_chunks && (f_m < 0 || f_chunk >= fe.first_chunk + fe.chunks)) {
+            f_m = find(f_m < 0 ? 0 : f_m + 1, f_chunk);
+            fe = table[f_m];
+            slot(fe, f_rl, f_c, f_owner);
+        }
+    };
+    auto fetch = [&](int d) {                  // step d of chunk f_chunk; past the end it re-reads a valid row
+        const int s = f_chunk < total_chunks ? (f_chunk - fe.first_chunk) * kDepth + d : 0;
+        const int row = f_owner ? min(s * fe.rs + f_rl, fe.out_w - 1) : 0;
+        return Q::load((const uint8_t*)(fe.w + static_cast<size_t>(row) * fe.row_bytes), f_c);
+    };
+
+    // ---- activation pump: matrix p_m is being staged in rounds of 2T pieces; `held` is the round in the holding pair
+    int p_m = -1, p_round = 0, p_rounds = 0, p_pieces = 0, held = -1;
+    const NNHIP_GLOBAL_PTR float4* p_x = nullptr;
+    float4 xh0 = make_float4(0.f, 0.f, 0.f, 0.f), xh1 = xh0;
+    bool staging_free = true;
+    auto pump_issue = [&]() {
+        const int base = p_round * 2 * T;
+        if (base + tid < p_pieces) xh0 = p_x[base + tid];
+        if (base + T + tid < p_pieces) xh1 = p_x[base + T + tid];
+        held = p_round;
+        p_round = uni(p_round + 1);
+    };
+    auto pump_store = [&]() {
+        const int L0 = held * 2 * T + tid, L1 = L0 + T;
+        if (L0 < p_pieces) xstage[L0 + (L0 >> 4)] = xh0;
+        if (L1 < p_pieces) xstage[L1 + (L1 >> 4)] = xh1;
+        held = -1;
+    };
+    auto pump_target = [&](int m) {
+        p_m = m;
+        p_x = (const NNHIP_GLOBAL_PTR float4*)table[m].x;
+        p_pieces = uni(table[m].in_w >> 2);
+        p_rounds = uni((p_pieces + 2 * T - 1) / (2 * T));
+        p_round = 0;
+        held = -1;
+    };
+    auto pump_beat = [&]() {
+        if (p_m >= 0) {
+            if (held >= 0) pump_store();
+            if (staging_free && p_round < p_rounds) pump_issue();
+        }
+    };
+
+    // ---- reduction side
+    int c_m = -1, c_rl = 0, c_c = 0, c_chunk = blockIdx.x;
+    bool c_owner = false;
+    BatchEntry ce{};
+    typename Q::X xr{};
+    int buf = 0;
+    auto enter = [&](int m) {
+        if (p_m != m) pump_target(m);        // nothing was pumped for this matrix (first matrix of the workgroup)
+        if (held >= 0) pump_store();
+        while (p_round < p_rounds) {          // what the pump did not get to: fetched here, the stream stalls
+            pump_issue();
+            pump_store();
+        }
+        c_m = m;
+        ce = table[m];
+        slot(ce, c_rl, c_c, c_owner);
+        __syncthreads();
+        xr = Q::load_x(xstage, c_owner ? c_c : 0);
+        staging_free = false;
+        // next matrix this workgroup will meet: its first chunk at or beyond the end of this matrix
+        p_m = -1;
+        const int end = ce.first_chunk + ce.chunks;
+        const int ahead = uni(c_chunk + (end - c_chunk + G - 1) / G * G);
+        if (ahead < total_chunks) pump_target(find(m + 1, ahead));
+    };
+    auto finish = [&](const typename Q::Regs& r, int d) {
+        const int st = (c_chunk - ce.first_chunk) * kDepth + d;
+        if (st < ce.steps) {                  // the last chunk of a matrix may be short (uniform)
+            part[buf][tid] = Q::dot(r, xr, c_c, grid);
+            __syncthreads();
+            staging_free = true;
+            for (int rr = wave; rr < ce.rs; rr += waves) {
+                const int row = st * ce.rs + rr;
+                if (row < ce.out_w) {
+                    float t = 0.0f;
+                    for (int u = lane; u < ce.upr; u += 64) t += part[buf][rr * ce.upr + u];
+                    t = wave_sum(t);
+                    const int urow = __builtin_amdgcn_readfirstlane(row);
+                    if (lane == 0) ce.y[urow] = (ce.bias ? ce.bias[urow] : 0.0f) + t;
+                }
+            }
+            buf ^= 1;
+        }
+    };
+
+    // One turn = one chunk.  At step d of the reduction the prefetch is kDepth - 1 steps ahead: steps d + kDepth - 1 of
+    // this chunk while they exist, then the first steps of the workgroup's next chunk.
+    typename Q::Regs regs[kDepth];
+    fetch_enter();
+#pragma unroll
+    for (int d = 0; d < kDepth - 1; ++d) regs[d] = fetch(d);
+    while (c_chunk < total_chunks) {
+        if (c_m < 0 || c_chunk >= ce.first_chunk + ce.chunks) enter(find(c_m < 0 ? 0 : c_m + 1, c_chunk));
+#pragma unroll
+        for (int d = 0; d < kDepth; ++d) {
+            if (d == 0) {
+                regs[kDepth - 1] = fetch(kDepth - 1);
+            } else {
+                if (d == 1) {
+                    f_chunk += G;
+                    fetch_enter();
+                }
+                regs[d - 1] = fetch(d - 1);
+            }
+            pump_beat();
+            finish(regs[d], d);
+        }
+        c_chunk += G;
+    }
+}
+
 // Slow path for Q8_0 rows with an odd number of blocks (row starts are then only 2-byte aligned and blocks cannot
 // be paired): one wave per output, lanes stride over single blocks.
 __global__ __launch_bounds__(256) void matvec_q8_0_oddrow_kernel(MatvecArgs a)
@@ -538,6 +727,36 @@ hipError_t launch_rowstep(Lane* lane, MatvecArgs args, int rows)
     return hipGetLastError();
 }
 
+
+// Builds the device table for the entries of one block format and launches the persistent kernel.
+template <class Q>
+hipError_t launch_batch_of(Lane* lane, int total_chunks, int max_in_w, size_t table_offset)
+{
+    const size_t lds = static_cast<size_t>(kChunkPieces) * (max_in_w / kUnitW) * sizeof(float4);
+    static bool big_lds_enabled = false;
+    if (lds > 48 * 1024 && !big_lds_enabled) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&matvec_batch_kernel<Q>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, kMaxDynamicLds);
+        if (e != hipSuccess) return e;
+        big_lds_enabled = true;
+    }
+    const BatchEntry* table = reinterpret_cast<const BatchEntry*>(static_cast<const char*>(lane->batch_table) + table_offset);
+    const int groups = total_chunks < lane->compute_units ? total_chunks : lane->compute_units;
+    hipLaunchKernelGGL(matvec_batch_kernel<Q>, dim3(groups), dim3(Shape<Q>::kMaxT), lds, lane->stream, table, total_chunks);
+    return hipGetLastError();
+}
+
+void shape_of(uint32_t type, int* max_t, int* depth)
+{
+    switch (type) {
+    case NNHIP_TYPE_Q8_0: *max_t = Shape<Q8_0Unit>::kMaxT; *depth = Shape<Q8_0Unit>::kDepth; break;
+    case NNHIP_TYPE_Q4_K: *max_t = Shape<Q4KUnit>::kMaxT; *depth = Shape<Q4KUnit>::kDepth; break;
+    case NNHIP_TYPE_Q5_K: *max_t = Shape<Q5KUnit>::kMaxT; *depth = Shape<Q5KUnit>::kDepth; break;
+    case NNHIP_TYPE_Q6_K: *max_t = Shape<Q6KUnit>::kMaxT; *depth = Shape<Q6KUnit>::kDepth; break;
+    default: *max_t = Shape<IQ2SUnit>::kMaxT; *depth = Shape<IQ2SUnit>::kDepth; break;
+    }
+}
+
 }  // namespace
 
 int matvec_max_in_w(uint32_t)
@@ -576,6 +795,104 @@ hipError_t launch_matvec(Lane* lane, uint32_t type, const float* x, const void* 
     case NNHIP_TYPE_IQ2_S: return launch_rowstep<IQ2SUnit>(lane, a, rows);
     default: return hipErrorInvalidValue;
     }
+}
+
+
+hipError_t launch_matvec_batch(Lane* lane, const nnhip_matvec_desc* descs, int count)
+{
+    static const uint32_t kTypes[5] = {NNHIP_TYPE_Q8_0, NNHIP_TYPE_Q4_K, NNHIP_TYPE_Q5_K, NNHIP_TYPE_Q6_K, NNHIP_TYPE_IQ2_S};
+    std::vector<BatchEntry> all;
+    struct Group { uint32_t type; size_t begin, end; int total_chunks, max_in_w; };
+    std::vector<Group> groups;
+    for (uint32_t type : kTypes) {
+        Group g{type, all.size(), all.size(), 0, 0};
+        int max_t = 0, depth = 0;
+        shape_of(type, &max_t, &depth);
+        for (int i = 0; i < count; ++i) {
+            const nnhip_matvec_desc& d = descs[i];
+            if (d.ggml_type != type) continue;
+            if (type == NNHIP_TYPE_Q8_0 && ((d.in_w / 32) & 1)) continue;   // launched one by one below
+            int elems = 0, bytes = 0;
+            type_block(type, &elems, &bytes);
+            const int upr = d.in_w / kUnitW;
+            int rs = max_t / upr;
+            if (rs > d.out_w) rs = d.out_w;
+            for (int r = 0; r < d.rows; ++r) {
+                BatchEntry e{};
+                e.x = (decltype(e.x))(d.x + static_cast<size_t>(r) * d.in_w);
+                e.w = (decltype(e.w))(d.w);
+                e.bias = (decltype(e.bias))(d.bias);
+                e.y = (decltype(e.y))(d.y + static_cast<size_t>(r) * d.out_w);
+                e.in_w = d.in_w;
+                e.out_w = d.out_w;
+                e.upr = upr;
+                e.rs = rs;
+                e.steps = (d.out_w + rs - 1) / rs;
+                e.row_bytes = static_cast<uint32_t>(d.in_w / elems) * static_cast<uint32_t>(bytes);
+                e.magic = static_cast<uint32_t>((0x100000000ull + upr - 1) / upr);
+                e.first_chunk = g.total_chunks;
+                e.chunks = (e.steps + depth - 1) / depth;
+                g.total_chunks += e.chunks;
+                if (d.in_w > g.max_in_w) g.max_in_w = d.in_w;
+                all.push_back(e);
+            }
+        }
+        g.end = all.size();
+        if (g.end > g.begin) groups.push_back(g);
+    }
+
+    // Upload the table unless it is the one already on the device.  The staging copy is pinned; a pending launch that
+    // still reads the old table is waited for before it is overwritten.
+    const size_t bytes = all.size() * sizeof(BatchEntry);
+    if (bytes) {
+        const bool same = lane->batch_table && bytes == lane->batch_table_used &&
+                          memcmp(lane->batch_table_host, all.data(), bytes) == 0;
+        if (!same) {
+            if (lane->capturing) return hipErrorStreamCaptureUnsupported;
+            hipError_t e = hipStreamSynchronize(lane->stream);
+            if (e != hipSuccess) return e;
+            if (bytes > lane->batch_table_bytes) {
+                if (lane->batch_table) (void)hipFree(lane->batch_table);
+                if (lane->batch_table_host) (void)hipHostFree(lane->batch_table_host);
+                lane->batch_table = nullptr;
+                lane->batch_table_host = nullptr;
+                lane->batch_table_bytes = 0;
+                const size_t cap = bytes * 2;
+                e = hipMalloc(&lane->batch_table, cap);
+                if (e != hipSuccess) return e;
+                e = hipHostMalloc(&lane->batch_table_host, cap, hipHostMallocDefault);
+                if (e != hipSuccess) return e;
+                lane->batch_table_bytes = cap;
+            }
+            memcpy(lane->batch_table_host, all.data(), bytes);
+            lane->batch_table_used = bytes;
+            e = hipMemcpyAsync(lane->batch_table, lane->batch_table_host, bytes, hipMemcpyHostToDevice, lane->stream);
+            if (e != hipSuccess) return e;
+        }
+    }
+
+    for (const Group& g : groups) {
+        hipError_t e = hipSuccess;
+        const size_t off = g.begin * sizeof(BatchEntry);
+        switch (g.type) {
+        case NNHIP_TYPE_Q8_0: e = launch_batch_of<Q8_0Unit>(lane, g.total_chunks, g.max_in_w, off); break;
+        case NNHIP_TYPE_Q4_K: e = launch_batch_of<Q4KUnit>(lane, g.total_chunks, g.max_in_w, off); break;
+        case NNHIP_TYPE_Q5_K: e = launch_batch_of<Q5KUnit>(lane, g.total_chunks, g.max_in_w, off); break;
+        case NNHIP_TYPE_Q6_K: e = launch_batch_of<Q6KUnit>(lane, g.total_chunks, g.max_in_w, off); break;
+        default: e = launch_batch_of<IQ2SUnit>(lane, g.total_chunks, g.max_in_w, off); break;
+        }
+        if (e != hipSuccess) return e;
+        lane->counters.kernel_launches += 1;
+    }
+    for (int i = 0; i < count; ++i) {
+        const nnhip_matvec_desc& d = descs[i];
+        if (d.ggml_type == NNHIP_TYPE_Q8_0 && ((d.in_w / 32) & 1)) {
+            hipError_t e = launch_matvec(lane, d.ggml_type, d.x, d.w, d.bias, d.y, d.rows, d.in_w, d.out_w);
+            if (e != hipSuccess) return e;
+            lane->counters.kernel_launches += 1;
+        }
+    }
+    return hipSuccess;
 }
 
 }  // namespace nnhip

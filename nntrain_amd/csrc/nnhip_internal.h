@@ -25,7 +25,8 @@ struct Lane {
     std::unordered_map<void*, size_t> buffers;  // device allocations still owned by the lane
     std::mutex mutex;                           // guards buffers + counters (uploads may come from loader threads)
     void* batch_table = nullptr;                // device copy of the descriptor table of the last batch launch
-    size_t batch_table_bytes = 0;
+    size_t batch_table_bytes = 0;               // capacity of both copies
+    size_t batch_table_used = 0;                // bytes of the table that is on the device now
     void* batch_table_host = nullptr;           // pinned staging for the table
 };
 

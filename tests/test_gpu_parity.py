@@ -263,3 +263,50 @@ def test_matvec_full_size_configs(lane, name, typ, in_w, out_w, wseed, xseed):
     ref, asum = oracle.linear_f64(typ, payload, x, None, 1, in_w, out_w)
     _check_against_f64(y, ref, asum)
     print(f"{name}: rel_l2 vs f64 = {oracle.rel_l2(y, ref):.3e}")
+
+
+# ----------------------------------------------------------------------------------------------- batched launch
+
+def test_matvec_batch_equals_single_launches_bitwise(lane):
+    """A batch (mixed formats, tiny and long matrices, rows > 1, bias) must reproduce per-matrix launches bit for bit."""
+    from ctypes import c_void_p
+    from nntrain_amd.native import MatvecDesc, check
+    rng = np.random.default_rng(2024)
+    shapes = [(GGML_Q8_0, 5376, 300, 1), (GGML_Q8_0, 4096, 37, 1), (GGML_Q8_0, 21504, 90, 1), (GGML_Q8_0, 64, 5, 2),
+              (GGML_Q4_K, 5120, 260, 1), (GGML_Q4_K, 256, 3, 3), (GGML_Q6_K, 1024, 130, 1), (GGML_Q5_K, 2048, 77, 1),
+              (GGML_IQ2_S, 17408, 40, 1), (GGML_Q8_0, 5376, 4100, 1), (GGML_Q8_0, 160, 9, 1), (GGML_Q4_K, 5120, 1, 1)]
+    items = []
+    for i, (typ, in_w, out_w, rows) in enumerate(shapes):
+        payload = _random_payload(typ, out_w, in_w, seed=900 + i)
+        x = rng.standard_normal((rows, in_w)).astype(np.float32)
+        bias = rng.standard_normal(out_w).astype(np.float32) if i % 2 else None
+        wb = lane.upload_raw(payload)
+        xb = lane.upload_raw(x)
+        bb = lane.upload_raw(bias) if bias is not None else None
+        y1 = lane.allocate(rows * out_w + 2)
+        y2 = lane.allocate(rows * out_w + 2)
+        lane.fill_u32(y1, NAN_BITS, rows * out_w + 2)
+        lane.fill_u32(y2, NAN_BITS, rows * out_w + 2)
+        items.append((typ, in_w, out_w, rows, payload, x, bias, wb, xb, bb, y1, y2))
+    lib, h = lane._lib, lane._handle
+    for typ, in_w, out_w, rows, payload, x, bias, wb, xb, bb, y1, y2 in items:
+        check(lib.nnhip_quant_matvec(h, typ, c_void_p(xb.ptr), c_void_p(wb.ptr), c_void_p(bb.ptr) if bb else None,
+                                     c_void_p(y1.ptr), rows, in_w, out_w), "quant_matvec")
+    descs = (MatvecDesc * len(items))()
+    for i, (typ, in_w, out_w, rows, payload, x, bias, wb, xb, bb, y1, y2) in enumerate(items):
+        descs[i] = MatvecDesc(xb.ptr, wb.ptr, bb.ptr if bb else None, y2.ptr, typ, rows, in_w, out_w)
+    for _ in range(2):      # the second call reuses the device table
+        check(lib.nnhip_quant_matvec_batch(h, descs, len(items)), "quant_matvec_batch")
+    lane.synchronize()
+    for typ, in_w, out_w, rows, payload, x, bias, wb, xb, bb, y1, y2 in items:
+        a, b = lane.read(y1), lane.read(y2)
+        assert np.isnan(b[-1]) and np.isnan(b[-2])
+        assert np.array_equal(_bits(a[:-2]), _bits(b[:-2])), (typ, in_w, out_w, rows)
+        ref, asum = oracle.linear_f64(typ, payload, x, bias, rows, in_w, out_w)
+        _check_against_f64(b[:-2].reshape(rows, out_w), ref, asum)
+    assert lib.nnhip_quant_matvec_batch(h, descs, 0) == 0
+    assert lib.nnhip_quant_matvec_batch(h, None, 3) == 1
+    for it in items:
+        for b in it[7:]:
+            if b is not None:
+                b.dispose()
