@@ -310,3 +310,60 @@ def test_matvec_batch_equals_single_launches_bitwise(lane):
         for b in it[7:]:
             if b is not None:
                 b.dispose()
+
+
+# ----------------------------------------------------------------------------------------------- prefill mat-mul
+
+PREFILL_BAR = 2e-3      # relative L2 against the float64 oracle fed the same bf16 activation bits
+
+
+@pytest.mark.parametrize("rows,in_w,out_w", [(16, 256, 16), (33, 512, 100), (128, 1024, 81), (200, 768, 160),
+                                             (512, 1024, 300), (700, 512, 75)])
+def test_prefill_matmul_q4k_vs_oracle(lane, rows, in_w, out_w):
+    payload = synth.k_quant_matrix(GGML_Q4_K, out_w, in_w, seed=rows + in_w + out_w)
+    xb = synth.to_bf16_bits(synth.activations(rows, in_w, seed=17))
+    bias = np.random.default_rng(5).standard_normal(out_w).astype(np.float32) * np.float32(0.01)
+    mat = HipQuantizedMatrix(payload, GGML_Q4_K, out_w, in_w)
+    x = lane.upload_raw(xb)
+    b = lane.upload_raw(bias)
+    y = lane.allocate(rows * out_w + 2)
+    lane.fill_u32(y, NAN_BITS, rows * out_w + 2)
+    mat.forward_bf16(lane, x, b, rows, out=y)
+    lane.synchronize()
+    got = lane.read(y)
+    assert np.isnan(got[-1]) and np.isnan(got[-2])
+    got = got[:-2].reshape(rows, out_w)
+    assert np.all(np.isfinite(got))
+    ref, _ = oracle.linear_f64(GGML_Q4_K, payload, xb, bias, rows, in_w, out_w, x_is_bf16=True)
+    rel = oracle.rel_l2(got, ref)
+    assert rel <= PREFILL_BAR, rel
+    for buf in (x, b, y):
+        buf.dispose()
+    mat.dispose()
+
+
+def test_prefill_matmul_rejects_other_types(lane):
+    mat = HipQuantizedMatrix(np.zeros(34 * 8, np.uint8), GGML_Q8_0, 1, 256)
+    x = lane.allocate(256)
+    with pytest.raises(NnHipError) as e:
+        mat.forward_bf16(lane, x, None, 1)
+    assert e.value.status == 2
+    x.dispose()
+    mat.dispose()
+
+
+def test_prefill_matmul_full_width_sample(lane):
+    """BASELINE prefill shape at M = 128: every output of 16 sampled rows against the oracle."""
+    in_w, out_w, rows = 5120, 17408, 128
+    payload = synth.matrix(GGML_Q4_K, out_w, in_w, 2001)
+    xb = synth.to_bf16_bits(synth.activations(rows, in_w, 4000))
+    mat = HipQuantizedMatrix(payload, GGML_Q4_K, out_w, in_w)
+    x = lane.upload_raw(xb)
+    got = lane.read(mat.forward_bf16(lane, x, None, rows)).reshape(rows, out_w)
+    pick = np.arange(0, rows, 8)
+    ref, _ = oracle.linear_f64(GGML_Q4_K, payload, xb[pick], None, len(pick), in_w, out_w, x_is_bf16=True)
+    rel = oracle.rel_l2(got[pick], ref)
+    print(f"prefill 128x5120x17408 rel-L2 = {rel:.3e}")
+    assert rel <= PREFILL_BAR
+    x.dispose()
+    mat.dispose()
