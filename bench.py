@@ -28,6 +28,10 @@ sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 BF16_PEAK_TFLOPS = 2500.0      # MI355X dense bf16 MFMA, published
+# HBM bytes one batched launch of the decode27b set moves, from two rocprofv3 --pmc runs (FETCH_SIZE x 2.000 and
+# WRITE_SIZE x 1.000, the factors a plain copy kernel of known size gives); summary in
+# profiles/matvec_batch_q8_0_decode27b_hbm_traffic.md.  Only valid for --mode batch.
+DECODE27B_BATCH_TRAFFIC_BYTES = 29_106_670_696
 
 
 def log(*a):
@@ -159,6 +163,15 @@ def run_decode27b(args, lane, nn, oracle):
             raise SystemExit(f"parity failure ({tag}): rel-L2 {worst:.3e} > 1e-5")
         return worst
 
+    if args.copy_calibration:
+        # a plain device-to-device copy of known size, so that a counter run (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)
+        # of this same command can scale the counters by what they read for it
+        n = weights[-1].nbytes
+        scratch = lane.allocate_bytes(n)
+        lane.copy(scratch, weights[-1], n)
+        lane.synchronize()
+        scratch.dispose()
+        log(f"[decode27b] calibration copy of {n} bytes done")
     for _ in range(max(args.warmup, 1)):
         token()
     lane.synchronize()
@@ -186,8 +199,9 @@ def run_decode27b(args, lane, nn, oracle):
                                "28,695,625,728 weight bytes/token resident in HBM, batch 1, fp32 activations",
                    "launch": args.mode, "launches_per_token": n_launch},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "matvec_rowstep_kernel<Q8_0Unit>",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4),
+                     "traffic": DECODE27B_BATCH_TRAFFIC_BYTES if args.mode == "batch" else None,
+                     "kernel": "matvec_batch_kernel<Q8_0Unit>" if args.mode == "batch" else "matvec_rowstep_kernel<Q8_0Unit>",
                      "bytes_per_launch": total_bytes // n_launch},
         "cpu_baseline": cpu,
         "parity": {"rel_l2_vs_f64_oracle_sampled": rel, "bar": 1e-5},
@@ -335,6 +349,8 @@ def main():
     ap.add_argument("--mode", choices=["forward", "graph", "batch"], default="batch",
                     help="decode27b: one launch per matrix, the same captured in a HIP graph, or the batched entry point")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="decode27b: also run one device-to-device copy of the lm_head weights (for counter runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("this build measures one GPU: the quantized linear path has no collectives and every box has a "
