@@ -373,13 +373,15 @@ struct IQ2SUnit {
 
 // ---------------------------------------------------------------------------------------------- the kernel
 // Launch shape of one block format: lanes per workgroup, waves per SIMD the register budget is sized for, and the
-// number of weight register sets that rotate (DEPTH - 1 row steps are in flight while one is reduced).
+// number of weight register sets that rotate (DEPTH - 1 row steps are in flight while one is reduced): kDepth for a
+// single mat-vec, kBatchDepth for the persistent batched kernel.  More bytes in flight than the memory system needs
+// to cover its latency lowers the rate it sustains, so the single launch keeps the ring short.
 template <class Q> struct Shape;
-template <> struct Shape<Q8_0Unit> { static constexpr int kMaxT = 768, kWavesPerEu = 3, kDepth = 3; };
-template <> struct Shape<Q4KUnit> { static constexpr int kMaxT = 1024, kWavesPerEu = 4, kDepth = 3; };
-template <> struct Shape<Q5KUnit> { static constexpr int kMaxT = 768, kWavesPerEu = 3, kDepth = 3; };
-template <> struct Shape<Q6KUnit> { static constexpr int kMaxT = 768, kWavesPerEu = 3, kDepth = 4; };
-template <> struct Shape<IQ2SUnit> { static constexpr int kMaxT = 1024, kWavesPerEu = 4, kDepth = 4; };
+template <> struct Shape<Q8_0Unit> { static constexpr int kMaxT = 768, kWavesPerEu = 3, kDepth = 2, kBatchDepth = 3; };
+template <> struct Shape<Q4KUnit> { static constexpr int kMaxT = 1024, kWavesPerEu = 4, kDepth = 3, kBatchDepth = 3; };
+template <> struct Shape<Q5KUnit> { static constexpr int kMaxT = 768, kWavesPerEu = 3, kDepth = 3, kBatchDepth = 3; };
+template <> struct Shape<Q6KUnit> { static constexpr int kMaxT = 768, kWavesPerEu = 3, kDepth = 2, kBatchDepth = 4; };
+template <> struct Shape<IQ2SUnit> { static constexpr int kMaxT = 1024, kWavesPerEu = 4, kDepth = 2, kBatchDepth = 4; };
 
 // grid.x = workgroups striding over row steps, grid.y = input rows, blockDim.x = T (a multiple of 64).
 template <class Q>
@@ -508,7 +510,7 @@ template <class Q>
 __global__ __launch_bounds__(Shape<Q>::kMaxT) __attribute__((amdgpu_waves_per_eu(Shape<Q>::kWavesPerEu, Shape<Q>::kWavesPerEu)))
 void matvec_batch_kernel(const BatchEntry* __restrict__ table, int total_chunks)
 {
-    constexpr int kDepth = Shape<Q>::kDepth;
+    constexpr int kDepth = Shape<Q>::kBatchDepth;
     __shared__ float part[2][kMaxWG];
     __shared__ uint64_t grid[Q::kGrid ? 1024 : 1];
     extern __shared__ float4 xstage[];
@@ -749,11 +751,11 @@ hipError_t launch_batch_of(Lane* lane, int total_chunks, int max_in_w, size_t ta
 void shape_of(uint32_t type, int* max_t, int* depth)
 {
     switch (type) {
-    case NNHIP_TYPE_Q8_0: *max_t = Shape<Q8_0Unit>::kMaxT; *depth = Shape<Q8_0Unit>::kDepth; break;
-    case NNHIP_TYPE_Q4_K: *max_t = Shape<Q4KUnit>::kMaxT; *depth = Shape<Q4KUnit>::kDepth; break;
-    case NNHIP_TYPE_Q5_K: *max_t = Shape<Q5KUnit>::kMaxT; *depth = Shape<Q5KUnit>::kDepth; break;
-    case NNHIP_TYPE_Q6_K: *max_t = Shape<Q6KUnit>::kMaxT; *depth = Shape<Q6KUnit>::kDepth; break;
-    default: *max_t = Shape<IQ2SUnit>::kMaxT; *depth = Shape<IQ2SUnit>::kDepth; break;
+    case NNHIP_TYPE_Q8_0: *max_t = Shape<Q8_0Unit>::kMaxT; *depth = Shape<Q8_0Unit>::kBatchDepth; break;
+    case NNHIP_TYPE_Q4_K: *max_t = Shape<Q4KUnit>::kMaxT; *depth = Shape<Q4KUnit>::kBatchDepth; break;
+    case NNHIP_TYPE_Q5_K: *max_t = Shape<Q5KUnit>::kMaxT; *depth = Shape<Q5KUnit>::kBatchDepth; break;
+    case NNHIP_TYPE_Q6_K: *max_t = Shape<Q6KUnit>::kMaxT; *depth = Shape<Q6KUnit>::kBatchDepth; break;
+    default: *max_t = Shape<IQ2SUnit>::kMaxT; *depth = Shape<IQ2SUnit>::kBatchDepth; break;
     }
 }
 

@@ -1,6 +1,6 @@
 """ctypes binding of libnnhip.so - one declaration per entry point of include/nnhip.h.
 
-This is the Python counterpart of the LibraryImport class a C# maintainer adds to NNtrain;
+This is the Python counterpart of the LibraryImport class a C# maintainer adds to NNtrain (bindings/csharp/NnHipNative.cs);
 it declares argument types only and converts non-zero statuses to exceptions the way OpenClNative.Check does
 (NNtrain.Arc/OpenClNative.cs:37-41).
 """
