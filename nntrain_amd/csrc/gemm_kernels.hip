@@ -2,19 +2,21 @@
 //
 // Replaces the XMX prefill launch of the reference (NNtrain.Arc/Kernels/qwen35_prefill_xmx.cl:112-184): weight tiles
 // are dequantized to bfloat16 in LDS and contracted on the matrix cores (v_mfma_f32_16x16x32_bf16) with FP32
-// accumulators.  The FP32 dequantization formula and rounding order are those of the CPU decoder
-// ((d*sc)*q - dmin*m, NNtrain.Core/Serialization/GgufQ4K.cs:34-41); the only rounding added is FP32 -> bf16 of the
-// weight, which is what the 2e-3 relative-L2 bar of this path allows for.
+// accumulators.  The weight is the CPU decoder's (d*sc)*q - dmin*m (NNtrain.Core/Serialization/GgufQ4K.cs:34-41)
+// evaluated in FP32 and rounded once to bf16, which is what the 2e-3 relative-L2 bar of this path allows for.
 //
-// Tiling.  A workgroup of 8 waves owns BM = 8 * RW rows (RW = 16, 32 or 64 rows per wave) and a strip of up to 80
-// output columns for the whole K range; the strip width is chosen on the host so that the strips split N evenly over
-// the compute units (17408 columns -> 256 strips of 68).  Every wave spans the whole strip, so a weight sub-block
-// is dequantized once per workgroup.  K advances in steps of 32 = one Q4_K sub-block per weight row:
-//   - x tile  [BM][32] bf16 and weight tile [80][32] bf16 live in LDS, double buffered (rows are 64 bytes, so the 16
-//     rows x 4 k-groups an MFMA operand needs form one contiguous, conflict-free 1 KiB read);
-//   - while the MFMAs of step i run, the x tile of step i+1 travels global -> registers -> LDS and threads
-//     0 .. 4*cols-1 each decode 8 weights of step i+1 (one 8-byte load of nibbles plus the block header);
-//   - one barrier per step.
+// Tiling.  A workgroup of 8 waves owns BM = 8 * RW rows (RW = 16 or 32 rows per wave) and a strip of up to 16 * CT
+// output columns (CT = 5 or 9 column tiles) for the whole K range; the strip width is chosen on the host so that
+// strips x row tiles split evenly over the compute units (17408 columns: 256 strips of 68 for M <= 256, 128 strips of
+// 136 for larger M).  Every wave spans the whole strip, so a weight sub-block is dequantized once per workgroup.
+// K advances 64 per iteration = the two Q4_K sub-blocks that share 32 bytes of nibbles:
+//   - per iteration two x sub-tiles [BM][32] bf16 and two weight sub-tiles [16 CT][32] bf16 live in LDS, double
+//     buffered (rows are 64 bytes, so the 16 rows x 4 k-groups an MFMA operand needs form one contiguous,
+//     conflict-free 1 KiB read);
+//   - while the MFMAs of iteration i run, the x tile of iteration i+1 travels global -> registers -> LDS and each
+//     thread decodes up to two weight items of iteration i+1 (8 bytes of nibbles -> 8 low-nibble and 8 high-nibble
+//     weights, plus the block header);
+//   - one barrier per iteration.
 #include "nnhip_internal.h"
 #include "quant_device.h"
 
@@ -26,8 +28,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kGemmThreads = 512;
-constexpr int kMaxCols = 80;            // five 16-column MFMA tiles
-constexpr int kRowBytes = 64;           // one tile row: 32 bf16
+constexpr int kRowBytes = 64;           // one sub-tile row: 32 bf16
 
 struct GemmArgs {
     const uint16_t* x;     // bf16 [M, K]
@@ -35,7 +36,7 @@ struct GemmArgs {
     const float* bias;
     float* y;
     int M, K, N;
-    int cols;              // strip width actually used, <= 80
+    int cols;              // strip width actually used, <= 16 * CT
     int strips;            // ceil(N / cols)
 };
 
@@ -47,116 +48,152 @@ __device__ __forceinline__ uint32_t pack_bf16(float a, float b)
     return __builtin_bit_cast(uint32_t, v);
 }
 
-template <int RW>
+// 6-bit scale and min of sub-block g from the three dwords holding the 12 packed bytes (GgufQ4K.cs:51-60).
+__device__ __forceinline__ void q4k_scale_min(uint32_t s0, uint32_t s1, uint32_t s2, int g, uint32_t& sc, uint32_t& mn)
+{
+    const int sh = (g & 3) * 8;
+    if (g < 4) {
+        sc = (s0 >> sh) & 63u;
+        mn = (s1 >> sh) & 63u;
+    } else {
+        sc = ((s2 >> sh) & 15u) | ((((s0 >> sh) >> 6) & 3u) << 4);
+        mn = (((s2 >> sh) >> 4) & 15u) | ((((s1 >> sh) >> 6) & 3u) << 4);
+    }
+}
+
+__device__ __forceinline__ u32x4 q4k_decode8(uint32_t q_lo, uint32_t q_hi, float scale, float mnv)
+{
+    // eight weights (d*sc)*q - dmin*m as one fused multiply-add each (the bf16 rounding that follows is 2^16 times
+    // coarser than the difference to the separately rounded form), packed to bf16 two at a time
+    q_lo = opaque(q_lo);
+    q_hi = opaque(q_hi);
+    const float w0 = fmaf(scale, ubyte0(q_lo), -mnv), w1 = fmaf(scale, ubyte1(q_lo), -mnv);
+    const float w2 = fmaf(scale, ubyte2(q_lo), -mnv), w3 = fmaf(scale, ubyte3(q_lo), -mnv);
+    const float w4 = fmaf(scale, ubyte0(q_hi), -mnv), w5 = fmaf(scale, ubyte1(q_hi), -mnv);
+    const float w6 = fmaf(scale, ubyte2(q_hi), -mnv), w7 = fmaf(scale, ubyte3(q_hi), -mnv);
+    return u32x4{pack_bf16(w0, w1), pack_bf16(w2, w3), pack_bf16(w4, w5), pack_bf16(w6, w7)};
+}
+
+template <int RW, int CT>
 __global__ __launch_bounds__(kGemmThreads) void matmul_q4k_bf16_kernel(GemmArgs a)
 {
     constexpr int BM = 8 * RW;
     constexpr int MT = RW / 16;                     // 16-row MFMA tiles per wave
-    constexpr int kXLoads = BM * kRowBytes / 16 / kGemmThreads;   // 16-byte pieces of the x tile per thread
+    constexpr int BN = 16 * CT;
+    constexpr int kXLoads = BM * 2 * kRowBytes / 16 / kGemmThreads;   // 16-byte pieces of the two x sub-tiles per thread
+    constexpr int kItems = (4 * BN + kGemmThreads - 1) / kGemmThreads;  // weight items (row, quarter) per thread
     static_assert(kXLoads >= 1, "tile too small for the thread count");
-    __shared__ __attribute__((aligned(16))) uint8_t xs[2][BM * kRowBytes];
-    __shared__ __attribute__((aligned(16))) uint8_t ws[2][kMaxCols * kRowBytes];
+    // [buffer][k sub-tile][row][32 bf16]
+    __shared__ __attribute__((aligned(16))) uint8_t xs[2][2][BM * kRowBytes];
+    __shared__ __attribute__((aligned(16))) uint8_t ws[2][2][BN * kRowBytes];
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int strip = blockIdx.x, m0 = blockIdx.y * BM;
     const int n0 = strip * a.cols;
     const int row_bytes = (a.K >> 8) * 144;
 
-    // x tile piece p of this thread: row p / 4 of the tile, 16-byte group p % 4
+    // x piece p of this thread: row p / 8 of the tile, 16-byte group p % 8 of the 64-value K slice
     const uint16_t* xsrc[kXLoads];
     int xdst[kXLoads];
 #pragma unroll
     for (int i = 0; i < kXLoads; ++i) {
         const int p = tid + i * kGemmThreads;
-        const int r = min(m0 + (p >> 2), a.M - 1);
-        xsrc[i] = a.x + static_cast<size_t>(r) * a.K + (p & 3) * 8;
-        xdst[i] = p * 16;
+        const int r = p >> 3, grp = p & 7;
+        xsrc[i] = a.x + static_cast<size_t>(min(m0 + r, a.M - 1)) * a.K + grp * 8;
+        xdst[i] = (grp >> 2) * (BM * kRowBytes) + r * kRowBytes + (grp & 3) * 16;
     }
-    // weight item of this thread: column tid / 4 of the strip, quarter tid % 4 of the sub-block
-    const bool decoder = tid < 4 * kMaxCols;
-    const int wn = tid >> 2, wq = tid & 3;
-    const uint8_t* wrow = a.w + static_cast<size_t>(min(n0 + wn, a.N - 1)) * row_bytes;
+    // weight item it of this thread: column (tid + it * 512) / 4 of the strip, quarter (tid + it * 512) % 4
+    const uint8_t* wrow[kItems];
+    int wdst[kItems], wqoff[kItems];
+    bool wact[kItems];
+#pragma unroll
+    for (int it = 0; it < kItems; ++it) {
+        const int id = tid + it * kGemmThreads;
+        const int wn = id >> 2, wq = id & 3;
+        wact[it] = id < 4 * BN;
+        wrow[it] = a.w + static_cast<size_t>(min(n0 + wn, a.N - 1)) * row_bytes;
+        wqoff[it] = wq * 8;
+        wdst[it] = wn * kRowBytes + wq * 16;
+    }
 
     u32x4 xreg[kXLoads];
-    u32x4 hdr{};
-    u32x2 qs{};
+    u32x4 hdr[kItems];
+    u32x2 qs[kItems];
     auto load_step = [&](int k0) {
 #pragma unroll
         for (int i = 0; i < kXLoads; ++i) xreg[i] = *reinterpret_cast<const u32x4*>(xsrc[i] + k0);
-        if (decoder) {
-            const uint8_t* blk = wrow + (k0 >> 8) * 144;
-            const int g = (k0 >> 5) & 7;
-            hdr = *reinterpret_cast<const u32x4*>(blk);
-            qs = *reinterpret_cast<const u32x2*>(blk + 16 + (g >> 1) * 32 + wq * 8);
+#pragma unroll
+        for (int it = 0; it < kItems; ++it) {
+            if (wact[it]) {
+                const uint8_t* blk = wrow[it] + (k0 >> 8) * 144;
+                hdr[it] = *reinterpret_cast<const u32x4*>(blk);
+                qs[it] = *reinterpret_cast<const u32x2*>(blk + 16 + ((k0 >> 6) & 3) * 32 + wqoff[it]);
+            }
         }
     };
     auto store_step = [&](int k0, int buf) {
 #pragma unroll
-        for (int i = 0; i < kXLoads; ++i) *reinterpret_cast<u32x4*>(&xs[buf][xdst[i]]) = xreg[i];
-        if (decoder) {
-            const int g = (k0 >> 5) & 7;
-            const float d = half_bits_to_float(hdr[0]), dmin = half_bits_to_float(hdr[0] >> 16);
-            // 6-bit scale and min of sub-block g from the 12 packed bytes (GgufQ4K.cs:51-60)
-            const uint32_t s0 = hdr[1], s1 = hdr[2], s2 = hdr[3];
-            const int sh = (g & 3) * 8;
-            uint32_t sc, mn;
-            if (g < 4) {
-                sc = (s0 >> sh) & 63u;
-                mn = (s1 >> sh) & 63u;
-            } else {
-                sc = ((s2 >> sh) & 15u) | (((s0 >> sh) >> 6 & 3u) << 4);
-                mn = ((s2 >> sh) >> 4 & 15u) | (((s1 >> sh) >> 6 & 3u) << 4);
-            }
-            const float scale = d * static_cast<float>(sc);
-            const float mnv = dmin * static_cast<float>(mn);
-            const int nib = (g & 1) * 4;
-            uint32_t out[4];
+        for (int i = 0; i < kXLoads; ++i) *reinterpret_cast<u32x4*>(&xs[buf][0][0] + xdst[i]) = xreg[i];
+        const int g = (k0 >> 5) & 7;      // even: sub-blocks g (low nibbles) and g + 1 (high nibbles)
 #pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                const uint32_t q4 = (qs[h] >> nib) & 0x0f0f0f0fu;
-                const float w0 = __fsub_rn(__fmul_rn(scale, ubyte0(q4)), mnv), w1 = __fsub_rn(__fmul_rn(scale, ubyte1(q4)), mnv);
-                const float w2 = __fsub_rn(__fmul_rn(scale, ubyte2(q4)), mnv), w3 = __fsub_rn(__fmul_rn(scale, ubyte3(q4)), mnv);
-                out[2 * h] = pack_bf16(w0, w1);
-                out[2 * h + 1] = pack_bf16(w2, w3);
+        for (int it = 0; it < kItems; ++it) {
+            if (wact[it]) {
+                const float d = half_bits_to_float(hdr[it][0]), dmin = half_bits_to_float(hdr[it][0] >> 16);
+                uint32_t sc0, mn0, sc1, mn1;
+                q4k_scale_min(hdr[it][1], hdr[it][2], hdr[it][3], g, sc0, mn0);
+                q4k_scale_min(hdr[it][1], hdr[it][2], hdr[it][3], g + 1, sc1, mn1);
+                const uint32_t a0 = qs[it][0], a1 = qs[it][1];
+                const u32x4 lo = q4k_decode8(a0 & 0x0f0f0f0fu, a1 & 0x0f0f0f0fu, d * static_cast<float>(sc0), dmin * static_cast<float>(mn0));
+                const u32x4 hi = q4k_decode8((a0 >> 4) & 0x0f0f0f0fu, (a1 >> 4) & 0x0f0f0f0fu, d * static_cast<float>(sc1), dmin * static_cast<float>(mn1));
+                *reinterpret_cast<u32x4*>(&ws[buf][0][wdst[it]]) = lo;
+                *reinterpret_cast<u32x4*>(&ws[buf][1][wdst[it]]) = hi;
             }
-            const u32x4 v = {out[0], out[1], out[2], out[3]};
-            *reinterpret_cast<u32x4*>(&ws[buf][wn * kRowBytes + wq * 16]) = v;
         }
     };
 
-    f32x4 acc[MT][5];
+    f32x4 acc[MT][CT];
 #pragma unroll
     for (int i = 0; i < MT; ++i)
 #pragma unroll
-        for (int j = 0; j < 5; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-    load_step(0);
-    store_step(0, 0);
-    __syncthreads();
+        for (int j = 0; j < CT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     // operand address of this lane inside a 16-row tile: row lane % 16, k-group lane / 16
     const int frag = (lane & 15) * kRowBytes + (lane >> 4) * 16;
-    int buf = 0;
-    for (int k0 = 0; k0 < a.K; k0 += 32) {
-        const bool more = k0 + 32 < a.K;
-        if (more) load_step(k0 + 32);
-        bf16x8 bfrag[5];
+    auto mfma_step = [&](int buf) {
 #pragma unroll
-        for (int j = 0; j < 5; ++j) bfrag[j] = *reinterpret_cast<const bf16x8*>(&ws[buf][j * 16 * kRowBytes + frag]);
+        for (int sub = 0; sub < 2; ++sub) {
+            bf16x8 afrag[MT];
 #pragma unroll
-        for (int i = 0; i < MT; ++i) {
-            const bf16x8 afrag = *reinterpret_cast<const bf16x8*>(&xs[buf][(wave * RW + i * 16) * kRowBytes + frag]);
+            for (int i = 0; i < MT; ++i)
+                afrag[i] = *reinterpret_cast<const bf16x8*>(&xs[buf][sub][(wave * RW + i * 16) * kRowBytes + frag]);
 #pragma unroll
-            for (int j = 0; j < 5; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag, bfrag[j], acc[i][j], 0, 0, 0);
+            for (int j = 0; j < CT; ++j) {
+                const bf16x8 bfrag = *reinterpret_cast<const bf16x8*>(&ws[buf][sub][j * 16 * kRowBytes + frag]);
+#pragma unroll
+                for (int i = 0; i < MT; ++i)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[i], bfrag, acc[i][j], 0, 0, 0);
+            }
         }
-        if (more) store_step(k0 + 32, buf ^ 1);
+    };
+
+    // Iteration i: request the data of iteration i + 1, contract iteration i from LDS, decode iteration i + 1 into the
+    // other LDS buffer.
+    load_step(0);
+    store_step(0, 0);
+    __syncthreads();
+    int buf = 0;
+    for (int k0 = 0; k0 < a.K; k0 += 64) {
+        const bool more = k0 + 64 < a.K;
+        if (more) load_step(k0 + 64);
+        mfma_step(buf);
+        if (more) store_step(k0 + 64, buf ^ 1);
         __syncthreads();
         buf ^= 1;
     }
 
     // accumulator element v of a tile: row 4 * (lane / 16) + v, column lane % 16
 #pragma unroll
-    for (int j = 0; j < 5; ++j) {
+    for (int j = 0; j < CT; ++j) {
         const int cn = j * 16 + (lane & 15);
         const int n = n0 + cn;
         if (cn < a.cols && n < a.N) {
@@ -187,18 +224,24 @@ hipError_t launch_matmul_bf16(Lane* lane, uint32_t type, const uint16_t* x, cons
     a.M = rows;
     a.K = in_w;
     a.N = out_w;
-    // strip width: as close to 80 columns as an even split of N over the compute units allows
-    int strips = (out_w + kMaxCols - 1) / kMaxCols;
-    const int even = (strips + lane->compute_units - 1) / lane->compute_units * lane->compute_units;
-    if ((out_w + even - 1) / even >= 56) strips = even;
+    // Row tile and strip width: BM = 128 rows for M <= 128, else 256; strips as wide as the column tiles allow, narrowed
+    // so that strips x row tiles is a whole number of rounds over the compute units when that keeps them >= 70 % wide.
+    const int bm = rows <= 128 ? 128 : 256;
+    const int m_tiles = (rows + bm - 1) / bm;
+    const int max_cols = (rows <= 256) ? 80 : 144;
+    int strips = (out_w + max_cols - 1) / max_cols;
+    const int per_round = lane->compute_units;
+    const int even = (strips * m_tiles + per_round - 1) / per_round * per_round / m_tiles;
+    if (even > strips && (out_w + even - 1) / even * 10 >= max_cols * 7) strips = even;
     a.cols = (out_w + strips - 1) / strips;
     a.strips = (out_w + a.cols - 1) / a.cols;
+    const dim3 grid(a.strips, m_tiles);
     if (rows <= 128) {
-        hipLaunchKernelGGL(matmul_q4k_bf16_kernel<16>, dim3(a.strips, (rows + 127) / 128), dim3(kGemmThreads), 0, lane->stream, a);
+        hipLaunchKernelGGL((matmul_q4k_bf16_kernel<16, 5>), grid, dim3(kGemmThreads), 0, lane->stream, a);
     } else if (rows <= 256) {
-        hipLaunchKernelGGL(matmul_q4k_bf16_kernel<32>, dim3(a.strips, (rows + 255) / 256), dim3(kGemmThreads), 0, lane->stream, a);
+        hipLaunchKernelGGL((matmul_q4k_bf16_kernel<32, 5>), grid, dim3(kGemmThreads), 0, lane->stream, a);
     } else {
-        hipLaunchKernelGGL(matmul_q4k_bf16_kernel<64>, dim3(a.strips, (rows + 511) / 512), dim3(kGemmThreads), 0, lane->stream, a);
+        hipLaunchKernelGGL((matmul_q4k_bf16_kernel<32, 9>), grid, dim3(kGemmThreads), 0, lane->stream, a);
     }
     return hipGetLastError();
 }
