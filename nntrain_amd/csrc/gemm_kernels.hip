@@ -5,10 +5,11 @@
 // accumulators.  The weight is the CPU decoder's (d*sc)*q - dmin*m (NNtrain.Core/Serialization/GgufQ4K.cs:34-41)
 // evaluated in FP32 and rounded once to bf16, which is what the 2e-3 relative-L2 bar of this path allows for.
 //
-// Tiling.  A workgroup of 8 waves owns BM = 8 * RW rows (RW = 16 or 32 rows per wave) and a strip of up to 16 * CT
-// output columns (CT = 5 or 9 column tiles) for the whole K range; the strip width is chosen on the host so that
+// Tiling.  A workgroup of 8 waves owns BM rows (128 or 256) and a strip of up to 16 * CT output columns (CT = 5 or 9
+// column tiles) for the whole K range; the waves are laid out 8 x 1 (16 or 32 rows each, whole strip) or 4 x 2 (64 rows,
+// 5 or 4 column tiles: squarer wave tiles re-read less of the LDS tiles); the strip width is chosen on the host so that
 // strips x row tiles split evenly over the compute units (17408 columns: 256 strips of 68 for M <= 256, 128 strips of
-// 136 for larger M).  Every wave spans the whole strip, so a weight sub-block is dequantized once per workgroup.
+// 136 for larger M).  A weight sub-block is dequantized once per workgroup.
 // K advances 64 per iteration = the two Q4_K sub-blocks that share 32 bytes of nibbles:
 //   - per iteration two x sub-tiles [BM][32] bf16 and two weight sub-tiles [16 CT][32] bf16 live in LDS, double
 //     buffered (rows are 64 bytes, so the 16 rows x 4 k-groups an MFMA operand needs form one contiguous,
@@ -74,12 +75,15 @@ __device__ __forceinline__ u32x4 q4k_decode8(uint32_t q_lo, uint32_t q_hi, float
     return u32x4{pack_bf16(w0, w1), pack_bf16(w2, w3), pack_bf16(w4, w5), pack_bf16(w6, w7)};
 }
 
-template <int RW, int CT>
+// WM x WN waves (8 in all); a wave owns RW rows and, when WN == 2, the first CTW or the remaining CT - CTW column tiles.
+template <int RW, int CT, int WN>
 __global__ __launch_bounds__(kGemmThreads) void matmul_q4k_bf16_kernel(GemmArgs a)
 {
-    constexpr int BM = 8 * RW;
+    constexpr int WM = 8 / WN;
+    constexpr int BM = WM * RW;
     constexpr int MT = RW / 16;                     // 16-row MFMA tiles per wave
     constexpr int BN = 16 * CT;
+    constexpr int CTW = (CT + WN - 1) / WN;         // column tiles of the widest wave
     constexpr int kXLoads = BM * 2 * kRowBytes / 16 / kGemmThreads;   // 16-byte pieces of the two x sub-tiles per thread
     constexpr int kItems = (4 * BN + kGemmThreads - 1) / kGemmThreads;  // weight items (row, quarter) per thread
     static_assert(kXLoads >= 1, "tile too small for the thread count");
@@ -88,6 +92,9 @@ __global__ __launch_bounds__(kGemmThreads) void matmul_q4k_bf16_kernel(GemmArgs 
     __shared__ __attribute__((aligned(16))) uint8_t ws[2][2][BN * kRowBytes];
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    // waves w and w + 4 usually share a SIMD: giving them different column halves balances the matrix pipes
+    const int wm = wave % WM, wn = wave / WM;
+    const int ct0 = wn * CTW, ct_n = wn == WN - 1 ? CT - ct0 : CTW;   // this wave's column tiles [ct0, ct0 + ct_n)
     const int strip = blockIdx.x, m0 = blockIdx.y * BM;
     const int n0 = strip * a.cols;
     const int row_bytes = (a.K >> 8) * 144;
@@ -151,11 +158,11 @@ __global__ __launch_bounds__(kGemmThreads) void matmul_q4k_bf16_kernel(GemmArgs 
         }
     };
 
-    f32x4 acc[MT][CT];
+    f32x4 acc[MT][CTW];
 #pragma unroll
     for (int i = 0; i < MT; ++i)
 #pragma unroll
-        for (int j = 0; j < CT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < CTW; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     // operand address of this lane inside a 16-row tile: row lane % 16, k-group lane / 16
     const int frag = (lane & 15) * kRowBytes + (lane >> 4) * 16;
@@ -165,13 +172,15 @@ __global__ __launch_bounds__(kGemmThreads) void matmul_q4k_bf16_kernel(GemmArgs 
             bf16x8 afrag[MT];
 #pragma unroll
             for (int i = 0; i < MT; ++i)
-                afrag[i] = *reinterpret_cast<const bf16x8*>(&xs[buf][sub][(wave * RW + i * 16) * kRowBytes + frag]);
+                afrag[i] = *reinterpret_cast<const bf16x8*>(&xs[buf][sub][(wm * RW + i * 16) * kRowBytes + frag]);
 #pragma unroll
-            for (int j = 0; j < CT; ++j) {
-                const bf16x8 bfrag = *reinterpret_cast<const bf16x8*>(&ws[buf][sub][j * 16 * kRowBytes + frag]);
+            for (int j = 0; j < CTW; ++j) {
+                if (j < ct_n) {        // wave-uniform: the last wave column may have one tile less
+                    const bf16x8 bfrag = *reinterpret_cast<const bf16x8*>(&ws[buf][sub][(ct0 + j) * 16 * kRowBytes + frag]);
 #pragma unroll
-                for (int i = 0; i < MT; ++i)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[i], bfrag, acc[i][j], 0, 0, 0);
+                    for (int i = 0; i < MT; ++i)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[i], bfrag, acc[i][j], 0, 0, 0);
+                }
             }
         }
     };
@@ -193,16 +202,16 @@ __global__ __launch_bounds__(kGemmThreads) void matmul_q4k_bf16_kernel(GemmArgs 
 
     // accumulator element v of a tile: row 4 * (lane / 16) + v, column lane % 16
 #pragma unroll
-    for (int j = 0; j < CT; ++j) {
-        const int cn = j * 16 + (lane & 15);
+    for (int j = 0; j < CTW; ++j) {
+        const int cn = (ct0 + j) * 16 + (lane & 15);
         const int n = n0 + cn;
-        if (cn < a.cols && n < a.N) {
+        if (j < ct_n && cn < a.cols && n < a.N) {
             const float b = a.bias ? a.bias[n] : 0.0f;
 #pragma unroll
             for (int i = 0; i < MT; ++i) {
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
-                    const int m = m0 + wave * RW + i * 16 + (lane >> 4) * 4 + v;
+                    const int m = m0 + wm * RW + i * 16 + (lane >> 4) * 4 + v;
                     if (m < a.M) a.y[static_cast<size_t>(m) * a.N + n] = acc[i][j][v] + b;
                 }
             }
@@ -237,11 +246,11 @@ hipError_t launch_matmul_bf16(Lane* lane, uint32_t type, const uint16_t* x, cons
     a.strips = (out_w + a.cols - 1) / a.cols;
     const dim3 grid(a.strips, m_tiles);
     if (rows <= 128) {
-        hipLaunchKernelGGL((matmul_q4k_bf16_kernel<16, 5>), grid, dim3(kGemmThreads), 0, lane->stream, a);
+        hipLaunchKernelGGL((matmul_q4k_bf16_kernel<16, 5, 1>), grid, dim3(kGemmThreads), 0, lane->stream, a);
     } else if (rows <= 256) {
-        hipLaunchKernelGGL((matmul_q4k_bf16_kernel<32, 5>), grid, dim3(kGemmThreads), 0, lane->stream, a);
+        hipLaunchKernelGGL((matmul_q4k_bf16_kernel<32, 5, 1>), grid, dim3(kGemmThreads), 0, lane->stream, a);
     } else {
-        hipLaunchKernelGGL((matmul_q4k_bf16_kernel<32, 9>), grid, dim3(kGemmThreads), 0, lane->stream, a);
+        hipLaunchKernelGGL((matmul_q4k_bf16_kernel<64, 9, 2>), grid, dim3(kGemmThreads), 0, lane->stream, a);
     }
     return hipGetLastError();
 }
