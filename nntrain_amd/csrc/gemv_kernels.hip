@@ -32,6 +32,8 @@ __device__ const uint64_t g_iq2s_grid[1024] = { NNHIP_IQ2S_GRID_VALUES };
 
 constexpr int kMaxWG = 1024;       // lanes per workgroup (16 waves: 4 per SIMD)
 constexpr int kUnitW = 64;         // weights per lane-unit
+constexpr int kYBuf = 1024;        // row results a workgroup holds back before storing them
+constexpr int kWaitVm0 = 0x0F70;   // s_waitcnt immediate: vmcnt(0), nothing else waited for
 constexpr int kMaxDynamicLds = 140 * 1024;   // staged activations; 16 KB of the 160 KB stay for the static arrays
 
 struct MatvecArgs {
@@ -435,8 +437,22 @@ void matvec_rowstep_kernel(MatvecArgs a, const float* __restrict__ bias)
     __syncthreads();
     typename Q::X xr = Q::load_x(xstage, owner ? c : 0);
 
+    // Row results are collected in LDS and stored to memory in bursts (when the buffer is full, and at the end), so
+    // the steady state has no vector-memory traffic besides the weight stream.
+    __shared__ float ybuf[kYBuf];
     const int wave = tid >> 6, lane = tid & 63, waves = T >> 6;
     int buf = 0;
+    int held = 0;                 // steps whose rows sit in ybuf
+    int first_held = step;        // step number of ybuf[0 .. rs)
+    auto flush = [&]() {
+        __syncthreads();
+        for (int i = tid; i < held * rs; i += T) {
+            const int j = i / rs;
+            const int row = (first_held + j * stride) * rs + (i - j * rs);
+            if (row < a.out_w) y[row] = ybuf[i];
+        }
+        held = 0;
+    };
     auto finish = [&](const typename Q::Regs& r, int st) {
         part[buf][tid] = Q::dot(r, xr, c, grid);
         __syncthreads();
@@ -449,21 +465,39 @@ void matvec_rowstep_kernel(MatvecArgs a, const float* __restrict__ bias)
                 // the row index is wave-uniform: the bias comes through the scalar cache and does not wait on the
                 // vector-memory counter that the prefetched weights are tracked by
                 const int urow = __builtin_amdgcn_readfirstlane(row);
-                if (lane == 0) y[urow] = (bias ? bias[urow] : 0.0f) + t;
+                if (lane == 0) ybuf[held * rs + rr] = (bias ? bias[urow] : 0.0f) + t;
             }
         }
         buf ^= 1;
+        ++held;
     };
 
-    while (step < a.steps) {
+    // The loop runs whole turns of the register ring and has one exit, at the turn boundary: an exit in the middle of
+    // a turn would join the loop's back edge right after a register set was refilled, and the wait for that set at the
+    // loop head would then have to be "everything has arrived", which drains the prefetch queue every turn.
+    while (step + (kDepth - 1) * stride < a.steps) {
 #pragma unroll
         for (int d = 0; d < kDepth; ++d) {
             regs[(d + kDepth - 1) % kDepth] = fetch(step + (kDepth - 1) * stride);
             finish(regs[d], step);
             step += stride;
-            if (step >= a.steps) break;
+        }
+        if ((held + kDepth) * rs > kYBuf) {         // rare: only matrices with very many rows per workgroup get here
+            flush();
+            __builtin_amdgcn_s_waitcnt(kWaitVm0);
+            __syncthreads();
+            first_held = step;
         }
     }
+    // fewer than kDepth steps are left, and their weights are already in flight
+#pragma unroll
+    for (int d = 0; d < kDepth - 1; ++d) {
+        if (step < a.steps) {
+            finish(regs[d], step);
+            step += stride;
+        }
+    }
+    flush();
 }
 
 // ------------------------------------------------------------------------------------------- batched kernel
@@ -472,8 +506,10 @@ void matvec_rowstep_kernel(MatvecArgs a, const float* __restrict__ bias)
 // the vector-memory one.  The device pass therefore declares them as global-address-space pointers.
 #if defined(__HIP_DEVICE_COMPILE__)
 #define NNHIP_GLOBAL_PTR __attribute__((address_space(1)))
+#define NNHIP_CONST_PTR __attribute__((address_space(4)))
 #else
 #define NNHIP_GLOBAL_PTR
+#define NNHIP_CONST_PTR
 #endif
 struct BatchEntry {
     const NNHIP_GLOBAL_PTR float* x;
@@ -508,9 +544,14 @@ struct BatchEntry {
 // pump did not get to is fetched at the switch (the stream stalls once).
 template <class Q>
 __global__ __launch_bounds__(Shape<Q>::kMaxT) __attribute__((amdgpu_waves_per_eu(Shape<Q>::kWavesPerEu, Shape<Q>::kWavesPerEu)))
-void matvec_batch_kernel(const BatchEntry* __restrict__ table, int total_chunks)
+void matvec_batch_kernel(const BatchEntry* __restrict__ table_arg, int total_chunks)
 {
     constexpr int kDepth = Shape<Q>::kBatchDepth;
+    // The table and the bias vectors are read-only for the whole launch and always indexed with workgroup-uniform
+    // values: reading them through the constant address space makes those reads scalar loads, which do not tick the
+    // vector-memory counter.  A vector load there would make its user wait for every prefetched weight load as well
+    // (the counter completes in order), draining the ring once per step.
+    const NNHIP_CONST_PTR BatchEntry* table = (const NNHIP_CONST_PTR BatchEntry*)table_arg;
     __shared__ float part[2][kMaxWG];
     __shared__ uint64_t grid[Q::kGrid ? 1024 : 1];
     extern __shared__ float4 xstage[];
@@ -619,7 +660,8 @@ void matvec_batch_kernel(const BatchEntry* __restrict__ table, int total_chunks)
                     for (int u = lane; u < ce.upr; u += 64) t += part[buf][rr * ce.upr + u];
                     t = wave_sum(t);
                     const int urow = __builtin_amdgcn_readfirstlane(row);
-                    if (lane == 0) ce.y[urow] = (ce.bias ? ce.bias[urow] : 0.0f) + t;
+                    const NNHIP_CONST_PTR float* cbias = (const NNHIP_CONST_PTR float*)ce.bias;
+                    if (lane == 0) ce.y[urow] = (cbias ? cbias[urow] : 0.0f) + t;
                 }
             }
             buf ^= 1;
