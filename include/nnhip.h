@@ -42,6 +42,7 @@ enum {
     NNHIP_TYPE_Q4_K = 12,
     NNHIP_TYPE_Q5_K = 13,
     NNHIP_TYPE_Q6_K = 14,
+    NNHIP_TYPE_IQ3_S = 21,
     NNHIP_TYPE_IQ2_S = 22
 };
 

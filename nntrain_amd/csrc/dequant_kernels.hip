@@ -3,7 +3,7 @@
 // Every product and difference is rounded to FP32 on its own (__fmul_rn / __fsub_rn, never fused), in the order the
 // managed decoders use: Q4_K/Q5_K (d*sc)*q - (dmin*m)   (NNtrain.Core/Serialization/GgufQ4K.cs:34-41),
 // Q6_K (d*scale)*q (GgufQ6K.cs:45-48), IQ2_S ((d*(0.5+s))*0.25)*mag*sign (NNtrain.Arc/Kernels/qwen35_iq.cl:411-419),
-// Q8_0 d*q.  One thread decodes four consecutive weights and stores one float4.
+// IQ3_S (d*(1+2s))*mag*sign (qwen35_iq.cl:421-429), Q8_0 d*q.  One thread decodes four consecutive weights and stores one float4.
 #include "nnhip_internal.h"
 #include "quant_device.h"
 
@@ -14,6 +14,7 @@ namespace nnhip {
 namespace {
 
 __device__ const uint64_t g_iq2s_grid_dq[1024] = { NNHIP_IQ2S_GRID_VALUES };
+__device__ const uint32_t g_iq3s_grid_dq[512] = { NNHIP_IQ3S_GRID_VALUES };
 
 __device__ __forceinline__ void k4_scale_min(const uint8_t* packed, int g, uint32_t& sc, uint32_t& mn)
 {
@@ -90,6 +91,28 @@ __device__ __forceinline__ float4 deq4_iq2_s(const uint8_t* w, int64_t e)
     return v;
 }
 
+// IQ3_S: d @0, qs[64] @2 (low 8 index bits, one per four weights), qh[8] @66 (ninth index bit), signs[32] @74 (one bit
+// per weight), scales[4] @106 (a nibble per 32 weights); the four weights of a quartet are the bytes of the 32-bit
+// codebook entry.
+__device__ __forceinline__ float4 deq4_iq3_s(const uint8_t* w, int64_t e)
+{
+    const uint8_t* p = w + (e >> 8) * 110;
+    const int i = static_cast<int>(e & 255), g = i >> 5, quartet = (i >> 2) & 7;
+    const float d = half_bits_to_float(ld16(p));
+    const uint32_t idx = p[2 + 8 * g + quartet] | (((p[66 + g] >> quartet) & 1u) << 8);
+    const uint32_t mags = g_iq3s_grid_dq[idx];
+    const uint32_t signs = p[74 + (i >> 3)] >> (i & 7);          // i & 7 is 0 or 4
+    const uint32_t sub = (p[106 + (g >> 1)] >> (4 * (g & 1))) & 15u;
+    const float db = __fmul_rn(d, static_cast<float>(1u + 2u * sub));
+    float4 v = make_float4(__fmul_rn(db, ubyte0(mags)), __fmul_rn(db, ubyte1(mags)), __fmul_rn(db, ubyte2(mags)),
+                           __fmul_rn(db, ubyte3(mags)));
+    v.x = __fmul_rn(v.x, (signs & 1u) ? -1.0f : 1.0f);
+    v.y = __fmul_rn(v.y, (signs & 2u) ? -1.0f : 1.0f);
+    v.z = __fmul_rn(v.z, (signs & 4u) ? -1.0f : 1.0f);
+    v.w = __fmul_rn(v.w, (signs & 8u) ? -1.0f : 1.0f);
+    return v;
+}
+
 template <uint32_t TYPE>
 __global__ __launch_bounds__(256) void dequantize_kernel(const uint8_t* __restrict__ w, float4* __restrict__ out,
                                                          int64_t quads)
@@ -102,6 +125,7 @@ __global__ __launch_bounds__(256) void dequantize_kernel(const uint8_t* __restri
         else if (TYPE == NNHIP_TYPE_Q4_K) v = deq4_q45_k<false>(w, e);
         else if (TYPE == NNHIP_TYPE_Q5_K) v = deq4_q45_k<true>(w, e);
         else if (TYPE == NNHIP_TYPE_Q6_K) v = deq4_q6_k(w, e);
+        else if (TYPE == NNHIP_TYPE_IQ3_S) v = deq4_iq3_s(w, e);
         else v = deq4_iq2_s(w, e);
         out[t] = v;
     }
@@ -135,6 +159,7 @@ hipError_t launch_dequantize(Lane* lane, uint32_t type, const void* w, float* ou
     case NNHIP_TYPE_Q4_K: return launch_deq<NNHIP_TYPE_Q4_K>(lane, w, out, elements);
     case NNHIP_TYPE_Q5_K: return launch_deq<NNHIP_TYPE_Q5_K>(lane, w, out, elements);
     case NNHIP_TYPE_Q6_K: return launch_deq<NNHIP_TYPE_Q6_K>(lane, w, out, elements);
+    case NNHIP_TYPE_IQ3_S: return launch_deq<NNHIP_TYPE_IQ3_S>(lane, w, out, elements);
     case NNHIP_TYPE_IQ2_S: return launch_deq<NNHIP_TYPE_IQ2_S>(lane, w, out, elements);
     default: return hipErrorInvalidValue;
     }

@@ -29,6 +29,7 @@ namespace nnhip {
 namespace {
 
 __device__ const uint64_t g_iq2s_grid[1024] = { NNHIP_IQ2S_GRID_VALUES };
+__device__ const uint32_t g_iq3s_grid[512] = { NNHIP_IQ3S_GRID_VALUES };
 
 constexpr int kMaxWG = 1024;       // lanes per workgroup (16 waves: 4 per SIMD)
 constexpr int kUnitW = 64;         // weights per lane-unit
@@ -91,7 +92,7 @@ __device__ __forceinline__ XChunk load_chunk(const float4* xs, int c)
 // ---------------------------------------------------------------------------------------------------- Q8_0
 // Unit = two consecutive 34-byte blocks (68 bytes, 4-byte aligned because a row holds an even number of blocks).
 struct Q8_0Unit {
-    static constexpr bool kGrid = false;
+    static constexpr int kGridWords = 0;          // no codebook
     struct X { XChunk c; };
     struct Regs { u32x4 a, b, c, d; uint32_t e; };
 
@@ -111,7 +112,7 @@ struct Q8_0Unit {
         return r;
     }
 
-    static __device__ __forceinline__ float dot(const Regs& r, const X& x, int, const uint64_t*)
+    static __device__ __forceinline__ float dot(const Regs& r, const X& x, int, const uint32_t*)
     {
         const uint32_t w[17] = {r.a[0], r.a[1], r.a[2], r.a[3], r.b[0], r.b[1], r.b[2], r.b[3], r.c[0], r.c[1], r.c[2],
                                 r.c[3], r.d[0], r.d[1], r.d[2], r.d[3], r.e};
@@ -133,7 +134,7 @@ struct Q8_0Unit {
 // Unit j of a super-block = sub-blocks 2j (low nibbles) and 2j+1 (high nibbles) of qs[32j .. 32j+31].
 // sum_k x (s*q - m) = s * sum(q x) - m * sum(x); the two 32-wide sums of x are taken once per lane.
 struct Q4KUnit {
-    static constexpr bool kGrid = false;
+    static constexpr int kGridWords = 0;          // no codebook
     struct X { XChunk c; float xs_lo, xs_hi; };
     struct Regs { u32x4 h, qa, qb; };
 
@@ -163,7 +164,7 @@ struct Q4KUnit {
         return r;
     }
 
-    static __device__ __forceinline__ float dot(const Regs& r, const X& x, int unit, const uint64_t*)
+    static __device__ __forceinline__ float dot(const Regs& r, const X& x, int unit, const uint32_t*)
     {
         const int j = unit & 3;
         const float d = half_bits_to_float(r.h[0]), dmin = half_bits_to_float(r.h[0] >> 16);
@@ -191,7 +192,7 @@ struct Q4KUnit {
 // ---------------------------------------------------------------------------------------------------- Q5_K
 // As Q4_K plus one high bit per weight: bit g of qh[i] belongs to element i of sub-block g.
 struct Q5KUnit {
-    static constexpr bool kGrid = false;
+    static constexpr int kGridWords = 0;          // no codebook
     using X = Q4KUnit::X;
     struct Regs { u32x4 h, ha, hb, qa, qb; };
 
@@ -210,7 +211,7 @@ struct Q5KUnit {
         return r;
     }
 
-    static __device__ __forceinline__ float dot(const Regs& r, const X& x, int unit, const uint64_t*)
+    static __device__ __forceinline__ float dot(const Regs& r, const X& x, int unit, const uint32_t*)
     {
         const int j = unit & 3;
         const float d = half_bits_to_float(r.h[0]), dmin = half_bits_to_float(r.h[0] >> 16);
@@ -241,7 +242,7 @@ struct Q5KUnit {
 // Unit (sb, half h, part p): elements 128h + 32e + 16p + i, i < 16, e < 4 - the four 16-runs that share
 // ql[64h+16p ..], ql[64h+32+16p ..] and qh[32h+16p ..].  w = d*scale*(q - 32): sum(q x) - 32 sum16(x).
 struct Q6KUnit {
-    static constexpr bool kGrid = false;
+    static constexpr int kGridWords = 0;          // no codebook
     struct X { float4 p[4][4]; float xs[4]; };   // [run e][piece]
     struct Regs { u32x4 la, lb, hh; u32x2 scw; uint32_t d; };
 
@@ -277,7 +278,7 @@ struct Q6KUnit {
         return r;
     }
 
-    static __device__ __forceinline__ float dot(const Regs& r, const X& x, int unit, const uint64_t*)
+    static __device__ __forceinline__ float dot(const Regs& r, const X& x, int unit, const uint32_t*)
     {
         const int p = unit & 1;
         const float d = half_bits_to_float(r.d);
@@ -309,7 +310,8 @@ struct Q6KUnit {
 // Unit gp of a super-block = 32-groups 2gp and 2gp+1.  Each octet: 10-bit index into the 1024-entry codebook held
 // in LDS (8 magnitude bytes), 8 sign bits, 4-bit sub-scale shared by two octets.
 struct IQ2SUnit {
-    static constexpr bool kGrid = true;
+    static constexpr int kGridWords = 2048;       // 1024 codebook entries of 8 magnitudes
+    static __device__ __forceinline__ const uint32_t* grid_table() { return reinterpret_cast<const uint32_t*>(g_iq2s_grid); }
     struct X { XChunk c; };
     struct Regs { u32x2 qs, sg; uint32_t qh, scl, d; };
 
@@ -339,8 +341,9 @@ struct IQ2SUnit {
         return __uint_as_float(__float_as_uint(mag) | sign);
     }
 
-    static __device__ __forceinline__ float dot(const Regs& r, const X& x, int, const uint64_t* grid)
+    static __device__ __forceinline__ float dot(const Regs& r, const X& x, int, const uint32_t* grid32)
     {
+        const uint64_t* grid = reinterpret_cast<const uint64_t*>(grid32);
         const float d = half_bits_to_float(r.d);
         float acc = 0.0f;
 #pragma unroll
@@ -373,6 +376,69 @@ struct IQ2SUnit {
     }
 };
 
+// ---------------------------------------------------------------------------------------------------- IQ3_S
+// Unit u of a 110-byte super-block = groups 2u and 2u+1 (32 weights each): 16 index bytes, 2 high-bit bytes, 8 sign
+// bytes, one byte holding both 4-bit scales.  w = (d * (1 + 2 s)) * magnitude * sign (qwen35_iq.cl:421-429).
+struct IQ3SUnit {
+    static constexpr int kGridWords = 512;        // 512 codebook entries of 4 magnitudes
+    static __device__ __forceinline__ const uint32_t* grid_table() { return g_iq3s_grid; }
+    struct X { XChunk c; };
+    struct Regs { u32x4 qs; u32x2 sg; uint32_t qh, scl, d; };
+
+    static __device__ __forceinline__ X load_x(const float4* x, int unit)
+    {
+        X r;
+        r.c = load_chunk(x, unit);
+        return r;
+    }
+
+    static __device__ __forceinline__ Regs load(const uint8_t* row, int unit)
+    {
+        const int sb = unit >> 2, u = unit & 3;
+        const uint8_t* blk = row + static_cast<uint32_t>(sb) * 110u;
+        Regs r;
+        r.qs = ld128(blk + 2 + 16 * u);
+        r.sg = ld64(blk + 74 + 8 * u);
+        r.qh = ld16(blk + 66 + 2 * u);
+        r.scl = blk[106 + u];
+        r.d = ld16(blk);
+        return r;
+    }
+
+    static __device__ __forceinline__ float signed_mag(float mag, uint32_t signs, int t)
+    {
+        const uint32_t sign = (signs << (31 - t)) & 0x80000000u;
+        return __uint_as_float(__float_as_uint(mag) | sign);
+    }
+
+    static __device__ __forceinline__ float dot(const Regs& r, const X& x, int, const uint32_t* grid)
+    {
+        const float d = half_bits_to_float(r.d);
+        float acc = 0.0f;
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+            const uint32_t hbits = (r.qh >> (8 * g)) & 0xffu;
+            const uint32_t s4 = r.sg[g];
+            float t = 0.0f;
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                const uint32_t word = r.qs[2 * g + (q >> 2)];
+                const uint32_t idx = ((word >> (8 * (q & 3))) & 0xffu) | (((hbits >> q) & 1u) << 8);
+                const uint32_t gv = grid[idx];
+                const uint32_t signs = (s4 >> (8 * (q >> 1) + 4 * (q & 1))) & 0xfu;
+                const float4 xa = x.c.p[8 * g + q];
+                t = fmaf(signed_mag(ubyte0(gv), signs, 0), xa.x, t);
+                t = fmaf(signed_mag(ubyte1(gv), signs, 1), xa.y, t);
+                t = fmaf(signed_mag(ubyte2(gv), signs, 2), xa.z, t);
+                t = fmaf(signed_mag(ubyte3(gv), signs, 3), xa.w, t);
+            }
+            const uint32_t sub = (r.scl >> (4 * g)) & 15u;
+            acc = fmaf(d * static_cast<float>(1u + 2u * sub), t, acc);
+        }
+        return acc;
+    }
+};
+
 // ---------------------------------------------------------------------------------------------- the kernel
 // Launch shape of one block format: lanes per workgroup, waves per SIMD the register budget is sized for, and the
 // number of weight register sets that rotate (DEPTH - 1 row steps are in flight while one is reduced): kDepth for a
@@ -384,6 +450,7 @@ template <> struct Shape<Q4KUnit> { static constexpr int kMaxT = 1024, kWavesPer
 template <> struct Shape<Q5KUnit> { static constexpr int kMaxT = 768, kWavesPerEu = 3, kDepth = 3, kBatchDepth = 3; };
 template <> struct Shape<Q6KUnit> { static constexpr int kMaxT = 768, kWavesPerEu = 3, kDepth = 2, kBatchDepth = 4; };
 template <> struct Shape<IQ2SUnit> { static constexpr int kMaxT = 1024, kWavesPerEu = 4, kDepth = 2, kBatchDepth = 4; };
+template <> struct Shape<IQ3SUnit> { static constexpr int kMaxT = 1024, kWavesPerEu = 4, kDepth = 2, kBatchDepth = 4; };
 
 // grid.x = workgroups striding over row steps, grid.y = input rows, blockDim.x = T (a multiple of 64).
 template <class Q>
@@ -392,7 +459,7 @@ void matvec_rowstep_kernel(MatvecArgs a, const float* __restrict__ bias)
 {
     constexpr int kDepth = Shape<Q>::kDepth;
     __shared__ float part[2][kMaxWG];
-    __shared__ uint64_t grid[Q::kGrid ? 1024 : 1];
+    __shared__ __attribute__((aligned(8))) uint32_t grid[Q::kGridWords ? Q::kGridWords : 2];
 
     const int tid = threadIdx.x;
     const int upr = a.units_per_row, rs = a.rows_per_step;
@@ -432,8 +499,8 @@ void matvec_rowstep_kernel(MatvecArgs a, const float* __restrict__ bias)
     if (tid < pieces) xstage[tid + (tid >> 4)] = xv0;
     if (tid + T < pieces) xstage[tid + T + ((tid + T) >> 4)] = xv1;
     for (int L = tid + 2 * T; L < pieces; L += T) xstage[L + (L >> 4)] = xg[L];
-    if (Q::kGrid)
-        for (int i = tid; i < 1024; i += T) grid[i] = g_iq2s_grid[i];
+    if constexpr (Q::kGridWords > 0)
+        for (int i = tid; i < Q::kGridWords; i += T) grid[i] = Q::grid_table()[i];
     __syncthreads();
     typename Q::X xr = Q::load_x(xstage, owner ? c : 0);
 
@@ -553,13 +620,13 @@ void matvec_batch_kernel(const BatchEntry* __restrict__ table_arg, int total_chu
     // (the counter completes in order), draining the ring once per step.
     const NNHIP_CONST_PTR BatchEntry* table = (const NNHIP_CONST_PTR BatchEntry*)table_arg;
     __shared__ float part[2][kMaxWG];
-    __shared__ uint64_t grid[Q::kGrid ? 1024 : 1];
+    __shared__ __attribute__((aligned(8))) uint32_t grid[Q::kGridWords ? Q::kGridWords : 2];
     extern __shared__ float4 xstage[];
 
     const int tid = threadIdx.x, T = blockDim.x, G = gridDim.x;
     const int wave = tid >> 6, lane = tid & 63, waves = T >> 6;
-    if (Q::kGrid)
-        for (int i = tid; i < 1024; i += T) grid[i] = g_iq2s_grid[i];
+    if constexpr (Q::kGridWords > 0)
+        for (int i = tid; i < Q::kGridWords; i += T) grid[i] = Q::grid_table()[i];
 
     auto uni = [](int v) { return __builtin_amdgcn_readfirstlane(v); };   // pins workgroup-uniform state to SGPRs
     auto slot = [&](const BatchEntry& e, int& rl, int& c, bool& owner) {
@@ -797,6 +864,7 @@ void shape_of(uint32_t type, int* max_t, int* depth)
     case NNHIP_TYPE_Q4_K: *max_t = Shape<Q4KUnit>::kMaxT; *depth = Shape<Q4KUnit>::kBatchDepth; break;
     case NNHIP_TYPE_Q5_K: *max_t = Shape<Q5KUnit>::kMaxT; *depth = Shape<Q5KUnit>::kBatchDepth; break;
     case NNHIP_TYPE_Q6_K: *max_t = Shape<Q6KUnit>::kMaxT; *depth = Shape<Q6KUnit>::kBatchDepth; break;
+    case NNHIP_TYPE_IQ3_S: *max_t = Shape<IQ3SUnit>::kMaxT; *depth = Shape<IQ3SUnit>::kBatchDepth; break;
     default: *max_t = Shape<IQ2SUnit>::kMaxT; *depth = Shape<IQ2SUnit>::kBatchDepth; break;
     }
 }
@@ -836,6 +904,7 @@ hipError_t launch_matvec(Lane* lane, uint32_t type, const float* x, const void* 
     case NNHIP_TYPE_Q4_K: return launch_rowstep<Q4KUnit>(lane, a, rows);
     case NNHIP_TYPE_Q5_K: return launch_rowstep<Q5KUnit>(lane, a, rows);
     case NNHIP_TYPE_Q6_K: return launch_rowstep<Q6KUnit>(lane, a, rows);
+    case NNHIP_TYPE_IQ3_S: return launch_rowstep<IQ3SUnit>(lane, a, rows);
     case NNHIP_TYPE_IQ2_S: return launch_rowstep<IQ2SUnit>(lane, a, rows);
     default: return hipErrorInvalidValue;
     }
@@ -844,7 +913,8 @@ hipError_t launch_matvec(Lane* lane, uint32_t type, const float* x, const void* 
 
 hipError_t launch_matvec_batch(Lane* lane, const nnhip_matvec_desc* descs, int count)
 {
-    static const uint32_t kTypes[5] = {NNHIP_TYPE_Q8_0, NNHIP_TYPE_Q4_K, NNHIP_TYPE_Q5_K, NNHIP_TYPE_Q6_K, NNHIP_TYPE_IQ2_S};
+    static const uint32_t kTypes[6] = {NNHIP_TYPE_Q8_0, NNHIP_TYPE_Q4_K, NNHIP_TYPE_Q5_K, NNHIP_TYPE_Q6_K, NNHIP_TYPE_IQ3_S,
+                                       NNHIP_TYPE_IQ2_S};
     std::vector<BatchEntry> all;
     struct Group { uint32_t type; size_t begin, end; int total_chunks, max_in_w; };
     std::vector<Group> groups;
@@ -923,6 +993,7 @@ hipError_t launch_matvec_batch(Lane* lane, const nnhip_matvec_desc* descs, int c
         case NNHIP_TYPE_Q4_K: e = launch_batch_of<Q4KUnit>(lane, g.total_chunks, g.max_in_w, off); break;
         case NNHIP_TYPE_Q5_K: e = launch_batch_of<Q5KUnit>(lane, g.total_chunks, g.max_in_w, off); break;
         case NNHIP_TYPE_Q6_K: e = launch_batch_of<Q6KUnit>(lane, g.total_chunks, g.max_in_w, off); break;
+        case NNHIP_TYPE_IQ3_S: e = launch_batch_of<IQ3SUnit>(lane, g.total_chunks, g.max_in_w, off); break;
         default: e = launch_batch_of<IQ2SUnit>(lane, g.total_chunks, g.max_in_w, off); break;
         }
         if (e != hipSuccess) return e;

@@ -65,6 +65,7 @@ bool type_block(uint32_t type, int* elems, int* bytes)
     case NNHIP_TYPE_Q4_K: e = 256; b = 144; break;
     case NNHIP_TYPE_Q5_K: e = 256; b = 176; break;
     case NNHIP_TYPE_Q6_K: e = 256; b = 210; break;
+    case NNHIP_TYPE_IQ3_S: e = 256; b = 110; break;
     case NNHIP_TYPE_IQ2_S: e = 256; b = 82; break;
     default: return false;
     }

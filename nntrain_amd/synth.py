@@ -9,7 +9,8 @@ from __future__ import annotations
 
 import numpy as np
 
-from .quantized_matrix import BLOCK_BYTES, BLOCK_ELEMS, GGML_IQ2_S, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_Q8_0
+from .quantized_matrix import (BLOCK_BYTES, BLOCK_ELEMS, GGML_IQ2_S, GGML_IQ3_S, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K,
+                               GGML_Q8_0)
 
 
 def _rng(seed: int) -> np.random.Generator:
@@ -46,7 +47,7 @@ def _half_abs_normal(rng, n: int, sigma: float) -> np.ndarray:
 
 
 def k_quant_matrix(ggml_type: int, out_w: int, in_w: int, seed: int, sigma: float = 0.01) -> np.ndarray:
-    """Random Q4_K / Q5_K / Q6_K / IQ2_S payload: fp16 scales from |N(0, sigma)|, every packed field uniform."""
+    """Random Q4_K / Q5_K / Q6_K / IQ2_S / IQ3_S payload: fp16 scales from |N(0, sigma)|, every packed field uniform."""
     rng = _rng(seed)
     bb = BLOCK_BYTES[ggml_type]
     n = out_w * (in_w // BLOCK_ELEMS[ggml_type])
@@ -56,7 +57,7 @@ def k_quant_matrix(ggml_type: int, out_w: int, in_w: int, seed: int, sigma: floa
         blocks[:, 2:4] = _half_abs_normal(rng, n, sigma)
     elif ggml_type == GGML_Q6_K:
         blocks[:, 208:210] = _half_abs_normal(rng, n, sigma)
-    elif ggml_type == GGML_IQ2_S:
+    elif ggml_type in (GGML_IQ2_S, GGML_IQ3_S):
         blocks[:, 0:2] = _half_abs_normal(rng, n, sigma)
     else:
         raise ValueError("not a super-block type")

@@ -10,12 +10,12 @@ import numpy as np
 import pytest
 
 import oracle
-from nntrain_amd import (BLOCK_BYTES, BLOCK_ELEMS, GGML_IQ2_S, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_Q8_0, GgufReader,
-                         HipExecutionLane, HipQuantizedMatrix, NnHipError, synth)
+from nntrain_amd import (BLOCK_BYTES, BLOCK_ELEMS, GGML_IQ2_S, GGML_IQ3_S, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_Q8_0,
+                         GgufReader, HipExecutionLane, HipQuantizedMatrix, NnHipError, synth)
 
 pytestmark = pytest.mark.gpu
 
-ALL_TYPES = [GGML_Q8_0, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_IQ2_S]
+ALL_TYPES = [GGML_Q8_0, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_IQ3_S, GGML_IQ2_S]
 NAN_BITS = 0x7FC00000
 REL_L2_BAR = 1e-5
 
@@ -94,10 +94,10 @@ def test_dequantize_q4k_q6k_bit_exact_vs_gguf_py(lane, golden_dir):
         assert seen == 4
 
 
-@pytest.mark.parametrize("typ", [GGML_Q5_K, GGML_IQ2_S])
+@pytest.mark.parametrize("typ", [GGML_Q5_K, GGML_IQ2_S, GGML_IQ3_S])
 def test_dequantize_bit_exact_vs_native_ggml_blocks(lane, golden_dir, typ):
     cases = [c for c in json.loads((golden_dir / "iq_quant_blocks.json").read_text())["cases"] if c["type"] == typ]
-    assert len(cases) == {GGML_Q5_K: 25, GGML_IQ2_S: 69}[typ]
+    assert len(cases) == {GGML_Q5_K: 25, GGML_IQ2_S: 69, GGML_IQ3_S: 45}[typ]
     raw = np.concatenate([np.frombuffer(base64.b64decode(c["encoded"]), np.uint8) for c in cases])
     want = np.concatenate([np.frombuffer(base64.b64decode(c["decodedFloat32Base64"]), "<f4") for c in cases])
     mat = HipQuantizedMatrix(raw, typ, len(cases), 256)

@@ -33,7 +33,7 @@ def test_abi_version_and_struct_layouts():
 def test_geometry_queries_without_a_gpu():
     lib = native.load_library()
     e, b = c_int(), c_int()
-    for typ, (elems, nbytes) in {8: (32, 34), 12: (256, 144), 13: (256, 176), 14: (256, 210), 22: (256, 82)}.items():
+    for typ, (elems, nbytes) in {8: (32, 34), 12: (256, 144), 13: (256, 176), 14: (256, 210), 21: (256, 110), 22: (256, 82)}.items():
         assert lib.nnhip_type_block(typ, byref(e), byref(b)) == 0
         assert (e.value, b.value) == (elems, nbytes)
     assert lib.nnhip_type_block(2, byref(e), byref(b)) == 2
@@ -70,7 +70,7 @@ def test_quantized_matrix_constructor_validation():
         nn.HipQuantizedMatrix(b"\0" * 145, nn.GGML_Q4_K, 1, 256)
     m = nn.HipQuantizedMatrix(b"\0" * (34 * 4), nn.GGML_Q8_0, 2, 64)
     assert (m.ggml_type, m.output_width, m.input_width, m.storage_bytes) == (8, 2, 64, 136)
-    for typ in (8, 12, 13, 14, 22):
+    for typ in (8, 12, 13, 14, 21, 22):
         nn.HipQuantizedMatrix(np.zeros(nn.BLOCK_BYTES[typ] * 3, np.uint8), typ, 3, nn.BLOCK_ELEMS[typ])
 
 
@@ -162,7 +162,7 @@ def test_synthetic_payload_generators():
     d = raw.reshape(-1, 34)[:, :2].copy().view(np.float16).astype(np.float32).reshape(4, 2)
     # half a quantisation step, plus up to 127 steps of the fp16 rounding of the scale (2^-11 relative)
     assert np.all(np.abs(back - w).reshape(4, 2, 32) <= 0.57 * d[:, :, None] + 1e-9)
-    for typ in (12, 13, 14, 22):
+    for typ in (12, 13, 14, 21, 22):
         p = synth.k_quant_matrix(typ, 5, 512, 3)
         assert p.size == 5 * 2 * nn.BLOCK_BYTES[typ]
         assert np.all(np.isfinite(oracle.dequantize(typ, p)))
