@@ -51,7 +51,7 @@ enum {
 enum {
     NNHIP_OK = 0,
     NNHIP_ERR_INVALID_ARGUMENT = 1,   /* null pointer, non-positive width, rows < 1 ...                */
-    NNHIP_ERR_UNSUPPORTED_TYPE = 2,   /* ggml_type is not one of the five above                         */
+    NNHIP_ERR_UNSUPPORTED_TYPE = 2,   /* ggml_type is not one of the six above                          */
     NNHIP_ERR_INCOMPLETE_BLOCKS = 3,  /* in_w (or elements) is not a whole number of blocks             */
     NNHIP_ERR_OUT_OF_MEMORY = 4,
     NNHIP_ERR_HIP = 5,                /* a HIP call failed                                               */
@@ -162,8 +162,8 @@ NNHIP_API int nnhip_lane_stream(void* lane, void** stream);
 /* --- compute ------------------------------------------------------------------------------------------------ */
 
 /* out[i] = decoded weight i, FP32, bit-identical to the managed decoders GgufQ4K.Dequantize / GgufQ6K.Dequantize
- * (NNtrain.Core/Serialization/GgufQ4K.cs:9-60, GgufQ6K.cs:9-54) and to native ggml for Q5_K / IQ2_S / Q8_0
- * (NNtrain.Arc/Kernels/qwen35_iq.cl:398-419).  Also the embedding-row lookup of
+ * (NNtrain.Core/Serialization/GgufQ4K.cs:9-60, GgufQ6K.cs:9-54) and to native ggml for Q5_K / IQ2_S / IQ3_S / Q8_0
+ * (NNtrain.Arc/Kernels/qwen35_iq.cl:398-429).  Also the embedding-row lookup of
  * Matrix.Embedding (Qwen35QuantizedModel.cs:1497-1521) when w points at one row.  `elements` must be a whole
  * number of blocks.  Asynchronous. */
 NNHIP_API int nnhip_dequantize(void* lane, uint32_t ggml_type, const void* w, float* out, int64_t elements);

@@ -222,6 +222,24 @@ class GgufReader:
             done += len(piece)
         return chunks[0] if len(chunks) == 1 else b"".join(chunks)
 
+    def read_tensor_range(self, tensor: GgufTensorInfo, start: int, byte_count: int) -> bytes:
+        """Bytes [start, start + byte_count) of a tensor's payload (positional, for streaming uploads)."""
+        total = tensor.byte_count()
+        if start < 0 or byte_count < 0 or start + byte_count > total:
+            raise ValueError("range is outside the tensor payload")
+        offset = self._data_offset + tensor.offset + start
+        if offset > self._size or byte_count > self._size - offset:
+            raise EOFError("tensor payload exceeds the file")
+        chunks = []
+        done = 0
+        while done < byte_count:
+            piece = os.pread(self._fd, min(byte_count - done, 1 << 28), offset + done)
+            if not piece:
+                raise EOFError("tensor payload exceeds the file")
+            chunks.append(piece)
+            done += len(piece)
+        return chunks[0] if len(chunks) == 1 else b"".join(chunks)
+
     def matrix_dims(self, tensor: GgufTensorInfo) -> tuple[int, int]:
         """(input_width, output_width) of a 2-D weight: GGUF stores ne0 = K first (Qwen35Gguf.cs:170-182)."""
         if len(tensor.shape) != 2:

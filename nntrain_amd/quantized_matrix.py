@@ -49,6 +49,31 @@ class HipQuantizedMatrix:
         self._lane: HipExecutionLane | None = None
         self._device_payload: HipBuffer | None = None
 
+    @classmethod
+    def from_device(cls, lane: HipExecutionLane, buffer: HipBuffer, ggml_type: int, output_width: int,
+                    input_width: int) -> "HipQuantizedMatrix":
+        """A matrix whose raw blocks are already in `buffer` on `lane` (streamed there piece by piece); the matrix
+        takes ownership of the buffer and is bound to that lane, like one whose host payload was dropped."""
+        if ggml_type not in BLOCK_ELEMS:
+            raise NotImplementedError(f"GGML type {ggml_type} is not a supported quantized matrix type.")
+        if output_width <= 0 or input_width <= 0:
+            raise ValueError("outputWidth and inputWidth must be positive.")
+        elems = BLOCK_ELEMS[ggml_type]
+        if input_width % elems != 0:
+            raise NotImplementedError(f"Quantized rows must contain complete {elems}-value blocks.")
+        expected = output_width * (input_width // elems) * BLOCK_BYTES[ggml_type]
+        if buffer.nbytes < expected:
+            raise ValueError(f"Quantized matrix payload has {buffer.nbytes} bytes; expected {expected}.")
+        self = cls.__new__(cls)
+        self._payload = None
+        self._storage_bytes = expected
+        self.ggml_type = ggml_type
+        self.output_width = output_width
+        self.input_width = input_width
+        self._lane = lane
+        self._device_payload = buffer
+        return self
+
     @property
     def storage_bytes(self) -> int:
         return int(self._payload.size) if self._payload is not None else self._storage_bytes

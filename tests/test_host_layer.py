@@ -167,3 +167,67 @@ def test_synthetic_payload_generators():
         assert p.size == 5 * 2 * nn.BLOCK_BYTES[typ]
         assert np.all(np.isfinite(oracle.dequantize(typ, p)))
     assert np.array_equal(synth.to_bf16_bits(np.array([1.0, -2.0], np.float32)), np.array([0x3F80, 0xC000], np.uint16))
+
+
+# ------------------------------------------------------------------------------------------------ tensor directory
+
+def test_tensor_directory_checks_follow_the_reference(tmp_path):
+    """Qwen35Gguf.ValidateDirectory (NNtrain.Core/Serialization/Qwen35Gguf.cs:110-193): the same cases, same kinds."""
+    from nntrain_amd import GgufTensorDirectory, NotSupportedError
+    tail = b"\0" * 4096
+    path = _gguf(tmp_path, tensors=[("a.weight", (512, 7), 12, 0), ("n.weight", (512,), 0, 2048), ("h.weight", (16,), 1, 4000)],
+                 tail=tail)
+    with GgufReader(path) as r:
+        d = GgufTensorDirectory(r)
+        assert d.matrix("a.weight", 512, 7).type == 12
+        assert d.dense("n.weight", 512).type == 0
+        with pytest.raises(InvalidDataError, match="missing"):
+            d.matrix("b.weight", 512, 7)
+        with pytest.raises(InvalidDataError, match=r"shape \[512,7\] does not match expected \[7,512\]"):
+            d.matrix("a.weight", 7, 512)                      # GGUF order is [input_width, output_width]
+        with pytest.raises(NotSupportedError, match="F32/F16/BF16"):
+            d.dense("a.weight", 512, 7)
+        with pytest.raises(NotSupportedError, match="storage; got type 0"):
+            nn.loader.check_matrix_storage(nn.GgufTensorInfo("f32.weight", (512, 1), 0, 0))
+        with pytest.raises(NotSupportedError, match="Unexpected tensor 'h.weight'"):
+            d.reject_unexpected()
+        d.dense("h.weight", 16)
+        d.reject_unexpected()
+    with GgufReader(_gguf(tmp_path, tensors=[("w", (256, 1), 12, 0), ("w", (256, 1), 12, 256)], tail=tail)) as r:
+        with pytest.raises(InvalidDataError, match="Duplicate GGUF tensor 'w'"):
+            GgufTensorDirectory(r)
+    with pytest.raises(InvalidDataError, match="divisible by 256"):
+        nn.loader.check_matrix_storage(nn.GgufTensorInfo("short", (128, 3), 12, 0))
+    with pytest.raises(InvalidDataError, match="divisible by 32"):
+        nn.loader.check_matrix_storage(nn.GgufTensorInfo("short", (48, 3), 8, 0))
+    with pytest.raises(NotSupportedError, match="payload limit"):
+        nn.loader.check_matrix_storage(nn.GgufTensorInfo("huge", (256, 1 << 24), 12, 0))     # 144 * 2^24 > 2^31 - 1
+    assert nn.loader.check_matrix_storage(nn.GgufTensorInfo("lm_head", (5376, 262144), 8, 0)) == 1_497_366_528
+    with pytest.raises(NotSupportedError, match="payload limit"):
+        nn.loader.check_dense_storage(nn.GgufTensorInfo("big", (1 << 30,), 0, 0))
+
+
+def test_dense_widening_is_exact():
+    from nntrain_amd.loader import widen_dense
+    f16 = np.array([0x0001, 0x03ff, 0x0400, 0x3c00, 0xbc00, 0x7bff, 0x8000, 0x7c00], np.uint16)
+    got = widen_dense(1, f16.tobytes())
+    assert np.array_equal(got.view(np.uint32), f16.view(np.float16).astype(np.float32).view(np.uint32))
+    assert got[0] == np.float32(2.0 ** -24) and np.isinf(got[-1])
+    bf16 = np.array([0x3f80, 0xc000, 0x0001, 0x7f80], np.uint16)
+    assert np.array_equal(widen_dense(30, bf16.tobytes()).view(np.uint32), bf16.astype(np.uint32) << 16)
+    f32 = np.array([1.5, -0.0, 3e-45], np.float32)
+    assert np.array_equal(widen_dense(0, f32.tobytes()).view(np.uint32), f32.view(np.uint32))
+
+
+def test_gguf_ranged_reads(tmp_path):
+    from gguf_writer import write_gguf
+    payload = bytes(range(256)) * 9                       # 16 Q4_K blocks = 2304 bytes
+    path = write_gguf(tmp_path / "r.gguf", [("pad", (32,), 8, b"\x11" * 34), ("w", (256, 16), 12, payload)])
+    with GgufReader(path) as r:
+        t = r.get_tensor("w")
+        assert r.read_tensor_bytes(t) == payload
+        assert r.read_tensor_range(t, 0, 10) == payload[:10]
+        assert r.read_tensor_range(t, 1000, 1304) == payload[1000:]
+        assert r.read_tensor_range(t, 2304, 0) == b""
+        with pytest.raises(ValueError):
+            r.read_tensor_range(t, 2300, 5)
