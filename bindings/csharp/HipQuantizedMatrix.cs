@@ -1,6 +1,6 @@
 // Immutable GGUF block-quantized matrix resident in HBM.  Same constructor checks, exceptions and Forward contract as
 // ArcQuantizedMatrix (NNtrain.Core/Serialization/ArcQuantizedMatrix.cs:16-60) and Qwen35QuantizedModel.Matrix.Forward
-// (NNtrain.Core/Modules/Qwen35QuantizedModel.cs:1210-1369), extended to GGML types 8, 12, 13, 14, 21 and 22.
+// (NNtrain.Core/Modules/Qwen35QuantizedModel.cs:1210-1369), extended to GGML types 8, 12, 13, 14, 21, 22 and 30 (bfloat16).
 namespace NNtrain.Hip;
 
 public sealed class HipQuantizedMatrix : IDisposable

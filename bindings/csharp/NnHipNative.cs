@@ -11,7 +11,7 @@ internal static unsafe partial class NnHipNative
     private const string Library = "nnhip";   // resolves to libnnhip.so / nnhip.dll
 
     internal const uint SupportedAbiMajor = 1;
-    internal const uint TypeQ8_0 = 8, TypeQ4K = 12, TypeQ5K = 13, TypeQ6K = 14, TypeIQ3S = 21, TypeIQ2S = 22;
+    internal const uint TypeQ8_0 = 8, TypeQ4K = 12, TypeQ5K = 13, TypeQ6K = 14, TypeIQ3S = 21, TypeIQ2S = 22, TypeBF16 = 30;
 
     [StructLayout(LayoutKind.Sequential)]
     internal struct ErrorInfo

@@ -43,7 +43,9 @@ enum {
     NNHIP_TYPE_Q5_K = 13,
     NNHIP_TYPE_Q6_K = 14,
     NNHIP_TYPE_IQ3_S = 21,
-    NNHIP_TYPE_IQ2_S = 22
+    NNHIP_TYPE_IQ2_S = 22,
+    NNHIP_TYPE_BF16 = 30    /* unquantized bfloat16 matrix storage (Qwen35Gguf.cs:12-13); one 2-byte "block" per weight, the
+                             * mat-vec needs rows of a multiple of 64 weights */
 };
 
 /* Status codes.  Positive values below 1000 are this library's own; HIP runtime errors are reported as
@@ -51,7 +53,7 @@ enum {
 enum {
     NNHIP_OK = 0,
     NNHIP_ERR_INVALID_ARGUMENT = 1,   /* null pointer, non-positive width, rows < 1 ...                */
-    NNHIP_ERR_UNSUPPORTED_TYPE = 2,   /* ggml_type is not one of the six above                          */
+    NNHIP_ERR_UNSUPPORTED_TYPE = 2,   /* ggml_type is not one of the seven above                        */
     NNHIP_ERR_INCOMPLETE_BLOCKS = 3,  /* in_w (or elements) is not a whole number of blocks             */
     NNHIP_ERR_OUT_OF_MEMORY = 4,
     NNHIP_ERR_HIP = 5,                /* a HIP call failed                                               */

@@ -10,7 +10,7 @@ Nothing here computes on the CPU: every operator call goes to the HIP library an
 """
 from .native import NnHipError, abi_version, library_path, load_library  # noqa: F401
 from .lane import HipBuffer, HipExecutionLane  # noqa: F401
-from .quantized_matrix import (BLOCK_BYTES, BLOCK_ELEMS, GGML_IQ2_S, GGML_IQ3_S, GGML_Q4_K, GGML_Q5_K,  # noqa: F401
-                               GGML_Q6_K, GGML_Q8_0, HipQuantizedMatrix)
+from .quantized_matrix import (BLOCK_BYTES, BLOCK_ELEMS, GGML_BF16, GGML_IQ2_S, GGML_IQ3_S, GGML_Q4_K,  # noqa: F401
+                               GGML_Q5_K, GGML_Q6_K, GGML_Q8_0, HipQuantizedMatrix)
 from .gguf import GgufReader, GgufReadLimits, GgufTensorInfo, InvalidDataError  # noqa: F401
 from .loader import GgufTensorDirectory, HipGgufLoader, NotSupportedError  # noqa: F401

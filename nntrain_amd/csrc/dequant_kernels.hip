@@ -113,6 +113,13 @@ __device__ __forceinline__ float4 deq4_iq3_s(const uint8_t* w, int64_t e)
     return v;
 }
 
+__device__ __forceinline__ float4 deq4_bf16(const uint8_t* w, int64_t e)
+{
+    const u32x2 v = ld64(w + 2 * e);        // four bfloat16: each is the upper half of its FP32 value
+    return make_float4(__uint_as_float(v[0] << 16), __uint_as_float(v[0] & 0xffff0000u), __uint_as_float(v[1] << 16),
+                       __uint_as_float(v[1] & 0xffff0000u));
+}
+
 template <uint32_t TYPE>
 __global__ __launch_bounds__(256) void dequantize_kernel(const uint8_t* __restrict__ w, float4* __restrict__ out,
                                                          int64_t quads)
@@ -126,6 +133,7 @@ __global__ __launch_bounds__(256) void dequantize_kernel(const uint8_t* __restri
         else if (TYPE == NNHIP_TYPE_Q5_K) v = deq4_q45_k<true>(w, e);
         else if (TYPE == NNHIP_TYPE_Q6_K) v = deq4_q6_k(w, e);
         else if (TYPE == NNHIP_TYPE_IQ3_S) v = deq4_iq3_s(w, e);
+        else if (TYPE == NNHIP_TYPE_BF16) v = deq4_bf16(w, e);
         else v = deq4_iq2_s(w, e);
         out[t] = v;
     }
@@ -161,6 +169,7 @@ hipError_t launch_dequantize(Lane* lane, uint32_t type, const void* w, float* ou
     case NNHIP_TYPE_Q6_K: return launch_deq<NNHIP_TYPE_Q6_K>(lane, w, out, elements);
     case NNHIP_TYPE_IQ3_S: return launch_deq<NNHIP_TYPE_IQ3_S>(lane, w, out, elements);
     case NNHIP_TYPE_IQ2_S: return launch_deq<NNHIP_TYPE_IQ2_S>(lane, w, out, elements);
+    case NNHIP_TYPE_BF16: return launch_deq<NNHIP_TYPE_BF16>(lane, w, out, elements);
     default: return hipErrorInvalidValue;
     }
 }

@@ -268,57 +268,63 @@ __global__ __launch_bounds__(kGemmAll) void matmul_q4k_bf16_kernel(GemmArgs a)
     // ---------------------------------------------------------------------------------------------- consumers
     // waves w and w + 4 usually share a SIMD: giving them different column halves balances the matrix pipes
     const int wm = wave % WM, wn = wave / WM;
-    const int ct0 = wn * CTW, ct_n = wn == WN - 1 ? CT - ct0 : CTW;   // this wave's column tiles [ct0, ct0 + ct_n)
-    f32x4 acc[MT][CTW];
-#pragma unroll
-    for (int i = 0; i < MT; ++i)
-#pragma unroll
-        for (int j = 0; j < CTW; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-
+    const int ct0 = wn * CTW;                       // this wave's column tiles start here
     // operand address of this lane inside a 16-row tile: row lane % 16, k-group lane / 16
     const int frag = (lane & 15) * kRowBytes + lds_slot(lane & 15, lane >> 4) * 16;
-    __syncthreads();        // the first raw blocks are staged
-    __syncthreads();        // their scales are staged
-    __syncthreads();        // the tiles of K slice 0 are ready
-    for (int it = 0; it < iters; ++it) {
-        const uint8_t* xb = xs + (it & 1) * 2 * kXTile;
-        const uint8_t* wb = ws + (it & 1) * 2 * kWTile;
+
+    // The whole consumer body is instantiated per tile count NT, so the loop is straight-line code: a wave-uniform
+    // "does this wave have a fifth tile" test inside the loop would put that tile's operand read and its wait in a
+    // block of their own, twice per iteration.
+    auto consume = [&](auto nt_tag) {
+        constexpr int NT = decltype(nt_tag)::value;
+        f32x4 acc[MT][NT];
 #pragma unroll
-        for (int sub = 0; sub < 2; ++sub) {
-            bf16x8 afrag[MT];
+        for (int i = 0; i < MT; ++i)
 #pragma unroll
-            for (int i = 0; i < MT; ++i)
-                afrag[i] = *reinterpret_cast<const bf16x8*>(xb + sub * kXTile + (wm * RW + i * 16) * kRowBytes + frag);
+            for (int j = 0; j < NT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        __syncthreads();        // the first raw blocks are staged
+        __syncthreads();        // their scales are staged
+        __syncthreads();        // the tiles of K slice 0 are ready
+        for (int it = 0; it < iters; ++it) {
+            const uint8_t* xb = xs + (it & 1) * 2 * kXTile + wm * RW * kRowBytes + frag;
+            const uint8_t* wb = ws + (it & 1) * 2 * kWTile + ct0 * 16 * kRowBytes + frag;
 #pragma unroll
-            for (int j = 0; j < CTW; ++j) {
-                if (j < ct_n) {        // wave-uniform: the last wave column may have one tile less
-                    const bf16x8 bfrag = *reinterpret_cast<const bf16x8*>(wb + sub * kWTile + (ct0 + j) * 16 * kRowBytes + frag);
+            for (int sub = 0; sub < 2; ++sub) {
+                bf16x8 afrag[MT];
+#pragma unroll
+                for (int i = 0; i < MT; ++i)
+                    afrag[i] = *reinterpret_cast<const bf16x8*>(xb + sub * kXTile + i * 16 * kRowBytes);
+#pragma unroll
+                for (int j = 0; j < NT; ++j) {
+                    const bf16x8 bfrag = *reinterpret_cast<const bf16x8*>(wb + sub * kWTile + j * 16 * kRowBytes);
 #pragma unroll
                     for (int i = 0; i < MT; ++i)
                         acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[i], bfrag, acc[i][j], 0, 0, 0);
                 }
             }
+            __syncthreads();
         }
-        __syncthreads();
-    }
-
-    // accumulator element v of a tile: row 4 * (lane / 16) + v, column lane % 16
+        // accumulator element v of a tile: row 4 * (lane / 16) + v, column lane % 16
 #pragma unroll
-    for (int j = 0; j < CTW; ++j) {
-        const int cn = (ct0 + j) * 16 + (lane & 15);
-        const int n = n0 + cn;
-        if (j < ct_n && cn < a.cols && n < a.N) {
-            const float b = a.bias ? a.bias[n] : 0.0f;
+        for (int j = 0; j < NT; ++j) {
+            const int cn = (ct0 + j) * 16 + (lane & 15);
+            const int n = n0 + cn;
+            if (cn < a.cols && n < a.N) {
+                const float b = a.bias ? a.bias[n] : 0.0f;
 #pragma unroll
-            for (int i = 0; i < MT; ++i) {
+                for (int i = 0; i < MT; ++i) {
 #pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    const int m = m0 + wm * RW + i * 16 + (lane >> 4) * 4 + v;
-                    if (m < a.M) a.y[static_cast<size_t>(m) * a.N + n] = acc[i][j][v] + b;
+                    for (int v = 0; v < 4; ++v) {
+                        const int m = m0 + wm * RW + i * 16 + (lane >> 4) * 4 + v;
+                        if (m < a.M) a.y[static_cast<size_t>(m) * a.N + n] = acc[i][j][v] + b;
+                    }
                 }
             }
         }
-    }
+    };
+    constexpr int kLastTiles = CT - (WN - 1) * CTW;     // tiles of the last wave column
+    if (kLastTiles == CTW || wn < WN - 1) consume(std::integral_constant<int, CTW>{});
+    else consume(std::integral_constant<int, kLastTiles>{});
 }
 
 template <int RW, int CT, int WN>

@@ -439,6 +439,49 @@ struct IQ3SUnit {
     }
 };
 
+// ---------------------------------------------------------------------------------------------------- BF16
+// Unquantized bfloat16 rows: a unit is 64 weights = 128 bytes; a bfloat16 is the upper half of its FP32 value.
+struct BF16Unit {
+    static constexpr int kGridWords = 0;
+    struct X { XChunk c; };
+    struct Regs { u32x4 v[8]; };
+
+    static __device__ __forceinline__ X load_x(const float4* x, int unit)
+    {
+        X r;
+        r.c = load_chunk(x, unit);
+        return r;
+    }
+
+    static __device__ __forceinline__ Regs load(const uint8_t* row, int unit)
+    {
+        const uint8_t* p = row + static_cast<uint32_t>(unit) * 128u;
+        Regs r;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) r.v[i] = *reinterpret_cast<const u32x4*>(p + 16 * i);
+        return r;
+    }
+
+    static __device__ __forceinline__ float dot(const Regs& r, const X& x, int, const uint32_t*)
+    {
+        float acc0 = 0.0f, acc1 = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const u32x4 w = r.v[i];
+            const float4 xa = x.c.p[2 * i], xb = x.c.p[2 * i + 1];
+            acc0 = fmaf(__uint_as_float(w[0] << 16), xa.x, acc0);
+            acc1 = fmaf(__uint_as_float(w[0] & 0xffff0000u), xa.y, acc1);
+            acc0 = fmaf(__uint_as_float(w[1] << 16), xa.z, acc0);
+            acc1 = fmaf(__uint_as_float(w[1] & 0xffff0000u), xa.w, acc1);
+            acc0 = fmaf(__uint_as_float(w[2] << 16), xb.x, acc0);
+            acc1 = fmaf(__uint_as_float(w[2] & 0xffff0000u), xb.y, acc1);
+            acc0 = fmaf(__uint_as_float(w[3] << 16), xb.z, acc0);
+            acc1 = fmaf(__uint_as_float(w[3] & 0xffff0000u), xb.w, acc1);
+        }
+        return acc0 + acc1;
+    }
+};
+
 // ---------------------------------------------------------------------------------------------- the kernel
 // Launch shape of one block format: lanes per workgroup, waves per SIMD the register budget is sized for, and the
 // number of weight register sets that rotate (DEPTH - 1 row steps are in flight while one is reduced): kDepth for a
@@ -451,6 +494,7 @@ template <> struct Shape<Q5KUnit> { static constexpr int kMaxT = 768, kWavesPerE
 template <> struct Shape<Q6KUnit> { static constexpr int kMaxT = 768, kWavesPerEu = 3, kDepth = 2, kBatchDepth = 4; };
 template <> struct Shape<IQ2SUnit> { static constexpr int kMaxT = 1024, kWavesPerEu = 4, kDepth = 2, kBatchDepth = 4; };
 template <> struct Shape<IQ3SUnit> { static constexpr int kMaxT = 1024, kWavesPerEu = 4, kDepth = 2, kBatchDepth = 4; };
+template <> struct Shape<BF16Unit> { static constexpr int kMaxT = 512, kWavesPerEu = 2, kDepth = 2, kBatchDepth = 2; };
 
 // grid.x = workgroups striding over row steps, grid.y = input rows, blockDim.x = T (a multiple of 64).
 template <class Q>
@@ -865,16 +909,18 @@ void shape_of(uint32_t type, int* max_t, int* depth)
     case NNHIP_TYPE_Q5_K: *max_t = Shape<Q5KUnit>::kMaxT; *depth = Shape<Q5KUnit>::kBatchDepth; break;
     case NNHIP_TYPE_Q6_K: *max_t = Shape<Q6KUnit>::kMaxT; *depth = Shape<Q6KUnit>::kBatchDepth; break;
     case NNHIP_TYPE_IQ3_S: *max_t = Shape<IQ3SUnit>::kMaxT; *depth = Shape<IQ3SUnit>::kBatchDepth; break;
+    case NNHIP_TYPE_BF16: *max_t = Shape<BF16Unit>::kMaxT; *depth = Shape<BF16Unit>::kBatchDepth; break;
     default: *max_t = Shape<IQ2SUnit>::kMaxT; *depth = Shape<IQ2SUnit>::kBatchDepth; break;
     }
 }
 
 }  // namespace
 
-int matvec_max_in_w(uint32_t)
+int matvec_max_in_w(uint32_t type)
 {
     const int by_lds = kMaxDynamicLds / (kChunkPieces * static_cast<int>(sizeof(float4))) * kUnitW;
-    const int by_lanes = 768 * kUnitW;   // the narrowest workgroup shape must still hold one row
+    // one row must fit the workgroup: 768 lanes for the narrowest block-format shape, 512 for bfloat16 rows
+    const int by_lanes = (type == NNHIP_TYPE_BF16 ? Shape<BF16Unit>::kMaxT : 768) * kUnitW;
     return by_lds < by_lanes ? by_lds : by_lanes;
 }
 
@@ -905,6 +951,7 @@ hipError_t launch_matvec(Lane* lane, uint32_t type, const float* x, const void* 
     case NNHIP_TYPE_Q5_K: return launch_rowstep<Q5KUnit>(lane, a, rows);
     case NNHIP_TYPE_Q6_K: return launch_rowstep<Q6KUnit>(lane, a, rows);
     case NNHIP_TYPE_IQ3_S: return launch_rowstep<IQ3SUnit>(lane, a, rows);
+    case NNHIP_TYPE_BF16: return launch_rowstep<BF16Unit>(lane, a, rows);
     case NNHIP_TYPE_IQ2_S: return launch_rowstep<IQ2SUnit>(lane, a, rows);
     default: return hipErrorInvalidValue;
     }
@@ -913,8 +960,8 @@ hipError_t launch_matvec(Lane* lane, uint32_t type, const float* x, const void* 
 
 hipError_t launch_matvec_batch(Lane* lane, const nnhip_matvec_desc* descs, int count)
 {
-    static const uint32_t kTypes[6] = {NNHIP_TYPE_Q8_0, NNHIP_TYPE_Q4_K, NNHIP_TYPE_Q5_K, NNHIP_TYPE_Q6_K, NNHIP_TYPE_IQ3_S,
-                                       NNHIP_TYPE_IQ2_S};
+    static const uint32_t kTypes[7] = {NNHIP_TYPE_Q8_0, NNHIP_TYPE_Q4_K, NNHIP_TYPE_Q5_K, NNHIP_TYPE_Q6_K, NNHIP_TYPE_IQ3_S,
+                                       NNHIP_TYPE_IQ2_S, NNHIP_TYPE_BF16};
     std::vector<BatchEntry> all;
     struct Group { uint32_t type; size_t begin, end; int total_chunks, max_in_w; };
     std::vector<Group> groups;
@@ -994,6 +1041,7 @@ hipError_t launch_matvec_batch(Lane* lane, const nnhip_matvec_desc* descs, int c
         case NNHIP_TYPE_Q5_K: e = launch_batch_of<Q5KUnit>(lane, g.total_chunks, g.max_in_w, off); break;
         case NNHIP_TYPE_Q6_K: e = launch_batch_of<Q6KUnit>(lane, g.total_chunks, g.max_in_w, off); break;
         case NNHIP_TYPE_IQ3_S: e = launch_batch_of<IQ3SUnit>(lane, g.total_chunks, g.max_in_w, off); break;
+        case NNHIP_TYPE_BF16: e = launch_batch_of<BF16Unit>(lane, g.total_chunks, g.max_in_w, off); break;
         default: e = launch_batch_of<IQ2SUnit>(lane, g.total_chunks, g.max_in_w, off); break;
         }
         if (e != hipSuccess) return e;

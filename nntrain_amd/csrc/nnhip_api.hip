@@ -49,7 +49,9 @@ int check_linear(uint32_t op, Lane* lane, uint32_t type, const void* x, const vo
         return fail(NNHIP_ERR_INCOMPLETE_BLOCKS, op, lane->device, 0, "quantized rows must contain complete %d-value blocks (in_w = %d)", elems, in_w);
     if ((reinterpret_cast<uintptr_t>(x) & 15u) || (reinterpret_cast<uintptr_t>(y) & 3u))
         return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0, "x must be 16-byte aligned and y 4-byte aligned");
-    const uintptr_t wa = (type == NNHIP_TYPE_Q4_K || type == NNHIP_TYPE_Q5_K) ? 15u : 3u;
+    if (type == NNHIP_TYPE_BF16 && op != NNHIP_OP_DEQUANTIZE && in_w % 64 != 0)
+        return fail(NNHIP_ERR_INCOMPLETE_BLOCKS, op, lane->device, 0, "bfloat16 rows must hold a multiple of 64 weights (in_w = %d)", in_w);
+    const uintptr_t wa = (type == NNHIP_TYPE_Q4_K || type == NNHIP_TYPE_Q5_K || type == NNHIP_TYPE_BF16) ? 15u : 3u;
     if (reinterpret_cast<uintptr_t>(w) & wa)
         return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0, "weight pointer must be %u-byte aligned", static_cast<unsigned>(wa + 1));
     return NNHIP_OK;
@@ -67,6 +69,7 @@ bool type_block(uint32_t type, int* elems, int* bytes)
     case NNHIP_TYPE_Q6_K: e = 256; b = 210; break;
     case NNHIP_TYPE_IQ3_S: e = 256; b = 110; break;
     case NNHIP_TYPE_IQ2_S: e = 256; b = 82; break;
+    case NNHIP_TYPE_BF16: e = 1; b = 2; break;
     default: return false;
     }
     if (elems) *elems = e;
@@ -342,6 +345,7 @@ int nnhip_dequantize(void* handle, uint32_t ggml_type, const void* w, float* out
     if (!type_block(ggml_type, &elems, &bytes))
         return fail(NNHIP_ERR_UNSUPPORTED_TYPE, NNHIP_OP_DEQUANTIZE, lane->device, 0, "GGML type %u is not a supported quantized matrix type", ggml_type);
     if (elements < 0) return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_DEQUANTIZE, lane->device, 0, "element count must be non-negative");
+    if (ggml_type == NNHIP_TYPE_BF16) elems = 4;     // decoded four at a time
     if (elements % elems != 0)
         return fail(NNHIP_ERR_INCOMPLETE_BLOCKS, NNHIP_OP_DEQUANTIZE, lane->device, 0, "element count must be a multiple of %d", elems);
     if (elements == 0) return NNHIP_OK;

@@ -29,7 +29,8 @@ class NotSupportedError(NotImplementedError):
 
 
 def is_quantized_matrix(tensor: GgufTensorInfo) -> bool:
-    """A 2-D tensor stored in one of the block formats the mat-vec kernels read."""
+    """A 2-D tensor stored in one of the formats the mat-vec kernels read (block formats and bfloat16; a 2-D F16 or
+    F32 tensor is a dense tensor, as in Qwen35Gguf.IsSupportedMatrixStorage)."""
     return len(tensor.shape) == 2 and tensor.type in BLOCK_ELEMS
 
 
@@ -83,7 +84,7 @@ def check_matrix_storage(tensor: GgufTensorInfo) -> int:
     if len(tensor.shape) != 2:
         raise InvalidDataError(f"GGUF tensor '{tensor.name}' is not a matrix.")
     if tensor.type not in BLOCK_ELEMS:
-        raise NotSupportedError(f"Matrix '{tensor.name}' requires Q8_0/Q4_K/Q5_K/Q6_K/IQ3_S/IQ2_S storage; got type "
+        raise NotSupportedError(f"Matrix '{tensor.name}' requires Q8_0/Q4_K/Q5_K/Q6_K/IQ3_S/IQ2_S/BF16 storage; got type "
                                 f"{tensor.type}.")
     input_width, output_width = int(tensor.shape[0]), int(tensor.shape[1])
     elems = BLOCK_ELEMS[tensor.type]

@@ -2,7 +2,7 @@
 
 Constructor checks, error kinds and `forward` semantics follow ArcQuantizedMatrix
 (NNtrain.Core/Serialization/ArcQuantizedMatrix.cs:16-60) and Qwen35QuantizedModel.Matrix.Forward
-(NNtrain.Core/Modules/Qwen35QuantizedModel.cs:1210-1369), extended from Q4_K/Q6_K to the six types of this path.
+(NNtrain.Core/Modules/Qwen35QuantizedModel.cs:1210-1369), extended from Q4_K/Q6_K to the seven storage types of this path (six block formats and bfloat16).
 Exceptions map as: NotSupportedException -> NotImplementedError, ArgumentOutOfRangeException/ArgumentException ->
 ValueError, InvalidDataException -> ValueError("... payload ...").
 """
@@ -16,9 +16,11 @@ from . import native
 from .lane import HipBuffer, HipExecutionLane
 from .native import check
 
-GGML_Q8_0, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_IQ3_S, GGML_IQ2_S = 8, 12, 13, 14, 21, 22
-BLOCK_ELEMS = {GGML_Q8_0: 32, GGML_Q4_K: 256, GGML_Q5_K: 256, GGML_Q6_K: 256, GGML_IQ3_S: 256, GGML_IQ2_S: 256}
-BLOCK_BYTES = {GGML_Q8_0: 34, GGML_Q4_K: 144, GGML_Q5_K: 176, GGML_Q6_K: 210, GGML_IQ3_S: 110, GGML_IQ2_S: 82}
+GGML_Q8_0, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_IQ3_S, GGML_IQ2_S, GGML_BF16 = 8, 12, 13, 14, 21, 22, 30
+BLOCK_ELEMS = {GGML_Q8_0: 32, GGML_Q4_K: 256, GGML_Q5_K: 256, GGML_Q6_K: 256, GGML_IQ3_S: 256, GGML_IQ2_S: 256,
+               GGML_BF16: 1}
+BLOCK_BYTES = {GGML_Q8_0: 34, GGML_Q4_K: 144, GGML_Q5_K: 176, GGML_Q6_K: 210, GGML_IQ3_S: 110, GGML_IQ2_S: 82,
+               GGML_BF16: 2}
 
 # rows at or above which forward() uses the bf16 MFMA mat-mul when asked to (Qwen35QuantizedModel.cs:1249: rows >= 16)
 PREFILL_MIN_ROWS = 16

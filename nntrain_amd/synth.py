@@ -9,8 +9,8 @@ from __future__ import annotations
 
 import numpy as np
 
-from .quantized_matrix import (BLOCK_BYTES, BLOCK_ELEMS, GGML_IQ2_S, GGML_IQ3_S, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K,
-                               GGML_Q8_0)
+from .quantized_matrix import (BLOCK_BYTES, BLOCK_ELEMS, GGML_BF16, GGML_IQ2_S, GGML_IQ3_S, GGML_Q4_K, GGML_Q5_K,
+                               GGML_Q6_K, GGML_Q8_0)
 
 
 def _rng(seed: int) -> np.random.Generator:
@@ -64,7 +64,15 @@ def k_quant_matrix(ggml_type: int, out_w: int, in_w: int, seed: int, sigma: floa
     return blocks.reshape(-1)
 
 
+def bf16_matrix(out_w: int, in_w: int, seed: int, sigma: float = 0.02) -> np.ndarray:
+    """bfloat16 weights N(0, sigma), as raw bytes."""
+    w = _rng(seed).standard_normal((out_w, in_w), dtype=np.float32) * np.float32(sigma)
+    return to_bf16_bits(w).reshape(-1).view(np.uint8)
+
+
 def matrix(ggml_type: int, out_w: int, in_w: int, seed: int) -> np.ndarray:
+    if ggml_type == GGML_BF16:
+        return bf16_matrix(out_w, in_w, seed)
     if ggml_type == GGML_Q8_0:
         return q8_0_matrix(out_w, in_w, seed)
     return k_quant_matrix(ggml_type, out_w, in_w, seed)

@@ -22,9 +22,9 @@ import numpy as np
 
 HERE = Path(__file__).resolve().parent
 
-Q8_0, Q4_K, Q5_K, Q6_K, IQ3_S, IQ2_S = 8, 12, 13, 14, 21, 22
-BLOCK_ELEMS = {Q8_0: 32, Q4_K: 256, Q5_K: 256, Q6_K: 256, IQ3_S: 256, IQ2_S: 256}
-BLOCK_BYTES = {Q8_0: 34, Q4_K: 144, Q5_K: 176, Q6_K: 210, IQ3_S: 110, IQ2_S: 82}
+Q8_0, Q4_K, Q5_K, Q6_K, IQ3_S, IQ2_S, BF16 = 8, 12, 13, 14, 21, 22, 30
+BLOCK_ELEMS = {Q8_0: 32, Q4_K: 256, Q5_K: 256, Q6_K: 256, IQ3_S: 256, IQ2_S: 256, BF16: 1}
+BLOCK_BYTES = {Q8_0: 34, Q4_K: 144, Q5_K: 176, Q6_K: 210, IQ3_S: 110, IQ2_S: 82, BF16: 2}
 
 _lib = None
 
@@ -169,6 +169,8 @@ def np_dequantize(ggml_type: int, raw) -> np.ndarray:
     b = raw.reshape(-1, bb)
     n = b.shape[0]
     f32 = np.float32
+    if ggml_type == BF16:
+        return (b.reshape(-1).view('<u2').astype(np.uint32) << 16).view(f32)
     if ggml_type == Q8_0:
         d = _half(b[:, 0:2])
         q = b[:, 2:34].view(np.int8).astype(f32)

@@ -39,7 +39,7 @@
 
 #define ORACLE_EXPORT __attribute__((visibility("default")))
 
-enum { T_Q8_0 = 8, T_Q4_K = 12, T_Q5_K = 13, T_Q6_K = 14, T_IQ3_S = 21, T_IQ2_S = 22 };
+enum { T_Q8_0 = 8, T_Q4_K = 12, T_Q5_K = 13, T_Q6_K = 14, T_IQ3_S = 21, T_IQ2_S = 22, T_BF16 = 30 };
 
 #include "iq_grids.inc"
 static const uint64_t iq2s_grid[1024] = { NNHIP_IQ2S_GRID_VALUES };
@@ -48,6 +48,7 @@ static const uint32_t iq3s_grid[512] = { NNHIP_IQ3S_GRID_VALUES };
 ORACLE_EXPORT int oracle_block_elems(uint32_t type)
 {
     switch (type) {
+    case T_BF16: return 1;
     case T_Q8_0: return 32;
     case T_Q4_K: case T_Q5_K: case T_Q6_K: case T_IQ3_S: case T_IQ2_S: return 256;
     default: return 0;
@@ -57,6 +58,7 @@ ORACLE_EXPORT int oracle_block_elems(uint32_t type)
 ORACLE_EXPORT int oracle_block_bytes(uint32_t type)
 {
     switch (type) {
+    case T_BF16: return 2;
     case T_Q8_0: return 34;
     case T_Q4_K: return 144;
     case T_Q5_K: return 176;
@@ -211,6 +213,11 @@ static void deq_iq3_s(const uint8_t* b, float* out)
 static int deq_block(uint32_t type, const uint8_t* b, float* out)
 {
     switch (type) {
+    case T_BF16: {   /* bfloat16 is the upper half of a binary32 (Qwen2Gguf.cs:349-356) */
+        uint32_t bits = ((uint32_t)b[0] | ((uint32_t)b[1] << 8)) << 16;
+        memcpy(out, &bits, 4);
+        return 0;
+    }
     case T_Q8_0: deq_q8_0(b, out); return 0;
     case T_Q4_K: deq_q4_k(b, out); return 0;
     case T_Q5_K: deq_q5_k(b, out); return 0;

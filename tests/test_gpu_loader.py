@@ -7,7 +7,7 @@ import pytest
 
 import oracle
 from gguf_writer import write_gguf
-from nntrain_amd import (BLOCK_BYTES, BLOCK_ELEMS, GGML_IQ2_S, GGML_IQ3_S, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_Q8_0,
+from nntrain_amd import (BLOCK_BYTES, BLOCK_ELEMS, GGML_BF16, GGML_IQ2_S, GGML_IQ3_S, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_Q8_0,
                          GgufReader, HipExecutionLane, HipGgufLoader, HipQuantizedMatrix, NotSupportedError, synth)
 
 pytestmark = pytest.mark.gpu
@@ -64,7 +64,7 @@ def test_loader_all_block_formats_and_dense_kinds(lane, tmp_path):
     byte-identical to a direct upload (same kernel results bit for bit), whatever the piece size."""
     rng = np.random.default_rng(77)
     specs = [(GGML_Q8_0, 160, 9), (GGML_Q4_K, 512, 5), (GGML_Q5_K, 256, 3), (GGML_Q6_K, 768, 4), (GGML_IQ3_S, 512, 6),
-             (GGML_IQ2_S, 256, 7)]
+             (GGML_IQ2_S, 256, 7), (GGML_BF16, 192, 5)]
     tensors, payloads = [], {}
     for typ, in_w, out_w in specs:
         p = synth.matrix(typ, out_w, in_w, 900 + typ)

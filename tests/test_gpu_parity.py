@@ -367,3 +367,40 @@ def test_prefill_matmul_full_width_sample(lane):
     assert rel <= PREFILL_BAR
     x.dispose()
     mat.dispose()
+
+
+# ----------------------------------------------------------------------------------------------- bfloat16 storage
+
+def test_bf16_matrix_storage(lane):
+    """Unquantized bfloat16 matrices (the reference's "bf16" matrix storage, Qwen35Gguf.cs:12-13): widening is exact,
+    the mat-vec meets the same bar as the block formats, rows are independent, the batched entry is bit-identical."""
+    from nntrain_amd import GGML_BF16
+    from nntrain_amd.native import MatvecDesc
+    from ctypes import c_void_p
+    for in_w, out_w, rows in [(64, 1, 1), (512, 7, 3), (5376, 131, 1), (21504, 33, 2)]:
+        payload = synth.matrix(GGML_BF16, out_w, in_w, 40 + out_w)
+        want = oracle.dequantize(GGML_BF16, payload)
+        assert np.array_equal(_bits(want), payload.view("<u2").astype(np.uint32) << 16)
+        mat = HipQuantizedMatrix(payload, GGML_BF16, out_w, in_w)
+        assert np.array_equal(_bits(lane.read(mat.dequantize(lane))), _bits(want))
+        assert np.array_equal(_bits(lane.read(mat.dequantize(lane, row=out_w - 1))), _bits(want[-in_w:]))
+        x = synth.activations(rows, in_w, 6)
+        bias = np.random.default_rng(3).standard_normal(out_w).astype(np.float32)
+        y = _run_matvec(lane, GGML_BF16, payload, x, bias, rows, in_w, out_w)
+        ref, asum = oracle.linear_f64(GGML_BF16, payload, x, bias, rows, in_w, out_w)
+        _check_against_f64(y, ref, asum)
+        y1 = np.stack([_run_matvec(lane, GGML_BF16, payload, x[r:r + 1], bias, 1, in_w, out_w)[0] for r in range(rows)])
+        assert np.array_equal(_bits(y), _bits(y1))
+        xb, bb, yb = lane.upload_raw(x), lane.upload_raw(bias), lane.allocate(rows * out_w)
+        desc = (MatvecDesc * 1)(MatvecDesc(xb.ptr, mat.device_payload(lane).ptr, bb.ptr, yb.ptr, GGML_BF16, rows, in_w, out_w))
+        assert lane._lib.nnhip_quant_matvec_batch(lane._handle, desc, 1) == 0
+        assert np.array_equal(_bits(lane.read(yb)), _bits(y.reshape(-1)))
+        for b in (xb, bb, yb):
+            b.dispose()
+        mat.dispose()
+    lib, h = lane._lib, lane._handle
+    buf = lane.allocate(4096)
+    assert lib.nnhip_quant_matvec(h, GGML_BF16, c_void_p(buf.ptr), c_void_p(buf.ptr), None, c_void_p(buf.ptr), 1, 96, 2) == 3
+    assert lib.nnhip_dequantize(h, GGML_BF16, c_void_p(buf.ptr), c_void_p(buf.ptr), 6) == 3
+    assert lib.nnhip_dequantize(h, GGML_BF16, c_void_p(buf.ptr), c_void_p(buf.ptr), 8) == 0
+    buf.dispose()
