@@ -9,21 +9,24 @@
 // for the whole K range; the strip width is chosen on the host so that strips x row tiles split evenly over the
 // compute units (17408 columns: 256 strips of 68 for M <= 256, 128 strips of 136 for larger M).  A weight sub-block
 // is dequantized once per workgroup.  K advances 64 per iteration = the two Q4_K sub-blocks that share 32 bytes of
-// nibbles; per iteration two x sub-tiles [BM][32] bf16 and two weight sub-tiles [16 CT][32] bf16 live in LDS, double
-// buffered (rows are 64 bytes, so the 16 rows x 4 k-groups an MFMA operand needs form one contiguous, conflict-free
-// 1 KiB read).
+// nibbles; a slice is two x sub-tiles [BM][32] bf16 and two weight sub-tiles [16 CT][32] bf16 in LDS (rows are 64
+// bytes, placed so that the 16 rows x 4 k-groups an MFMA operand needs are one conflict-free read), in three stages:
+// the slice being multiplied, the finished next one, and the one being made.
 //
 // The 13 waves of a workgroup are specialised:
 //   - 8 consumer waves (8 x 1, or 4 x 2 with 64-row, 5- or 4-tile wave tiles) only read operands from LDS and issue
-//     MFMAs;
+//     MFMAs.  Operand reads run ahead of their use, also across the barrier into the finished next slice, so the
+//     matrix pipe restarts right after a barrier;
 //   - 5 producer waves fill LDS.  Four of them move the x tile (requested two iterations ahead into registers, then
-//     written to the swizzled sub-tiles).  The raw Q4_K blocks of the strip are staged in LDS one 256-block ahead
-//     (144 contiguous bytes per column instead of 8-byte pieces per K slice, which keeps the cache-line count per
-//     load instruction low), their eight (d * scale, dmin * min) pairs are computed once per block, and two threads
-//     per column turn the 32 nibble bytes of a K slice into 32 low-nibble and 32 high-nibble bf16 weights.
+//     written to the sub-tiles).  Two threads per column decode: each keeps the 16 nibble bytes of its next two slices
+//     and the (d * scale, dmin * min) pairs of the current 256-block in registers (the header of the next block is
+//     requested a block ahead), and turns a slice into 16 low-nibble and 16 high-nibble bf16 weights.  Nothing a
+//     producer needs after a barrier has to be waited for.
 // One barrier per iteration joins the two groups: while the consumers multiply slice i, the producers build slice
-// i + 1 in the other LDS buffer.  Measured with either group switched off, the consumers alone take about 1.0 us per
-// iteration (72 MFMAs per SIMD) and the producers alone about 1.2 us; together 1.6 us.
+// i + 2.  Measured with either group switched off (M = 512, 80 iterations): consumers alone 0.85 us per iteration
+// (72 MFMAs per SIMD; 0.62 us at the back-to-back MFMA rate), producers alone 1.04 us, together 1.43 us.  LDS is about
+// as busy as the matrix pipe: 144 KB of operand reads (4 cycles per 1 KB wave read) and 50 KB of tile writes (13
+// cycles per 1 KB wave write) per iteration.
 #include <type_traits>
 
 #include "nnhip_internal.h"
@@ -91,6 +94,7 @@ constexpr int kConsumers = 512;         // 8 MFMA waves
 constexpr int kProducers = 320;         // 5 waves that fetch, decode and fill LDS
 constexpr int kXThreads = 256;          // the producer threads that also move the x tile
 constexpr int kGemmAll = kConsumers + kProducers;
+constexpr int kStages = 3;              // LDS tile stages: multiplied, ready (being pre-read), being made
 
 // Consumer waves are laid out WM x WN (8 in all); a wave owns RW rows and, when WN == 2, the first CTW or the
 // remaining CT - CTW column tiles.
@@ -104,14 +108,10 @@ __global__ __launch_bounds__(kGemmAll) void matmul_q4k_bf16_kernel(GemmArgs a)
     constexpr int CTW = (CT + WN - 1) / WN;         // column tiles of the widest wave
     constexpr int kXTile = BM * kRowBytes;          // bytes of one x sub-tile
     constexpr int kWTile = BN * kRowBytes;          // bytes of one weight sub-tile
-    constexpr int kRawBytes = BN * 144;             // one Q4_K block of every strip column
-    constexpr int kSclBytes = BN * 64;              // its eight (scale, min) pairs
-    // dynamic LDS: xs[buffer][k sub-tile][row][32 bf16] then ws[buffer][k sub-tile][column][32 bf16]
+    // dynamic LDS: xs[stage][k sub-tile][row][32 bf16] then ws[stage][k sub-tile][column][32 bf16], kStages stages
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint8_t* xs = smem;
-    uint8_t* ws = smem + 4 * kXTile;
-    uint8_t* raw = ws + 4 * kWTile;                 // raw[buffer][column][144]: the Q4_K blocks of two K blocks
-    uint8_t* scl = raw + 2 * kRawBytes;             // scl[buffer][column][sub-block][d * scale, dmin * min] as FP32
+    uint8_t* ws = smem + kStages * 2 * kXTile;
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int strip = blockIdx.x, m0 = blockIdx.y * BM;
@@ -121,8 +121,6 @@ __global__ __launch_bounds__(kGemmAll) void matmul_q4k_bf16_kernel(GemmArgs a)
     if (wave >= kConsumers / 64) {
         // ------------------------------------------------------------------------------------------ producers
         constexpr int kXLoads = 2 * kXTile / 16 / kXThreads;                   // 16-byte pieces of x per thread
-        constexpr int kRawPieces = BN * 9;                                     // 16-byte pieces of one block column set
-        constexpr int kRawLoads = (kRawPieces + kProducers - 1) / kProducers;
         static_assert(kXLoads >= 1, "tile too small for the producer count");
         static_assert(2 * BN <= kProducers, "two decoding threads per column");
         const int p = tid - kConsumers;
@@ -139,22 +137,17 @@ __global__ __launch_bounds__(kGemmAll) void matmul_q4k_bf16_kernel(GemmArgs a)
             xsrc[i] = static_cast<uint32_t>((min(r, a.M - 1 - m0) * a.K + grp * 8) * 2);
             xdst[i] = (grp >> 2) * kXTile + r * kRowBytes + lds_slot(r, grp & 3) * 16;
         }
-        // raw piece id of this thread: 16-byte part id % 9 of the 144-byte block of strip column id / 9; the staging
-        // area is [column][144 bytes], so piece id lands at byte 16 * id
-        const uint8_t* wbase = a.w + static_cast<size_t>(n0) * row_bytes;                               // wave-uniform
-        uint32_t rsrc[kRawLoads];   // byte offsets from wbase
-#pragma unroll
-        for (int i = 0; i < kRawLoads; ++i) {
-            const int id = min(p + i * kProducers, kRawPieces - 1);
-            const int col = id / 9, part = id - col * 9;
-            rsrc[i] = static_cast<uint32_t>(min(col, a.N - 1 - n0) * row_bytes + part * 16);
-        }
-        // decoding: thread (column dc, half dh) owns bytes [16 dh, 16 dh + 16) of the 32 nibble bytes of a K slice
+        // decoding: thread (column dc, half dh) owns bytes [16 dh, 16 dh + 16) of the 32 nibble bytes of a K slice:
+        // 16 low-nibble weights of sub-block 2J and 16 high-nibble weights of sub-block 2J + 1
         const bool d_role = p < 2 * BN;
         const int dc = d_role ? p >> 1 : 0, dh = p & 1;
+        const uint8_t* wbase = a.w + static_cast<size_t>(n0) * row_bytes;                               // wave-uniform
+        const uint32_t wrow = static_cast<uint32_t>(min(dc, a.N - 1 - n0) * row_bytes);                 // byte offset
         const int nblocks = a.K >> 8;
-        u32x4 xset[2][kXLoads];
-        u32x4 rawreg[kRawLoads];
+        u32x4 xset[2][kXLoads];     // x pieces of K slices t and t + 1
+        u32x4 nq[2];                // nibble bytes of K slices t and t + 1
+        u32x4 hdr;                  // header (d, dmin, packed scales) of the next 256-block
+        float sm[16];               // (d * scale, dmin * min) of the eight sub-blocks of the current block
         auto load_x = [&](u32x4* set, int t) {
             uint32_t koff = static_cast<uint32_t>(min(t, iters - 1)) << 7;     // past the end: a harmless repeat of the last slice
             asm volatile("" : "+s"(koff));      // keeps the address as scalar base + 32-bit lane offset
@@ -162,104 +155,88 @@ __global__ __launch_bounds__(kGemmAll) void matmul_q4k_bf16_kernel(GemmArgs a)
 #pragma unroll
             for (int i = 0; i < kXLoads; ++i) set[i] = *reinterpret_cast<const u32x4*>(src + opaque(xsrc[i]));
         };
-        auto load_raw = [&](int blk) {
-            uint32_t boff = static_cast<uint32_t>(min(blk, nblocks - 1)) * 144u;
-            asm volatile("" : "+s"(boff));
-            const uint8_t* src = wbase + boff;
-#pragma unroll
-            for (int i = 0; i < kRawLoads; ++i) rawreg[i] = ld128(src + opaque(rsrc[i]));
+        auto load_q = [&](int t) {
+            const int tt = min(t, iters - 1);
+            uint32_t off = static_cast<uint32_t>(tt >> 2) * 144u + 16u + static_cast<uint32_t>(tt & 3) * 32u;
+            asm volatile("" : "+s"(off));
+            return ld128(wbase + off + opaque(wrow + static_cast<uint32_t>(dh) * 16u));
         };
-        auto store_raw = [&](int buf) {
-            uint8_t* dst = raw + buf * kRawBytes;
-#pragma unroll
-            for (int i = 0; i < kRawLoads; ++i) {
-                const int id = p + i * kProducers;
-                if (id < kRawPieces) *reinterpret_cast<u32x4*>(dst + id * 16) = rawreg[i];
-            }
+        auto load_hdr = [&](int blk) {
+            uint32_t off = static_cast<uint32_t>(min(blk, nblocks - 1)) * 144u;
+            asm volatile("" : "+s"(off));
+            hdr = ld128(wbase + off + opaque(wrow));
         };
-        // (d * scale, dmin * min) of sub-blocks 4 dh .. 4 dh + 3 of the staged block, as FP32, for the decoding steps
-        auto make_scales = [&](int buf) {
-            if (!d_role) return;
-            const u32x4 hdr = *reinterpret_cast<const u32x4*>(raw + buf * kRawBytes + dc * 144);
+        // FP32 (d * scale, dmin * min) of all eight sub-blocks from a block header; 6-bit fields as in GgufQ4K.cs:51-60:
+        // sub-blocks 0-3 sit in the low six bits of bytes j and 4 + j, 4-7 are split between bytes 8 + j (low nibble
+        // scale, high nibble min) and the top two bits of bytes j and 4 + j
+        auto make_scales = [&]() {
             const float d = half_bits_to_float(hdr[0]), dmin = half_bits_to_float(hdr[0] >> 16);
-            float v[8];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                // 6-bit fields (GgufQ4K.cs:51-60): sub-blocks 0-3 sit in the low six bits of bytes j and 4 + j; 4-7 are
-                // split between bytes 8 + j (low nibble scale, high nibble min) and the top two bits of bytes j, 4 + j
                 const uint32_t b0 = (hdr[1] >> (8 * j)) & 255u, b1 = (hdr[2] >> (8 * j)) & 255u, b2 = (hdr[3] >> (8 * j)) & 255u;
-                const uint32_t sc = dh ? ((b2 & 15u) | ((b0 >> 6) << 4)) : (b0 & 63u);
-                const uint32_t mn = dh ? ((b2 >> 4) | ((b1 >> 6) << 4)) : (b1 & 63u);
-                v[2 * j] = d * static_cast<float>(sc);
-                v[2 * j + 1] = dmin * static_cast<float>(mn);
+                sm[2 * j] = d * static_cast<float>(b0 & 63u);
+                sm[2 * j + 1] = dmin * static_cast<float>(b1 & 63u);
+                sm[8 + 2 * j] = d * static_cast<float>((b2 & 15u) | ((b0 >> 6) << 4));
+                sm[8 + 2 * j + 1] = dmin * static_cast<float>((b2 >> 4) | ((b1 >> 6) << 4));
             }
-            float* dst = reinterpret_cast<float*>(scl + buf * kSclBytes + dc * 64 + dh * 32);
-            *reinterpret_cast<f32x4*>(dst) = f32x4{v[0], v[1], v[2], v[3]};
-            *reinterpret_cast<f32x4*>(dst + 4) = f32x4{v[4], v[5], v[6], v[7]};
         };
-        // One production step makes the LDS tiles of K slice t: J = t % 4 is the 64-wide slice inside the Q4_K block
-        // (sub-blocks 2J in the low nibbles and 2J + 1 in the high nibbles of its 32 bytes).
-        // The decode inputs of a step are read from LDS one step early (before the barrier that ends the previous
-        // step), so that after the barrier the step starts with arithmetic, not with an LDS round trip.
-        u32x4 nq;
-        f32x4 nsm;
-        auto fetch_inputs = [&](int t, int j) {      // for K slice t, j = t % 4
-            if (!d_role) return;
-            const int buf = (t >> 2) & 1;
-            nq = *reinterpret_cast<const u32x4*>(raw + buf * kRawBytes + dc * 144 + 16 + j * 32 + dh * 16);
-            nsm = *reinterpret_cast<const f32x4*>(scl + buf * kSclBytes + dc * 64 + j * 16);
-        };
-        auto step = [&](int t, auto jt) {
+        // One production step makes the LDS tiles of K slice t in stage `stage`; J = t % 4 is the 64-wide slice inside
+        // the Q4_K block.  Everything it consumes was requested two steps earlier.
+        auto step = [&](int t, int stage, auto jt) {
             constexpr int J = decltype(jt)::value;
-            const int blk = t >> 2;
-            if (J == 0) load_raw(blk + 1);
             if (d_role) {
-                const u32x4 q = nq;
-                const f32x4 sm = nsm;
-                uint8_t* wb = ws + (t & 1) * 2 * kWTile + dc * kRowBytes;
+                const u32x4 q = nq[J & 1];
+                uint8_t* wb = ws + stage * 2 * kWTile + dc * kRowBytes;
 #pragma unroll
                 for (int g = 0; g < 2; ++g) {
                     const uint32_t a0 = q[2 * g], a1 = q[2 * g + 1];
                     const int slot = lds_slot(dc, 2 * dh + g) * 16;
-                    *reinterpret_cast<u32x4*>(wb + slot) = q4k_decode8(a0 & 0x0f0f0f0fu, a1 & 0x0f0f0f0fu, sm[0], sm[1]);
+                    *reinterpret_cast<u32x4*>(wb + slot) =
+                        q4k_decode8(a0 & 0x0f0f0f0fu, a1 & 0x0f0f0f0fu, sm[4 * J], sm[4 * J + 1]);
                     *reinterpret_cast<u32x4*>(wb + kWTile + slot) =
-                        q4k_decode8((a0 >> 4) & 0x0f0f0f0fu, (a1 >> 4) & 0x0f0f0f0fu, sm[2], sm[3]);
+                        q4k_decode8((a0 >> 4) & 0x0f0f0f0fu, (a1 >> 4) & 0x0f0f0f0fu, sm[4 * J + 2], sm[4 * J + 3]);
                 }
+                nq[J & 1] = load_q(t + 2);
+                if (J == 0) load_hdr((t >> 2) + 1);
+                if (J == 3) make_scales();
             }
+            // (writing the x tile before the decode was measured slower: 137 against 114 us at M = 512)
             if (x_role) {
-                u32x4* set = xset[t & 1];
-                uint8_t* xb = xs + (t & 1) * 2 * kXTile;
+                u32x4* set = xset[J & 1];
+                uint8_t* xb = xs + stage * 2 * kXTile;
 #pragma unroll
                 for (int i = 0; i < kXLoads; ++i) *reinterpret_cast<u32x4*>(xb + xdst[i]) = set[i];
                 load_x(set, t + 2);
             }
-            // the next block: requested at J = 0, staged at J = 1, its scales made at J = 2, all visible from J = 3 on
-            if (J == 1) store_raw((blk + 1) & 1);
-            if (J == 2) make_scales((blk + 1) & 1);
-            fetch_inputs(t + 1, (J + 1) & 3);
         };
         using std::integral_constant;
-        load_raw(0);
+        load_hdr(0);
+        nq[0] = load_q(0);
+        nq[1] = load_q(1);
         if (x_role) {
             load_x(xset[0], 0);
             load_x(xset[1], 1);
         }
-        store_raw(0);
+        make_scales();
+        // tiles 0 and 1 before the consumers start; from then on tile i + 2 is made while tile i is multiplied
+        step(0, 0, integral_constant<int, 0>{});
+        step(1, 1, integral_constant<int, 1>{});
         __syncthreads();
-        make_scales(0);
-        __syncthreads();
-        fetch_inputs(0, 0);
-        step(0, integral_constant<int, 0>{});
-        __syncthreads();
-        // K is a whole number of 256-blocks, so iters is a multiple of 4 and the last step of the last group is skipped
+        // K is a whole number of 256-blocks, so iters is a multiple of 4
+        int stage = 2;
+        auto next_stage = [&]() { stage = stage == kStages - 1 ? 0 : stage + 1; };
         for (int i = 0; i < iters; i += 4) {
-            step(i + 1, integral_constant<int, 1>{});
+            if (i + 2 < iters) step(i + 2, stage, integral_constant<int, 2>{});
+            next_stage();
             __syncthreads();
-            step(i + 2, integral_constant<int, 2>{});
+            if (i + 3 < iters) step(i + 3, stage, integral_constant<int, 3>{});
+            next_stage();
             __syncthreads();
-            step(i + 3, integral_constant<int, 3>{});
+            if (i + 4 < iters) step(i + 4, stage, integral_constant<int, 0>{});
+            next_stage();
             __syncthreads();
-            if (i + 4 < iters) step(i + 4, integral_constant<int, 0>{});
+            if (i + 5 < iters) step(i + 5, stage, integral_constant<int, 1>{});
+            next_stage();
             __syncthreads();
         }
         return;
@@ -282,26 +259,43 @@ __global__ __launch_bounds__(kGemmAll) void matmul_q4k_bf16_kernel(GemmArgs a)
         for (int i = 0; i < MT; ++i)
 #pragma unroll
             for (int j = 0; j < NT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-        __syncthreads();        // the first raw blocks are staged
-        __syncthreads();        // their scales are staged
-        __syncthreads();        // the tiles of K slice 0 are ready
-        for (int it = 0; it < iters; ++it) {
-            const uint8_t* xb = xs + (it & 1) * 2 * kXTile + wm * RW * kRowBytes + frag;
-            const uint8_t* wb = ws + (it & 1) * 2 * kWTile + ct0 * 16 * kRowBytes + frag;
+        const uint8_t* xrow = xs + wm * RW * kRowBytes + frag;
+        const uint8_t* wcol = ws + ct0 * 16 * kRowBytes + frag;
+        __syncthreads();        // tiles 0 and 1 are ready
+        // Operand fetches run ahead of the matrix instructions that use them: a weight fragment is read one tile ahead
+        // (two registers sets alternate), the x fragments of a half-slice while the previous half is multiplied, and
+        // both continue across the barrier into the next slice, which was completed one iteration earlier.  The
+        // scheduling barriers keep the compiler from sinking the reads back down to their first use.
+        bf16x8 afrag[MT], afrag1[MT], bfrag[2];
 #pragma unroll
-            for (int sub = 0; sub < 2; ++sub) {
-                bf16x8 afrag[MT];
+        for (int i = 0; i < MT; ++i) afrag[i] = *reinterpret_cast<const bf16x8*>(xrow + i * 16 * kRowBytes);
+        bfrag[0] = *reinterpret_cast<const bf16x8*>(wcol);
+        int stage = 0;
+        for (int it = 0; it < iters; ++it) {
+            const uint8_t* xb = xrow + stage * 2 * kXTile;
+            const uint8_t* wb = wcol + stage * 2 * kWTile;
+            const int nstage = stage == kStages - 1 ? 0 : stage + 1;
+            const uint8_t* xn = xrow + nstage * 2 * kXTile;
+            const uint8_t* wn_ = wcol + nstage * 2 * kWTile;
+#pragma unroll
+            for (int i = 0; i < MT; ++i) afrag1[i] = *reinterpret_cast<const bf16x8*>(xb + kXTile + i * 16 * kRowBytes);
+#pragma unroll
+            for (int t = 0; t < 2 * NT; ++t) {
+                // tile t: columns t % NT of half-slice t / NT; fetch tile t + 1 (or the next slice's first) meanwhile
+                const uint8_t* nb = t + 1 < NT ? wb + (t + 1) * 16 * kRowBytes
+                                    : t + 1 < 2 * NT ? wb + kWTile + (t + 1 - NT) * 16 * kRowBytes : wn_;
+                bfrag[(t + 1) & 1] = *reinterpret_cast<const bf16x8*>(nb);
 #pragma unroll
                 for (int i = 0; i < MT; ++i)
-                    afrag[i] = *reinterpret_cast<const bf16x8*>(xb + sub * kXTile + i * 16 * kRowBytes);
+                    acc[i][t % NT] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(t < NT ? afrag[i] : afrag1[i], bfrag[t & 1],
+                                                                             acc[i][t % NT], 0, 0, 0);
+                if (t == NT - 1) {
 #pragma unroll
-                for (int j = 0; j < NT; ++j) {
-                    const bf16x8 bfrag = *reinterpret_cast<const bf16x8*>(wb + sub * kWTile + j * 16 * kRowBytes);
-#pragma unroll
-                    for (int i = 0; i < MT; ++i)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[i], bfrag, acc[i][j], 0, 0, 0);
+                    for (int i = 0; i < MT; ++i) afrag[i] = *reinterpret_cast<const bf16x8*>(xn + i * 16 * kRowBytes);
                 }
+                __builtin_amdgcn_sched_barrier(0);
             }
+            stage = nstage;
             __syncthreads();
         }
         // accumulator element v of a tile: row 4 * (lane / 16) + v, column lane % 16
@@ -331,7 +325,7 @@ template <int RW, int CT, int WN>
 hipError_t launch_gemm(Lane* lane, const GemmArgs& a, dim3 grid)
 {
     constexpr int BM = (8 / WN) * RW, BN = 16 * CT;
-    constexpr size_t lds = 4 * static_cast<size_t>(BM + BN) * kRowBytes + 2 * static_cast<size_t>(BN) * (144 + 64);
+    constexpr size_t lds = static_cast<size_t>(kStages) * 2 * (BM + BN) * kRowBytes;
     static bool configured = false;
     if (lds > 48 * 1024 && !configured) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&matmul_q4k_bf16_kernel<RW, CT, WN>),
