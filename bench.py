@@ -31,7 +31,7 @@ BF16_PEAK_TFLOPS = 2500.0      # MI355X dense bf16 MFMA, published
 # HBM bytes one batched launch of the decode27b set moves, from two rocprofv3 --pmc runs (FETCH_SIZE x 2.000 and
 # WRITE_SIZE x 1.000, the factors a plain copy kernel of known size gives); summary in
 # profiles/matvec_batch_q8_0_decode27b_hbm_traffic.md.  Only valid for --mode batch.
-DECODE27B_BATCH_TRAFFIC_BYTES = 29_106_670_696
+DECODE27B_BATCH_TRAFFIC_BYTES = 29_074_665_059
 
 
 def log(*a):
