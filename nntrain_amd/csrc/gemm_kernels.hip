@@ -13,20 +13,21 @@
 // bytes, placed so that the 16 rows x 4 k-groups an MFMA operand needs are one conflict-free read), in three stages:
 // the slice being multiplied, the finished next one, and the one being made.
 //
-// The 13 waves of a workgroup are specialised:
+// The 16 waves of a workgroup are specialised, each role with a code path (and so a register allocation) of its own:
 //   - 8 consumer waves (8 x 1, or 4 x 2 with 64-row, 5- or 4-tile wave tiles) only read operands from LDS and issue
-//     MFMAs.  Operand reads run ahead of their use, also across the barrier into the finished next slice, so the
-//     matrix pipe restarts right after a barrier;
-//   - 5 producer waves fill LDS.  Four of them move the x tile (requested two iterations ahead into registers, then
-//     written to the sub-tiles).  Two threads per column decode: each keeps the 16 nibble bytes of its next two slices
-//     and the (d * scale, dmin * min) pairs of the current 256-block in registers (the header of the next block is
-//     requested a block ahead), and turns a slice into 16 low-nibble and 16 high-nibble bf16 weights.  Nothing a
-//     producer needs after a barrier has to be waited for.
-// One barrier per iteration joins the two groups: while the consumers multiply slice i, the producers build slice
-// i + 2.  Measured with either group switched off (M = 512, 80 iterations): consumers alone 0.85 us per iteration
-// (72 MFMAs per SIMD; 0.62 us at the back-to-back MFMA rate), producers alone 1.04 us, together 1.43 us.  LDS is about
-// as busy as the matrix pipe: 144 KB of operand reads (4 cycles per 1 KB wave read) and 50 KB of tile writes (13
-// cycles per 1 KB wave write) per iteration.
+//     MFMAs.  Operand reads run one tile ahead of their use, also across the barrier into the finished next slice, so
+//     the matrix pipe restarts right after a barrier;
+//   - 5 decoder waves, two threads per strip column: each keeps the 16 nibble bytes of its next two slices and the
+//     (d * scale, dmin * min) pairs of the current 256-block in registers (the header of the next block is requested a
+//     block ahead), and turns a slice into 16 low-nibble and 16 high-nibble bf16 weights;
+//   - 3 waves move the x tile: requested two iterations ahead into registers, then written to the sub-tiles.
+//     Nothing a producer needs after a barrier has to be waited for.
+// One barrier per iteration joins the groups: while the consumers multiply slice i, the producers build slice i + 2.
+// Measured with groups switched off (M = 512, 80 iterations): consumers alone 0.83 us per iteration (72 MFMAs per SIMD;
+// 0.62 us at the back-to-back MFMA rate; 0.76 us without the weight-operand reads), decoders alone 0.72 us, x movers
+// alone 0.64 us, all producers 0.88 us, everything together 1.33 us.  LDS is about as busy as the matrix pipe: 144 KB
+// of operand reads (4 cycles per 1 KB wave read) and 50 KB of tile writes (13 cycles per 1 KB wave write, 8 cycles per
+// 512-byte write: 64-bit writes gain nothing) per iteration.
 #include <type_traits>
 
 #include "nnhip_internal.h"
@@ -91,8 +92,9 @@ __device__ __forceinline__ u32x4 q4k_decode8(uint32_t q_lo, uint32_t q_hi, float
 __device__ __forceinline__ int lds_slot(int row, int group) { return group ^ ((row >> 1) & 3); }
 
 constexpr int kConsumers = 512;         // 8 MFMA waves
-constexpr int kProducers = 320;         // 5 waves that fetch, decode and fill LDS
-constexpr int kXThreads = 256;          // the producer threads that also move the x tile
+constexpr int kProducers = 512;         // 8 waves that fill LDS: waves 8-12 decode weights, waves 13-15 move the x tile
+constexpr int kDecoders = 320;          // producer threads reserved for decoding (two per strip column are used)
+constexpr int kXThreads = kProducers - kDecoders;
 constexpr int kGemmAll = kConsumers + kProducers;
 constexpr int kStages = 3;              // LDS tile stages: multiplied, ready (being pre-read), being made
 
@@ -120,41 +122,84 @@ __global__ __launch_bounds__(kGemmAll) void matmul_q4k_bf16_kernel(GemmArgs a)
 
     if (wave >= kConsumers / 64) {
         // ------------------------------------------------------------------------------------------ producers
-        constexpr int kXLoads = 2 * kXTile / 16 / kXThreads;                   // 16-byte pieces of x per thread
-        static_assert(kXLoads >= 1, "tile too small for the producer count");
-        static_assert(2 * BN <= kProducers, "two decoding threads per column");
+        // Both producer roles make slices 0 and 1 before the first barrier and then, between two barriers, slice
+        // i + 2 while slice i is multiplied.  Everything a role consumes was requested two slices earlier.  The
+        // roles are separate code paths so that each is allocated only its own registers.
         const int p = tid - kConsumers;
-        const int row_bytes = (a.K >> 8) * 144;
-        // x piece q of this thread: row q / 8 of the tile, 16-byte group q % 8 of the 64-value K slice
-        const bool x_role = p < kXThreads;
-        const uint8_t* xbase = reinterpret_cast<const uint8_t*>(a.x + static_cast<size_t>(m0) * a.K);   // wave-uniform
-        uint32_t xsrc[kXLoads];     // byte offsets from xbase (a tile spans at most 256 rows)
-        int xdst[kXLoads];
+        // K is a whole number of 256-blocks, so iters is a multiple of 4; `make(t, stage)` is given t % 4 statically
+        auto run = [&](auto&& make) {
+            using std::integral_constant;
+            make(0, 0, integral_constant<int, 0>{});
+            make(1, 1, integral_constant<int, 1>{});
+            __syncthreads();
+            int stage = 2;
+            auto next_stage = [&]() { stage = stage == kStages - 1 ? 0 : stage + 1; };
+            for (int i = 0; i < iters; i += 4) {
+                if (i + 2 < iters) make(i + 2, stage, integral_constant<int, 2>{});
+                next_stage();
+                __syncthreads();
+                if (i + 3 < iters) make(i + 3, stage, integral_constant<int, 3>{});
+                next_stage();
+                __syncthreads();
+                if (i + 4 < iters) make(i + 4, stage, integral_constant<int, 0>{});
+                next_stage();
+                __syncthreads();
+                if (i + 5 < iters) make(i + 5, stage, integral_constant<int, 1>{});
+                next_stage();
+                __syncthreads();
+            }
+        };
+
+        if (p >= kDecoders) {
+            // ---- x movers (waves 13-15): piece q of a slice = row q / 8 of the tile, 16-byte group q % 8 of its 64
+            // values; a thread moves pieces xp, xp + 192, ...
+            constexpr int kXPieces = 2 * kXTile / 16;
+            constexpr int kXLoads = (kXPieces + kXThreads - 1) / kXThreads;
+            const int xp = p - kDecoders;
+            const uint8_t* xbase = reinterpret_cast<const uint8_t*>(a.x + static_cast<size_t>(m0) * a.K);   // wave-uniform
+            uint32_t xsrc[kXLoads];     // byte offsets from xbase (a tile spans at most 256 rows)
+            int xdst[kXLoads];
 #pragma unroll
-        for (int i = 0; i < kXLoads; ++i) {
-            const int q = (x_role ? p : 0) + i * kXThreads;
-            const int r = q >> 3, grp = q & 7;
-            xsrc[i] = static_cast<uint32_t>((min(r, a.M - 1 - m0) * a.K + grp * 8) * 2);
-            xdst[i] = (grp >> 2) * kXTile + r * kRowBytes + lds_slot(r, grp & 3) * 16;
+            for (int i = 0; i < kXLoads; ++i) {
+                const int q = min(xp + i * kXThreads, kXPieces - 1);       // the last round is partly idle (not stored)
+                const int r = q >> 3, grp = q & 7;
+                xsrc[i] = static_cast<uint32_t>((min(r, a.M - 1 - m0) * a.K + grp * 8) * 2);
+                xdst[i] = (grp >> 2) * kXTile + r * kRowBytes + lds_slot(r, grp & 3) * 16;
+            }
+            u32x4 xset[2][kXLoads];     // x pieces of K slices t and t + 1
+            auto load_x = [&](u32x4* set, int t) {
+                uint32_t koff = static_cast<uint32_t>(min(t, iters - 1)) << 7;     // past the end: a harmless repeat
+                asm volatile("" : "+s"(koff));      // keeps the address as scalar base + 32-bit lane offset
+                const uint8_t* src = xbase + koff;
+#pragma unroll
+                for (int i = 0; i < kXLoads; ++i) set[i] = *reinterpret_cast<const u32x4*>(src + opaque(xsrc[i]));
+            };
+            load_x(xset[0], 0);
+            load_x(xset[1], 1);
+            run([&](int t, int stage, auto jt) {
+                constexpr int J = decltype(jt)::value;
+                u32x4* set = xset[J & 1];
+                uint8_t* xb = xs + stage * 2 * kXTile;
+#pragma unroll
+                for (int i = 0; i < kXLoads; ++i)
+                    if (xp + i * kXThreads < kXPieces) *reinterpret_cast<u32x4*>(xb + xdst[i]) = set[i];
+                load_x(set, t + 2);
+            });
+            return;
         }
-        // decoding: thread (column dc, half dh) owns bytes [16 dh, 16 dh + 16) of the 32 nibble bytes of a K slice:
-        // 16 low-nibble weights of sub-block 2J and 16 high-nibble weights of sub-block 2J + 1
+
+        // ---- decoders (waves 8-12): thread (column dc, half dh) owns bytes [16 dh, 16 dh + 16) of the 32 nibble bytes
+        // of a K slice: 16 low-nibble weights of sub-block 2J and 16 high-nibble weights of sub-block 2J + 1
+        static_assert(2 * BN <= kDecoders, "two decoding threads per column");
+        const int row_bytes = (a.K >> 8) * 144;
         const bool d_role = p < 2 * BN;
         const int dc = d_role ? p >> 1 : 0, dh = p & 1;
         const uint8_t* wbase = a.w + static_cast<size_t>(n0) * row_bytes;                               // wave-uniform
         const uint32_t wrow = static_cast<uint32_t>(min(dc, a.N - 1 - n0) * row_bytes);                 // byte offset
         const int nblocks = a.K >> 8;
-        u32x4 xset[2][kXLoads];     // x pieces of K slices t and t + 1
         u32x4 nq[2];                // nibble bytes of K slices t and t + 1
         u32x4 hdr;                  // header (d, dmin, packed scales) of the next 256-block
         float sm[16];               // (d * scale, dmin * min) of the eight sub-blocks of the current block
-        auto load_x = [&](u32x4* set, int t) {
-            uint32_t koff = static_cast<uint32_t>(min(t, iters - 1)) << 7;     // past the end: a harmless repeat of the last slice
-            asm volatile("" : "+s"(koff));      // keeps the address as scalar base + 32-bit lane offset
-            const uint8_t* src = xbase + koff;
-#pragma unroll
-            for (int i = 0; i < kXLoads; ++i) set[i] = *reinterpret_cast<const u32x4*>(src + opaque(xsrc[i]));
-        };
         auto load_q = [&](int t) {
             const int tt = min(t, iters - 1);
             uint32_t off = static_cast<uint32_t>(tt >> 2) * 144u + 16u + static_cast<uint32_t>(tt & 3) * 32u;
@@ -180,65 +225,28 @@ __global__ __launch_bounds__(kGemmAll) void matmul_q4k_bf16_kernel(GemmArgs a)
                 sm[8 + 2 * j + 1] = dmin * static_cast<float>((b2 >> 4) | ((b1 >> 6) << 4));
             }
         };
-        // One production step makes the LDS tiles of K slice t in stage `stage`; J = t % 4 is the 64-wide slice inside
-        // the Q4_K block.  Everything it consumes was requested two steps earlier.
-        auto step = [&](int t, int stage, auto jt) {
-            constexpr int J = decltype(jt)::value;
-            if (d_role) {
-                const u32x4 q = nq[J & 1];
-                uint8_t* wb = ws + stage * 2 * kWTile + dc * kRowBytes;
-#pragma unroll
-                for (int g = 0; g < 2; ++g) {
-                    const uint32_t a0 = q[2 * g], a1 = q[2 * g + 1];
-                    const int slot = lds_slot(dc, 2 * dh + g) * 16;
-                    *reinterpret_cast<u32x4*>(wb + slot) =
-                        q4k_decode8(a0 & 0x0f0f0f0fu, a1 & 0x0f0f0f0fu, sm[4 * J], sm[4 * J + 1]);
-                    *reinterpret_cast<u32x4*>(wb + kWTile + slot) =
-                        q4k_decode8((a0 >> 4) & 0x0f0f0f0fu, (a1 >> 4) & 0x0f0f0f0fu, sm[4 * J + 2], sm[4 * J + 3]);
-                }
-                nq[J & 1] = load_q(t + 2);
-                if (J == 0) load_hdr((t >> 2) + 1);
-                if (J == 3) make_scales();
-            }
-            // (writing the x tile before the decode was measured slower: 137 against 114 us at M = 512)
-            if (x_role) {
-                u32x4* set = xset[J & 1];
-                uint8_t* xb = xs + stage * 2 * kXTile;
-#pragma unroll
-                for (int i = 0; i < kXLoads; ++i) *reinterpret_cast<u32x4*>(xb + xdst[i]) = set[i];
-                load_x(set, t + 2);
-            }
-        };
-        using std::integral_constant;
         load_hdr(0);
         nq[0] = load_q(0);
         nq[1] = load_q(1);
-        if (x_role) {
-            load_x(xset[0], 0);
-            load_x(xset[1], 1);
-        }
         make_scales();
-        // tiles 0 and 1 before the consumers start; from then on tile i + 2 is made while tile i is multiplied
-        step(0, 0, integral_constant<int, 0>{});
-        step(1, 1, integral_constant<int, 1>{});
-        __syncthreads();
-        // K is a whole number of 256-blocks, so iters is a multiple of 4
-        int stage = 2;
-        auto next_stage = [&]() { stage = stage == kStages - 1 ? 0 : stage + 1; };
-        for (int i = 0; i < iters; i += 4) {
-            if (i + 2 < iters) step(i + 2, stage, integral_constant<int, 2>{});
-            next_stage();
-            __syncthreads();
-            if (i + 3 < iters) step(i + 3, stage, integral_constant<int, 3>{});
-            next_stage();
-            __syncthreads();
-            if (i + 4 < iters) step(i + 4, stage, integral_constant<int, 0>{});
-            next_stage();
-            __syncthreads();
-            if (i + 5 < iters) step(i + 5, stage, integral_constant<int, 1>{});
-            next_stage();
-            __syncthreads();
-        }
+        run([&](int t, int stage, auto jt) {
+            constexpr int J = decltype(jt)::value;
+            if (!d_role) return;
+            const u32x4 q = nq[J & 1];
+            uint8_t* wb = ws + stage * 2 * kWTile + dc * kRowBytes;
+#pragma unroll
+            for (int g = 0; g < 2; ++g) {
+                const uint32_t a0 = q[2 * g], a1 = q[2 * g + 1];
+                const int slot = lds_slot(dc, 2 * dh + g) * 16;
+                *reinterpret_cast<u32x4*>(wb + slot) =
+                    q4k_decode8(a0 & 0x0f0f0f0fu, a1 & 0x0f0f0f0fu, sm[4 * J], sm[4 * J + 1]);
+                *reinterpret_cast<u32x4*>(wb + kWTile + slot) =
+                    q4k_decode8((a0 >> 4) & 0x0f0f0f0fu, (a1 >> 4) & 0x0f0f0f0fu, sm[4 * J + 2], sm[4 * J + 3]);
+            }
+            nq[J & 1] = load_q(t + 2);
+            if (J == 0) load_hdr((t >> 2) + 1);
+            if (J == 3) make_scales();
+        });
         return;
     }
 
