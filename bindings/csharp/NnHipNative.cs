@@ -57,6 +57,10 @@ internal static unsafe partial class NnHipNative
     [LibraryImport(Library)] internal static partial int nnhip_quant_matvec(nint lane, uint ggmlType, nint x, nint w, nint bias, nint y, int rows, int inW, int outW);
     [LibraryImport(Library)] internal static partial int nnhip_quant_matvec_batch(nint lane, MatvecDesc* descs, int count);
     [LibraryImport(Library)] internal static partial int nnhip_quant_matmul_bf16(nint lane, uint ggmlType, nint xBf16, nint w, nint bias, nint y, int rows, int inW, int outW);
+    [LibraryImport(Library)] internal static partial int nnhip_rms_norm(nint lane, nint input, nint weight, nint output, int rows, int width, int inputStride, float epsilon);
+    [LibraryImport(Library)] internal static partial int nnhip_add_rms_norm(nint lane, nint destination, nint residual, nint weight, nint output, int rows, int width, int inputStride, float epsilon);
+    [LibraryImport(Library)] internal static partial int nnhip_silu_multiply(nint lane, nint gate, nint up, nint output, int length);
+    [LibraryImport(Library)] internal static partial int nnhip_add_in_place(nint lane, nint destination, nint source, int length);
     [LibraryImport(Library)] internal static partial int nnhip_event_create(nint lane, out nint evt);
     [LibraryImport(Library)] internal static partial int nnhip_event_destroy(nint lane, nint evt);
     [LibraryImport(Library)] internal static partial int nnhip_event_record(nint lane, nint evt);

@@ -67,7 +67,8 @@ enum {
     NNHIP_OP_NONE = 0, NNHIP_OP_LANE_CREATE, NNHIP_OP_LANE_DESTROY, NNHIP_OP_ALLOC, NNHIP_OP_FREE,
     NNHIP_OP_UPLOAD, NNHIP_OP_DOWNLOAD, NNHIP_OP_COPY, NNHIP_OP_SYNCHRONIZE, NNHIP_OP_DEQUANTIZE,
     NNHIP_OP_MATVEC, NNHIP_OP_MATVEC_BATCH, NNHIP_OP_MATMUL_BF16, NNHIP_OP_EVENT, NNHIP_OP_GRAPH,
-    NNHIP_OP_DEVICE_QUERY, NNHIP_OP_FILL
+    NNHIP_OP_DEVICE_QUERY, NNHIP_OP_FILL, NNHIP_OP_RMS_NORM, NNHIP_OP_SILU_MULTIPLY, NNHIP_OP_ADD_IN_PLACE,
+    NNHIP_OP_MATVEC_FUSED
 };
 
 /* Same field order as the reference's NativeErrorInfo (CudaNativeGateway.cs:1360-1371). */
@@ -192,6 +193,32 @@ NNHIP_API int nnhip_quant_matvec_batch(void* lane, const nnhip_matvec_desc* desc
  * NNtrain.Arc/Kernels/qwen35_prefill_xmx.cl:112-184).  Asynchronous. */
 NNHIP_API int nnhip_quant_matmul_bf16(void* lane, uint32_t ggml_type, const uint16_t* x_bf16, const void* w,
                                       const float* bias, float* y, int rows, int in_w, int out_w);
+
+/* --- FP32 row operations around the mat-vec ------------------------------------------------------------------ */
+
+/* output[r, j] = input[r * input_stride + j] * inverse_r * weight[j], inverse_r = 1 / sqrt(sum_j x^2 / width + epsilon),
+ * for `rows` rows.  Replaces q35a_rms_norm (NNtrain.Arc/Kernels/qwen35_attention.cl:16-36; host wrapper
+ * Qwen35Gpu.RmsNorm, NNtrain.Core/Modules/Qwen35Gpu.Attention.cs:11-36) with the same summation order (128
+ * lane-strided partial sums, halving tree), so results have the bits of that kernel evaluated with IEEE arithmetic.
+ * epsilon must be finite and >= 0 (ValidateAttentionEpsilon, Qwen35Gpu.Attention.cs:181-184).  Asynchronous. */
+NNHIP_API int nnhip_rms_norm(void* lane, const float* input, const float* weight, float* output, int rows, int width,
+                             int input_stride, float epsilon);
+
+/* destination[r, j] += residual[r, j] (stored), then output = RMSNorm(destination) * weight as above.  Replaces
+ * q35a_add_rms_norm (qwen35_attention.cl:55-78; call site AddResidualAndRmsNorm,
+ * NNtrain.Core/Modules/Qwen35QuantizedModel.cs:527-546).  destination and residual rows are input_stride apart.
+ * Asynchronous. */
+NNHIP_API int nnhip_add_rms_norm(void* lane, float* destination, const float* residual, const float* weight,
+                                 float* output, int rows, int width, int input_stride, float epsilon);
+
+/* output[i] = gate[i] * sigmoid(gate[i]) * up[i] with the overflow-free two-sided sigmoid.  Replaces
+ * q35a_silu_multiply (qwen35_attention.cl:9-14,38-43; Qwen35Gpu.SiluMultiply, Qwen35Gpu.Attention.cs:38-50).
+ * Asynchronous. */
+NNHIP_API int nnhip_silu_multiply(void* lane, const float* gate, const float* up, float* output, int length);
+
+/* destination[i] += source[i].  Replaces q35a_add_in_place (qwen35_attention.cl:45-49; Qwen35Gpu.AddInPlace,
+ * Qwen35Gpu.Attention.cs:52-58).  Asynchronous. */
+NNHIP_API int nnhip_add_in_place(void* lane, float* destination, const float* source, int length);
 
 /* --- timing and replay --------------------------------------------------------------------------------------- */
 

@@ -1,4 +1,5 @@
 // C ABI of libnnhip.so: lanes, device memory, transfers, error record, and validated dispatch to the kernels.
+#include <cmath>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -370,6 +371,67 @@ int nnhip_quant_matvec(void* handle, uint32_t ggml_type, const float* x, const v
     if (rows > 65535) return fail(NNHIP_ERR_TOO_LARGE, NNHIP_OP_MATVEC, lane->device, 0, "rows %d exceeds 65535", rows);
     hipError_t e = launch_matvec(lane, ggml_type, x, w, bias, y, rows, in_w, out_w);
     if (e != hipSuccess) return hip_fail(e, NNHIP_OP_MATVEC, lane->device, "mat-vec launch");
+    lane->counters.kernel_launches += 1;
+    return NNHIP_OK;
+}
+
+static int check_norm(uint32_t op, nnhip::Lane* lane, const void* input, const void* weight, const void* output, int rows,
+                      int width, int input_stride, float epsilon)
+{
+    using namespace nnhip;
+    if (!input || !weight || !output)
+        return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0, "input, weight and output must be non-null");
+    if (rows < 1 || width < 1 || input_stride < width)
+        return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0, "rows and width must be positive and input_stride >= width");
+    if (!(epsilon >= 0.0f) || !std::isfinite(epsilon))
+        return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0, "epsilon must be finite and not negative");
+    if (rows > 65535) return fail(NNHIP_ERR_TOO_LARGE, op, lane->device, 0, "rows %d exceeds 65535", rows);
+    return NNHIP_OK;
+}
+
+int nnhip_rms_norm(void* handle, const float* input, const float* weight, float* output, int rows, int width,
+                   int input_stride, float epsilon)
+{
+    NNHIP_LANE(handle, NNHIP_OP_RMS_NORM)
+    int rc = check_norm(NNHIP_OP_RMS_NORM, lane, input, weight, output, rows, width, input_stride, epsilon);
+    if (rc != NNHIP_OK) return rc;
+    hipError_t e = launch_rms_norm(lane, const_cast<float*>(input), nullptr, weight, output, rows, width, input_stride, epsilon);
+    if (e != hipSuccess) return hip_fail(e, NNHIP_OP_RMS_NORM, lane->device, "RMSNorm launch");
+    lane->counters.kernel_launches += 1;
+    return NNHIP_OK;
+}
+
+int nnhip_add_rms_norm(void* handle, float* destination, const float* residual, const float* weight, float* output,
+                       int rows, int width, int input_stride, float epsilon)
+{
+    NNHIP_LANE(handle, NNHIP_OP_RMS_NORM)
+    int rc = check_norm(NNHIP_OP_RMS_NORM, lane, destination, weight, output, rows, width, input_stride, epsilon);
+    if (rc != NNHIP_OK) return rc;
+    if (!residual) return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_RMS_NORM, lane->device, 0, "residual must be non-null");
+    hipError_t e = launch_rms_norm(lane, destination, residual, weight, output, rows, width, input_stride, epsilon);
+    if (e != hipSuccess) return hip_fail(e, NNHIP_OP_RMS_NORM, lane->device, "add + RMSNorm launch");
+    lane->counters.kernel_launches += 1;
+    return NNHIP_OK;
+}
+
+int nnhip_silu_multiply(void* handle, const float* gate, const float* up, float* output, int length)
+{
+    NNHIP_LANE(handle, NNHIP_OP_SILU_MULTIPLY)
+    if (!gate || !up || !output || length < 1)
+        return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_SILU_MULTIPLY, lane->device, 0, "pointers must be non-null and length positive");
+    hipError_t e = launch_silu_multiply(lane, gate, up, output, length);
+    if (e != hipSuccess) return hip_fail(e, NNHIP_OP_SILU_MULTIPLY, lane->device, "SiLU multiply launch");
+    lane->counters.kernel_launches += 1;
+    return NNHIP_OK;
+}
+
+int nnhip_add_in_place(void* handle, float* destination, const float* source, int length)
+{
+    NNHIP_LANE(handle, NNHIP_OP_ADD_IN_PLACE)
+    if (!destination || !source || length < 1)
+        return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_ADD_IN_PLACE, lane->device, 0, "pointers must be non-null and length positive");
+    hipError_t e = launch_add_in_place(lane, destination, source, length);
+    if (e != hipSuccess) return hip_fail(e, NNHIP_OP_ADD_IN_PLACE, lane->device, "add launch");
     lane->counters.kernel_launches += 1;
     return NNHIP_OK;
 }

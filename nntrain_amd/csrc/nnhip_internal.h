@@ -54,6 +54,11 @@ hipError_t launch_matvec(Lane* lane, uint32_t type, const float* x, const void* 
 hipError_t launch_matvec_batch(Lane* lane, const nnhip_matvec_desc* descs, int count);
 hipError_t launch_matmul_bf16(Lane* lane, uint32_t type, const uint16_t* x, const void* w, const float* bias,
                               float* y, int rows, int in_w, int out_w);
+// FP32 row operations (rowop_kernels.hip).  residual == nullptr: plain RMSNorm of io (not modified).
+hipError_t launch_rms_norm(Lane* lane, float* io, const float* residual, const float* weight, float* output, int rows,
+                           int width, int input_stride, float epsilon);
+hipError_t launch_silu_multiply(Lane* lane, const float* gate, const float* up, float* output, int length);
+hipError_t launch_add_in_place(Lane* lane, float* destination, const float* source, int length);
 hipError_t launch_fill_u32(Lane* lane, uint32_t* p, uint32_t value, size_t count);
 
 // Largest in_w the mat-vec kernels can stage in LDS.

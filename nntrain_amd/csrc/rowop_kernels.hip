@@ -1,0 +1,96 @@
+// FP32 row operations that sit on either side of the quantized mat-vec in the decode path: RMSNorm, residual add +
+// RMSNorm, SiLU(gate) * up, in-place add (NNtrain.Arc/Kernels/qwen35_attention.cl:9-78).
+//
+// The reductions follow the reference's order, so a result has the bits of a plain CPU restatement: lane t of 128 adds
+// x[t]^2, x[t+128]^2, ... in that order, the 128 partial sums meet in a halving tree (64, 32, .. 1), and
+// inverse = 1 / sqrt(sum / width + eps) uses IEEE division and square root.  The build keeps multiply and add
+// separate (-ffp-contract=off).
+#include "nnhip_internal.h"
+#include "quant_device.h"
+
+namespace nnhip {
+
+namespace {
+
+constexpr int kNormLanes = 128;
+
+// ADD: destination[row] += residual[row] first (and is stored), as q35a_add_rms_norm does.
+template <bool ADD>
+__global__ __launch_bounds__(kNormLanes) void rms_norm_kernel(float* io, const float* residual, const float* weight,
+                                                              float* output, int width, int input_stride, float epsilon)
+{
+    __shared__ float sums[kNormLanes];
+    const int tid = threadIdx.x;
+    float* x = io + static_cast<size_t>(blockIdx.x) * input_stride;
+    const float* res = ADD ? residual + static_cast<size_t>(blockIdx.x) * input_stride : nullptr;
+    float* out = output + static_cast<size_t>(blockIdx.x) * width;
+    float sum = 0.0f;
+    for (int j = tid; j < width; j += kNormLanes) {
+        float v = x[j];
+        if (ADD) {
+            v = v + res[j];
+            x[j] = v;
+        }
+        sum += v * v;
+    }
+    sums[tid] = sum;
+    __syncthreads();
+    for (int stride = kNormLanes / 2; stride > 0; stride >>= 1) {
+        if (tid < stride) sums[tid] += sums[tid + stride];
+        __syncthreads();
+    }
+    const float inverse = 1.0f / sqrtf(sums[0] / static_cast<float>(width) + epsilon);
+    // every lane re-reads the components it wrote itself
+    for (int j = tid; j < width; j += kNormLanes) out[j] = x[j] * inverse * weight[j];
+}
+
+// Two-sided form: exp never sees a positive argument, so neither side overflows (qwen35_attention.cl:9-14).
+__device__ __forceinline__ float stable_sigmoid(float x)
+{
+    if (x >= 0.0f) return 1.0f / (1.0f + expf(-x));
+    const float e = expf(x);
+    return e / (1.0f + e);
+}
+
+__global__ __launch_bounds__(256) void silu_multiply_kernel(const float* gate, const float* up, float* output, int length)
+{
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < length) {
+        const float g = gate[i];
+        output[i] = g * stable_sigmoid(g) * up[i];
+    }
+}
+
+__global__ __launch_bounds__(256) void add_in_place_kernel(float* destination, const float* source, int length)
+{
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < length) destination[i] += source[i];
+}
+
+}  // namespace
+
+hipError_t launch_rms_norm(Lane* lane, float* io, const float* residual, const float* weight, float* output, int rows,
+                           int width, int input_stride, float epsilon)
+{
+    if (residual)
+        hipLaunchKernelGGL(rms_norm_kernel<true>, dim3(rows), dim3(kNormLanes), 0, lane->stream, io, residual, weight, output,
+                           width, input_stride, epsilon);
+    else
+        hipLaunchKernelGGL(rms_norm_kernel<false>, dim3(rows), dim3(kNormLanes), 0, lane->stream, io, residual, weight, output,
+                           width, input_stride, epsilon);
+    return hipGetLastError();
+}
+
+hipError_t launch_silu_multiply(Lane* lane, const float* gate, const float* up, float* output, int length)
+{
+    hipLaunchKernelGGL(silu_multiply_kernel, dim3((length + 255) / 256), dim3(256), 0, lane->stream, gate, up, output, length);
+    return hipGetLastError();
+}
+
+hipError_t launch_add_in_place(Lane* lane, float* destination, const float* source, int length)
+{
+    hipLaunchKernelGGL(add_in_place_kernel, dim3((length + 255) / 256), dim3(256), 0, lane->stream, destination, source, length);
+    return hipGetLastError();
+}
+
+}  // namespace nnhip

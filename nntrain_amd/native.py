@@ -68,6 +68,10 @@ PROTOTYPES = {
     "nnhip_quant_matvec": (c_int, [c_void_p, c_uint32, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int]),
     "nnhip_quant_matvec_batch": (c_int, [c_void_p, POINTER(MatvecDesc), c_int]),
     "nnhip_quant_matmul_bf16": (c_int, [c_void_p, c_uint32, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int]),
+    "nnhip_rms_norm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float]),
+    "nnhip_add_rms_norm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float]),
+    "nnhip_silu_multiply": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int]),
+    "nnhip_add_in_place": (c_int, [c_void_p, c_void_p, c_void_p, c_int]),
     "nnhip_event_create": (c_int, [c_void_p, POINTER(c_void_p)]),
     "nnhip_event_destroy": (c_int, [c_void_p, c_void_p]),
     "nnhip_event_record": (c_int, [c_void_p, c_void_p]),

@@ -1,0 +1,92 @@
+"""Resident FP32 row operations of the decode path, shaped like the reference's Qwen35Gpu helpers
+(NNtrain.Core/Modules/Qwen35Gpu.Attention.cs:11-58) and AddResidualAndRmsNorm
+(NNtrain.Core/Modules/Qwen35QuantizedModel.cs:527-546).  Callers own returned buffers; nothing crosses to the host.
+"""
+from __future__ import annotations
+
+import math
+from ctypes import c_void_p
+
+from .lane import HipBuffer, HipExecutionLane
+from .native import check
+
+
+def _positive(value: int, name: str) -> None:
+    if value <= 0:
+        raise ValueError(f"{name} must be positive (ArgumentOutOfRangeException in the reference).")
+
+
+def _validate_epsilon(eps: float) -> None:
+    if not math.isfinite(eps) or eps < 0.0:
+        raise ValueError("eps must be finite and not negative.")
+
+
+def _validate_buffer(buffer: HipBuffer, elements: int, name: str) -> None:
+    if buffer is None:
+        raise TypeError(f"{name} is null.")
+    if buffer.disposed or buffer.nbytes < elements * 4:
+        raise ValueError(f"The buffer '{name}' is disposed or too small for its declared dimensions.")
+
+
+def rms_norm(lane: HipExecutionLane, input: HipBuffer, weight: HipBuffer, rows: int, width: int, eps: float,
+             input_stride: int | None = None) -> HipBuffer:
+    """Qwen35Gpu.RmsNorm: output[r] = input[r] * inverse_rms(input[r]) * weight."""
+    _positive(rows, "rows")
+    _positive(width, "width")
+    _validate_epsilon(eps)
+    stride = width if input_stride is None else input_stride
+    if stride < width:
+        raise ValueError("input_stride must be at least width.")
+    _validate_buffer(input, (rows - 1) * stride + width, "input")
+    _validate_buffer(weight, width, "weight")
+    output = lane.allocate(rows * width)
+    try:
+        check(lane._lib.nnhip_rms_norm(lane._handle, c_void_p(input._require()), c_void_p(weight._require()),
+                                       c_void_p(output._require()), rows, width, stride, eps), "rms_norm")
+        return output
+    except BaseException:
+        output.dispose()
+        raise
+
+
+def add_residual_and_rms_norm(lane: HipExecutionLane, hidden: HipBuffer, residual: HipBuffer, weight: HipBuffer,
+                              width: int, eps: float) -> HipBuffer:
+    """AddResidualAndRmsNorm (fused form): hidden += residual in place, returns RMSNorm(hidden) * weight."""
+    _positive(width, "width")
+    _validate_epsilon(eps)
+    _validate_buffer(hidden, width, "hidden")
+    _validate_buffer(residual, width, "residual")
+    _validate_buffer(weight, width, "weight")
+    output = lane.allocate(width)
+    try:
+        check(lane._lib.nnhip_add_rms_norm(lane._handle, c_void_p(hidden._require()), c_void_p(residual._require()),
+                                           c_void_p(weight._require()), c_void_p(output._require()), 1, width, width,
+                                           eps), "add_rms_norm")
+        return output
+    except BaseException:
+        output.dispose()
+        raise
+
+
+def silu_multiply(lane: HipExecutionLane, gate: HipBuffer, up: HipBuffer, length: int) -> HipBuffer:
+    """Qwen35Gpu.SiluMultiply: gate * sigmoid(gate) * up."""
+    _positive(length, "length")
+    _validate_buffer(gate, length, "gate")
+    _validate_buffer(up, length, "up")
+    output = lane.allocate(length)
+    try:
+        check(lane._lib.nnhip_silu_multiply(lane._handle, c_void_p(gate._require()), c_void_p(up._require()),
+                                            c_void_p(output._require()), length), "silu_multiply")
+        return output
+    except BaseException:
+        output.dispose()
+        raise
+
+
+def add_in_place(lane: HipExecutionLane, destination: HipBuffer, source: HipBuffer, length: int) -> None:
+    """Qwen35Gpu.AddInPlace: destination += source."""
+    _positive(length, "length")
+    _validate_buffer(destination, length, "destination")
+    _validate_buffer(source, length, "source")
+    check(lane._lib.nnhip_add_in_place(lane._handle, c_void_p(destination._require()), c_void_p(source._require()),
+                                       length), "add_in_place")

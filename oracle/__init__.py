@@ -54,6 +54,12 @@ def lib() -> ctypes.CDLL:
                                         ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                         ctypes.c_int]
         L.oracle_max_threads.restype = ctypes.c_int
+        vp, ci, cf = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
+        L.oracle_rms_norm.argtypes = [vp, vp, vp, ci, ci, ci, cf]
+        L.oracle_add_rms_norm.argtypes = [vp, vp, vp, vp, ci, ci, ci, cf]
+        L.oracle_rms_norm_serial.argtypes = [vp, vp, vp, ci, ci, cf]
+        L.oracle_silu_multiply.argtypes = [vp, vp, vp, ci]
+        L.oracle_add_in_place.argtypes = [vp, vp, ci]
         _lib = L
     return _lib
 
@@ -266,3 +272,77 @@ def bf16_round(x: np.ndarray) -> np.ndarray:
 
 def bf16_widen(b: np.ndarray) -> np.ndarray:
     return (np.ascontiguousarray(b, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+# ------------------------------------------------------------------ FP32 row operations around the mat-vec
+# C statements in norm_oracle.c (which cites the reference kernels); the np_* functions are written separately.
+
+def _f32(a) -> np.ndarray:
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def rms_norm(x, weight, rows: int, width: int, eps: float, input_stride: int | None = None) -> np.ndarray:
+    """q35a_rms_norm: x holds `rows` rows `input_stride` apart; returns [rows, width]."""
+    stride = width if input_stride is None else input_stride
+    x, weight = _f32(x), _f32(weight)
+    assert x.size >= (rows - 1) * stride + width and weight.size == width
+    out = np.empty(rows * width, dtype=np.float32)
+    lib().oracle_rms_norm(_ptr(x), _ptr(weight), _ptr(out), rows, width, stride, eps)
+    return out.reshape(rows, width)
+
+
+def add_rms_norm(destination, residual, weight, rows: int, width: int, eps: float,
+                 input_stride: int | None = None):
+    """q35a_add_rms_norm: returns (destination + residual, normalized [rows, width])."""
+    stride = width if input_stride is None else input_stride
+    dest = _f32(destination).copy()
+    residual, weight = _f32(residual), _f32(weight)
+    out = np.empty(rows * width, dtype=np.float32)
+    lib().oracle_add_rms_norm(_ptr(dest), _ptr(residual), _ptr(weight), _ptr(out), rows, width, stride, eps)
+    return dest, out.reshape(rows, width)
+
+
+def rms_norm_serial(x, weight, rows: int, width: int, eps: float) -> np.ndarray:
+    """Qwen35Math.RmsNorm: one running sum per row."""
+    x, weight = _f32(x), _f32(weight)
+    out = np.empty(rows * width, dtype=np.float32)
+    lib().oracle_rms_norm_serial(_ptr(x), _ptr(weight), _ptr(out), rows, width, eps)
+    return out.reshape(rows, width)
+
+
+def silu_multiply(gate, up) -> np.ndarray:
+    gate, up = _f32(gate), _f32(up)
+    out = np.empty(gate.size, dtype=np.float32)
+    lib().oracle_silu_multiply(_ptr(gate), _ptr(up), _ptr(out), gate.size)
+    return out
+
+
+def add_in_place(destination, source) -> np.ndarray:
+    dest, source = _f32(destination).copy(), _f32(source)
+    lib().oracle_add_in_place(_ptr(dest), _ptr(source), dest.size)
+    return dest
+
+
+def np_tree_sum_of_squares(x: np.ndarray) -> np.float32:
+    """The 128-lane strided partial sums and the halving tree, with numpy float32 scalars (separate from the C)."""
+    x = np.asarray(x, dtype=np.float32)
+    sums = np.zeros(128, dtype=np.float32)
+    for j in range(x.size):                      # lane j % 128 meets its elements in increasing j
+        sums[j % 128] = np.float32(sums[j % 128] + np.float32(x[j] * x[j]))
+    stride = 64
+    while stride > 0:
+        sums[:stride] = sums[:stride] + sums[stride:2 * stride]
+        stride >>= 1
+    return sums[0]
+
+
+def np_rms_norm(x, weight, rows: int, width: int, eps: float, input_stride: int | None = None) -> np.ndarray:
+    stride = width if input_stride is None else input_stride
+    x, weight = np.asarray(x, dtype=np.float32), np.asarray(weight, dtype=np.float32)
+    out = np.empty((rows, width), dtype=np.float32)
+    for r in range(rows):
+        row = x[r * stride:r * stride + width]
+        mean = np.float32(np_tree_sum_of_squares(row) / np.float32(width))
+        inverse = np.float32(np.float32(1.0) / np.sqrt(np.float32(mean + np.float32(eps))))
+        out[r] = (row * inverse) * weight
+    return out
