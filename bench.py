@@ -317,6 +317,83 @@ def run_gemv(args, lane, nn, oracle):
     return out
 
 
+def run_ffn(args, lane, nn, oracle):
+    """Feed-forward half of a decode layer (hidden += attention; n = RMSNorm(hidden); hidden += W_down(SiLU(W_gate n) *
+    W_up n), NNtrain.Core/Modules/Qwen35QuantizedModel.cs:486-498) at hidden 5120 / feed-forward 17408 in Q4_K: the six
+    launches the reference issues against the three fused ones.  Eight layers' weights rotate (1.2 GB) so they stream
+    from HBM.  Both forms end in the same bits."""
+    from nntrain_amd import synth
+    from nntrain_amd.native import FusedMatvecDesc, PRE_RMS_NORM, PRE_SILU_MULTIPLY
+    import ctypes
+    typ, width, ffn, layers, eps = nn.GGML_Q4_K, 5120, 17408, 8, 1e-6
+    lib, h, chk = lane._lib, lane._handle, nn.native.check
+    up = lane.upload_raw
+    base = {"gate": up(synth.matrix(typ, ffn, width, 11)), "up": up(synth.matrix(typ, ffn, width, 12)),
+            "down": up(synth.matrix(typ, width, ffn, 13))}
+    weights = [base]
+    for _ in range(layers - 1):
+        layer = {}
+        for k, b in base.items():
+            layer[k] = lane.allocate_bytes(b.nbytes)
+            lane.copy(layer[k], b, b.nbytes)
+        weights.append(layer)
+    rng = np.random.default_rng(5)
+    hidden0 = (rng.standard_normal(width) * 2).astype(np.float32)
+    attn, gamma = up(rng.standard_normal(width).astype(np.float32)), up(rng.uniform(0.5, 1.5, width).astype(np.float32))
+    hid, hid2, norm, g, u, act, down = (lane.allocate(n) for n in (width, width, width, ffn, ffn, ffn, width))
+    P = lambda b: c_void_p(b.ptr) if b is not None else None                     # noqa: E731
+
+    def matvec(w, x, y, in_w, out_w):
+        chk(lib.nnhip_quant_matvec(h, typ, P(x), P(w), None, P(y), 1, in_w, out_w), "quant_matvec")
+
+    def fused(w, in_w, out_w, **kw):
+        d = FusedMatvecDesc(struct_size=ctypes.sizeof(FusedMatvecDesc), ggml_type=typ, w=P(w), in_w=in_w, out_w=out_w,
+                            **{k: (P(v) if hasattr(v, "ptr") else v) for k, v in kw.items()})
+        chk(lib.nnhip_quant_matvec_fused(h, ctypes.byref(d)), "quant_matvec_fused")
+
+    def layer_unfused(w):
+        chk(lib.nnhip_add_rms_norm(h, P(hid), P(attn), P(gamma), P(norm), 1, width, width, eps), "add_rms_norm")
+        matvec(w["gate"], norm, g, width, ffn)
+        matvec(w["up"], norm, u, width, ffn)
+        chk(lib.nnhip_silu_multiply(h, P(g), P(u), P(act), ffn), "silu_multiply")
+        matvec(w["down"], act, down, ffn, width)
+        chk(lib.nnhip_add_in_place(h, P(hid), P(down), width), "add_in_place")
+
+    state = {"cur": hid, "nxt": hid2}
+
+    def layer_fused(w):
+        cur, nxt = state["cur"], state["nxt"]
+        fused(w["gate"], width, ffn, pre_op=PRE_RMS_NORM, x=cur, x2=attn, norm_weight=gamma, epsilon=eps, x_out=norm, sum_out=nxt, y=g)
+        matvec(w["up"], norm, u, width, ffn)
+        fused(w["down"], ffn, width, pre_op=PRE_SILU_MULTIPLY, x=g, x2=u, addend=nxt, y=nxt)
+        state["cur"], state["nxt"] = nxt, cur
+
+    results = {}
+    finals = {}
+    for name, fn in (("unfused_6_launches", layer_unfused), ("fused_3_launches", layer_fused)):
+        lane.write(hid, hidden0)
+        state["cur"], state["nxt"] = hid, hid2
+        for w in weights:
+            fn(w)
+        lane.synchronize()
+        finals[name] = lane.read(state["cur"] if name.startswith("fused") else hid, np.uint32)
+        samples = []
+        for _ in range(9):
+            ms, _ = timed(lane, lambda: [fn(w) for w in weights], 1)
+            samples.append(ms * 1e3 / layers)
+        results[name] = round(float(np.median(samples)), 2)
+    if not np.array_equal(finals["unfused_6_launches"], finals["fused_3_launches"]):
+        raise SystemExit("ffn: fused and unfused layers differ bitwise")
+    wbytes = sum(b.nbytes for b in base.values())
+    out = {"config": "Q4_K, hidden 5120, feed-forward 17408, 8 layers' weights rotated", "us_per_layer": results,
+           "weight_bytes_per_layer": wbytes,
+           "gb_per_s_fused": round(wbytes / results["fused_3_launches"] / 1e3, 1),
+           "gb_per_s_unfused": round(wbytes / results["unfused_6_launches"] / 1e3, 1), "bitwise_equal": True}
+    log(f"[ffn] per layer: unfused {results['unfused_6_launches']:.2f} us, fused {results['fused_3_launches']:.2f} us "
+        f"({wbytes / results['fused_3_launches'] / 1e3:.0f} GB/s)")
+    return out
+
+
 def run_prefill(args, lane, nn, oracle):
     """Q4_K 17408x5120 bf16-MFMA prefill mat-mul at M = 128, 256, 512, 2048 (BASELINE configs[3])."""
     from nntrain_amd import synth
@@ -365,7 +442,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", choices=["decode27b", "gemv", "prefill", "all"], default="all")
+    ap.add_argument("--workload", choices=["decode27b", "gemv", "prefill", "ffn", "all"], default="all")
     ap.add_argument("--mode", choices=["forward", "graph", "batch"], default="batch",
                     help="decode27b: one launch per matrix, the same captured in a HIP graph, or the batched entry point")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -386,6 +463,8 @@ def main():
         also["gemv_single_matrix"] = run_gemv(args, lane, nn, oracle)
     if args.workload in ("prefill", "all"):
         also["prefill_q4k_bf16_mfma"] = run_prefill(args, lane, nn, oracle)
+    if args.workload in ("ffn", "all"):
+        also["ffn_layer_half_fused_epilogues"] = run_ffn(args, lane, nn, oracle)
     if args.workload in ("decode27b", "all"):
         res = run_decode27b(args, lane, nn, oracle)
     else:

@@ -34,6 +34,17 @@ internal static unsafe partial class NnHipNative
         internal uint GgmlType; internal int Rows; internal int InW; internal int OutW;
     }
 
+    internal const uint PreNone = 0, PreRmsNorm = 1, PreSiluMultiply = 2;
+
+    [StructLayout(LayoutKind.Sequential)]
+    internal struct FusedMatvecDesc
+    {
+        internal uint StructSize; internal uint GgmlType; internal uint PreOp; internal float Epsilon;
+        internal nint X; internal nint X2; internal nint NormWeight; internal nint XOut; internal nint SumOut;
+        internal nint W; internal nint Bias; internal nint Addend; internal nint Y;
+        internal int InW; internal int OutW;
+    }
+
     [LibraryImport(Library)] internal static partial uint nnhip_abi_version();
     [LibraryImport(Library)] internal static partial int nnhip_last_error(out ErrorInfo info, nuint size);
     [LibraryImport(Library)] internal static partial int nnhip_last_error_message(byte* buffer, int capacity);
@@ -56,6 +67,7 @@ internal static unsafe partial class NnHipNative
     [LibraryImport(Library)] internal static partial int nnhip_dequantize(nint lane, uint ggmlType, nint w, nint output, long elements);
     [LibraryImport(Library)] internal static partial int nnhip_quant_matvec(nint lane, uint ggmlType, nint x, nint w, nint bias, nint y, int rows, int inW, int outW);
     [LibraryImport(Library)] internal static partial int nnhip_quant_matvec_batch(nint lane, MatvecDesc* descs, int count);
+    [LibraryImport(Library)] internal static partial int nnhip_quant_matvec_fused(nint lane, FusedMatvecDesc* desc);
     [LibraryImport(Library)] internal static partial int nnhip_quant_matmul_bf16(nint lane, uint ggmlType, nint xBf16, nint w, nint bias, nint y, int rows, int inW, int outW);
     [LibraryImport(Library)] internal static partial int nnhip_rms_norm(nint lane, nint input, nint weight, nint output, int rows, int width, int inputStride, float epsilon);
     [LibraryImport(Library)] internal static partial int nnhip_add_rms_norm(nint lane, nint destination, nint residual, nint weight, nint output, int rows, int width, int inputStride, float epsilon);

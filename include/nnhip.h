@@ -220,6 +220,43 @@ NNHIP_API int nnhip_silu_multiply(void* lane, const float* gate, const float* up
  * Qwen35Gpu.Attention.cs:52-58).  Asynchronous. */
 NNHIP_API int nnhip_add_in_place(void* lane, float* destination, const float* source, int length);
 
+/* One decode mat-vec with the row operations on either side of it fused into the launch, for the feed-forward half
+ * of a layer as ForwardTokenDevice issues it (NNtrain.Core/Modules/Qwen35QuantizedModel.cs:482-498):
+ *   pre_op NNHIP_PRE_RMS_NORM       v = RMSNorm(x + x2) * norm_weight   (x2 may be null: plain RMSNorm of x); replaces
+ *                                   q35a_add_rms_norm / q35a_rms_norm followed by the projection; sum_out (may be null)
+ *                                   receives x + x2, x_out (may be null) the normalized vector, bit-identical to
+ *                                   nnhip_add_rms_norm / nnhip_rms_norm;
+ *   pre_op NNHIP_PRE_SILU_MULTIPLY  v = x * sigmoid(x) * x2 (gate, up); replaces q35a_silu_multiply followed by the
+ *                                   down projection; x_out (may be null) receives v;
+ *   pre_op NNHIP_PRE_NONE           v = x;
+ *   then  y[o] = addend[o] + (bias[o] + sum_k v[k] * w[o, k]); addend may be null, and may be y itself (the
+ *   residual stream: replaces q35a_add_in_place after the down projection).  bias may be null.
+ * The mat-vec part is bit-identical to nnhip_quant_matvec on the same v.  x, x2, norm_weight hold in_w floats;
+ * x_out and sum_out must not overlap x or x2 (every workgroup reads those while workgroup 0 writes).  Q8_0 rows with
+ * an odd number of blocks are not covered (NNHIP_ERR_INVALID_ARGUMENT).  struct_size = sizeof of this structure.
+ * This fusion has no single counterpart in the reference, which launches the parts one by one.  Asynchronous. */
+enum { NNHIP_PRE_NONE = 0, NNHIP_PRE_RMS_NORM = 1, NNHIP_PRE_SILU_MULTIPLY = 2 };
+
+typedef struct nnhip_fused_matvec_desc {
+    uint32_t struct_size;
+    uint32_t ggml_type;
+    uint32_t pre_op;
+    float epsilon;              /* RMSNorm only: finite, >= 0 */
+    const float* x;
+    const float* x2;
+    const float* norm_weight;   /* RMSNorm only */
+    float* x_out;
+    float* sum_out;             /* RMSNorm with x2 only */
+    const void* w;
+    const float* bias;
+    const float* addend;
+    float* y;
+    int32_t in_w;
+    int32_t out_w;
+} nnhip_fused_matvec_desc;
+
+NNHIP_API int nnhip_quant_matvec_fused(void* lane, const nnhip_fused_matvec_desc* desc);
+
 /* --- timing and replay --------------------------------------------------------------------------------------- */
 
 /* Device events on the lane's stream.  Replace the per-kernel OpenCL event timing of

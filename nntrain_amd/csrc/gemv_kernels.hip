@@ -49,7 +49,36 @@ struct MatvecArgs {
     int steps;             // ceil(out_w / RS)
     uint32_t row_bytes;
     uint32_t magic;        // ceil(2^32 / units_per_row): t / units_per_row == umulhi(t, magic) for t < 2^32 / upr
+    // fused variants only (null / unused otherwise)
+    const float* x2;       // RMSNorm: residual added to x first (or null); SiLU: the `up` vector
+    const float* gamma;    // RMSNorm weight
+    float* x_out;          // where the vector that was multiplied is stored (or null)
+    float* sum_out;        // RMSNorm: where x + residual is stored (or null)
+    const float* addend;   // y = addend + (bias + W x) (or null)
+    float epsilon;
 };
+
+enum : int { kPreNone = 0, kPreRmsNorm = 1, kPreSiluMultiply = 2 };
+
+__device__ __forceinline__ float4 add4(const float4 a, const float4 b) { return make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w); }
+
+// gate * sigmoid(gate) * up with the two-sided sigmoid of the reference (NNtrain.Arc/Kernels/qwen35_attention.cl:9-14,
+// 38-43): exp never sees a positive argument.
+__device__ __forceinline__ float silu_mul1(float g, float u)
+{
+    float sig;
+    if (g >= 0.0f) {
+        sig = 1.0f / (1.0f + expf(-g));
+    } else {
+        const float e = expf(g);
+        sig = e / (1.0f + e);
+    }
+    return g * sig * u;
+}
+__device__ __forceinline__ float4 silu_mul4(const float4 g, const float4 u)
+{
+    return make_float4(silu_mul1(g.x, u.x), silu_mul1(g.y, u.y), silu_mul1(g.z, u.z), silu_mul1(g.w, u.w));
+}
 
 __device__ __forceinline__ float dot4s(uint32_t v, const float4 x, float acc)  // 4 signed bytes . x
 {
@@ -497,7 +526,11 @@ template <> struct Shape<IQ3SUnit> { static constexpr int kMaxT = 1024, kWavesPe
 template <> struct Shape<BF16Unit> { static constexpr int kMaxT = 512, kWavesPerEu = 2, kDepth = 2, kBatchDepth = 2; };
 
 // grid.x = workgroups striding over row steps, grid.y = input rows, blockDim.x = T (a multiple of 64).
-template <class Q>
+// PRE selects what is done to the activations while they are staged: nothing; (x + residual) -> RMSNorm * gamma in the
+// summation order of q35a_add_rms_norm / q35a_rms_norm (NNtrain.Arc/Kernels/qwen35_attention.cl:16-78: 128 lane-strided
+// partial sums, halving tree); SiLU(x) * x2 (qwen35_attention.cl:38-43).  Every workgroup prepares the whole vector
+// for itself; workgroup 0 also stores it (and the residual sum) where the caller asked.
+template <class Q, int PRE = kPreNone>
 __global__ __launch_bounds__(Shape<Q>::kMaxT) __attribute__((amdgpu_waves_per_eu(Shape<Q>::kWavesPerEu, Shape<Q>::kWavesPerEu)))
 void matvec_rowstep_kernel(MatvecArgs a, const float* __restrict__ bias)
 {
@@ -529,6 +562,18 @@ void matvec_rowstep_kernel(MatvecArgs a, const float* __restrict__ bias)
     const int T = blockDim.x;
     float4 xv0 = tid < pieces ? xg[tid] : make_float4(0.f, 0.f, 0.f, 0.f);
     float4 xv1 = tid + T < pieces ? xg[tid + T] : make_float4(0.f, 0.f, 0.f, 0.f);
+    const float4* x2g = reinterpret_cast<const float4*>(a.x2);
+    const float4* gg = reinterpret_cast<const float4*>(a.gamma);
+    const bool second = PRE == kPreSiluMultiply || (PRE == kPreRmsNorm && a.x2 != nullptr);
+    float4 sv0 = make_float4(0.f, 0.f, 0.f, 0.f), sv1 = sv0, gv0 = sv0, gv1 = sv0;
+    if constexpr (PRE != kPreNone) {
+        if (second && tid < pieces) sv0 = x2g[tid];
+        if (second && tid + T < pieces) sv1 = x2g[tid + T];
+    }
+    if constexpr (PRE == kPreRmsNorm) {
+        if (tid < pieces) gv0 = gg[tid];
+        if (tid + T < pieces) gv1 = gg[tid + T];
+    }
     // The compute unit returns vector-memory data in the order the requests were queued, across waves.  This barrier
     // (no memory wait, just a rendezvous) puts every wave's activation requests ahead of every wave's weight
     // requests, so staging does not wait for the first weight rows to come back from HBM.
@@ -540,9 +585,78 @@ void matvec_rowstep_kernel(MatvecArgs a, const float* __restrict__ bias)
 #pragma unroll
     for (int d = 0; d < kDepth - 1; ++d) regs[d] = fetch(step + d * stride);
 
-    if (tid < pieces) xstage[tid + (tid >> 4)] = xv0;
-    if (tid + T < pieces) xstage[tid + T + ((tid + T) >> 4)] = xv1;
-    for (int L = tid + 2 * T; L < pieces; L += T) xstage[L + (L >> 4)] = xg[L];
+    const bool scribe = blockIdx.x == 0;      // the workgroup that stores the prepared vector
+    if constexpr (PRE == kPreSiluMultiply) {
+        float4* xo = scribe ? reinterpret_cast<float4*>(a.x_out) : nullptr;
+        xv0 = silu_mul4(xv0, sv0);
+        xv1 = silu_mul4(xv1, sv1);
+        if (tid < pieces) { xstage[tid + (tid >> 4)] = xv0; if (xo) xo[tid] = xv0; }
+        if (tid + T < pieces) { xstage[tid + T + ((tid + T) >> 4)] = xv1; if (xo) xo[tid + T] = xv1; }
+        for (int L = tid + 2 * T; L < pieces; L += T) {
+            const float4 v = silu_mul4(xg[L], x2g[L]);
+            xstage[L + (L >> 4)] = v;
+            if (xo) xo[L] = v;
+        }
+    } else if constexpr (PRE == kPreRmsNorm) {
+        float4* so = scribe ? reinterpret_cast<float4*>(a.sum_out) : nullptr;
+        float4* xo = scribe ? reinterpret_cast<float4*>(a.x_out) : nullptr;
+        // the residual stream first
+        if (second) {                      // (without a residual the input keeps its bits: -0 stays -0)
+            xv0 = add4(xv0, sv0);
+            xv1 = add4(xv1, sv1);
+        }
+        if (tid < pieces) { xstage[tid + (tid >> 4)] = xv0; if (so) so[tid] = xv0; }
+        if (tid + T < pieces) { xstage[tid + T + ((tid + T) >> 4)] = xv1; if (so) so[tid + T] = xv1; }
+        for (int L = tid + 2 * T; L < pieces; L += T) {
+            const float4 v = second ? add4(xg[L], x2g[L]) : xg[L];
+            xstage[L + (L >> 4)] = v;
+            if (so) so[L] = v;
+        }
+        __syncthreads();
+        // 128 lane-strided partial sums of squares ...
+        const float* xs = reinterpret_cast<const float*>(xstage);
+        float sq = 0.0f;
+        if (tid < 128)
+            for (int j = tid; j < a.in_w; j += 128) {
+                const int L = j >> 2;
+                const float v = xs[4 * (L + (L >> 4)) + (j & 3)];
+                sq += v * v;
+            }
+        // ... then the halving tree: 64 through LDS (the two waves that hold the partials), 32 .. 1 inside wave 0
+        if (tid >= 64 && tid < 128) part[0][tid - 64] = sq;
+        __syncthreads();
+        if (tid < 64) {
+            sq += part[0][tid];
+            const uint32_t u = __float_as_uint(sq);
+            auto s32 = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+            sq = __uint_as_float(s32[0]) + __uint_as_float(s32[1]);              // lanes 0-31: s[t] + s[t+32]
+            const uint32_t v = __float_as_uint(sq);
+            auto s16 = __builtin_amdgcn_permlane16_swap(v, v, false, false);
+            sq = __uint_as_float(s16[0]) + __uint_as_float(s16[1]);              // lanes 0-15: s[t] + s[t+16]
+            sq += dpp_mov<0x108>(sq);                                             // row_shl:8  s[t] + s[t+8]
+            sq += dpp_mov<0x104>(sq);                                             // row_shl:4
+            sq += dpp_mov<0x102>(sq);                                             // row_shl:2
+            sq += dpp_mov<0x101>(sq);                                             // row_shl:1
+            if (tid == 0) part[1][0] = sq;
+        }
+        __syncthreads();
+        const float inverse = 1.0f / sqrtf(part[1][0] / static_cast<float>(a.in_w) + a.epsilon);
+        auto normalize = [&](float4 h, const float4 g) {
+            return make_float4(h.x * inverse * g.x, h.y * inverse * g.y, h.z * inverse * g.z, h.w * inverse * g.w);
+        };
+        // every lane rewrites the pieces it staged itself
+        if (tid < pieces) { xv0 = normalize(xv0, gv0); xstage[tid + (tid >> 4)] = xv0; if (xo) xo[tid] = xv0; }
+        if (tid + T < pieces) { xv1 = normalize(xv1, gv1); xstage[tid + T + ((tid + T) >> 4)] = xv1; if (xo) xo[tid + T] = xv1; }
+        for (int L = tid + 2 * T; L < pieces; L += T) {
+            const float4 v = normalize(xstage[L + (L >> 4)], gg[L]);
+            xstage[L + (L >> 4)] = v;
+            if (xo) xo[L] = v;
+        }
+    } else {
+        if (tid < pieces) xstage[tid + (tid >> 4)] = xv0;
+        if (tid + T < pieces) xstage[tid + T + ((tid + T) >> 4)] = xv1;
+        for (int L = tid + 2 * T; L < pieces; L += T) xstage[L + (L >> 4)] = xg[L];
+    }
     if constexpr (Q::kGridWords > 0)
         for (int i = tid; i < Q::kGridWords; i += T) grid[i] = Q::grid_table()[i];
     __syncthreads();
@@ -560,7 +674,9 @@ void matvec_rowstep_kernel(MatvecArgs a, const float* __restrict__ bias)
         for (int i = tid; i < held * rs; i += T) {
             const int j = i / rs;
             const int row = (first_held + j * stride) * rs + (i - j * rs);
-            if (row < a.out_w) y[row] = ybuf[i];
+            if (row < a.out_w) {
+                y[row] = a.addend ? a.addend[row] + ybuf[i] : ybuf[i];
+            }
         }
         held = 0;
     };
@@ -863,22 +979,23 @@ bool plan(int in_w, int out_w, int compute_units, int max_t, Geometry* g)
     return true;
 }
 
-template <class Q>
+template <class Q, int PRE = kPreNone>
 hipError_t launch_rowstep(Lane* lane, MatvecArgs args, int rows)
 {
     Geometry g;
     if (!plan(args.in_w, args.out_w, lane->compute_units, Shape<Q>::kMaxT, &g)) return hipErrorInvalidValue;
+    if (PRE == kPreRmsNorm && g.threads < 128) g.threads = 128;     // the norm's partial sums take 128 lanes
     args.rows_per_step = g.rows_per_step;
     args.steps = g.steps;
     const size_t lds = static_cast<size_t>(kChunkPieces) * args.units_per_row * sizeof(float4);
     static bool big_lds_enabled = false;
     if (lds > 48 * 1024 && !big_lds_enabled) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&matvec_rowstep_kernel<Q>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&matvec_rowstep_kernel<Q, PRE>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, kMaxDynamicLds);
         if (e != hipSuccess) return e;
         big_lds_enabled = true;
     }
-    hipLaunchKernelGGL(matvec_rowstep_kernel<Q>, dim3(g.groups, rows), dim3(g.threads), lds, lane->stream, args, args.bias);
+    hipLaunchKernelGGL((matvec_rowstep_kernel<Q, PRE>), dim3(g.groups, rows), dim3(g.threads), lds, lane->stream, args, args.bias);
     return hipGetLastError();
 }
 
@@ -957,6 +1074,54 @@ hipError_t launch_matvec(Lane* lane, uint32_t type, const float* x, const void* 
     }
 }
 
+
+template <int PRE>
+hipError_t launch_fused_of(Lane* lane, uint32_t type, const MatvecArgs& a)
+{
+    switch (type) {
+    case NNHIP_TYPE_Q8_0: return launch_rowstep<Q8_0Unit, PRE>(lane, a, 1);
+    case NNHIP_TYPE_Q4_K: return launch_rowstep<Q4KUnit, PRE>(lane, a, 1);
+    case NNHIP_TYPE_Q5_K: return launch_rowstep<Q5KUnit, PRE>(lane, a, 1);
+    case NNHIP_TYPE_Q6_K: return launch_rowstep<Q6KUnit, PRE>(lane, a, 1);
+    case NNHIP_TYPE_IQ3_S: return launch_rowstep<IQ3SUnit, PRE>(lane, a, 1);
+    case NNHIP_TYPE_BF16: return launch_rowstep<BF16Unit, PRE>(lane, a, 1);
+    case NNHIP_TYPE_IQ2_S: return launch_rowstep<IQ2SUnit, PRE>(lane, a, 1);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+bool matvec_fused_supported(uint32_t type, int in_w)
+{
+    return !(type == NNHIP_TYPE_Q8_0 && ((in_w / 32) & 1));     // rows of an odd number of Q8_0 blocks take another kernel
+}
+
+hipError_t launch_matvec_fused(Lane* lane, const nnhip_fused_matvec_desc& d)
+{
+    int elems = 0, bytes = 0;
+    type_block(d.ggml_type, &elems, &bytes);
+    MatvecArgs a{};
+    a.x = d.x;
+    a.w = static_cast<const uint8_t*>(d.w);
+    a.bias = d.bias;
+    a.y = d.y;
+    a.in_w = d.in_w;
+    a.out_w = d.out_w;
+    a.row_bytes = static_cast<uint32_t>(d.in_w / elems) * static_cast<uint32_t>(bytes);
+    a.units_per_row = d.in_w / kUnitW;
+    a.magic = static_cast<uint32_t>((0x100000000ull + a.units_per_row - 1) / a.units_per_row);
+    a.x2 = d.x2;
+    a.gamma = d.norm_weight;
+    a.x_out = d.x_out;
+    a.sum_out = d.sum_out;
+    a.addend = d.addend;
+    a.epsilon = d.epsilon;
+    switch (d.pre_op) {
+    case NNHIP_PRE_NONE: return launch_fused_of<kPreNone>(lane, d.ggml_type, a);
+    case NNHIP_PRE_RMS_NORM: return launch_fused_of<kPreRmsNorm>(lane, d.ggml_type, a);
+    case NNHIP_PRE_SILU_MULTIPLY: return launch_fused_of<kPreSiluMultiply>(lane, d.ggml_type, a);
+    default: return hipErrorInvalidValue;
+    }
+}
 
 hipError_t launch_matvec_batch(Lane* lane, const nnhip_matvec_desc* descs, int count)
 {

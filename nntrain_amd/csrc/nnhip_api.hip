@@ -436,6 +436,56 @@ int nnhip_add_in_place(void* handle, float* destination, const float* source, in
     return NNHIP_OK;
 }
 
+int nnhip_quant_matvec_fused(void* handle, const nnhip_fused_matvec_desc* d)
+{
+    NNHIP_LANE(handle, NNHIP_OP_MATVEC_FUSED)
+    const uint32_t op = NNHIP_OP_MATVEC_FUSED;
+    if (!d || d->struct_size != sizeof(nnhip_fused_matvec_desc))
+        return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0, "descriptor is null or has the wrong struct_size");
+    int rc = check_linear(op, lane, d->ggml_type, d->x, d->w, d->y, 1, d->in_w, d->out_w);
+    if (rc != NNHIP_OK) return rc;
+    if (d->in_w > matvec_max_in_w(d->ggml_type))
+        return fail(NNHIP_ERR_TOO_LARGE, op, lane->device, 0, "in_w %d exceeds the %d values one workgroup can stage", d->in_w, matvec_max_in_w(d->ggml_type));
+    if (!matvec_fused_supported(d->ggml_type, d->in_w))
+        return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0, "Q8_0 rows with an odd number of blocks are not covered by the fused mat-vec");
+    auto aligned = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
+    if (!aligned(d->x2) || !aligned(d->norm_weight) || !aligned(d->x_out) || !aligned(d->sum_out))
+        return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0, "x2, norm_weight, x_out and sum_out must be 16-byte aligned");
+    switch (d->pre_op) {
+    case NNHIP_PRE_NONE:
+        if (d->x2 || d->norm_weight || d->x_out || d->sum_out)
+            return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0, "x2, norm_weight, x_out and sum_out must be null without a pre-op");
+        break;
+    case NNHIP_PRE_RMS_NORM:
+        if (!d->norm_weight) return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0, "norm_weight is null");
+        if (!(d->epsilon >= 0.0f) || !std::isfinite(d->epsilon))
+            return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0, "epsilon must be finite and not negative");
+        if (d->sum_out && !d->x2) return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0, "sum_out needs a residual (x2)");
+        break;
+    case NNHIP_PRE_SILU_MULTIPLY:
+        if (!d->x2) return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0, "the up vector (x2) is null");
+        if (d->norm_weight || d->sum_out)
+            return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0, "norm_weight and sum_out must be null for SiLU * up");
+        break;
+    default:
+        return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0, "unknown pre_op %u", d->pre_op);
+    }
+    const size_t xbytes = static_cast<size_t>(d->in_w) * sizeof(float);
+    auto overlaps = [&](const float* out, const float* in) {
+        if (!out || !in) return false;
+        const char* a = reinterpret_cast<const char*>(out);
+        const char* b = reinterpret_cast<const char*>(in);
+        return a < b + xbytes && b < a + xbytes;
+    };
+    if (overlaps(d->x_out, d->x) || overlaps(d->x_out, d->x2) || overlaps(d->sum_out, d->x) || overlaps(d->sum_out, d->x2) ||
+        overlaps(d->x_out, d->sum_out))
+        return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0, "x_out and sum_out must not overlap the inputs or each other");
+    hipError_t e = launch_matvec_fused(lane, *d);
+    if (e != hipSuccess) return hip_fail(e, op, lane->device, "fused mat-vec launch");
+    lane->counters.kernel_launches += 1;
+    return NNHIP_OK;
+}
+
 int nnhip_quant_matvec_batch(void* handle, const nnhip_matvec_desc* descs, int count)
 {
     NNHIP_LANE(handle, NNHIP_OP_MATVEC_BATCH)

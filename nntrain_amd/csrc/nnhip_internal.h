@@ -51,6 +51,9 @@ int fail(int status, uint32_t op, int device, uint32_t hip_error, const char* fm
 hipError_t launch_dequantize(Lane* lane, uint32_t type, const void* w, float* out, int64_t elements);
 hipError_t launch_matvec(Lane* lane, uint32_t type, const float* x, const void* w, const float* bias, float* y,
                          int rows, int in_w, int out_w);
+// Mat-vec with the activation preparation and the residual add fused in (descriptor checked by the caller).
+bool matvec_fused_supported(uint32_t type, int in_w);
+hipError_t launch_matvec_fused(Lane* lane, const nnhip_fused_matvec_desc& d);
 hipError_t launch_matvec_batch(Lane* lane, const nnhip_matvec_desc* descs, int count);
 hipError_t launch_matmul_bf16(Lane* lane, uint32_t type, const uint16_t* x, const void* w, const float* bias,
                               float* y, int rows, int in_w, int out_w);

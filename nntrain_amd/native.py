@@ -43,6 +43,15 @@ class MatvecDesc(Structure):
                 ("rows", c_int32), ("in_w", c_int32), ("out_w", c_int32)]
 
 
+class FusedMatvecDesc(Structure):
+    _fields_ = [("struct_size", c_uint32), ("ggml_type", c_uint32), ("pre_op", c_uint32), ("epsilon", c_float),
+                ("x", c_void_p), ("x2", c_void_p), ("norm_weight", c_void_p), ("x_out", c_void_p), ("sum_out", c_void_p),
+                ("w", c_void_p), ("bias", c_void_p), ("addend", c_void_p), ("y", c_void_p), ("in_w", c_int32),
+                ("out_w", c_int32)]
+
+
+PRE_NONE, PRE_RMS_NORM, PRE_SILU_MULTIPLY = 0, 1, 2
+
 # name -> (restype, argtypes); exactly the prototypes of include/nnhip.h
 PROTOTYPES = {
     "nnhip_abi_version": (c_uint32, []),
@@ -67,6 +76,7 @@ PROTOTYPES = {
     "nnhip_dequantize": (c_int, [c_void_p, c_uint32, c_void_p, c_void_p, c_int64]),
     "nnhip_quant_matvec": (c_int, [c_void_p, c_uint32, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int]),
     "nnhip_quant_matvec_batch": (c_int, [c_void_p, POINTER(MatvecDesc), c_int]),
+    "nnhip_quant_matvec_fused": (c_int, [c_void_p, POINTER(FusedMatvecDesc)]),
     "nnhip_quant_matmul_bf16": (c_int, [c_void_p, c_uint32, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int]),
     "nnhip_rms_norm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float]),
     "nnhip_add_rms_norm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float]),

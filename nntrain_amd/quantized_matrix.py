@@ -8,13 +8,14 @@ ValueError, InvalidDataException -> ValueError("... payload ...").
 """
 from __future__ import annotations
 
+import ctypes
 from ctypes import c_void_p
 
 import numpy as np
 
 from . import native
 from .lane import HipBuffer, HipExecutionLane
-from .native import check
+from .native import PRE_NONE, PRE_RMS_NORM, PRE_SILU_MULTIPLY, FusedMatvecDesc, check  # noqa: F401
 
 GGML_Q8_0, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_IQ3_S, GGML_IQ2_S, GGML_BF16 = 8, 12, 13, 14, 21, 22, 30
 BLOCK_ELEMS = {GGML_Q8_0: 32, GGML_Q4_K: 256, GGML_Q5_K: 256, GGML_Q6_K: 256, GGML_IQ3_S: 256, GGML_IQ2_S: 256,
@@ -115,6 +116,33 @@ class HipQuantizedMatrix:
         check(lane._lib.nnhip_quant_matvec(lane._handle, self.ggml_type, c_void_p(x._require()), c_void_p(w._require()),
                                            c_void_p(bias._require()) if bias is not None else None,
                                            c_void_p(y._require()), rows, self.input_width, self.output_width), "quant_matvec")
+        return y
+
+    def forward_fused(self, lane: HipExecutionLane, x: HipBuffer, *, pre_op: int = PRE_NONE, x2: HipBuffer | None = None,
+                      norm_weight: HipBuffer | None = None, epsilon: float = 0.0, x_out: HipBuffer | None = None,
+                      sum_out: HipBuffer | None = None, bias: HipBuffer | None = None, addend: HipBuffer | None = None,
+                      out: HipBuffer | None = None) -> HipBuffer:
+        """One decode mat-vec with its neighbours fused into the launch: v = RMSNorm(x + x2) * norm_weight
+        (PRE_RMS_NORM; x2 optional) or SiLU(x) * x2 (PRE_SILU_MULTIPLY) or x, then y = addend + bias + W v.
+        x_out / sum_out receive v and x + x2 when given.  `out` may be `addend` (the residual stream updated in place)."""
+        n_in, n_out = 4 * self.input_width, 4 * self.output_width
+        for name, buf, need in (("x", x, n_in), ("x2", x2, n_in), ("norm_weight", norm_weight, n_in), ("x_out", x_out, n_in),
+                                ("sum_out", sum_out, n_in), ("bias", bias, n_out), ("addend", addend, n_out), ("out", out, n_out)):
+            if buf is not None and buf.nbytes < need:
+                raise ValueError(f"Quantized linear '{name}' width mismatch.")
+        w = self.device_payload(lane)
+        y = out if out is not None else lane.allocate(self.output_width)
+        ptr = lambda b: c_void_p(b._require()) if b is not None else None   # noqa: E731
+        desc = FusedMatvecDesc(struct_size=ctypes.sizeof(FusedMatvecDesc), ggml_type=self.ggml_type, pre_op=pre_op,
+                               epsilon=epsilon, x=ptr(x), x2=ptr(x2), norm_weight=ptr(norm_weight), x_out=ptr(x_out),
+                               sum_out=ptr(sum_out), w=ptr(w), bias=ptr(bias), addend=ptr(addend), y=ptr(y),
+                               in_w=self.input_width, out_w=self.output_width)
+        try:
+            check(lane._lib.nnhip_quant_matvec_fused(lane._handle, ctypes.byref(desc)), "quant_matvec_fused")
+        except BaseException:
+            if out is None:
+                y.dispose()
+            raise
         return y
 
     def forward_bf16(self, lane: HipExecutionLane, x_bf16: HipBuffer, bias: HipBuffer | None, rows: int,

@@ -1,0 +1,159 @@
+"""GPU parity of the fused decode mat-vec (activation preparation + mat-vec + residual add in one launch).
+
+Bar: bit-identical to the unfused sequence of this library's own entry points (nnhip_add_rms_norm / nnhip_rms_norm /
+nnhip_silu_multiply, nnhip_quant_matvec, nnhip_add_in_place), each of which is checked against the oracle elsewhere;
+and, end to end, within the mat-vec bar (relative L2 <= 1e-5) of the float64 oracle fed the oracle's own FP32
+preparation.
+"""
+import numpy as np
+import pytest
+
+import oracle
+from nntrain_amd import (GGML_BF16, GGML_IQ2_S, GGML_IQ3_S, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_Q8_0, HipExecutionLane,
+                         HipQuantizedMatrix, NnHipError, qwen35_gpu, synth)
+from nntrain_amd.quantized_matrix import PRE_NONE, PRE_RMS_NORM, PRE_SILU_MULTIPLY
+
+pytestmark = pytest.mark.gpu
+
+TYPES = [GGML_Q8_0, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_IQ3_S, GGML_IQ2_S, GGML_BF16]
+SHAPES = [(256, 8), (1024, 67), (5120, 131)]           # (in_w, out_w); 17408 is covered separately (staging loop)
+EPS = 1e-6
+
+
+@pytest.fixture(scope="module")
+def lane():
+    with HipExecutionLane(0) as ln:
+        yield ln
+
+
+def _bits(a):
+    return np.ascontiguousarray(a, dtype=np.float32).view(np.uint32)
+
+
+def _matrix(typ, out_w, in_w, seed):
+    return HipQuantizedMatrix(synth.matrix(typ, out_w, in_w, seed), typ, out_w, in_w)
+
+
+def _vectors(in_w, out_w, seed):
+    rng = np.random.default_rng(seed)
+    f = lambda n, s=1.0: (rng.standard_normal(n) * s).astype(np.float32)     # noqa: E731
+    return dict(hidden=f(in_w, 3), residual=f(in_w), gamma=rng.uniform(-2, 2, in_w).astype(np.float32), gate=f(in_w, 4),
+                up=f(in_w), bias=f(out_w, 0.1), stream=f(out_w, 2))
+
+
+@pytest.mark.parametrize("typ", TYPES)
+@pytest.mark.parametrize("in_w,out_w", SHAPES)
+def test_rms_norm_projection_equals_the_unfused_sequence_bitwise(lane, typ, in_w, out_w):
+    v = _vectors(in_w, out_w, in_w + typ)
+    m = _matrix(typ, out_w, in_w, 3)
+    up = lambda a: lane.upload_raw(a)                                           # noqa: E731
+    for with_residual in (True, False):
+        hid_a, hid_b, res, gam, bias = up(v["hidden"]), up(v["hidden"]), up(v["residual"]), up(v["gamma"]), up(v["bias"])
+        # unfused: (hidden += residual) -> RMSNorm -> mat-vec
+        if with_residual:
+            norm = qwen35_gpu.add_residual_and_rms_norm(lane, hid_a, res, gam, in_w, EPS)
+        else:
+            norm = qwen35_gpu.rms_norm(lane, hid_a, gam, 1, in_w, EPS)
+        y_ref = m.forward(lane, norm, bias)
+        # fused
+        x_out, sum_out = lane.allocate(in_w), lane.allocate(in_w)
+        y = m.forward_fused(lane, hid_b, pre_op=PRE_RMS_NORM, x2=res if with_residual else None, norm_weight=gam,
+                            epsilon=EPS, x_out=x_out, sum_out=sum_out if with_residual else None, bias=bias)
+        assert np.array_equal(_bits(lane.read(x_out, count=in_w)), _bits(lane.read(norm, count=in_w)))
+        if with_residual:
+            assert np.array_equal(_bits(lane.read(sum_out, count=in_w)), _bits(lane.read(hid_a, count=in_w)))
+        assert np.array_equal(_bits(lane.read(hid_b, count=in_w)), _bits(v["hidden"]))      # the fused form writes elsewhere
+        assert np.array_equal(_bits(lane.read(y, count=out_w)), _bits(lane.read(y_ref, count=out_w)))
+        for b in (hid_a, hid_b, res, gam, bias, norm, y_ref, x_out, sum_out, y):
+            b.dispose()
+    m.dispose()
+
+
+@pytest.mark.parametrize("typ", TYPES)
+@pytest.mark.parametrize("in_w,out_w", SHAPES + [(17408, 33)])
+def test_silu_down_projection_and_residual_add_equal_the_unfused_sequence_bitwise(lane, typ, in_w, out_w):
+    v = _vectors(in_w, out_w, in_w + 7 * typ)
+    m = _matrix(typ, out_w, in_w, 4)
+    gate, upv, stream_a, stream_b = (lane.upload_raw(v[k]) for k in ("gate", "up", "stream", "stream"))
+    act = qwen35_gpu.silu_multiply(lane, gate, upv, in_w)
+    down = m.forward(lane, act, None)
+    qwen35_gpu.add_in_place(lane, stream_a, down, out_w)
+    x_out = lane.allocate(in_w)
+    y = m.forward_fused(lane, gate, pre_op=PRE_SILU_MULTIPLY, x2=upv, x_out=x_out, addend=stream_b, out=stream_b)
+    assert y is stream_b
+    assert np.array_equal(_bits(lane.read(x_out, count=in_w)), _bits(lane.read(act, count=in_w)))
+    assert np.array_equal(_bits(lane.read(stream_b, count=out_w)), _bits(lane.read(stream_a, count=out_w)))
+    for b in (gate, upv, stream_a, stream_b, act, down, x_out):
+        b.dispose()
+    m.dispose()
+
+
+@pytest.mark.parametrize("typ", [GGML_Q8_0, GGML_Q4_K, GGML_IQ2_S])
+def test_plain_with_addend_and_without_outputs(lane, typ):
+    in_w, out_w = 2048, 517
+    v = _vectors(in_w, out_w, 11)
+    m = _matrix(typ, out_w, in_w, 5)
+    x, bias, stream = lane.upload_raw(v["gate"]), lane.upload_raw(v["bias"]), lane.upload_raw(v["stream"])
+    y_ref = lane.read(m.forward(lane, x, bias), count=out_w)
+    y = m.forward_fused(lane, x, pre_op=PRE_NONE, bias=bias, addend=stream)
+    assert np.array_equal(_bits(lane.read(y, count=out_w)), _bits(v["stream"] + y_ref))
+    # pre-ops without the optional outputs
+    gam = lane.upload_raw(v["gamma"][:in_w])
+    a = m.forward_fused(lane, x, pre_op=PRE_RMS_NORM, norm_weight=gam, epsilon=EPS)
+    norm = qwen35_gpu.rms_norm(lane, x, gam, 1, in_w, EPS)
+    assert np.array_equal(_bits(lane.read(a, count=out_w)), _bits(lane.read(m.forward(lane, norm, None), count=out_w)))
+    m.dispose()
+
+
+@pytest.mark.parametrize("typ", [GGML_Q8_0, GGML_Q4_K, GGML_Q6_K])
+def test_feed_forward_half_of_a_layer_against_the_float64_oracle(lane, typ):
+    # hidden += attention; n = RMSNorm(hidden); hidden += W_down (SiLU(W_gate n) * (W_up n))   (Qwen35QuantizedModel.cs:486-498)
+    width, ffn = 1024, 2816 if typ == GGML_Q8_0 else 2816 - 2816 % 256
+    rng = np.random.default_rng(21)
+    hidden = (rng.standard_normal(width) * 2).astype(np.float32)
+    attn = rng.standard_normal(width).astype(np.float32)
+    gamma = rng.uniform(0.5, 1.5, width).astype(np.float32)
+    raw = {k: synth.matrix(typ, o, i, s) for k, (o, i, s) in dict(gate=(ffn, width, 1), up=(ffn, width, 2), down=(width, ffn, 3)).items()}
+    mats = {k: HipQuantizedMatrix(raw[k], typ, *(dict(gate=(ffn, width), up=(ffn, width), down=(width, ffn))[k])) for k in raw}
+    hb, ab, gb = lane.upload_raw(hidden), lane.upload_raw(attn), lane.upload_raw(gamma)
+    stream, normed = lane.allocate(width), lane.allocate(width)
+    launches = lane.counters()["kernel_launches"]
+    g = mats["gate"].forward_fused(lane, hb, pre_op=PRE_RMS_NORM, x2=ab, norm_weight=gb, epsilon=EPS, x_out=normed, sum_out=stream)
+    u = mats["up"].forward(lane, normed, None)
+    mats["down"].forward_fused(lane, g, pre_op=PRE_SILU_MULTIPLY, x2=u, addend=stream, out=stream)
+    assert lane.counters()["kernel_launches"] - launches == 3              # the reference issues six
+    got = lane.read(stream, count=width)
+    # oracle: FP32 row operations, float64 mat-vecs
+    summed, n = oracle.add_rms_norm(hidden, attn, gamma, 1, width, EPS)
+    g64, _ = oracle.linear_f64(typ, raw["gate"], n.ravel(), None, 1, width, ffn)
+    u64, _ = oracle.linear_f64(typ, raw["up"], n.ravel(), None, 1, width, ffn)
+    act = oracle.silu_multiply(g64.astype(np.float32).ravel(), u64.astype(np.float32).ravel())
+    d64, _ = oracle.linear_f64(typ, raw["down"], act, None, 1, ffn, width)
+    want = summed.astype(np.float64) + d64.ravel()
+    assert oracle.rel_l2(got, want) <= 1e-5
+    for m in mats.values():
+        m.dispose()
+
+
+def test_argument_checks(lane):
+    m = _matrix(GGML_Q4_K, 8, 256, 1)
+    x, small = lane.allocate(256), lane.allocate(8)
+    with pytest.raises(NnHipError):
+        m.forward_fused(lane, x, pre_op=PRE_RMS_NORM)                              # no norm weight
+    with pytest.raises(NnHipError):
+        m.forward_fused(lane, x, pre_op=PRE_RMS_NORM, norm_weight=x, epsilon=-1.0)
+    with pytest.raises(NnHipError):
+        m.forward_fused(lane, x, pre_op=PRE_SILU_MULTIPLY)                         # no up vector
+    with pytest.raises(NnHipError):
+        m.forward_fused(lane, x, pre_op=PRE_SILU_MULTIPLY, x2=x, x_out=x)          # output over an input
+    with pytest.raises(NnHipError):
+        m.forward_fused(lane, x, pre_op=PRE_NONE, x2=x)
+    with pytest.raises(NnHipError):
+        m.forward_fused(lane, x, pre_op=7)
+    with pytest.raises(ValueError):
+        m.forward_fused(lane, x, pre_op=PRE_SILU_MULTIPLY, x2=small)
+    odd = HipQuantizedMatrix(synth.matrix(GGML_Q8_0, 4, 96, 1), GGML_Q8_0, 4, 96)
+    with pytest.raises(NnHipError):
+        odd.forward_fused(lane, x, pre_op=PRE_NONE)                                # three Q8_0 blocks per row
+    m.dispose()
+    odd.dispose()
