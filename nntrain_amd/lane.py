@@ -42,6 +42,17 @@ class HipBuffer:
             raise ValueError("buffer has been disposed")
         return self.ptr
 
+    def view(self, offset_bytes: int, nbytes: int) -> "HipBuffer":
+        """A window of this allocation that does not own it (disposing the view frees nothing)."""
+        if offset_bytes < 0 or nbytes <= 0 or offset_bytes + nbytes > self.nbytes:
+            raise ValueError("view exceeds the buffer")
+        return _HipBufferView(self.lane, self._require() + offset_bytes, nbytes)
+
+
+class _HipBufferView(HipBuffer):
+    def dispose(self) -> None:
+        self.ptr = 0
+
 
 class HipEvent:
     def __init__(self, lane: "HipExecutionLane"):

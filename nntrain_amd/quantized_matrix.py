@@ -77,6 +77,30 @@ class HipQuantizedMatrix:
         self._device_payload = buffer
         return self
 
+    @classmethod
+    def stacked(cls, lane: HipExecutionLane, matrices) -> "HipQuantizedMatrix":
+        """One device matrix holding the rows of `matrices` one after the other (same storage type and input width):
+        projections that consume the same vector, such as the gate and up matrices of a feed-forward block
+        (Qwen35QuantizedModel.cs:488-489), then cost one launch, and row i of matrix k is output row offset_k + i with
+        the bits it has alone.  Raw blocks are copied device to device; the inputs stay usable."""
+        matrices = list(matrices)
+        if not matrices:
+            raise ValueError("no matrices to stack")
+        first = matrices[0]
+        if any(m.ggml_type != first.ggml_type or m.input_width != first.input_width for m in matrices):
+            raise ValueError("stacked matrices must share the storage type and the input width")
+        total = sum(m.storage_bytes for m in matrices)
+        buffer = lane.allocate_bytes(total)
+        try:
+            offset = 0
+            for m in matrices:
+                lane.copy(buffer, m.device_payload(lane), m.storage_bytes, dst_offset=offset)
+                offset += m.storage_bytes
+        except BaseException:
+            buffer.dispose()
+            raise
+        return cls.from_device(lane, buffer, first.ggml_type, sum(m.output_width for m in matrices), first.input_width)
+
     @property
     def storage_bytes(self) -> int:
         return int(self._payload.size) if self._payload is not None else self._storage_bytes

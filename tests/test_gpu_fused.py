@@ -157,3 +157,36 @@ def test_argument_checks(lane):
         odd.forward_fused(lane, x, pre_op=PRE_NONE)                                # three Q8_0 blocks per row
     m.dispose()
     odd.dispose()
+
+
+@pytest.mark.parametrize("typ", [GGML_Q8_0, GGML_Q4_K, GGML_Q6_K, GGML_IQ2_S])
+def test_stacked_gate_and_up_make_a_two_launch_feed_forward(lane, typ):
+    width, ffn = 1024, 2816 if typ == GGML_Q8_0 else 2560
+    rng = np.random.default_rng(31)
+    hidden = (rng.standard_normal(width) * 2).astype(np.float32)
+    attn = rng.standard_normal(width).astype(np.float32)
+    gamma = rng.uniform(0.5, 1.5, width).astype(np.float32)
+    gate, up, down = _matrix(typ, ffn, width, 1), _matrix(typ, ffn, width, 2), _matrix(typ, width, ffn, 3)
+    hb, ab, gb = lane.upload_raw(hidden), lane.upload_raw(attn), lane.upload_raw(gamma)
+    # three launches, separate gate and up
+    stream, normed = lane.allocate(width), lane.allocate(width)
+    g = gate.forward_fused(lane, hb, pre_op=PRE_RMS_NORM, x2=ab, norm_weight=gb, epsilon=EPS, x_out=normed, sum_out=stream)
+    u = up.forward(lane, normed, None)
+    down.forward_fused(lane, g, pre_op=PRE_SILU_MULTIPLY, x2=u, addend=stream, out=stream)
+    want = lane.read(stream, count=width)
+    # two launches: gate and up stacked; the down projection reads the two halves of one output
+    both = HipQuantizedMatrix.stacked(lane, [gate, up])
+    assert (both.output_width, both.input_width, both.storage_bytes) == (2 * ffn, width, gate.storage_bytes + up.storage_bytes)
+    stream2 = lane.allocate(width)
+    launches = lane.counters()["kernel_launches"]
+    gu = both.forward_fused(lane, hb, pre_op=PRE_RMS_NORM, x2=ab, norm_weight=gb, epsilon=EPS, sum_out=stream2)
+    assert np.array_equal(_bits(lane.read(gu, count=ffn)), _bits(lane.read(g, count=ffn)))
+    assert np.array_equal(_bits(lane.read(gu, count=ffn, offset=4 * ffn)), _bits(lane.read(u, count=ffn)))
+    up_half = gu.view(4 * ffn, 4 * ffn)
+    down.forward_fused(lane, gu, pre_op=PRE_SILU_MULTIPLY, x2=up_half, addend=stream2, out=stream2)
+    assert lane.counters()["kernel_launches"] - launches == 2
+    assert np.array_equal(_bits(lane.read(stream2, count=width)), _bits(want))
+    with pytest.raises(ValueError):
+        HipQuantizedMatrix.stacked(lane, [gate, down])
+    for m in (gate, up, down, both):
+        m.dispose()
