@@ -43,6 +43,7 @@ internal static unsafe partial class NnHipNative
         internal nint X; internal nint X2; internal nint NormWeight; internal nint XOut; internal nint SumOut;
         internal nint W; internal nint Bias; internal nint Addend; internal nint Y;
         internal int InW; internal int OutW;
+        internal nint LoraZ; internal nint LoraB; internal int LoraRank; internal float LoraScale;
     }
 
     [LibraryImport(Library)] internal static partial uint nnhip_abi_version();
@@ -73,6 +74,8 @@ internal static unsafe partial class NnHipNative
     [LibraryImport(Library)] internal static partial int nnhip_add_rms_norm(nint lane, nint destination, nint residual, nint weight, nint output, int rows, int width, int inputStride, float epsilon);
     [LibraryImport(Library)] internal static partial int nnhip_silu_multiply(nint lane, nint gate, nint up, nint output, int length);
     [LibraryImport(Library)] internal static partial int nnhip_add_in_place(nint lane, nint destination, nint source, int length);
+    [LibraryImport(Library)] internal static partial int nnhip_lora_a(nint lane, nint x, nint a, nint z, int rows, int width, int rank);
+    [LibraryImport(Library)] internal static partial int nnhip_lora_b(nint lane, nint z, nint b, nint y, int rows, int output, int rank, float scale);
     [LibraryImport(Library)] internal static partial int nnhip_event_create(nint lane, out nint evt);
     [LibraryImport(Library)] internal static partial int nnhip_event_destroy(nint lane, nint evt);
     [LibraryImport(Library)] internal static partial int nnhip_event_record(nint lane, nint evt);

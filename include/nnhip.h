@@ -68,7 +68,7 @@ enum {
     NNHIP_OP_UPLOAD, NNHIP_OP_DOWNLOAD, NNHIP_OP_COPY, NNHIP_OP_SYNCHRONIZE, NNHIP_OP_DEQUANTIZE,
     NNHIP_OP_MATVEC, NNHIP_OP_MATVEC_BATCH, NNHIP_OP_MATMUL_BF16, NNHIP_OP_EVENT, NNHIP_OP_GRAPH,
     NNHIP_OP_DEVICE_QUERY, NNHIP_OP_FILL, NNHIP_OP_RMS_NORM, NNHIP_OP_SILU_MULTIPLY, NNHIP_OP_ADD_IN_PLACE,
-    NNHIP_OP_MATVEC_FUSED
+    NNHIP_OP_MATVEC_FUSED, NNHIP_OP_LORA
 };
 
 /* Same field order as the reference's NativeErrorInfo (CudaNativeGateway.cs:1360-1371). */
@@ -229,8 +229,11 @@ NNHIP_API int nnhip_add_in_place(void* lane, float* destination, const float* so
  *   pre_op NNHIP_PRE_SILU_MULTIPLY  v = x * sigmoid(x) * x2 (gate, up); replaces q35a_silu_multiply followed by the
  *                                   down projection; x_out (may be null) receives v;
  *   pre_op NNHIP_PRE_NONE           v = x;
- *   then  y[o] = addend[o] + (bias[o] + sum_k v[k] * w[o, k]); addend may be null, and may be y itself (the
- *   residual stream: replaces q35a_add_in_place after the down projection).  bias may be null.
+ *   then  y[o] = addend[o] + ((bias[o] + sum_k v[k] * w[o, k]) + lora_scale * sum_r lora_z[r] * lora_b[o, r]);
+ *   the low-rank term is the fused adapter branch of q35l_*_sg16_lora (NNtrain.Arc/Kernels/qwen35_linear_fast.cl:
+ *   217-275; Matrix.ForwardFusedLora, Qwen35QuantizedModel.cs:1387) and is bit-identical to nnhip_lora_b applied to
+ *   the plain result; addend may be null, and may be y itself (the residual stream: replaces q35a_add_in_place after
+ *   the down projection).  bias may be null.
  * The mat-vec part is bit-identical to nnhip_quant_matvec on the same v.  x, x2, norm_weight hold in_w floats;
  * x_out and sum_out must not overlap x or x2 (every workgroup reads those while workgroup 0 writes).  Q8_0 rows with
  * an odd number of blocks are not covered (NNHIP_ERR_INVALID_ARGUMENT).  struct_size = sizeof of this structure.
@@ -253,9 +256,20 @@ typedef struct nnhip_fused_matvec_desc {
     float* y;
     int32_t in_w;
     int32_t out_w;
+    const float* lora_z;        /* low-rank branch (null / 0 for none): lora_rank floats, z = A x of the adapter       */
+    const float* lora_b;        /* [out_w, lora_rank] FP32                                                             */
+    int32_t lora_rank;
+    float lora_scale;
 } nnhip_fused_matvec_desc;
 
 NNHIP_API int nnhip_quant_matvec_fused(void* lane, const nnhip_fused_matvec_desc* desc);
+
+/* Low-rank adapter halves.  z[t, r] = sum_j x[t, j] * a[r, j] (q35l_lora_a_coop, NNtrain.Arc/Kernels/qwen35_lora.cl:
+ * 2-11: 128 lane-strided fused multiply-add chains, halving tree) and y[t, o] += scale * sum_r z[t, r] * b[o, r]
+ * (q35l_lora_b, qwen35_lora.cl:68-74).  Asynchronous. */
+NNHIP_API int nnhip_lora_a(void* lane, const float* x, const float* a, float* z, int rows, int width, int rank);
+NNHIP_API int nnhip_lora_b(void* lane, const float* z, const float* b, float* y, int rows, int output, int rank,
+                           float scale);
 
 /* --- timing and replay --------------------------------------------------------------------------------------- */
 

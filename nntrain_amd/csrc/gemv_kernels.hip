@@ -56,6 +56,10 @@ struct MatvecArgs {
     float* sum_out;        // RMSNorm: where x + residual is stored (or null)
     const float* addend;   // y = addend + (bias + W x) (or null)
     float epsilon;
+    const float* lora_z;   // low-rank branch: y += lora_scale * sum_r lora_z[r] * lora_b[o, r] before the addend
+    const float* lora_b;
+    int lora_rank;         // 0: no low-rank branch
+    float lora_scale;
 };
 
 enum : int { kPreNone = 0, kPreRmsNorm = 1, kPreSiluMultiply = 2 };
@@ -675,7 +679,14 @@ void matvec_rowstep_kernel(MatvecArgs a, const float* __restrict__ bias)
             const int j = i / rs;
             const int row = (first_held + j * stride) * rs + (i - j * rs);
             if (row < a.out_w) {
-                y[row] = a.addend ? a.addend[row] + ybuf[i] : ybuf[i];
+                float v = ybuf[i];
+                if (a.lora_rank > 0) {      // the branch of q35l_*_sg16_lora (NNtrain.Arc/Kernels/qwen35_linear_fast.cl:262-268)
+                    const float* br = a.lora_b + static_cast<size_t>(row) * a.lora_rank;
+                    float sum = 0.0f;
+                    for (int r = 0; r < a.lora_rank; ++r) sum = fmaf(a.lora_z[r], br[r], sum);
+                    v = v + a.lora_scale * sum;
+                }
+                y[row] = a.addend ? a.addend[row] + v : v;
             }
         }
         held = 0;
@@ -1115,6 +1126,10 @@ hipError_t launch_matvec_fused(Lane* lane, const nnhip_fused_matvec_desc& d)
     a.sum_out = d.sum_out;
     a.addend = d.addend;
     a.epsilon = d.epsilon;
+    a.lora_z = d.lora_z;
+    a.lora_b = d.lora_b;
+    a.lora_rank = d.lora_rank;
+    a.lora_scale = d.lora_scale;
     switch (d.pre_op) {
     case NNHIP_PRE_NONE: return launch_fused_of<kPreNone>(lane, d.ggml_type, a);
     case NNHIP_PRE_RMS_NORM: return launch_fused_of<kPreRmsNorm>(lane, d.ggml_type, a);

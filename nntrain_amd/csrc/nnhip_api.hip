@@ -470,6 +470,10 @@ int nnhip_quant_matvec_fused(void* handle, const nnhip_fused_matvec_desc* d)
     default:
         return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0, "unknown pre_op %u", d->pre_op);
     }
+    if (d->lora_rank < 0 || (d->lora_rank > 0 && (!d->lora_z || !d->lora_b)) || (d->lora_rank == 0 && (d->lora_z || d->lora_b)))
+        return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0, "lora_z and lora_b go with a positive lora_rank, and only with one");
+    if (d->lora_rank > 0 && !std::isfinite(d->lora_scale))
+        return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0, "lora_scale must be finite");
     const size_t xbytes = static_cast<size_t>(d->in_w) * sizeof(float);
     auto overlaps = [&](const float* out, const float* in) {
         if (!out || !in) return false;
@@ -482,6 +486,32 @@ int nnhip_quant_matvec_fused(void* handle, const nnhip_fused_matvec_desc* d)
         return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0, "x_out and sum_out must not overlap the inputs or each other");
     hipError_t e = launch_matvec_fused(lane, *d);
     if (e != hipSuccess) return hip_fail(e, op, lane->device, "fused mat-vec launch");
+    lane->counters.kernel_launches += 1;
+    return NNHIP_OK;
+}
+
+int nnhip_lora_a(void* handle, const float* x, const float* a, float* z, int rows, int width, int rank)
+{
+    NNHIP_LANE(handle, NNHIP_OP_LORA)
+    if (!x || !a || !z || rows < 1 || width < 1 || rank < 1)
+        return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_LORA, lane->device, 0, "pointers must be non-null and rows, width, rank positive");
+    if (static_cast<int64_t>(rows) * rank > 0x7fffffff)
+        return fail(NNHIP_ERR_TOO_LARGE, NNHIP_OP_LORA, lane->device, 0, "rows * rank exceeds one launch");
+    hipError_t e = launch_lora_a(lane, x, a, z, rows, width, rank);
+    if (e != hipSuccess) return hip_fail(e, NNHIP_OP_LORA, lane->device, "adapter A launch");
+    lane->counters.kernel_launches += 1;
+    return NNHIP_OK;
+}
+
+int nnhip_lora_b(void* handle, const float* z, const float* b, float* y, int rows, int output, int rank, float scale)
+{
+    NNHIP_LANE(handle, NNHIP_OP_LORA)
+    if (!z || !b || !y || rows < 1 || output < 1 || rank < 1)
+        return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_LORA, lane->device, 0, "pointers must be non-null and rows, output, rank positive");
+    if (static_cast<int64_t>(rows) * output > 0x7fffffff)
+        return fail(NNHIP_ERR_TOO_LARGE, NNHIP_OP_LORA, lane->device, 0, "rows * output exceeds one launch");
+    hipError_t e = launch_lora_b(lane, z, b, y, rows, output, rank, scale);
+    if (e != hipSuccess) return hip_fail(e, NNHIP_OP_LORA, lane->device, "adapter B launch");
     lane->counters.kernel_launches += 1;
     return NNHIP_OK;
 }

@@ -1,5 +1,6 @@
 // FP32 row operations that sit on either side of the quantized mat-vec in the decode path: RMSNorm, residual add +
-// RMSNorm, SiLU(gate) * up, in-place add (NNtrain.Arc/Kernels/qwen35_attention.cl:9-78).
+// RMSNorm, SiLU(gate) * up, in-place add (NNtrain.Arc/Kernels/qwen35_attention.cl:9-78), and the two halves of a low-rank
+// adapter (NNtrain.Arc/Kernels/qwen35_lora.cl:2-11,68-74).
 //
 // The reductions follow the reference's order, so a result has the bits of a plain CPU restatement: lane t of 128 adds
 // x[t]^2, x[t+128]^2, ... in that order, the 128 partial sums meet in a halving tree (64, 32, .. 1), and
@@ -67,7 +68,51 @@ __global__ __launch_bounds__(256) void add_in_place_kernel(float* destination, c
     if (i < length) destination[i] += source[i];
 }
 
+// z[t, r] = sum_j x[t, j] * a[r, j]: one workgroup per (t, r); 128 lane-strided fused multiply-add chains, then the
+// halving tree (NNtrain.Arc/Kernels/qwen35_lora.cl:2-11).
+__global__ __launch_bounds__(kNormLanes) void lora_a_kernel(const float* x, const float* a, float* z, int width, int rank)
+{
+    __shared__ float partial[kNormLanes];
+    const int item = blockIdx.x, tid = threadIdx.x;
+    const int t = item / rank, r = item - t * rank;
+    const float* xr = x + static_cast<size_t>(t) * width;
+    const float* ar = a + static_cast<size_t>(r) * width;
+    float sum = 0.0f;
+    for (int j = tid; j < width; j += kNormLanes) sum = fmaf(xr[j], ar[j], sum);
+    partial[tid] = sum;
+    __syncthreads();
+    for (int s = kNormLanes / 2; s > 0; s >>= 1) {
+        if (tid < s) partial[tid] += partial[tid + s];
+        __syncthreads();
+    }
+    if (tid == 0) z[item] = partial[0];
+}
+
+// y[t, o] += scale * sum_r z[t, r] * b[o, r] (qwen35_lora.cl:68-74).
+__global__ __launch_bounds__(256) void lora_b_kernel(const float* z, const float* b, float* y, int rows, int output, int rank,
+                                                     float scale)
+{
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= rows * output) return;
+    const int t = i / output, o = i - t * output;
+    float sum = 0.0f;
+    for (int r = 0; r < rank; ++r) sum = fmaf(z[t * rank + r], b[static_cast<size_t>(o) * rank + r], sum);
+    y[i] = y[i] + scale * sum;
+}
+
 }  // namespace
+
+hipError_t launch_lora_a(Lane* lane, const float* x, const float* a, float* z, int rows, int width, int rank)
+{
+    hipLaunchKernelGGL(lora_a_kernel, dim3(rows * rank), dim3(kNormLanes), 0, lane->stream, x, a, z, width, rank);
+    return hipGetLastError();
+}
+
+hipError_t launch_lora_b(Lane* lane, const float* z, const float* b, float* y, int rows, int output, int rank, float scale)
+{
+    hipLaunchKernelGGL(lora_b_kernel, dim3((rows * output + 255) / 256), dim3(256), 0, lane->stream, z, b, y, rows, output, rank, scale);
+    return hipGetLastError();
+}
 
 hipError_t launch_rms_norm(Lane* lane, float* io, const float* residual, const float* weight, float* output, int rows,
                            int width, int input_stride, float epsilon)

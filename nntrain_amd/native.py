@@ -47,7 +47,8 @@ class FusedMatvecDesc(Structure):
     _fields_ = [("struct_size", c_uint32), ("ggml_type", c_uint32), ("pre_op", c_uint32), ("epsilon", c_float),
                 ("x", c_void_p), ("x2", c_void_p), ("norm_weight", c_void_p), ("x_out", c_void_p), ("sum_out", c_void_p),
                 ("w", c_void_p), ("bias", c_void_p), ("addend", c_void_p), ("y", c_void_p), ("in_w", c_int32),
-                ("out_w", c_int32)]
+                ("out_w", c_int32), ("lora_z", c_void_p), ("lora_b", c_void_p), ("lora_rank", c_int32),
+                ("lora_scale", c_float)]
 
 
 PRE_NONE, PRE_RMS_NORM, PRE_SILU_MULTIPLY = 0, 1, 2
@@ -82,6 +83,8 @@ PROTOTYPES = {
     "nnhip_add_rms_norm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float]),
     "nnhip_silu_multiply": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int]),
     "nnhip_add_in_place": (c_int, [c_void_p, c_void_p, c_void_p, c_int]),
+    "nnhip_lora_a": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int]),
+    "nnhip_lora_b": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float]),
     "nnhip_event_create": (c_int, [c_void_p, POINTER(c_void_p)]),
     "nnhip_event_destroy": (c_int, [c_void_p, c_void_p]),
     "nnhip_event_record": (c_int, [c_void_p, c_void_p]),

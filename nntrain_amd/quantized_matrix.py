@@ -145,10 +145,18 @@ class HipQuantizedMatrix:
     def forward_fused(self, lane: HipExecutionLane, x: HipBuffer, *, pre_op: int = PRE_NONE, x2: HipBuffer | None = None,
                       norm_weight: HipBuffer | None = None, epsilon: float = 0.0, x_out: HipBuffer | None = None,
                       sum_out: HipBuffer | None = None, bias: HipBuffer | None = None, addend: HipBuffer | None = None,
-                      out: HipBuffer | None = None) -> HipBuffer:
+                      out: HipBuffer | None = None, lora_z: HipBuffer | None = None, lora_b: HipBuffer | None = None,
+                      lora_rank: int = 0, lora_scale: float = 0.0) -> HipBuffer:
         """One decode mat-vec with its neighbours fused into the launch: v = RMSNorm(x + x2) * norm_weight
         (PRE_RMS_NORM; x2 optional) or SiLU(x) * x2 (PRE_SILU_MULTIPLY) or x, then y = addend + bias + W v.
-        x_out / sum_out receive v and x + x2 when given.  `out` may be `addend` (the residual stream updated in place)."""
+        x_out / sum_out receive v and x + x2 when given.  `out` may be `addend` (the residual stream updated in place).
+        lora_z [rank] and lora_b [out, rank] add the low-rank adapter branch lora_scale * z . b^T before the addend
+        (Matrix.ForwardFusedLora, Qwen35QuantizedModel.cs:1387)."""
+        if lora_rank < 0:
+            raise ValueError("lora_rank must not be negative.")
+        if lora_rank > 0 and (lora_z is None or lora_b is None or lora_z.nbytes < 4 * lora_rank
+                              or lora_b.nbytes < 4 * lora_rank * self.output_width):
+            raise ValueError("LoRA buffers do not match lora_rank.")
         n_in, n_out = 4 * self.input_width, 4 * self.output_width
         for name, buf, need in (("x", x, n_in), ("x2", x2, n_in), ("norm_weight", norm_weight, n_in), ("x_out", x_out, n_in),
                                 ("sum_out", sum_out, n_in), ("bias", bias, n_out), ("addend", addend, n_out), ("out", out, n_out)):
@@ -160,7 +168,8 @@ class HipQuantizedMatrix:
         desc = FusedMatvecDesc(struct_size=ctypes.sizeof(FusedMatvecDesc), ggml_type=self.ggml_type, pre_op=pre_op,
                                epsilon=epsilon, x=ptr(x), x2=ptr(x2), norm_weight=ptr(norm_weight), x_out=ptr(x_out),
                                sum_out=ptr(sum_out), w=ptr(w), bias=ptr(bias), addend=ptr(addend), y=ptr(y),
-                               in_w=self.input_width, out_w=self.output_width)
+                               in_w=self.input_width, out_w=self.output_width, lora_z=ptr(lora_z), lora_b=ptr(lora_b),
+                               lora_rank=lora_rank, lora_scale=lora_scale)
         try:
             check(lane._lib.nnhip_quant_matvec_fused(lane._handle, ctypes.byref(desc)), "quant_matvec_fused")
         except BaseException:

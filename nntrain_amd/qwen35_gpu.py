@@ -90,3 +90,33 @@ def add_in_place(lane: HipExecutionLane, destination: HipBuffer, source: HipBuff
     _validate_buffer(source, length, "source")
     check(lane._lib.nnhip_add_in_place(lane._handle, c_void_p(destination._require()), c_void_p(source._require()),
                                        length), "add_in_place")
+
+
+def lora_project_a(lane: HipExecutionLane, x: HipBuffer, a: HipBuffer, rows: int, width: int, rank: int) -> HipBuffer:
+    """z[rows, rank] = x . a^T, the first half of a low-rank adapter (q35l_lora_a_coop)."""
+    _positive(rows, "rows")
+    _positive(width, "width")
+    _positive(rank, "rank")
+    _validate_buffer(x, rows * width, "x")
+    _validate_buffer(a, rank * width, "a")
+    z = lane.allocate(rows * rank)
+    try:
+        check(lane._lib.nnhip_lora_a(lane._handle, c_void_p(x._require()), c_void_p(a._require()), c_void_p(z._require()),
+                                     rows, width, rank), "lora_a")
+        return z
+    except BaseException:
+        z.dispose()
+        raise
+
+
+def lora_apply_b(lane: HipExecutionLane, z: HipBuffer, b: HipBuffer, y: HipBuffer, rows: int, output: int, rank: int,
+                 scale: float) -> None:
+    """y[rows, output] += scale * z . b^T, the second half (q35l_lora_b)."""
+    _positive(rows, "rows")
+    _positive(output, "output")
+    _positive(rank, "rank")
+    _validate_buffer(z, rows * rank, "z")
+    _validate_buffer(b, output * rank, "b")
+    _validate_buffer(y, rows * output, "y")
+    check(lane._lib.nnhip_lora_b(lane._handle, c_void_p(z._require()), c_void_p(b._require()), c_void_p(y._require()),
+                                 rows, output, rank, scale), "lora_b")

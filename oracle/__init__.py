@@ -60,6 +60,8 @@ def lib() -> ctypes.CDLL:
         L.oracle_rms_norm_serial.argtypes = [vp, vp, vp, ci, ci, cf]
         L.oracle_silu_multiply.argtypes = [vp, vp, vp, ci]
         L.oracle_add_in_place.argtypes = [vp, vp, ci]
+        L.oracle_lora_a.argtypes = [vp, vp, vp, ci, ci, ci]
+        L.oracle_lora_b.argtypes = [vp, vp, vp, ci, ci, ci, cf]
         _lib = L
     return _lib
 
@@ -321,6 +323,23 @@ def add_in_place(destination, source) -> np.ndarray:
     dest, source = _f32(destination).copy(), _f32(source)
     lib().oracle_add_in_place(_ptr(dest), _ptr(source), dest.size)
     return dest
+
+
+def lora_a(x, a, rows: int, width: int, rank: int) -> np.ndarray:
+    """q35l_lora_a_coop: z[rows, rank] = x[rows, width] . a[rank, width]^T."""
+    x, a = _f32(x), _f32(a)
+    assert x.size == rows * width and a.size == rank * width
+    z = np.empty(rows * rank, dtype=np.float32)
+    lib().oracle_lora_a(_ptr(x), _ptr(a), _ptr(z), rows, width, rank)
+    return z.reshape(rows, rank)
+
+
+def lora_b(z, b, y, rows: int, output: int, rank: int, scale: float) -> np.ndarray:
+    """q35l_lora_b: returns y[rows, output] + scale * z[rows, rank] . b[output, rank]^T."""
+    z, b, out = _f32(z), _f32(b), _f32(y).copy()
+    assert z.size == rows * rank and b.size == output * rank and out.size == rows * output
+    lib().oracle_lora_b(_ptr(z), _ptr(b), _ptr(out), rows, output, rank, scale)
+    return out.reshape(rows, output)
 
 
 def np_tree_sum_of_squares(x: np.ndarray) -> np.float32:

@@ -9,10 +9,14 @@
  *   silu_multiply    qwen35_attention.cl:9-14,38-43: gate * sigmoid(gate) * up with the two-sided sigmoid
  *   add_in_place     qwen35_attention.cl:45-49
  *   rms_norm_serial  NNtrain.Core/Modules/Qwen35Math.cs:19-35 (the CPU statement: one running sum per row)
+ *   lora_a           NNtrain.Arc/Kernels/qwen35_lora.cl:2-11 (q35l_lora_a_coop): z[t, r] = sum_j x[t, j] a[r, j] as 128
+ *                    lane-strided fma chains and the halving tree
+ *   lora_b           qwen35_lora.cl:68-74 (q35l_lora_b): y[t, o] += scale * (fma chain over r of z[t, r] b[o, r])
  *
  * Pinning (tests/test_oracle_norm.py): the reference's own vector Qwen35Math.RmsNorm([3,4,-3,-4],[2,.5],0,2) and the
  * zero row (Qwen35MathTests.cs:10-12), the sigmoid limits of Qwen35MathTests.cs:29-37, closed forms (constant rows,
  * powers of two), an independent pure-Python statement of the 128-lane tree on inputs whose sum depends on the order,
+ * exact rational arithmetic (fractions) on small low-rank cases,
  * and float64 evaluation within 2e-5 (the reference's GPU-vs-CPU bound, Qwen35GpuAttentionTests.cs:26-28).
  */
 #include <math.h>
@@ -82,4 +86,30 @@ ORACLE_EXPORT void oracle_silu_multiply(const float* gate, const float* up, floa
 ORACLE_EXPORT void oracle_add_in_place(float* destination, const float* source, int length)
 {
     for (int i = 0; i < length; ++i) destination[i] += source[i];
+}
+
+ORACLE_EXPORT void oracle_lora_a(const float* x, const float* a, float* z, int rows, int width, int rank)
+{
+    for (int t = 0; t < rows; ++t)
+        for (int r = 0; r < rank; ++r) {
+            float partial[128];
+            for (int lane = 0; lane < 128; ++lane) {
+                float sum = 0.0f;
+                for (int j = lane; j < width; j += 128) sum = fmaf(x[(long)t * width + j], a[(long)r * width + j], sum);
+                partial[lane] = sum;
+            }
+            for (int s = 64; s > 0; s >>= 1)
+                for (int lane = 0; lane < s; ++lane) partial[lane] += partial[lane + s];
+            z[t * rank + r] = partial[0];
+        }
+}
+
+ORACLE_EXPORT void oracle_lora_b(const float* z, const float* b, float* y, int rows, int output, int rank, float scale)
+{
+    for (int t = 0; t < rows; ++t)
+        for (int o = 0; o < output; ++o) {
+            float sum = 0.0f;
+            for (int r = 0; r < rank; ++r) sum = fmaf(z[t * rank + r], b[(long)o * rank + r], sum);
+            y[(long)t * output + o] += scale * sum;
+        }
 }

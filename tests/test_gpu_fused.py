@@ -190,3 +190,49 @@ def test_stacked_gate_and_up_make_a_two_launch_feed_forward(lane, typ):
         HipQuantizedMatrix.stacked(lane, [gate, down])
     for m in (gate, up, down, both):
         m.dispose()
+
+
+@pytest.mark.parametrize("typ", [GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_IQ2_S, GGML_IQ3_S, GGML_Q8_0])
+def test_fused_projection_matches_separate_base_and_lora_bitwise(lane, typ):
+    # the shapes, value ranges and scales of Qwen35InferenceFusedLoraTests.cs:35-63 (decode rows only)
+    for in_w, out_w, rank in ((256, 5, 3), (512, 7, 8), (5120, 33, 8), (17408, 9, 3)):
+        rng = np.random.default_rng(975 + in_w + typ)
+        val = lambda n: rng.uniform(-0.4, 0.4, n).astype(np.float32)          # noqa: E731
+        m = _matrix(typ, out_w, in_w, 6)
+        m.device_payload(lane)
+        x, bias, a, b = (lane.upload_raw(val(n)) for n in (in_w, out_w, rank * in_w, out_w * rank))
+        z = qwen35_gpu.lora_project_a(lane, x, a, 1, in_w, rank)
+        want_z = oracle.lora_a(lane.read(x, count=in_w), lane.read(a, count=rank * in_w), 1, in_w, rank)
+        assert np.array_equal(_bits(lane.read(z, count=rank)), _bits(want_z.ravel()))
+        for scale in (2.0, -0.75, 0.0):
+            sentinel = np.full(out_w + 2, np.nan, dtype=np.float32)
+            baseline, fused = lane.upload_raw(sentinel), lane.upload_raw(sentinel)
+            before = lane.counters()
+            m.forward(lane, x, bias, out=baseline)
+            qwen35_gpu.lora_apply_b(lane, z, b, baseline, 1, out_w, rank, scale)
+            m.forward_fused(lane, x, bias=bias, out=fused, lora_z=z, lora_b=b, lora_rank=rank, lora_scale=scale)
+            after = lane.counters()
+            assert (before["h2d_bytes"], before["d2h_bytes"], before["allocated_bytes"]) == \
+                   (after["h2d_bytes"], after["d2h_bytes"], after["allocated_bytes"])
+            e, g = lane.read(baseline, count=out_w + 2), lane.read(fused, count=out_w + 2)
+            assert np.all(np.isfinite(g[:out_w])) and np.array_equal(_bits(e[:out_w]), _bits(g[:out_w]))
+            assert np.all(np.isnan(e[out_w:])) and np.all(np.isnan(g[out_w:]))
+            # the low-rank step itself against the oracle
+            plain = lane.read(m.forward(lane, x, bias), count=out_w)
+            want = oracle.lora_b(want_z, lane.read(b, count=out_w * rank), plain, 1, out_w, rank, scale)
+            assert np.array_equal(_bits(e[:out_w]), _bits(want.ravel()))
+        m.dispose()
+
+
+def test_lora_argument_checks(lane):
+    m = _matrix(GGML_Q4_K, 8, 256, 1)
+    x, z, b = lane.allocate(256), lane.allocate(4), lane.allocate(32)
+    with pytest.raises(ValueError):
+        m.forward_fused(lane, x, lora_z=z, lora_b=b, lora_rank=8)           # z too small for the rank
+    with pytest.raises(NnHipError):
+        m.forward_fused(lane, x, lora_z=z, lora_b=b, lora_rank=0)           # buffers without a rank
+    with pytest.raises(NnHipError):
+        m.forward_fused(lane, x, lora_z=z, lora_b=b, lora_rank=4, lora_scale=float("inf"))
+    with pytest.raises(ValueError):
+        qwen35_gpu.lora_project_a(lane, x, x, 1, 256, 2)
+    m.dispose()

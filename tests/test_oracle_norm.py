@@ -84,3 +84,63 @@ def test_silu_limits_and_float64():
     got = oracle.silu_multiply(g, u)
     assert np.abs(got - want).max() <= 2e-5
     assert (np.abs(got - want) / np.maximum(np.abs(want), 1e-30)).max() < 1e-6
+
+
+def _round_to_f32(q):
+    """Correctly rounded (nearest, ties to even) float32 of a fractions.Fraction, via integer arithmetic only."""
+    from fractions import Fraction
+    if q == 0:
+        return np.float32(0.0)
+    sign = -1 if q < 0 else 1
+    q = abs(q)
+    e = q.numerator.bit_length() - q.denominator.bit_length()
+    if Fraction(2) ** e > q:
+        e -= 1                                        # 2^e <= q < 2^(e+1)
+    e = max(e, -126)                                  # subnormal range keeps the exponent of 2^-126
+    scaled = q / Fraction(2) ** (e - 23)              # mantissa units
+    n, rem = divmod(scaled.numerator, scaled.denominator)
+    twice = 2 * rem
+    if twice > scaled.denominator or (twice == scaled.denominator and n % 2 == 1):
+        n += 1
+    return np.float32(sign * float(Fraction(n) * Fraction(2) ** (e - 23)))
+
+
+def _fma32(a, b, c):
+    from fractions import Fraction
+    return _round_to_f32(Fraction(float(a)) * Fraction(float(b)) + Fraction(float(c)))
+
+
+def test_lora_halves_against_exact_rational_arithmetic():
+    rng = np.random.default_rng(12)
+    rows, width, rank, output = 2, 300, 3, 5
+    x = rng.uniform(-0.4, 0.4, rows * width).astype(np.float32)
+    a = rng.uniform(-0.4, 0.4, rank * width).astype(np.float32)
+    z = oracle.lora_a(x, a, rows, width, rank)
+    for t in range(rows):
+        for r in range(rank):
+            partial = []
+            for lane in range(128):
+                s = np.float32(0.0)
+                for j in range(lane, width, 128):
+                    s = _fma32(x[t * width + j], a[r * width + j], s)
+                partial.append(s)
+            stride = 64
+            while stride:
+                for lane in range(stride):
+                    partial[lane] = np.float32(partial[lane] + partial[lane + stride])
+                stride >>= 1
+            assert bits(z[t, r]) == bits(partial[0])
+    b = rng.uniform(-0.4, 0.4, output * rank).astype(np.float32)
+    y = rng.uniform(-1, 1, rows * output).astype(np.float32)
+    for scale in (2.0, -0.75, 0.0):
+        got = oracle.lora_b(z, b, y, rows, output, rank, scale)
+        for t in range(rows):
+            for o in range(output):
+                s = np.float32(0.0)
+                for r in range(rank):
+                    s = _fma32(z[t, r], b[o * rank + r], s)
+                want = np.float32(y[t * output + o] + np.float32(np.float32(scale) * s))
+                assert bits(got[t, o]) == bits(want)
+    # and against float64
+    z64 = x.reshape(rows, width).astype(np.float64) @ a.reshape(rank, width).astype(np.float64).T
+    assert np.abs(z - z64).max() < 1e-5
