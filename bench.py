@@ -414,6 +414,121 @@ def run_ffn(args, lane, nn, oracle):
     return out
 
 
+def run_decode_loop(args, lane, nn, oracle):
+    """Per-token timing of the decode loop (nntrain_amd.decoder) over a synthetic llama-style GGUF file written to a
+    temporary directory and loaded through the streaming loader: 4 layers of hidden 5120 / feed-forward 17408 / 40 query
+    and 8 key-value heads of 128 in Q4_K, vocabulary 32000.  Three forms of the same step, same bits: one launch per
+    operation (the reference's sequence), the fused launches, and the fused launches replayed from a HIP graph."""
+    import struct
+    import tempfile
+    from nntrain_amd import synth
+    from nntrain_amd.decoder import QuantizedDecoder
+    layers, emb, ffn, heads, kv, hw, vocab, typ = 4, 5120, 17408, 40, 8, 128, 32000, nn.GGML_Q4_K
+
+    def kvp(key, value):
+        if isinstance(value, str):
+            b = value.encode()
+            return key, 8, struct.pack("<Q", len(b)) + b
+        return (key, 6, struct.pack("<f", value)) if isinstance(value, float) else (key, 4, struct.pack("<I", value))
+
+    tensors = []
+    rng = np.random.default_rng(8)
+
+    def mat(name, out_w, in_w, seed):
+        tensors.append((name, (in_w, out_w), typ, synth.matrix(typ, out_w, in_w, seed)))
+
+    def vec(name):
+        tensors.append((name, (emb,), 0, rng.uniform(0.5, 1.5, emb).astype(np.float32)))
+
+    mat("token_embd.weight", vocab, emb, 1)
+    for i in range(layers):
+        p = f"blk.{i}."
+        vec(p + "attn_norm.weight")
+        mat(p + "attn_q.weight", heads * hw, emb, 10 + i)
+        mat(p + "attn_k.weight", kv * hw, emb, 20 + i)
+        mat(p + "attn_v.weight", kv * hw, emb, 30 + i)
+        mat(p + "attn_output.weight", emb, heads * hw, 40 + i)
+        vec(p + "ffn_norm.weight")
+        mat(p + "ffn_gate.weight", ffn, emb, 50 + i)
+        mat(p + "ffn_up.weight", ffn, emb, 60 + i)
+        mat(p + "ffn_down.weight", emb, ffn, 70 + i)
+    vec("output_norm.weight")
+    mat("output.weight", vocab, emb, 2)
+    kvs = [kvp("general.architecture", "llama"), kvp("llama.block_count", layers), kvp("llama.embedding_length", emb),
+           kvp("llama.feed_forward_length", ffn), kvp("llama.attention.head_count", heads),
+           kvp("llama.attention.head_count_kv", kv), kvp("llama.attention.key_length", hw),
+           kvp("llama.attention.layer_norm_rms_epsilon", 1e-6)]
+
+    def s(x):
+        b = x.encode()
+        return struct.pack("<Q", len(b)) + b
+
+    out = {}
+    with tempfile.TemporaryDirectory() as tmp:
+        # GGUF v3, tensor data aligned to 32 bytes
+        offsets, cursor = [], 0
+        for _, _, _, payload in tensors:
+            offsets.append(cursor)
+            cursor = (cursor + payload.nbytes + 31) // 32 * 32
+        head = struct.pack("<IIQQ", 0x46554747, 3, len(tensors), len(kvs))
+        for k, t, v in kvs:
+            head += s(k) + struct.pack("<I", t) + v
+        for (name, shape, ttype, _), off in zip(tensors, offsets):
+            head += s(name) + struct.pack("<I", len(shape)) + b"".join(struct.pack("<Q", d) for d in shape) + struct.pack("<IQ", ttype, off)
+        data_start = (len(head) + 31) // 32 * 32
+        path = os.path.join(tmp, "synthetic.gguf")
+        with open(path, "wb") as f:
+            f.write(head + b"\0" * (data_start - len(head)))
+            for (_, _, _, payload), off in zip(tensors, offsets):
+                f.seek(data_start + off)
+                f.write(payload.tobytes())
+        file_bytes = os.path.getsize(path)
+        del tensors
+        t0 = time.perf_counter()
+        with nn.GgufReader(path) as reader:
+            plain = QuantizedDecoder(lane, reader, fused=False)
+            load_s = time.perf_counter() - t0
+            fused = QuantizedDecoder(lane, reader, fused=True)
+        lane.synchronize()
+    weight_bytes = plain.quantized_bytes - plain.embedding.storage_bytes      # streamed per token (the embedding is one row)
+    tokens = [3, 1000, 31999, 17, 4242, 9, 30000, 512]
+    ref = [lane.read(plain.forward_token(t), np.uint32, count=vocab) for t in tokens[:2]]
+    for t, r in zip(tokens[:2], ref):
+        if not np.array_equal(lane.read(fused.forward_token(t), np.uint32, count=vocab), r):
+            raise SystemExit("decode loop: fused and unfused logits differ bitwise")
+
+    def per_token(dec):
+        samples = []
+        for _ in range(5):
+            ms, _ = timed(lane, lambda: [dec.forward_token(t) for t in tokens], 1)
+            samples.append(ms / len(tokens))
+        return float(np.median(samples))
+
+    ms_plain, ms_fused = per_token(plain), per_token(fused)
+    fused.capture_graph()
+    if not np.array_equal(lane.read(fused.forward_token(tokens[0]), np.uint32, count=vocab), ref[0]):
+        raise SystemExit("decode loop: graph replay differs bitwise")
+    ms_graph = per_token(fused)
+    toks, timing = fused.generate(5, 16)
+    out = {"config": f"llama-style, {layers} layers, hidden {emb}, feed-forward {ffn}, heads {heads}/{kv} x {hw}, vocabulary {vocab}, Q4_K",
+           "gguf_file_bytes": file_bytes, "load_seconds_file_to_hbm": round(load_s, 2),
+           "weight_bytes_streamed_per_token": weight_bytes,
+           "ms_per_token": {"one_launch_per_operation": round(ms_plain, 4), "fused_launches": round(ms_fused, 4),
+                            "fused_launches_hip_graph": round(ms_graph, 4)},
+           "launches_per_token": {"one_launch_per_operation": 1 + 12 * layers + 2, "fused_launches": 1 + 5 * layers + 1},
+           "gb_per_s_fused_graph": round(weight_bytes / ms_graph / 1e6, 1),
+           "frac_of_8TBs_fused_graph": round(weight_bytes / ms_graph / 1e6 / HBM_PEAK_GBS, 4),
+           "greedy_generation_with_host_argmax": {"tokens": timing.generated_tokens,
+                                                  "first_token_ms": round(timing.first_token_milliseconds, 3),
+                                                  "decode_tokens_per_s": round(timing.decode_tokens_per_second, 1)},
+           "bitwise_equal": True}
+    log(f"[decode_loop] per token: {ms_plain * 1e3:.1f} us unfused, {ms_fused * 1e3:.1f} us fused, {ms_graph * 1e3:.1f} us fused + graph "
+        f"({weight_bytes / ms_graph / 1e6:.0f} GB/s); load {load_s:.1f} s for {file_bytes / 1e9:.2f} GB")
+    plain.dispose()
+    fused.dispose()
+    return out
+
+
 def run_prefill(args, lane, nn, oracle):
     """Q4_K 17408x5120 bf16-MFMA prefill mat-mul at M = 128, 256, 512, 2048 (BASELINE configs[3])."""
     from nntrain_amd import synth
@@ -462,7 +577,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", choices=["decode27b", "gemv", "prefill", "ffn", "all"], default="all")
+    ap.add_argument("--workload", choices=["decode27b", "gemv", "prefill", "ffn", "decode_loop", "all"], default="all")
     ap.add_argument("--mode", choices=["forward", "graph", "batch"], default="batch",
                     help="decode27b: one launch per matrix, the same captured in a HIP graph, or the batched entry point")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -485,6 +600,8 @@ def main():
         also["prefill_q4k_bf16_mfma"] = run_prefill(args, lane, nn, oracle)
     if args.workload in ("ffn", "all"):
         also["ffn_layer_half_fused_epilogues"] = run_ffn(args, lane, nn, oracle)
+    if args.workload in ("decode_loop", "all"):
+        also["decode_loop_gguf_file"] = run_decode_loop(args, lane, nn, oracle)
     if args.workload in ("decode27b", "all"):
         res = run_decode27b(args, lane, nn, oracle)
     else:

@@ -74,6 +74,7 @@ internal static unsafe partial class NnHipNative
     [LibraryImport(Library)] internal static partial int nnhip_add_rms_norm(nint lane, nint destination, nint residual, nint weight, nint output, int rows, int width, int inputStride, float epsilon);
     [LibraryImport(Library)] internal static partial int nnhip_silu_multiply(nint lane, nint gate, nint up, nint output, int length);
     [LibraryImport(Library)] internal static partial int nnhip_add_in_place(nint lane, nint destination, nint source, int length);
+    [LibraryImport(Library)] internal static partial int nnhip_first_token_attention(nint lane, nint v, nint output, int heads, int kvHeads, int headWidth);
     [LibraryImport(Library)] internal static partial int nnhip_lora_a(nint lane, nint x, nint a, nint z, int rows, int width, int rank);
     [LibraryImport(Library)] internal static partial int nnhip_lora_b(nint lane, nint z, nint b, nint y, int rows, int output, int rank, float scale);
     [LibraryImport(Library)] internal static partial int nnhip_event_create(nint lane, out nint evt);

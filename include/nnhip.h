@@ -68,7 +68,7 @@ enum {
     NNHIP_OP_UPLOAD, NNHIP_OP_DOWNLOAD, NNHIP_OP_COPY, NNHIP_OP_SYNCHRONIZE, NNHIP_OP_DEQUANTIZE,
     NNHIP_OP_MATVEC, NNHIP_OP_MATVEC_BATCH, NNHIP_OP_MATMUL_BF16, NNHIP_OP_EVENT, NNHIP_OP_GRAPH,
     NNHIP_OP_DEVICE_QUERY, NNHIP_OP_FILL, NNHIP_OP_RMS_NORM, NNHIP_OP_SILU_MULTIPLY, NNHIP_OP_ADD_IN_PLACE,
-    NNHIP_OP_MATVEC_FUSED, NNHIP_OP_LORA
+    NNHIP_OP_MATVEC_FUSED, NNHIP_OP_LORA, NNHIP_OP_ATTENTION
 };
 
 /* Same field order as the reference's NativeErrorInfo (CudaNativeGateway.cs:1360-1371). */
@@ -263,6 +263,13 @@ typedef struct nnhip_fused_matvec_desc {
 } nnhip_fused_matvec_desc;
 
 NNHIP_API int nnhip_quant_matvec_fused(void* lane, const nnhip_fused_matvec_desc* desc);
+
+/* out[h, :] = v[h / (heads / kv_heads), :] for h < heads: the result of causal grouped-query attention for the first
+ * token of a sequence (a single key has softmax weight 1 whatever the query), which lets a decode loop exercise every
+ * projection of a layer without a key/value cache (the attention core itself, Qwen35Gpu.AttentionStep,
+ * NNtrain.Core/Modules/Qwen35Gpu.Attention.cs:60-120, is outside this library).  heads must be a multiple of kv_heads.
+ * Asynchronous. */
+NNHIP_API int nnhip_first_token_attention(void* lane, const float* v, float* out, int heads, int kv_heads, int head_width);
 
 /* Low-rank adapter halves.  z[t, r] = sum_j x[t, j] * a[r, j] (q35l_lora_a_coop, NNtrain.Arc/Kernels/qwen35_lora.cl:
  * 2-11: 128 lane-strided fused multiply-add chains, halving tree) and y[t, o] += scale * sum_r z[t, r] * b[o, r]

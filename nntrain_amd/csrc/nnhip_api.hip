@@ -490,6 +490,19 @@ int nnhip_quant_matvec_fused(void* handle, const nnhip_fused_matvec_desc* d)
     return NNHIP_OK;
 }
 
+int nnhip_first_token_attention(void* handle, const float* v, float* out, int heads, int kv_heads, int head_width)
+{
+    NNHIP_LANE(handle, NNHIP_OP_ATTENTION)
+    if (!v || !out || heads < 1 || kv_heads < 1 || head_width < 1 || heads % kv_heads != 0)
+        return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_ATTENTION, lane->device, 0, "pointers must be non-null, counts positive and heads a multiple of kv_heads");
+    if (static_cast<int64_t>(heads) * head_width > 0x7fffffff)
+        return fail(NNHIP_ERR_TOO_LARGE, NNHIP_OP_ATTENTION, lane->device, 0, "heads * head_width exceeds one launch");
+    hipError_t e = launch_first_token_attention(lane, v, out, heads, kv_heads, head_width);
+    if (e != hipSuccess) return hip_fail(e, NNHIP_OP_ATTENTION, lane->device, "first-token attention launch");
+    lane->counters.kernel_launches += 1;
+    return NNHIP_OK;
+}
+
 int nnhip_lora_a(void* handle, const float* x, const float* a, float* z, int rows, int width, int rank)
 {
     NNHIP_LANE(handle, NNHIP_OP_LORA)

@@ -62,6 +62,7 @@ hipError_t launch_rms_norm(Lane* lane, float* io, const float* residual, const f
                            int width, int input_stride, float epsilon);
 hipError_t launch_silu_multiply(Lane* lane, const float* gate, const float* up, float* output, int length);
 hipError_t launch_add_in_place(Lane* lane, float* destination, const float* source, int length);
+hipError_t launch_first_token_attention(Lane* lane, const float* v, float* out, int heads, int kv_heads, int head_width);
 hipError_t launch_lora_a(Lane* lane, const float* x, const float* a, float* z, int rows, int width, int rank);
 hipError_t launch_lora_b(Lane* lane, const float* z, const float* b, float* y, int rows, int output, int rank, float scale);
 hipError_t launch_fill_u32(Lane* lane, uint32_t* p, uint32_t value, size_t count);

@@ -100,7 +100,24 @@ __global__ __launch_bounds__(256) void lora_b_kernel(const float* z, const float
     y[i] = y[i] + scale * sum;
 }
 
+// out[h, :] = v[h / (heads / kv_heads), :]: what causal grouped-query attention returns for the first token of a
+// sequence (one key: the softmax weight is 1, whatever the query), so a decode loop can run without a cache.
+__global__ __launch_bounds__(256) void first_token_attention_kernel(const float* v, float* out, int heads, int kv_heads, int head_width)
+{
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= heads * head_width) return;
+    const int h = i / head_width, c = i - h * head_width;
+    out[i] = v[(h / (heads / kv_heads)) * head_width + c];
+}
+
 }  // namespace
+
+hipError_t launch_first_token_attention(Lane* lane, const float* v, float* out, int heads, int kv_heads, int head_width)
+{
+    hipLaunchKernelGGL(first_token_attention_kernel, dim3((heads * head_width + 255) / 256), dim3(256), 0, lane->stream, v, out,
+                       heads, kv_heads, head_width);
+    return hipGetLastError();
+}
 
 hipError_t launch_lora_a(Lane* lane, const float* x, const float* a, float* z, int rows, int width, int rank)
 {

@@ -5,6 +5,7 @@ Allocate :241, AllocateBytes :271, Read :334, Synchronize :658, the byte counter
 """
 from __future__ import annotations
 
+import contextlib
 import ctypes
 from ctypes import byref, c_float, c_int, c_uint64, c_void_p
 
@@ -82,6 +83,14 @@ class HipExecutionLane:
         check(self._lib.nnhip_device_info(device, byref(cu), byref(mem)), "device_info")
         self.compute_units = cu.value
         self.total_memory_bytes = mem.value
+        # per-kernel device timing (ArcExecutionLane.KernelMilliseconds / KernelTimings, ArcExecutionLane.cs:87-92):
+        # off by default; when on, every operation is bracketed by two events that synchronize() turns into times
+        self.collect_kernel_events = False
+        self.kernel_milliseconds = 0.0
+        self.kernel_timings: dict[str, float] = {}
+        self._pending_events: list = []
+        self._event_pool: list = []
+        self._capturing = False
 
     # ---- enumeration (ArcDevices.Enumerate) ----
     @staticmethod
@@ -104,6 +113,12 @@ class HipExecutionLane:
 
     def dispose(self) -> None:
         if self._handle is not None:
+            for _, start, stop in self._pending_events:
+                self._event_pool += [start, stop]
+            self._pending_events.clear()
+            for e in self._event_pool:
+                e.dispose()
+            self._event_pool.clear()
             h, self._handle = self._handle, None
             check(self._lib.nnhip_lane_destroy(h), "lane_destroy")
 
@@ -161,6 +176,38 @@ class HipExecutionLane:
 
     def synchronize(self) -> None:
         check(self._lib.nnhip_synchronize(self._handle), "synchronize")
+        self._drain_events()
+
+    # ---- per-kernel timing (ArcExecutionLane.RecordKernelTime, ArcExecutionLane.cs:727-742) ----
+    @contextlib.contextmanager
+    def kernel(self, name: str):
+        """Brackets one operation with device events when collect_kernel_events is set (not while a graph is captured)."""
+        if not self.collect_kernel_events or self._capturing:
+            yield
+            return
+        start = self._event_pool.pop() if self._event_pool else HipEvent(self)
+        stop = self._event_pool.pop() if self._event_pool else HipEvent(self)
+        start.record()
+        try:
+            yield
+        finally:
+            stop.record()
+            self._pending_events.append((name, start, stop))
+
+    def _drain_events(self) -> None:
+        for name, start, stop in self._pending_events:
+            ms = self.elapsed_ms(start, stop)
+            self.kernel_milliseconds += ms
+            self.kernel_timings[name] = self.kernel_timings.get(name, 0.0) + ms
+            self._event_pool += [start, stop]
+        self._pending_events.clear()
+
+    def reset_profile(self) -> None:
+        """ArcExecutionLane.ResetProfile (ArcExecutionLane.cs:56-65): only with nothing pending."""
+        if self._pending_events:
+            raise RuntimeError("Synchronize before resetting the profile.")
+        self.kernel_milliseconds = 0.0
+        self.kernel_timings.clear()
 
     # ---- counters (ArcExecutionLane.H2DBytes etc.) ----
     def counters(self) -> dict:
@@ -180,9 +227,11 @@ class HipExecutionLane:
 
     def graph_begin(self) -> None:
         check(self._lib.nnhip_graph_begin(self._handle), "graph_begin")
+        self._capturing = True
 
     def graph_end(self):
         g = c_void_p()
+        self._capturing = False
         check(self._lib.nnhip_graph_end(self._handle, byref(g)), "graph_end")
         return g
 

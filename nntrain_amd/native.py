@@ -83,6 +83,7 @@ PROTOTYPES = {
     "nnhip_add_rms_norm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float]),
     "nnhip_silu_multiply": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int]),
     "nnhip_add_in_place": (c_int, [c_void_p, c_void_p, c_void_p, c_int]),
+    "nnhip_first_token_attention": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int]),
     "nnhip_lora_a": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int]),
     "nnhip_lora_b": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float]),
     "nnhip_event_create": (c_int, [c_void_p, POINTER(c_void_p)]),

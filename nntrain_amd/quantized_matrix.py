@@ -137,9 +137,10 @@ class HipQuantizedMatrix:
         y = out if out is not None else lane.allocate(rows * self.output_width)
         if y.nbytes < 4 * rows * self.output_width:
             raise ValueError("output buffer too small")
-        check(lane._lib.nnhip_quant_matvec(lane._handle, self.ggml_type, c_void_p(x._require()), c_void_p(w._require()),
-                                           c_void_p(bias._require()) if bias is not None else None,
-                                           c_void_p(y._require()), rows, self.input_width, self.output_width), "quant_matvec")
+        with lane.kernel("quant_matvec"):
+            check(lane._lib.nnhip_quant_matvec(lane._handle, self.ggml_type, c_void_p(x._require()), c_void_p(w._require()),
+                                               c_void_p(bias._require()) if bias is not None else None,
+                                               c_void_p(y._require()), rows, self.input_width, self.output_width), "quant_matvec")
         return y
 
     def forward_fused(self, lane: HipExecutionLane, x: HipBuffer, *, pre_op: int = PRE_NONE, x2: HipBuffer | None = None,
@@ -171,7 +172,8 @@ class HipQuantizedMatrix:
                                in_w=self.input_width, out_w=self.output_width, lora_z=ptr(lora_z), lora_b=ptr(lora_b),
                                lora_rank=lora_rank, lora_scale=lora_scale)
         try:
-            check(lane._lib.nnhip_quant_matvec_fused(lane._handle, ctypes.byref(desc)), "quant_matvec_fused")
+            with lane.kernel("quant_matvec_fused"):
+                check(lane._lib.nnhip_quant_matvec_fused(lane._handle, ctypes.byref(desc)), "quant_matvec_fused")
         except BaseException:
             if out is None:
                 y.dispose()
@@ -189,14 +191,15 @@ class HipQuantizedMatrix:
             raise ValueError("Quantized linear bias width mismatch.")
         w = self.device_payload(lane)
         y = out if out is not None else lane.allocate(rows * self.output_width)
-        check(lane._lib.nnhip_quant_matmul_bf16(lane._handle, self.ggml_type, c_void_p(x_bf16._require()),
-                                                c_void_p(w._require()),
-                                                c_void_p(bias._require()) if bias is not None else None,
-                                                c_void_p(y._require()), rows, self.input_width, self.output_width),
-              "quant_matmul_bf16")
+        with lane.kernel("quant_matmul_bf16"):
+            check(lane._lib.nnhip_quant_matmul_bf16(lane._handle, self.ggml_type, c_void_p(x_bf16._require()),
+                                                    c_void_p(w._require()),
+                                                    c_void_p(bias._require()) if bias is not None else None,
+                                                    c_void_p(y._require()), rows, self.input_width, self.output_width),
+                  "quant_matmul_bf16")
         return y
 
-    def dequantize(self, lane: HipExecutionLane, row: int | None = None) -> HipBuffer:
+    def dequantize(self, lane: HipExecutionLane, row: int | None = None, out: HipBuffer | None = None) -> HipBuffer:
         """Decode the whole matrix, or one row (the embedding lookup of Matrix.Embedding,
         Qwen35QuantizedModel.cs:1497-1521), to FP32 on the device."""
         w = self.device_payload(lane)
@@ -207,9 +210,12 @@ class HipQuantizedMatrix:
             if not 0 <= row < self.output_width:
                 raise IndexError(f"Embedding index {row} is outside the vocabulary.")
             elements, offset = self.input_width, row * row_bytes
-        out = lane.allocate(elements)
-        check(lane._lib.nnhip_dequantize(lane._handle, self.ggml_type, c_void_p(w._require() + offset),
-                                         c_void_p(out._require()), elements), "dequantize")
+        out = lane.allocate(elements) if out is None else out
+        if out.nbytes < 4 * elements:
+            raise ValueError("output buffer too small")
+        with lane.kernel("dequantize"):
+            check(lane._lib.nnhip_dequantize(lane._handle, self.ggml_type, c_void_p(w._require() + offset),
+                                             c_void_p(out._require()), elements), "dequantize")
         return out
 
     def dispose(self) -> None:

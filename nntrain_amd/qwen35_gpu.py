@@ -28,8 +28,15 @@ def _validate_buffer(buffer: HipBuffer, elements: int, name: str) -> None:
         raise ValueError(f"The buffer '{name}' is disposed or too small for its declared dimensions.")
 
 
+def _output(lane: HipExecutionLane, out: HipBuffer | None, elements: int) -> HipBuffer:
+    if out is None:
+        return lane.allocate(elements)
+    _validate_buffer(out, elements, "out")
+    return out
+
+
 def rms_norm(lane: HipExecutionLane, input: HipBuffer, weight: HipBuffer, rows: int, width: int, eps: float,
-             input_stride: int | None = None) -> HipBuffer:
+             input_stride: int | None = None, out: HipBuffer | None = None) -> HipBuffer:
     """Qwen35Gpu.RmsNorm: output[r] = input[r] * inverse_rms(input[r]) * weight."""
     _positive(rows, "rows")
     _positive(width, "width")
@@ -39,47 +46,54 @@ def rms_norm(lane: HipExecutionLane, input: HipBuffer, weight: HipBuffer, rows: 
         raise ValueError("input_stride must be at least width.")
     _validate_buffer(input, (rows - 1) * stride + width, "input")
     _validate_buffer(weight, width, "weight")
-    output = lane.allocate(rows * width)
+    output = _output(lane, out, rows * width)
     try:
-        check(lane._lib.nnhip_rms_norm(lane._handle, c_void_p(input._require()), c_void_p(weight._require()),
-                                       c_void_p(output._require()), rows, width, stride, eps), "rms_norm")
+        with lane.kernel("rms_norm"):
+            check(lane._lib.nnhip_rms_norm(lane._handle, c_void_p(input._require()), c_void_p(weight._require()),
+                                           c_void_p(output._require()), rows, width, stride, eps), "rms_norm")
         return output
     except BaseException:
-        output.dispose()
+        if out is None:
+            output.dispose()
         raise
 
 
 def add_residual_and_rms_norm(lane: HipExecutionLane, hidden: HipBuffer, residual: HipBuffer, weight: HipBuffer,
-                              width: int, eps: float) -> HipBuffer:
+                              width: int, eps: float, out: HipBuffer | None = None) -> HipBuffer:
     """AddResidualAndRmsNorm (fused form): hidden += residual in place, returns RMSNorm(hidden) * weight."""
     _positive(width, "width")
     _validate_epsilon(eps)
     _validate_buffer(hidden, width, "hidden")
     _validate_buffer(residual, width, "residual")
     _validate_buffer(weight, width, "weight")
-    output = lane.allocate(width)
+    output = _output(lane, out, width)
     try:
-        check(lane._lib.nnhip_add_rms_norm(lane._handle, c_void_p(hidden._require()), c_void_p(residual._require()),
-                                           c_void_p(weight._require()), c_void_p(output._require()), 1, width, width,
-                                           eps), "add_rms_norm")
+        with lane.kernel("add_rms_norm"):
+            check(lane._lib.nnhip_add_rms_norm(lane._handle, c_void_p(hidden._require()), c_void_p(residual._require()),
+                                               c_void_p(weight._require()), c_void_p(output._require()), 1, width, width,
+                                               eps), "add_rms_norm")
         return output
     except BaseException:
-        output.dispose()
+        if out is None:
+            output.dispose()
         raise
 
 
-def silu_multiply(lane: HipExecutionLane, gate: HipBuffer, up: HipBuffer, length: int) -> HipBuffer:
+def silu_multiply(lane: HipExecutionLane, gate: HipBuffer, up: HipBuffer, length: int,
+                  out: HipBuffer | None = None) -> HipBuffer:
     """Qwen35Gpu.SiluMultiply: gate * sigmoid(gate) * up."""
     _positive(length, "length")
     _validate_buffer(gate, length, "gate")
     _validate_buffer(up, length, "up")
-    output = lane.allocate(length)
+    output = _output(lane, out, length)
     try:
-        check(lane._lib.nnhip_silu_multiply(lane._handle, c_void_p(gate._require()), c_void_p(up._require()),
-                                            c_void_p(output._require()), length), "silu_multiply")
+        with lane.kernel("silu_multiply"):
+            check(lane._lib.nnhip_silu_multiply(lane._handle, c_void_p(gate._require()), c_void_p(up._require()),
+                                                c_void_p(output._require()), length), "silu_multiply")
         return output
     except BaseException:
-        output.dispose()
+        if out is None:
+            output.dispose()
         raise
 
 
@@ -88,8 +102,9 @@ def add_in_place(lane: HipExecutionLane, destination: HipBuffer, source: HipBuff
     _positive(length, "length")
     _validate_buffer(destination, length, "destination")
     _validate_buffer(source, length, "source")
-    check(lane._lib.nnhip_add_in_place(lane._handle, c_void_p(destination._require()), c_void_p(source._require()),
-                                       length), "add_in_place")
+    with lane.kernel("add_in_place"):
+        check(lane._lib.nnhip_add_in_place(lane._handle, c_void_p(destination._require()), c_void_p(source._require()),
+                                           length), "add_in_place")
 
 
 def lora_project_a(lane: HipExecutionLane, x: HipBuffer, a: HipBuffer, rows: int, width: int, rank: int) -> HipBuffer:
@@ -101,8 +116,9 @@ def lora_project_a(lane: HipExecutionLane, x: HipBuffer, a: HipBuffer, rows: int
     _validate_buffer(a, rank * width, "a")
     z = lane.allocate(rows * rank)
     try:
-        check(lane._lib.nnhip_lora_a(lane._handle, c_void_p(x._require()), c_void_p(a._require()), c_void_p(z._require()),
-                                     rows, width, rank), "lora_a")
+        with lane.kernel("lora_a"):
+            check(lane._lib.nnhip_lora_a(lane._handle, c_void_p(x._require()), c_void_p(a._require()), c_void_p(z._require()),
+                                         rows, width, rank), "lora_a")
         return z
     except BaseException:
         z.dispose()
@@ -118,5 +134,29 @@ def lora_apply_b(lane: HipExecutionLane, z: HipBuffer, b: HipBuffer, y: HipBuffe
     _validate_buffer(z, rows * rank, "z")
     _validate_buffer(b, output * rank, "b")
     _validate_buffer(y, rows * output, "y")
-    check(lane._lib.nnhip_lora_b(lane._handle, c_void_p(z._require()), c_void_p(b._require()), c_void_p(y._require()),
-                                 rows, output, rank, scale), "lora_b")
+    with lane.kernel("lora_b"):
+        check(lane._lib.nnhip_lora_b(lane._handle, c_void_p(z._require()), c_void_p(b._require()), c_void_p(y._require()),
+                                     rows, output, rank, scale), "lora_b")
+
+
+def first_token_attention(lane: HipExecutionLane, value: HipBuffer, heads: int, kv_heads: int, head_width: int,
+                          out: HipBuffer | None = None) -> HipBuffer:
+    """Causal grouped-query attention for the first token of a sequence: every query head receives its group's value
+    head (the single key has softmax weight 1).  The general attention step (Qwen35Gpu.AttentionStep) is not part of
+    this library."""
+    _positive(heads, "heads")
+    _positive(kv_heads, "kv_heads")
+    _positive(head_width, "head_width")
+    if heads % kv_heads != 0:
+        raise ValueError("heads must be a multiple of kv_heads.")
+    _validate_buffer(value, kv_heads * head_width, "value")
+    output = _output(lane, out, heads * head_width)
+    try:
+        with lane.kernel("first_token_attention"):
+            check(lane._lib.nnhip_first_token_attention(lane._handle, c_void_p(value._require()), c_void_p(output._require()),
+                                                        heads, kv_heads, head_width), "first_token_attention")
+        return output
+    except BaseException:
+        if out is None:
+            output.dispose()
+        raise
