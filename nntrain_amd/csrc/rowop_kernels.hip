@@ -26,7 +26,26 @@ __global__ __launch_bounds__(kNormLanes) void rms_norm_kernel(float* io, const f
     const float* res = ADD ? residual + static_cast<size_t>(blockIdx.x) * input_stride : nullptr;
     float* out = output + static_cast<size_t>(blockIdx.x) * width;
     float sum = 0.0f;
-    for (int j = tid; j < width; j += kNormLanes) {
+    // eight loads in flight per lane; the additions keep their order
+    constexpr int kAhead = 8;
+    int j = tid;
+    for (; j + (kAhead - 1) * kNormLanes < width; j += kAhead * kNormLanes) {
+        float v[kAhead], r[kAhead];
+#pragma unroll
+        for (int u = 0; u < kAhead; ++u) {
+            v[u] = x[j + u * kNormLanes];
+            r[u] = ADD ? res[j + u * kNormLanes] : 0.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < kAhead; ++u) {
+            if (ADD) {
+                v[u] = v[u] + r[u];
+                x[j + u * kNormLanes] = v[u];
+            }
+            sum += v[u] * v[u];
+        }
+    }
+    for (; j < width; j += kNormLanes) {
         float v = x[j];
         if (ADD) {
             v = v + res[j];
@@ -42,7 +61,47 @@ __global__ __launch_bounds__(kNormLanes) void rms_norm_kernel(float* io, const f
     }
     const float inverse = 1.0f / sqrtf(sums[0] / static_cast<float>(width) + epsilon);
     // every lane re-reads the components it wrote itself
-    for (int j = tid; j < width; j += kNormLanes) out[j] = x[j] * inverse * weight[j];
+#pragma unroll 8
+    for (int k = tid; k < width; k += kNormLanes) out[k] = x[k] * inverse * weight[k];
+}
+
+// The same arithmetic for wide rows with 1024 lanes: the row (plus residual) is staged in LDS by all lanes at once, lanes
+// 0-127 take the strided partial sums from LDS in the same order, and all lanes write the output.  One workgroup of
+// 128 lanes spends its time waiting for forty dependent batches of loads; this form needs one.
+constexpr int kWideLanes = 1024;
+constexpr int kWideMaxWidth = 15360;          // floats staged in LDS (60 KB)
+
+template <bool ADD>
+__global__ __launch_bounds__(kWideLanes) void rms_norm_wide_kernel(float* io, const float* residual, const float* weight,
+                                                                   float* output, int width, int input_stride, float epsilon)
+{
+    extern __shared__ float row[];
+    __shared__ float sums[kNormLanes];
+    const int tid = threadIdx.x;
+    float* x = io + static_cast<size_t>(blockIdx.x) * input_stride;
+    const float* res = ADD ? residual + static_cast<size_t>(blockIdx.x) * input_stride : nullptr;
+    float* out = output + static_cast<size_t>(blockIdx.x) * width;
+    for (int j = tid; j < width; j += kWideLanes) {
+        float v = x[j];
+        if (ADD) {
+            v = v + res[j];
+            x[j] = v;
+        }
+        row[j] = v;
+    }
+    __syncthreads();
+    if (tid < kNormLanes) {
+        float sum = 0.0f;
+        for (int j = tid; j < width; j += kNormLanes) sum += row[j] * row[j];
+        sums[tid] = sum;
+    }
+    __syncthreads();
+    for (int stride = kNormLanes / 2; stride > 0; stride >>= 1) {
+        if (tid < stride) sums[tid] += sums[tid + stride];
+        __syncthreads();
+    }
+    const float inverse = 1.0f / sqrtf(sums[0] / static_cast<float>(width) + epsilon);
+    for (int j = tid; j < width; j += kWideLanes) out[j] = row[j] * inverse * weight[j];
 }
 
 // Two-sided form: exp never sees a positive argument, so neither side overflows (qwen35_attention.cl:9-14).
@@ -134,6 +193,26 @@ hipError_t launch_lora_b(Lane* lane, const float* z, const float* b, float* y, i
 hipError_t launch_rms_norm(Lane* lane, float* io, const float* residual, const float* weight, float* output, int rows,
                            int width, int input_stride, float epsilon)
 {
+    if (width >= 2 * kWideLanes && width <= kWideMaxWidth) {
+        const size_t lds = static_cast<size_t>(width) * sizeof(float);
+        static bool big_lds_enabled = false;
+        if (!big_lds_enabled) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&rms_norm_wide_kernel<true>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, kWideMaxWidth * sizeof(float));
+            if (e == hipSuccess)
+                e = hipFuncSetAttribute(reinterpret_cast<const void*>(&rms_norm_wide_kernel<false>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, kWideMaxWidth * sizeof(float));
+            if (e != hipSuccess) return e;
+            big_lds_enabled = true;
+        }
+        if (residual)
+            hipLaunchKernelGGL(rms_norm_wide_kernel<true>, dim3(rows), dim3(kWideLanes), lds, lane->stream, io, residual, weight,
+                               output, width, input_stride, epsilon);
+        else
+            hipLaunchKernelGGL(rms_norm_wide_kernel<false>, dim3(rows), dim3(kWideLanes), lds, lane->stream, io, residual, weight,
+                               output, width, input_stride, epsilon);
+        return hipGetLastError();
+    }
     if (residual)
         hipLaunchKernelGGL(rms_norm_kernel<true>, dim3(rows), dim3(kNormLanes), 0, lane->stream, io, residual, weight, output,
                            width, input_stride, epsilon);
