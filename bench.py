@@ -530,14 +530,26 @@ def run_decode_loop(args, lane, nn, oracle):
 
 
 def run_prefill(args, lane, nn, oracle):
-    """Q4_K 17408x5120 bf16-MFMA prefill mat-mul at M = 128, 256, 512, 2048 (BASELINE configs[3])."""
+    """Q4_K 17408x5120 bf16-MFMA prefill mat-mul at M = 128, 256, 512, 2048 (BASELINE configs[3]); the other formats
+    the kernel decodes (Q5_K, Q6_K, Q8_0) at M = 512 under "other_formats"."""
+    out = _prefill_of(lane, nn, oracle, nn.GGML_Q4_K, "Q4_K", (128, 256, 512, 2048))
+    if out is not None:
+        out["other_formats"] = {}
+        for tname in ("Q5_K", "Q6_K", "Q8_0"):
+            res = _prefill_of(lane, nn, oracle, getattr(nn, "GGML_" + tname), tname, (512,))
+            if res is not None:
+                out["other_formats"][tname] = res["M=512"]
+    return out
+
+
+def _prefill_of(lane, nn, oracle, typ, tname, ms_list):
     from nntrain_amd import synth
-    typ, in_w, out_w = nn.GGML_Q4_K, 5120, 17408
+    in_w, out_w = 5120, 17408
     payload = synth.matrix(typ, out_w, in_w, 2001)
     mat = nn.HipQuantizedMatrix(payload, typ, out_w, in_w)
     mat.device_payload(lane)
     out = {}
-    for m in (128, 256, 512, 2048):
+    for m in ms_list:
         xb = synth.to_bf16_bits(synth.activations(m, in_w, 4000))
         x = lane.upload_raw(xb)
         y = lane.allocate(m * out_w)
@@ -555,7 +567,7 @@ def run_prefill(args, lane, nn, oracle):
         ref, _ = oracle.linear_f64(typ, payload, xb[:rows], None, rows, in_w, out_w, x_is_bf16=True)
         rel = oracle.rel_l2(got, ref)
         if not rel <= 2e-3:
-            raise SystemExit(f"prefill M={m}: parity failure, rel-L2 {rel:.3e} > 2e-3")
+            raise SystemExit(f"prefill {tname} M={m}: parity failure, rel-L2 {rel:.3e} > 2e-3")
         samples = []
         for _ in range(7):
             ms, _ = timed(lane, lambda: mat.forward_bf16(lane, x, None, m, out=y), 3)
@@ -565,7 +577,7 @@ def run_prefill(args, lane, nn, oracle):
         out[f"M={m}"] = {"ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 1),
                          "mfma_util_vs_2500_TFLOPs_bf16": round(flops / ms / 1e9 / BF16_PEAK_TFLOPS, 4),
                          "rel_l2_vs_f64_oracle": rel}
-        log(f"[prefill] M={m}: {ms:.3f} ms, {flops / ms / 1e9:.0f} TFLOP/s, rel-L2 {rel:.2e}")
+        log(f"[prefill] {tname} M={m}: {ms:.3f} ms, {flops / ms / 1e9:.0f} TFLOP/s, rel-L2 {rel:.2e}")
         x.dispose()
         y.dispose()
     mat.dispose()

@@ -1,15 +1,18 @@
-// Prefill mat-mul for raw GGUF Q4_K weights on gfx950: y[M, N] = bias + x[M, K] (bf16) . W[N, K]^T.
+// Prefill mat-mul for raw GGUF block-quantized weights (Q4_K, Q5_K, Q6_K, Q8_0) on gfx950:
+// y[M, N] = bias + x[M, K] (bf16) . W[N, K]^T.
 //
-// Replaces the XMX prefill launch of the reference (NNtrain.Arc/Kernels/qwen35_prefill_xmx.cl:112-184): weight tiles
-// are dequantized to bfloat16 in LDS and contracted on the matrix cores (v_mfma_f32_16x16x32_bf16) with FP32
-// accumulators.  The weight is the CPU decoder's (d*sc)*q - dmin*m (NNtrain.Core/Serialization/GgufQ4K.cs:34-41)
-// evaluated in FP32 and rounded once to bf16, which is what the 2e-3 relative-L2 bar of this path allows for.
+// Replaces the XMX prefill launches of the reference (NNtrain.Arc/Kernels/qwen35_prefill_xmx.cl:112-184, the
+// q35l_prefill_xmx_<format>_f16x2 family): weight tiles are dequantized to bfloat16 in LDS and contracted on the matrix
+// cores (v_mfma_f32_16x16x32_bf16) with FP32 accumulators.  A weight is the CPU decoder's value, e.g. (d*sc)*q - dmin*m
+// for Q4_K (NNtrain.Core/Serialization/GgufQ4K.cs:34-41), evaluated in FP32 and rounded once to bf16, which is what the
+// 2e-3 relative-L2 bar of this path allows for (the rounding alone is 1.6e-3 rms; against a product taken with
+// bf16-rounded weights the kernel agrees to FP32 accumulation accuracy).
 //
 // Tiling.  A workgroup owns BM rows (128 or 256) and a strip of up to 16 * CT output columns (CT = 5 or 9 column tiles)
 // for the whole K range; the strip width is chosen on the host so that strips x row tiles split evenly over the
 // compute units (17408 columns: 256 strips of 68 for M <= 256, 128 strips of 136 for larger M).  A weight sub-block
-// is dequantized once per workgroup.  K advances 64 per iteration = the two Q4_K sub-blocks that share 32 bytes of
-// nibbles; a slice is two x sub-tiles [BM][32] bf16 and two weight sub-tiles [16 CT][32] bf16 in LDS (rows are 64
+// is dequantized once per workgroup.  K advances 64 per iteration (for Q4_K the two sub-blocks that share 32 bytes of
+// nibbles); a slice is two x sub-tiles [BM][32] bf16 and two weight sub-tiles [16 CT][32] bf16 in LDS (rows are 64
 // bytes, placed so that the 16 rows x 4 k-groups an MFMA operand needs are one conflict-free read), in three stages:
 // the slice being multiplied, the finished next one, and the one being made.
 //
@@ -91,6 +94,251 @@ __device__ __forceinline__ u32x4 q4k_decode8(uint32_t q_lo, uint32_t q_hi, float
 // 4 cycles per 128-bit read against 6.6 for the plain row-major placement), and writes stay row-contiguous.
 __device__ __forceinline__ int lds_slot(int row, int group) { return group ^ ((row >> 1) & 3); }
 
+// ---------------------------------------------------------------------------------------------------- decoders
+// A decoding thread (column dc of the strip, half dh) turns its share of every 64-weight K slice into bf16 in the two
+// weight sub-tiles of a stage (`lo`: weights 0-31 of the slice, `hi`: weights 32-63; a column is one 64-byte row of
+// each).  What it needs for a slice was requested two slices earlier, block headers a block earlier.  One struct per
+// storage format: `start()` issues the first loads, `make<J>(t, lo, hi)` writes slice t (J = t % 4) and requests ahead.
+struct DecodeCtx {
+    const uint8_t* wbase;    // first row of the strip (wave-uniform)
+    uint32_t wrow;           // byte offset of this thread's row
+    int dc, dh;
+    int iters;               // K / 64
+    int nblocks;             // K / 256
+};
+
+__device__ __forceinline__ u32x4 gld128(const DecodeCtx& c, uint32_t uniform_off, uint32_t lane_off)
+{
+    asm volatile("" : "+s"(uniform_off));      // keeps the address as scalar base + 32-bit lane offset
+    return ld128(c.wbase + uniform_off + opaque(c.wrow + lane_off));
+}
+
+// (d * scale, dmin * min) of the eight sub-blocks of a Q4_K / Q5_K block header; 6-bit fields as in GgufQ4K.cs:51-60:
+// sub-blocks 0-3 sit in the low six bits of bytes j and 4 + j, 4-7 are split between bytes 8 + j (low nibble scale, high
+// nibble min) and the top two bits of bytes j and 4 + j.
+__device__ __forceinline__ void k4_block_scales(const u32x4 hdr, float sm[16])
+{
+    const float d = half_bits_to_float(hdr[0]), dmin = half_bits_to_float(hdr[0] >> 16);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t b0 = (hdr[1] >> (8 * j)) & 255u, b1 = (hdr[2] >> (8 * j)) & 255u, b2 = (hdr[3] >> (8 * j)) & 255u;
+        sm[2 * j] = d * static_cast<float>(b0 & 63u);
+        sm[2 * j + 1] = dmin * static_cast<float>(b1 & 63u);
+        sm[8 + 2 * j] = d * static_cast<float>((b2 & 15u) | ((b0 >> 6) << 4));
+        sm[8 + 2 * j + 1] = dmin * static_cast<float>((b2 >> 4) | ((b1 >> 6) << 4));
+    }
+}
+
+// Q4_K: the thread owns bytes [16 dh, 16 dh + 16) of the 32 nibble bytes of a slice: 16 low-nibble weights of sub-block 2J
+// and 16 high-nibble weights of sub-block 2J + 1.
+struct Q4KDecode {
+    static constexpr int kBlockBytes = 144;
+    u32x4 nq[2];                // nibble bytes of K slices t and t + 1
+    u32x4 hdr;                  // header (d, dmin, packed scales) of the next 256-block
+    float sm[16];               // (d * scale, dmin * min) of the eight sub-blocks of the current block
+
+    __device__ __forceinline__ u32x4 load_q(const DecodeCtx& c, int t)
+    {
+        const int tt = min(t, c.iters - 1);
+        return gld128(c, static_cast<uint32_t>(tt >> 2) * 144u + 16u + static_cast<uint32_t>(tt & 3) * 32u,
+                      static_cast<uint32_t>(c.dh) * 16u);
+    }
+    __device__ __forceinline__ void load_hdr(const DecodeCtx& c, int blk)
+    {
+        hdr = gld128(c, static_cast<uint32_t>(min(blk, c.nblocks - 1)) * 144u, 0u);
+    }
+    __device__ __forceinline__ void start(const DecodeCtx& c)
+    {
+        load_hdr(c, 0);
+        nq[0] = load_q(c, 0);
+        nq[1] = load_q(c, 1);
+        k4_block_scales(hdr, sm);
+    }
+    template <int J>
+    __device__ __forceinline__ void make(const DecodeCtx& c, int t, uint8_t* lo, uint8_t* hi)
+    {
+        const u32x4 q = nq[J & 1];
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+            const uint32_t a0 = q[2 * g], a1 = q[2 * g + 1];
+            const int slot = lds_slot(c.dc, 2 * c.dh + g) * 16;
+            *reinterpret_cast<u32x4*>(lo + slot) = q4k_decode8(a0 & 0x0f0f0f0fu, a1 & 0x0f0f0f0fu, sm[4 * J], sm[4 * J + 1]);
+            *reinterpret_cast<u32x4*>(hi + slot) =
+                q4k_decode8((a0 >> 4) & 0x0f0f0f0fu, (a1 >> 4) & 0x0f0f0f0fu, sm[4 * J + 2], sm[4 * J + 3]);
+        }
+        nq[J & 1] = load_q(c, t + 2);
+        if (J == 0) load_hdr(c, (t >> 2) + 1);
+        if (J == 3) k4_block_scales(hdr, sm);
+    }
+};
+
+// Q5_K: as Q4_K with one more bit per weight: bit g of qh[i] belongs to element i of sub-block g (qh: 32 bytes after
+// the header, nibbles after that).  The thread keeps bytes [16 dh, 16 dh + 16) of qh for the whole block.
+struct Q5KDecode {
+    static constexpr int kBlockBytes = 176;
+    u32x4 nq[2];
+    u32x4 hdr, qh_next;         // of the next block
+    u32x4 qh;                   // high bits of the current block
+    float sm[16];
+
+    __device__ __forceinline__ u32x4 load_q(const DecodeCtx& c, int t)
+    {
+        const int tt = min(t, c.iters - 1);
+        return gld128(c, static_cast<uint32_t>(tt >> 2) * 176u + 48u + static_cast<uint32_t>(tt & 3) * 32u,
+                      static_cast<uint32_t>(c.dh) * 16u);
+    }
+    __device__ __forceinline__ void load_hdr(const DecodeCtx& c, int blk)
+    {
+        const uint32_t off = static_cast<uint32_t>(min(blk, c.nblocks - 1)) * 176u;
+        hdr = gld128(c, off, 0u);
+        qh_next = gld128(c, off + 16u, static_cast<uint32_t>(c.dh) * 16u);
+    }
+    __device__ __forceinline__ void start(const DecodeCtx& c)
+    {
+        load_hdr(c, 0);
+        nq[0] = load_q(c, 0);
+        nq[1] = load_q(c, 1);
+        k4_block_scales(hdr, sm);
+        qh = qh_next;
+    }
+    template <int J>
+    __device__ __forceinline__ void make(const DecodeCtx& c, int t, uint8_t* lo, uint8_t* hi)
+    {
+        const u32x4 q = nq[J & 1];
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+            const uint32_t a0 = q[2 * g], a1 = q[2 * g + 1], h0 = qh[2 * g], h1 = qh[2 * g + 1];
+            const int slot = lds_slot(c.dc, 2 * c.dh + g) * 16;
+            *reinterpret_cast<u32x4*>(lo + slot) =
+                q4k_decode8((a0 & 0x0f0f0f0fu) | (((h0 >> (2 * J)) & 0x01010101u) << 4),
+                            (a1 & 0x0f0f0f0fu) | (((h1 >> (2 * J)) & 0x01010101u) << 4), sm[4 * J], sm[4 * J + 1]);
+            *reinterpret_cast<u32x4*>(hi + slot) =
+                q4k_decode8(((a0 >> 4) & 0x0f0f0f0fu) | (((h0 >> (2 * J + 1)) & 0x01010101u) << 4),
+                            ((a1 >> 4) & 0x0f0f0f0fu) | (((h1 >> (2 * J + 1)) & 0x01010101u) << 4), sm[4 * J + 2], sm[4 * J + 3]);
+        }
+        nq[J & 1] = load_q(c, t + 2);
+        if (J == 0) load_hdr(c, (t >> 2) + 1);
+        if (J == 3) {
+            k4_block_scales(hdr, sm);
+            qh = qh_next;
+        }
+    }
+};
+
+// Q6_K (GgufQ6K.cs:9-54): a block is two halves of 128 weights; in a half, weights 0-31 / 32-63 take the low nibbles of
+// ql[l] / ql[32 + l] with bits 0-1 / 2-3 of qh[l], weights 64-95 / 96-127 the high nibbles with bits 4-5 / 6-7; weight =
+// d * scale[16-group] * (q - 32).  Slice J of a block is half J / 2, nibble J % 2.  The thread keeps bytes
+// [16 dh, 16 dh + 16) of both ql runs and of qh for a half (two slices), and the 16 scales and d for a block.
+struct Q6KDecode {
+    static constexpr int kBlockBytes = 210;
+    u32x4 qa[2], qb[2], qhv[2];     // [half parity]: ql[l], ql[32 + l], qh[l] runs of the current and the next half
+    u32x4 sc_next;                  // the 16 scale bytes of the next block
+    uint32_t d_next;
+    float ds[8];                    // d * scale of the thread's 16-weight groups: [half][group of the half]
+
+    __device__ __forceinline__ void load_half(const DecodeCtx& c, int half_index, int set)
+    {
+        const int hh = min(half_index, 2 * c.nblocks - 1);
+        const uint32_t blk = static_cast<uint32_t>(hh >> 1) * 210u, h = static_cast<uint32_t>(hh & 1);
+        const uint32_t lane_off = static_cast<uint32_t>(c.dh) * 16u;
+        qa[set] = gld128(c, blk + 64u * h, lane_off);
+        qb[set] = gld128(c, blk + 64u * h + 32u, lane_off);
+        qhv[set] = gld128(c, blk + 128u + 32u * h, lane_off);
+    }
+    __device__ __forceinline__ void load_tail(const DecodeCtx& c, int blk)
+    {
+        uint32_t off = static_cast<uint32_t>(min(blk, c.nblocks - 1)) * 210u;
+        sc_next = gld128(c, off + 192u, 0u);
+        asm volatile("" : "+s"(off));
+        d_next = ld16(c.wbase + off + 208u + opaque(c.wrow));
+    }
+    int dh_sel;
+    __device__ __forceinline__ void block_scales()
+    {
+        const float d = half_bits_to_float(d_next);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            // group i = 4 * half + group-of-the-half uses scale byte 2 i + dh of the 16
+            const uint32_t two = (sc_next[i >> 1] >> (16 * (i & 1))) & 0xffffu;
+            ds[i] = d * static_cast<float>(static_cast<int8_t>(dh_sel ? (two >> 8) : (two & 0xffu)));
+        }
+    }
+    __device__ __forceinline__ void start(const DecodeCtx& c)
+    {
+        dh_sel = c.dh;
+        load_tail(c, 0);
+        load_half(c, 0, 0);
+        load_half(c, 1, 1);
+        block_scales();
+    }
+    // 16 weights: bytes q (6-bit values) -> d * scale * (q - 32), as one fused multiply-add each (exact: 32 * ds is a
+    // power-of-two multiple of ds, so the result is ds * (q - 32) rounded once, the reference's value)
+    static __device__ __forceinline__ void put16(uint8_t* row, int dc, int group0, const u32x4 bytes, float dsv)
+    {
+        const float off = 32.0f * dsv;
+#pragma unroll
+        for (int g = 0; g < 2; ++g)
+            *reinterpret_cast<u32x4*>(row + lds_slot(dc, group0 + g) * 16) = q4k_decode8(bytes[2 * g], bytes[2 * g + 1], dsv, off);
+    }
+    template <int J>
+    __device__ __forceinline__ void make(const DecodeCtx& c, int t, uint8_t* lo, uint8_t* hi)
+    {
+        constexpr int H = J >> 1, P = J & 1;        // half of the block, nibble
+        const u32x4 a = qa[H], b = qb[H], h = qhv[H];
+        u32x4 lo_b, hi_b;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            lo_b[i] = ((a[i] >> (4 * P)) & 0x0f0f0f0fu) | (((h[i] >> (4 * P)) & 0x03030303u) << 4);
+            hi_b[i] = ((b[i] >> (4 * P)) & 0x0f0f0f0fu) | (((h[i] >> (4 * P + 2)) & 0x03030303u) << 4);
+        }
+        put16(lo, c.dc, 2 * c.dh, lo_b, ds[4 * H + 2 * P]);
+        put16(hi, c.dc, 2 * c.dh, hi_b, ds[4 * H + 2 * P + 1]);
+        if (P == 1) load_half(c, (t >> 1) + 2, H);          // this half's registers are free: request the half after next
+        if (J == 0) load_tail(c, (t >> 2) + 1);
+        if (J == 3) block_scales();
+    }
+};
+
+// Q8_0: a slice is two 34-byte blocks (d, 32 signed bytes); thread dh decodes block dh of the slice, a whole 64-byte
+// row of its sub-tile.
+struct Q8_0Decode {
+    static constexpr int kBlockBytes = 34 * 8;     // bytes per 256 weights
+    u32x4 q0[2], q1[2];
+    uint32_t dbits[2];
+
+    __device__ __forceinline__ void load(const DecodeCtx& c, int t, int set)
+    {
+        uint32_t off = static_cast<uint32_t>(min(t, c.iters - 1)) * 68u;
+        const uint32_t lane_off = static_cast<uint32_t>(c.dh) * 34u;
+        q0[set] = gld128(c, off + 2u, lane_off);
+        q1[set] = gld128(c, off + 18u, lane_off);
+        asm volatile("" : "+s"(off));
+        dbits[set] = ld16(c.wbase + off + opaque(c.wrow + lane_off));
+    }
+    __device__ __forceinline__ void start(const DecodeCtx& c)
+    {
+        load(c, 0, 0);
+        load(c, 1, 1);
+    }
+    static __device__ __forceinline__ u32x4 decode8(uint32_t a, uint32_t b, float d)
+    {
+        return u32x4{pack_bf16(d * sbyte0(a), d * sbyte1(a)), pack_bf16(d * sbyte2(a), d * sbyte3(a)),
+                     pack_bf16(d * sbyte0(b), d * sbyte1(b)), pack_bf16(d * sbyte2(b), d * sbyte3(b))};
+    }
+    template <int J>
+    __device__ __forceinline__ void make(const DecodeCtx& c, int t, uint8_t* lo, uint8_t* hi)
+    {
+        const float d = half_bits_to_float(dbits[J & 1]);
+        uint8_t* row = c.dh ? hi : lo;
+        const u32x4 a = q0[J & 1], b = q1[J & 1];
+        *reinterpret_cast<u32x4*>(row + lds_slot(c.dc, 0) * 16) = decode8(a[0], a[1], d);
+        *reinterpret_cast<u32x4*>(row + lds_slot(c.dc, 1) * 16) = decode8(a[2], a[3], d);
+        *reinterpret_cast<u32x4*>(row + lds_slot(c.dc, 2) * 16) = decode8(b[0], b[1], d);
+        *reinterpret_cast<u32x4*>(row + lds_slot(c.dc, 3) * 16) = decode8(b[2], b[3], d);
+        load(c, t + 2, J & 1);
+    }
+};
+
 constexpr int kConsumers = 512;         // 8 MFMA waves
 constexpr int kProducers = 512;         // 8 waves that fill LDS: waves 8-12 decode weights, waves 13-15 move the x tile
 constexpr int kDecoders = 320;          // producer threads reserved for decoding (two per strip column are used)
@@ -100,8 +348,8 @@ constexpr int kStages = 3;              // LDS tile stages: multiplied, ready (b
 
 // Consumer waves are laid out WM x WN (8 in all); a wave owns RW rows and, when WN == 2, the first CTW or the
 // remaining CT - CTW column tiles.
-template <int RW, int CT, int WN>
-__global__ __launch_bounds__(kGemmAll) void matmul_q4k_bf16_kernel(GemmArgs a)
+template <class F, int RW, int CT, int WN>
+__global__ __launch_bounds__(kGemmAll) void matmul_bf16_kernel(GemmArgs a)
 {
     constexpr int WM = 8 / WN;
     constexpr int BM = WM * RW;
@@ -188,64 +436,24 @@ __global__ __launch_bounds__(kGemmAll) void matmul_q4k_bf16_kernel(GemmArgs a)
             return;
         }
 
-        // ---- decoders (waves 8-12): thread (column dc, half dh) owns bytes [16 dh, 16 dh + 16) of the 32 nibble bytes
-        // of a K slice: 16 low-nibble weights of sub-block 2J and 16 high-nibble weights of sub-block 2J + 1
+        // ---- decoders (waves 8-12): two threads per strip column, see the format's decoder struct
         static_assert(2 * BN <= kDecoders, "two decoding threads per column");
-        const int row_bytes = (a.K >> 8) * 144;
+        const int row_bytes = (a.K >> 8) * F::kBlockBytes;
         const bool d_role = p < 2 * BN;
-        const int dc = d_role ? p >> 1 : 0, dh = p & 1;
-        const uint8_t* wbase = a.w + static_cast<size_t>(n0) * row_bytes;                               // wave-uniform
-        const uint32_t wrow = static_cast<uint32_t>(min(dc, a.N - 1 - n0) * row_bytes);                 // byte offset
-        const int nblocks = a.K >> 8;
-        u32x4 nq[2];                // nibble bytes of K slices t and t + 1
-        u32x4 hdr;                  // header (d, dmin, packed scales) of the next 256-block
-        float sm[16];               // (d * scale, dmin * min) of the eight sub-blocks of the current block
-        auto load_q = [&](int t) {
-            const int tt = min(t, iters - 1);
-            uint32_t off = static_cast<uint32_t>(tt >> 2) * 144u + 16u + static_cast<uint32_t>(tt & 3) * 32u;
-            asm volatile("" : "+s"(off));
-            return ld128(wbase + off + opaque(wrow + static_cast<uint32_t>(dh) * 16u));
-        };
-        auto load_hdr = [&](int blk) {
-            uint32_t off = static_cast<uint32_t>(min(blk, nblocks - 1)) * 144u;
-            asm volatile("" : "+s"(off));
-            hdr = ld128(wbase + off + opaque(wrow));
-        };
-        // FP32 (d * scale, dmin * min) of all eight sub-blocks from a block header; 6-bit fields as in GgufQ4K.cs:51-60:
-        // sub-blocks 0-3 sit in the low six bits of bytes j and 4 + j, 4-7 are split between bytes 8 + j (low nibble
-        // scale, high nibble min) and the top two bits of bytes j and 4 + j
-        auto make_scales = [&]() {
-            const float d = half_bits_to_float(hdr[0]), dmin = half_bits_to_float(hdr[0] >> 16);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const uint32_t b0 = (hdr[1] >> (8 * j)) & 255u, b1 = (hdr[2] >> (8 * j)) & 255u, b2 = (hdr[3] >> (8 * j)) & 255u;
-                sm[2 * j] = d * static_cast<float>(b0 & 63u);
-                sm[2 * j + 1] = dmin * static_cast<float>(b1 & 63u);
-                sm[8 + 2 * j] = d * static_cast<float>((b2 & 15u) | ((b0 >> 6) << 4));
-                sm[8 + 2 * j + 1] = dmin * static_cast<float>((b2 >> 4) | ((b1 >> 6) << 4));
-            }
-        };
-        load_hdr(0);
-        nq[0] = load_q(0);
-        nq[1] = load_q(1);
-        make_scales();
+        DecodeCtx c;
+        c.dc = d_role ? p >> 1 : 0;
+        c.dh = p & 1;
+        c.wbase = a.w + static_cast<size_t>(n0) * row_bytes;                               // wave-uniform
+        c.wrow = static_cast<uint32_t>(min(c.dc, a.N - 1 - n0) * row_bytes);              // byte offset
+        c.iters = iters;
+        c.nblocks = a.K >> 8;
+        F dec;
+        dec.start(c);
         run([&](int t, int stage, auto jt) {
             constexpr int J = decltype(jt)::value;
             if (!d_role) return;
-            const u32x4 q = nq[J & 1];
-            uint8_t* wb = ws + stage * 2 * kWTile + dc * kRowBytes;
-#pragma unroll
-            for (int g = 0; g < 2; ++g) {
-                const uint32_t a0 = q[2 * g], a1 = q[2 * g + 1];
-                const int slot = lds_slot(dc, 2 * dh + g) * 16;
-                *reinterpret_cast<u32x4*>(wb + slot) =
-                    q4k_decode8(a0 & 0x0f0f0f0fu, a1 & 0x0f0f0f0fu, sm[4 * J], sm[4 * J + 1]);
-                *reinterpret_cast<u32x4*>(wb + kWTile + slot) =
-                    q4k_decode8((a0 >> 4) & 0x0f0f0f0fu, (a1 >> 4) & 0x0f0f0f0fu, sm[4 * J + 2], sm[4 * J + 3]);
-            }
-            nq[J & 1] = load_q(t + 2);
-            if (J == 0) load_hdr((t >> 2) + 1);
-            if (J == 3) make_scales();
+            uint8_t* wb = ws + stage * 2 * kWTile + c.dc * kRowBytes;
+            dec.template make<J>(c, t, wb, wb + kWTile);
         });
         return;
     }
@@ -329,28 +537,26 @@ __global__ __launch_bounds__(kGemmAll) void matmul_q4k_bf16_kernel(GemmArgs a)
     else consume(std::integral_constant<int, kLastTiles>{});
 }
 
-template <int RW, int CT, int WN>
+template <class F, int RW, int CT, int WN>
 hipError_t launch_gemm(Lane* lane, const GemmArgs& a, dim3 grid)
 {
     constexpr int BM = (8 / WN) * RW, BN = 16 * CT;
     constexpr size_t lds = static_cast<size_t>(kStages) * 2 * (BM + BN) * kRowBytes;
     static bool configured = false;
     if (lds > 48 * 1024 && !configured) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&matmul_q4k_bf16_kernel<RW, CT, WN>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&matmul_bf16_kernel<F, RW, CT, WN>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
         if (e != hipSuccess) return e;
         configured = true;
     }
-    hipLaunchKernelGGL((matmul_q4k_bf16_kernel<RW, CT, WN>), grid, dim3(kGemmAll), lds, lane->stream, a);
+    hipLaunchKernelGGL((matmul_bf16_kernel<F, RW, CT, WN>), grid, dim3(kGemmAll), lds, lane->stream, a);
     return hipGetLastError();
 }
 
-}  // namespace
-
-hipError_t launch_matmul_bf16(Lane* lane, uint32_t type, const uint16_t* x, const void* w, const float* bias, float* y,
-                              int rows, int in_w, int out_w)
+template <class F>
+hipError_t launch_matmul_of(Lane* lane, const uint16_t* x, const void* w, const float* bias, float* y, int rows, int in_w,
+                            int out_w)
 {
-    if (type != NNHIP_TYPE_Q4_K) return hipErrorNotSupported;
     GemmArgs a{};
     a.x = x;
     a.w = static_cast<const uint8_t*>(w);
@@ -371,9 +577,31 @@ hipError_t launch_matmul_bf16(Lane* lane, uint32_t type, const uint16_t* x, cons
     a.cols = (out_w + strips - 1) / strips;
     a.strips = (out_w + a.cols - 1) / a.cols;
     const dim3 grid(a.strips, m_tiles);
-    if (rows <= 128) return launch_gemm<16, 5, 1>(lane, a, grid);
-    if (rows <= 256) return launch_gemm<32, 5, 1>(lane, a, grid);
-    return launch_gemm<64, 9, 2>(lane, a, grid);
+    if (rows <= 128) return launch_gemm<F, 16, 5, 1>(lane, a, grid);
+    if (rows <= 256) return launch_gemm<F, 32, 5, 1>(lane, a, grid);
+    return launch_gemm<F, 64, 9, 2>(lane, a, grid);
+}
+
+}  // namespace
+
+bool matmul_bf16_supported(uint32_t type, int in_w)
+{
+    switch (type) {
+    case NNHIP_TYPE_Q4_K: case NNHIP_TYPE_Q5_K: case NNHIP_TYPE_Q6_K: case NNHIP_TYPE_Q8_0: return in_w % 256 == 0;
+    default: return false;
+    }
+}
+
+hipError_t launch_matmul_bf16(Lane* lane, uint32_t type, const uint16_t* x, const void* w, const float* bias, float* y,
+                              int rows, int in_w, int out_w)
+{
+    switch (type) {
+    case NNHIP_TYPE_Q4_K: return launch_matmul_of<Q4KDecode>(lane, x, w, bias, y, rows, in_w, out_w);
+    case NNHIP_TYPE_Q5_K: return launch_matmul_of<Q5KDecode>(lane, x, w, bias, y, rows, in_w, out_w);
+    case NNHIP_TYPE_Q6_K: return launch_matmul_of<Q6KDecode>(lane, x, w, bias, y, rows, in_w, out_w);
+    case NNHIP_TYPE_Q8_0: return launch_matmul_of<Q8_0Decode>(lane, x, w, bias, y, rows, in_w, out_w);
+    default: return hipErrorNotSupported;
+    }
 }
 
 }  // namespace nnhip

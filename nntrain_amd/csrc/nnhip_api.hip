@@ -553,6 +553,8 @@ int nnhip_quant_matmul_bf16(void* handle, uint32_t ggml_type, const uint16_t* x_
     NNHIP_LANE(handle, NNHIP_OP_MATMUL_BF16)
     int rc = check_linear(NNHIP_OP_MATMUL_BF16, lane, ggml_type, x_bf16, w, y, rows, in_w, out_w);
     if (rc != NNHIP_OK) return rc;
+    if (in_w % 256 != 0 && matmul_bf16_supported(ggml_type, 256))
+        return fail(NNHIP_ERR_INCOMPLETE_BLOCKS, NNHIP_OP_MATMUL_BF16, lane->device, 0, "the bf16 prefill mat-mul needs in_w to be a multiple of 256 (got %d)", in_w);
     hipError_t e = launch_matmul_bf16(lane, ggml_type, x_bf16, w, bias, y, rows, in_w, out_w);
     if (e == hipErrorNotSupported)
         return fail(NNHIP_ERR_UNSUPPORTED_TYPE, NNHIP_OP_MATMUL_BF16, lane->device, 0, "bf16 prefill mat-mul does not support GGML type %u", ggml_type);

@@ -65,6 +65,8 @@ hipError_t launch_add_in_place(Lane* lane, float* destination, const float* sour
 hipError_t launch_first_token_attention(Lane* lane, const float* v, float* out, int heads, int kv_heads, int head_width);
 hipError_t launch_lora_a(Lane* lane, const float* x, const float* a, float* z, int rows, int width, int rank);
 hipError_t launch_lora_b(Lane* lane, const float* z, const float* b, float* y, int rows, int output, int rank, float scale);
+// Storage types and widths the bf16 prefill mat-mul covers.
+bool matmul_bf16_supported(uint32_t type, int in_w);
 hipError_t launch_fill_u32(Lane* lane, uint32_t* p, uint32_t value, size_t count);
 
 // Largest in_w the mat-vec kernels can stage in LDS.
