@@ -531,11 +531,11 @@ def run_decode_loop(args, lane, nn, oracle):
 
 def run_prefill(args, lane, nn, oracle):
     """Q4_K 17408x5120 bf16-MFMA prefill mat-mul at M = 128, 256, 512, 2048 (BASELINE configs[3]); the other formats
-    the kernel decodes (Q5_K, Q6_K, Q8_0) at M = 512 under "other_formats"."""
+    the kernel decodes (Q5_K, Q6_K, Q8_0, IQ2_S, IQ3_S) at M = 512 under "other_formats"."""
     out = _prefill_of(lane, nn, oracle, nn.GGML_Q4_K, "Q4_K", (128, 256, 512, 2048))
     if out is not None:
         out["other_formats"] = {}
-        for tname in ("Q5_K", "Q6_K", "Q8_0"):
+        for tname in ("Q5_K", "Q6_K", "Q8_0", "IQ2_S", "IQ3_S"):
             res = _prefill_of(lane, nn, oracle, getattr(nn, "GGML_" + tname), tname, (512,))
             if res is not None:
                 out["other_formats"][tname] = res["M=512"]

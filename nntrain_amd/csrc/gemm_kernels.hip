@@ -1,4 +1,4 @@
-// Prefill mat-mul for raw GGUF block-quantized weights (Q4_K, Q5_K, Q6_K, Q8_0) on gfx950:
+// Prefill mat-mul for raw GGUF block-quantized weights (Q4_K, Q5_K, Q6_K, Q8_0, IQ2_S, IQ3_S) on gfx950:
 // y[M, N] = bias + x[M, K] (bf16) . W[N, K]^T.
 //
 // Replaces the XMX prefill launches of the reference (NNtrain.Arc/Kernels/qwen35_prefill_xmx.cl:112-184, the
@@ -35,6 +35,8 @@
 
 #include "nnhip_internal.h"
 #include "quant_device.h"
+
+#include "iq_grids.inc"
 
 namespace nnhip {
 
@@ -339,6 +341,172 @@ struct Q8_0Decode {
     }
 };
 
+// The codebooks of the IQ formats (read through the vector caches: the LDS of this kernel is taken by the tile stages).
+__device__ const uint64_t g_iq2s_grid_mm[1024] = { NNHIP_IQ2S_GRID_VALUES };
+__device__ const uint32_t g_iq3s_grid_mm[512] = { NNHIP_IQ3S_GRID_VALUES };
+
+// bf16 pair of two magnitudes times db with their sign bits (bit 0 of `signs`: first weight, bit 1: second)
+__device__ __forceinline__ uint32_t iq_pair(float db, float m0, float m1, uint32_t signs)
+{
+    return pack_bf16(db * m0, db * m1) ^ (((signs & 1u) << 15) | ((signs & 2u) << 30));
+}
+
+// IQ2_S (82 bytes: d, 32 index bytes, 32 sign bytes, qh[8], scales[8]; NNtrain.Arc/Kernels/qwen35_iq.cl:411-419): thread
+// dh decodes 32-weight group 2 (t % 4) + dh of block t / 4, a whole 64-byte row of its sub-tile = four codebook entries
+// of eight magnitudes.  Index and sign bytes are requested three slices ahead, the codebook entries one slice ahead (from
+// indices that arrived two slices earlier), qh / scales / d of a block a block ahead.
+struct IQ2SDecode {
+    static constexpr int kBlockBytes = 82;
+    uint32_t qs[4], sg[4];      // index and sign bytes of slices t .. t + 3 (set = slice % 4)
+    u32x2 grid[2][4];           // codebook entries of slices t, t + 1 (set = slice % 2)
+    u32x4 tail, tail_next;      // qh[8] | scales[8] of the current and the next block
+    uint32_t dbits, dbits_next;
+
+    __device__ __forceinline__ void load_raw(const DecodeCtx& c, int t, int set)
+    {
+        const int tt = min(t, c.iters - 1);
+        uint32_t off = static_cast<uint32_t>(tt >> 2) * 82u + static_cast<uint32_t>(tt & 3) * 8u;
+        asm volatile("" : "+s"(off));
+        const uint8_t* p = c.wbase + off + opaque(c.wrow + static_cast<uint32_t>(c.dh) * 4u);
+        qs[set] = ld32(p + 2);
+        sg[set] = ld32(p + 34);
+    }
+    __device__ __forceinline__ void load_hdr(const DecodeCtx& c, int blk)
+    {
+        uint32_t off = static_cast<uint32_t>(min(blk, c.nblocks - 1)) * 82u;
+        tail_next = gld128(c, off + 66u, 0u);
+        asm volatile("" : "+s"(off));
+        dbits_next = ld16(c.wbase + off + opaque(c.wrow));
+    }
+    // requests the entries of group 2 J + dh whose index bytes are `q`, high bits taken from `tl`
+    template <int J>
+    __device__ __forceinline__ void load_grid(const DecodeCtx& c, uint32_t q, const u32x4& tl, u32x2* out)
+    {
+        const uint32_t qh = (tl[J >> 1] >> (16 * (J & 1) + 8 * c.dh)) & 0xffu;
+#pragma unroll
+        for (int o = 0; o < 4; ++o) {
+            const uint32_t idx = ((q >> (8 * o)) & 0xffu) | (((qh >> (2 * o)) & 3u) << 8);
+            const uint64_t v = g_iq2s_grid_mm[idx];
+            out[o] = u32x2{static_cast<uint32_t>(v), static_cast<uint32_t>(v >> 32)};
+        }
+    }
+    __device__ __forceinline__ void start(const DecodeCtx& c)
+    {
+        load_hdr(c, 0);
+        tail = tail_next;
+        dbits = dbits_next;
+        load_hdr(c, 1);
+        load_raw(c, 0, 0);
+        load_raw(c, 1, 1);
+        load_raw(c, 2, 2);
+        load_grid<0>(c, qs[0], tail, grid[0]);
+    }
+    template <int J>
+    __device__ __forceinline__ void make(const DecodeCtx& c, int t, uint8_t* lo, uint8_t* hi)
+    {
+        const float d = half_bits_to_float(dbits);
+        const uint32_t scl = (tail[2 + (J >> 1)] >> (16 * (J & 1) + 8 * c.dh)) & 0xffu;
+        const float db_lo = (d * (0.5f + static_cast<float>(scl & 15u))) * 0.25f;
+        const float db_hi = (d * (0.5f + static_cast<float>(scl >> 4))) * 0.25f;
+        uint8_t* row = c.dh ? hi : lo;
+        const uint32_t signs = sg[J];
+#pragma unroll
+        for (int o = 0; o < 4; ++o) {
+            const uint32_t m0 = grid[J & 1][o][0], m1 = grid[J & 1][o][1], sb = signs >> (8 * o);
+            const float db = o < 2 ? db_lo : db_hi;
+            *reinterpret_cast<u32x4*>(row + lds_slot(c.dc, o) * 16) =
+                u32x4{iq_pair(db, ubyte0(m0), ubyte1(m0), sb), iq_pair(db, ubyte2(m0), ubyte3(m0), sb >> 2),
+                      iq_pair(db, ubyte0(m1), ubyte1(m1), sb >> 4), iq_pair(db, ubyte2(m1), ubyte3(m1), sb >> 6)};
+        }
+        // slice t + 1 belongs to the next block when J == 3
+        load_grid<(J + 1) & 3>(c, qs[(J + 1) & 3], J == 3 ? tail_next : tail, grid[(J + 1) & 1]);
+        load_raw(c, t + 3, (J + 3) & 3);
+        if (J == 3) {
+            tail = tail_next;
+            dbits = dbits_next;
+        }
+        if (J == 0) load_hdr(c, (t >> 2) + 1);
+    }
+};
+
+// IQ3_S (110 bytes: d, 64 index bytes, qh[8], 32 sign bytes, scales[4]; qwen35_iq.cl:421-429): as IQ2_S with eight
+// codebook entries of four magnitudes per 32-weight group and w = (d * (1 + 2 s)) * magnitude * sign.
+struct IQ3SDecode {
+    static constexpr int kBlockBytes = 110;
+    u32x2 qs[4];                // eight index bytes of slices t .. t + 3
+    uint32_t sg[4];
+    uint32_t grid[2][8];
+    u32x2 qh, qh_next;          // ninth index bits, a byte per group
+    uint32_t scales, scales_next;
+    uint32_t dbits, dbits_next;
+
+    __device__ __forceinline__ void load_raw(const DecodeCtx& c, int t, int set)
+    {
+        const int tt = min(t, c.iters - 1);
+        uint32_t off = static_cast<uint32_t>(tt >> 2) * 110u;
+        const uint32_t g = static_cast<uint32_t>(tt & 3) * 2u + static_cast<uint32_t>(c.dh);
+        asm volatile("" : "+s"(off));
+        const uint8_t* p = c.wbase + off;
+        qs[set] = ld64(p + 2 + opaque(c.wrow + g * 8u));
+        sg[set] = ld32(p + 74 + opaque(c.wrow + g * 4u));
+    }
+    __device__ __forceinline__ void load_hdr(const DecodeCtx& c, int blk)
+    {
+        uint32_t off = static_cast<uint32_t>(min(blk, c.nblocks - 1)) * 110u;
+        asm volatile("" : "+s"(off));
+        const uint8_t* p = c.wbase + off + opaque(c.wrow);
+        qh_next = ld64(p + 66);
+        scales_next = ld32(p + 106);
+        dbits_next = ld16(p);
+    }
+    template <int J>
+    __device__ __forceinline__ void load_grid(const DecodeCtx& c, const u32x2 q, const u32x2 high, uint32_t* out)
+    {
+        const uint32_t hb = (high[J >> 1] >> (16 * (J & 1) + 8 * c.dh)) & 0xffu;
+#pragma unroll
+        for (int o = 0; o < 8; ++o) {
+            const uint32_t idx = ((q[o >> 2] >> (8 * (o & 3))) & 0xffu) | (((hb >> o) & 1u) << 8);
+            out[o] = g_iq3s_grid_mm[idx];
+        }
+    }
+    __device__ __forceinline__ void start(const DecodeCtx& c)
+    {
+        load_hdr(c, 0);
+        qh = qh_next;
+        scales = scales_next;
+        dbits = dbits_next;
+        load_hdr(c, 1);
+        load_raw(c, 0, 0);
+        load_raw(c, 1, 1);
+        load_raw(c, 2, 2);
+        load_grid<0>(c, qs[0], qh, grid[0]);
+    }
+    template <int J>
+    __device__ __forceinline__ void make(const DecodeCtx& c, int t, uint8_t* lo, uint8_t* hi)
+    {
+        // group 2 J + dh: its scale nibble is nibble (2 J + dh) of the four scale bytes
+        const uint32_t sub = (scales >> (8 * J + 4 * c.dh)) & 15u;
+        const float db = half_bits_to_float(dbits) * static_cast<float>(1u + 2u * sub);
+        uint8_t* row = c.dh ? hi : lo;
+        const uint32_t signs = sg[J];
+#pragma unroll
+        for (int o = 0; o < 4; ++o) {
+            const uint32_t m0 = grid[J & 1][2 * o], m1 = grid[J & 1][2 * o + 1], sb = signs >> (8 * o);
+            *reinterpret_cast<u32x4*>(row + lds_slot(c.dc, o) * 16) =
+                u32x4{iq_pair(db, ubyte0(m0), ubyte1(m0), sb), iq_pair(db, ubyte2(m0), ubyte3(m0), sb >> 2),
+                      iq_pair(db, ubyte0(m1), ubyte1(m1), sb >> 4), iq_pair(db, ubyte2(m1), ubyte3(m1), sb >> 6)};
+        }
+        load_grid<(J + 1) & 3>(c, qs[(J + 1) & 3], J == 3 ? qh_next : qh, grid[(J + 1) & 1]);
+        load_raw(c, t + 3, (J + 3) & 3);
+        if (J == 3) {
+            qh = qh_next;
+            scales = scales_next;
+            dbits = dbits_next;
+        }
+        if (J == 0) load_hdr(c, (t >> 2) + 1);
+    }
+};
+
 constexpr int kConsumers = 512;         // 8 MFMA waves
 constexpr int kProducers = 512;         // 8 waves that fill LDS: waves 8-12 decode weights, waves 13-15 move the x tile
 constexpr int kDecoders = 320;          // producer threads reserved for decoding (two per strip column are used)
@@ -587,7 +755,8 @@ hipError_t launch_matmul_of(Lane* lane, const uint16_t* x, const void* w, const 
 bool matmul_bf16_supported(uint32_t type, int in_w)
 {
     switch (type) {
-    case NNHIP_TYPE_Q4_K: case NNHIP_TYPE_Q5_K: case NNHIP_TYPE_Q6_K: case NNHIP_TYPE_Q8_0: return in_w % 256 == 0;
+    case NNHIP_TYPE_Q4_K: case NNHIP_TYPE_Q5_K: case NNHIP_TYPE_Q6_K: case NNHIP_TYPE_Q8_0: case NNHIP_TYPE_IQ2_S:
+    case NNHIP_TYPE_IQ3_S: return in_w % 256 == 0;
     default: return false;
     }
 }
@@ -600,6 +769,8 @@ hipError_t launch_matmul_bf16(Lane* lane, uint32_t type, const uint16_t* x, cons
     case NNHIP_TYPE_Q5_K: return launch_matmul_of<Q5KDecode>(lane, x, w, bias, y, rows, in_w, out_w);
     case NNHIP_TYPE_Q6_K: return launch_matmul_of<Q6KDecode>(lane, x, w, bias, y, rows, in_w, out_w);
     case NNHIP_TYPE_Q8_0: return launch_matmul_of<Q8_0Decode>(lane, x, w, bias, y, rows, in_w, out_w);
+    case NNHIP_TYPE_IQ2_S: return launch_matmul_of<IQ2SDecode>(lane, x, w, bias, y, rows, in_w, out_w);
+    case NNHIP_TYPE_IQ3_S: return launch_matmul_of<IQ3SDecode>(lane, x, w, bias, y, rows, in_w, out_w);
     default: return hipErrorNotSupported;
     }
 }

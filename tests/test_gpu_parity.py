@@ -329,7 +329,7 @@ def _bf16_weight_product(typ, payload, xb, bias, rows, in_w, out_w):
     return y if bias is None else y + np.asarray(bias, dtype=np.float64)
 
 
-PREFILL_TYPES = [GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_Q8_0]
+PREFILL_TYPES = [GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_Q8_0, GGML_IQ2_S, GGML_IQ3_S]
 
 
 @pytest.mark.parametrize("typ", PREFILL_TYPES)
@@ -361,11 +361,12 @@ def test_prefill_matmul_vs_oracle(lane, typ, rows, in_w, out_w):
 
 
 def test_prefill_matmul_rejects_other_types_and_widths(lane):
-    mat = HipQuantizedMatrix(synth.matrix(GGML_IQ2_S, 1, 256, 1), GGML_IQ2_S, 1, 256)
+    from nntrain_amd import GGML_BF16
+    mat = HipQuantizedMatrix(np.zeros(2 * 256, np.uint8), GGML_BF16, 1, 256)
     x = lane.allocate(256)
     with pytest.raises(NnHipError) as e:
         mat.forward_bf16(lane, x, None, 1)
-    assert e.value.status == 2                      # no codebook formats in the prefill mat-mul
+    assert e.value.status == 2                      # unquantized bfloat16 matrices have no prefill mat-mul
     mat.dispose()
     mat = HipQuantizedMatrix(np.zeros(34 * 4, np.uint8), GGML_Q8_0, 1, 128)
     with pytest.raises(NnHipError) as e:
@@ -375,7 +376,7 @@ def test_prefill_matmul_rejects_other_types_and_widths(lane):
     mat.dispose()
 
 
-@pytest.mark.parametrize("typ", [GGML_Q5_K, GGML_Q6_K, GGML_Q8_0])
+@pytest.mark.parametrize("typ", [GGML_Q5_K, GGML_Q6_K, GGML_Q8_0, GGML_IQ2_S, GGML_IQ3_S])
 def test_prefill_matmul_model_width_sample(lane, typ):
     """A 5120-wide strip at M = 512 (the 256-row tiles, nine column tiles) for the other formats."""
     in_w, out_w, rows = 5120, 1500, 512
