@@ -541,6 +541,9 @@ __global__ __launch_bounds__(kGemmAll) void matmul_bf16_kernel(GemmArgs a)
         // Both producer roles make slices 0 and 1 before the first barrier and then, between two barriers, slice
         // i + 2 while slice i is multiplied.  Everything a role consumes was requested two slices earlier.  The
         // roles are separate code paths so that each is allocated only its own registers.
+        // With 128-row tiles the decoders are what an iteration waits for, with 256-row tiles the matrix pipes:
+        // the group on the critical path gets the higher issue priority (measured: +3 % at M = 128, +2.5 % at M = 2048).
+        if constexpr (BM <= 128) __builtin_amdgcn_s_setprio(3);
         const int p = tid - kConsumers;
         // K is a whole number of 256-blocks, so iters is a multiple of 4; `make(t, stage)` is given t % 4 statically
         auto run = [&](auto&& make) {
@@ -628,6 +631,7 @@ __global__ __launch_bounds__(kGemmAll) void matmul_bf16_kernel(GemmArgs a)
 
     // ---------------------------------------------------------------------------------------------- consumers
     // waves w and w + 4 usually share a SIMD: giving them different column halves balances the matrix pipes
+    if constexpr (BM > 128) __builtin_amdgcn_s_setprio(3);
     const int wm = wave % WM, wn = wave / WM;
     const int ct0 = wn * CTW;                       // this wave's column tiles start here
     // operand address of this lane inside a 16-row tile: row lane % 16, k-group lane / 16
