@@ -191,8 +191,8 @@ NNHIP_API int nnhip_quant_matvec_batch(void* lane, const nnhip_matvec_desc* desc
  * weight tiles are dequantized to bfloat16 in LDS and contracted on MFMA with FP32 accumulators.  Replaces the
  * XMX prefill launch of Matrix.Forward for rows >= 16 (Qwen35QuantizedModel.cs:1249-1317, kernels
  * q35l_prefill_xmx_<format>_f16x2, NNtrain.Arc/Kernels/qwen35_prefill_xmx.cl:112-184).  Storage types Q4_K, Q5_K,
- * Q6_K, Q8_0, IQ2_S and IQ3_S with in_w a multiple of 256 (NNHIP_ERR_INCOMPLETE_BLOCKS otherwise); unquantized
- * bfloat16 returns NNHIP_ERR_UNSUPPORTED_TYPE (its rows go through nnhip_quant_matvec).  Asynchronous. */
+ * Q6_K, Q8_0, IQ2_S, IQ3_S and unquantized bfloat16 with in_w a multiple of 256 (NNHIP_ERR_INCOMPLETE_BLOCKS
+ * otherwise).  Asynchronous. */
 NNHIP_API int nnhip_quant_matmul_bf16(void* lane, uint32_t ggml_type, const uint16_t* x_bf16, const void* w,
                                       const float* bias, float* y, int rows, int in_w, int out_w);
 

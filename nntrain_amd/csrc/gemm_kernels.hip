@@ -1,4 +1,4 @@
-// Prefill mat-mul for raw GGUF block-quantized weights (Q4_K, Q5_K, Q6_K, Q8_0, IQ2_S, IQ3_S) on gfx950:
+// Prefill mat-mul for raw GGUF block-quantized weights (Q4_K, Q5_K, Q6_K, Q8_0, IQ2_S, IQ3_S) and bfloat16 matrices on gfx950:
 // y[M, N] = bias + x[M, K] (bf16) . W[N, K]^T.
 //
 // Replaces the XMX prefill launches of the reference (NNtrain.Arc/Kernels/qwen35_prefill_xmx.cl:112-184, the
@@ -507,6 +507,34 @@ struct IQ3SDecode {
     }
 };
 
+// Unquantized bfloat16 weights (matrix storage type 30, and the scratch copy the two-pass path decodes into): thread dh
+// copies weights [32 dh, 32 dh + 32) of the slice, a whole 64-byte row of its sub-tile.
+struct BF16Decode {
+    static constexpr int kBlockBytes = 512;        // bytes per 256 weights
+    u32x4 q[2][4];
+
+    __device__ __forceinline__ void load(const DecodeCtx& c, int t, int set)
+    {
+        const uint32_t off = static_cast<uint32_t>(min(t, c.iters - 1)) * 128u;
+        const uint32_t lane_off = static_cast<uint32_t>(c.dh) * 64u;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) q[set][g] = gld128(c, off + 16u * g, lane_off);
+    }
+    __device__ __forceinline__ void start(const DecodeCtx& c)
+    {
+        load(c, 0, 0);
+        load(c, 1, 1);
+    }
+    template <int J>
+    __device__ __forceinline__ void make(const DecodeCtx& c, int t, uint8_t* lo, uint8_t* hi)
+    {
+        uint8_t* row = c.dh ? hi : lo;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) *reinterpret_cast<u32x4*>(row + lds_slot(c.dc, g) * 16) = q[J & 1][g];
+        load(c, t + 2, J & 1);
+    }
+};
+
 constexpr int kConsumers = 512;         // 8 MFMA waves
 constexpr int kProducers = 512;         // 8 waves that fill LDS: waves 8-12 decode weights, waves 13-15 move the x tile
 constexpr int kDecoders = 320;          // producer threads reserved for decoding (two per strip column are used)
@@ -760,7 +788,7 @@ bool matmul_bf16_supported(uint32_t type, int in_w)
 {
     switch (type) {
     case NNHIP_TYPE_Q4_K: case NNHIP_TYPE_Q5_K: case NNHIP_TYPE_Q6_K: case NNHIP_TYPE_Q8_0: case NNHIP_TYPE_IQ2_S:
-    case NNHIP_TYPE_IQ3_S: return in_w % 256 == 0;
+    case NNHIP_TYPE_IQ3_S: case NNHIP_TYPE_BF16: return in_w % 256 == 0;
     default: return false;
     }
 }
@@ -775,6 +803,7 @@ hipError_t launch_matmul_bf16(Lane* lane, uint32_t type, const uint16_t* x, cons
     case NNHIP_TYPE_Q8_0: return launch_matmul_of<Q8_0Decode>(lane, x, w, bias, y, rows, in_w, out_w);
     case NNHIP_TYPE_IQ2_S: return launch_matmul_of<IQ2SDecode>(lane, x, w, bias, y, rows, in_w, out_w);
     case NNHIP_TYPE_IQ3_S: return launch_matmul_of<IQ3SDecode>(lane, x, w, bias, y, rows, in_w, out_w);
+    case NNHIP_TYPE_BF16: return launch_matmul_of<BF16Decode>(lane, x, w, bias, y, rows, in_w, out_w);
     default: return hipErrorNotSupported;
     }
 }

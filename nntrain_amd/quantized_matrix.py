@@ -182,8 +182,8 @@ class HipQuantizedMatrix:
 
     def forward_bf16(self, lane: HipExecutionLane, x_bf16: HipBuffer, bias: HipBuffer | None, rows: int,
                      out: HipBuffer | None = None) -> HipBuffer:
-        """Prefill: x holds bfloat16 bit patterns [rows, in]; bf16 MFMA with FP32 accumulation.  Every block format
-        with in_w a multiple of 256; unquantized bfloat16 matrices raise NnHipError (unsupported type)."""
+        """Prefill: x holds bfloat16 bit patterns [rows, in]; bf16 MFMA with FP32 accumulation.  Every storage
+        type with in_w a multiple of 256."""
         if rows < 1:
             raise ValueError("rows must be positive.")
         if x_bf16.nbytes < 2 * rows * self.input_width:

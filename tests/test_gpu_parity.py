@@ -361,13 +361,15 @@ def test_prefill_matmul_vs_oracle(lane, typ, rows, in_w, out_w):
 
 
 def test_prefill_matmul_rejects_other_types_and_widths(lane):
-    from nntrain_amd import GGML_BF16
-    mat = HipQuantizedMatrix(np.zeros(2 * 256, np.uint8), GGML_BF16, 1, 256)
+    from ctypes import c_void_p
     x = lane.allocate(256)
-    with pytest.raises(NnHipError) as e:
-        mat.forward_bf16(lane, x, None, 1)
-    assert e.value.status == 2                      # unquantized bfloat16 matrices have no prefill mat-mul
-    mat.dispose()
+    w = lane.allocate(256)
+    y = lane.allocate(4)
+    # GGML type 2 (Q4_0) is no matrix storage of the reference (Qwen35Gguf.cs:12-13)
+    status = lane._lib.nnhip_quant_matmul_bf16(lane._handle, 2, c_void_p(x.ptr), c_void_p(w.ptr), None, c_void_p(y.ptr), 1, 256, 1)
+    assert status == 2
+    w.dispose()
+    y.dispose()
     mat = HipQuantizedMatrix(np.zeros(34 * 4, np.uint8), GGML_Q8_0, 1, 128)
     with pytest.raises(NnHipError) as e:
         mat.forward_bf16(lane, x, None, 1)
@@ -411,6 +413,25 @@ def test_prefill_matmul_full_width_sample(lane):
 
 
 # ----------------------------------------------------------------------------------------------- bfloat16 storage
+
+def test_prefill_matmul_bf16_weights(lane):
+    """Unquantized bfloat16 matrices through the prefill mat-mul: the weights are exact, so the product agrees with
+    float64 to FP32 accumulation accuracy."""
+    from nntrain_amd import GGML_BF16
+    for rows, in_w, out_w in [(16, 256, 16), (200, 768, 160), (512, 1024, 300), (300, 2304, 130)]:
+        rng = np.random.default_rng(rows + in_w)
+        wb = synth.to_bf16_bits(rng.standard_normal((out_w, in_w), dtype=np.float32) * np.float32(0.02))
+        xb = synth.to_bf16_bits(synth.activations(rows, in_w, seed=29))
+        bias = rng.standard_normal(out_w).astype(np.float32) * np.float32(0.01)
+        mat = HipQuantizedMatrix(wb.view(np.uint8).reshape(-1), GGML_BF16, out_w, in_w)
+        x, b = lane.upload_raw(xb), lane.upload_raw(bias)
+        got = lane.read(mat.forward_bf16(lane, x, b, rows)).reshape(rows, out_w)
+        ref = oracle.bf16_widen(xb).astype(np.float64) @ oracle.bf16_widen(wb).astype(np.float64).T + bias.astype(np.float64)
+        assert oracle.rel_l2(got, ref) <= PREFILL_TIGHT_BAR
+        x.dispose()
+        b.dispose()
+        mat.dispose()
+
 
 def test_bf16_matrix_storage(lane):
     """Unquantized bfloat16 matrices (the reference's "bf16" matrix storage, Qwen35Gguf.cs:12-13): widening is exact,
