@@ -17,6 +17,7 @@
 //     the row's partials in a fixed order (lane-strided, then a DPP butterfly) and stores y.  The order depends only
 //     on in_w, never on the launch geometry, so a row's result is bit-identical for any `rows`, out_w or batching.
 #include <cstring>
+#include <type_traits>
 #include <vector>
 
 #include "nnhip_internal.h"
@@ -49,6 +50,7 @@ struct MatvecArgs {
     int steps;             // ceil(out_w / RS)
     uint32_t row_bytes;
     uint32_t magic;        // ceil(2^32 / units_per_row): t / units_per_row == umulhi(t, magic) for t < 2^32 / upr
+    int rows;              // input rows of the call (grid.y covers them MR at a time)
     // fused variants only (null / unused otherwise)
     const float* x2;       // RMSNorm: residual added to x first (or null); SiLU: the `up` vector
     const float* gamma;    // RMSNorm weight
@@ -534,12 +536,18 @@ template <> struct Shape<BF16Unit> { static constexpr int kMaxT = 512, kWavesPer
 // summation order of q35a_add_rms_norm / q35a_rms_norm (NNtrain.Arc/Kernels/qwen35_attention.cl:16-78: 128 lane-strided
 // partial sums, halving tree); SiLU(x) * x2 (qwen35_attention.cl:38-43).  Every workgroup prepares the whole vector
 // for itself; workgroup 0 also stores it (and the residual sum) where the caller asked.
-template <class Q, int PRE = kPreNone>
+// MR > 1 (plain launches with several input rows; the reference routes 1 < rows to a row-tiled kernel,
+// NNtrain.Core/Modules/Qwen35QuantizedModel.cs:1340-1344): a workgroup multiplies every row step by MR input rows, so the
+// weights are streamed once per MR rows.  A lane cannot hold MR x 64 activations in registers: the vectors stay in LDS and
+// the lane re-reads its 64 values of a row for every step; the arithmetic and the summation order per input row are
+// those of MR = 1, so results do not depend on how the rows were grouped.
+template <class Q, int PRE = kPreNone, int MR = 1>
 __global__ __launch_bounds__(Shape<Q>::kMaxT) __attribute__((amdgpu_waves_per_eu(Shape<Q>::kWavesPerEu, Shape<Q>::kWavesPerEu)))
 void matvec_rowstep_kernel(MatvecArgs a, const float* __restrict__ bias)
 {
+    static_assert(MR == 1 || PRE == kPreNone, "row tiling is for plain launches");
     constexpr int kDepth = Shape<Q>::kDepth;
-    __shared__ float part[2][kMaxWG];
+    __shared__ float part[2][MR * kMaxWG];
     __shared__ __attribute__((aligned(8))) uint32_t grid[Q::kGridWords ? Q::kGridWords : 2];
 
     const int tid = threadIdx.x;
@@ -547,8 +555,9 @@ void matvec_rowstep_kernel(MatvecArgs a, const float* __restrict__ bias)
     const int rl = upr == 1 ? tid : static_cast<int>(__umulhi(static_cast<uint32_t>(tid), a.magic));  // row within a step
     const int c = tid - rl * upr;                                                                    // unit within the row
     const bool owner = rl < rs;
-    const float* x = a.x + static_cast<size_t>(blockIdx.y) * a.in_w;
-    float* y = a.y + static_cast<size_t>(blockIdx.y) * a.out_w;
+    const int row0 = blockIdx.y * MR;                          // first input row of this workgroup
+    const float* x = a.x + static_cast<size_t>(row0) * a.in_w;
+    float* y = a.y + static_cast<size_t>(row0) * a.out_w;
     const int last_row = a.out_w - 1;
 
     // Loads are unconditional: rows past the end re-read the last row, spare lanes re-read row 0 (both stay in L2),
@@ -660,11 +669,19 @@ void matvec_rowstep_kernel(MatvecArgs a, const float* __restrict__ bias)
         if (tid < pieces) xstage[tid + (tid >> 4)] = xv0;
         if (tid + T < pieces) xstage[tid + T + ((tid + T) >> 4)] = xv1;
         for (int L = tid + 2 * T; L < pieces; L += T) xstage[L + (L >> 4)] = xg[L];
+        // the other input rows of the tile, each in a staging area of its own (rows past the last one: zeros)
+        for (int m = 1; m < MR; ++m) {
+            float4* xm = xstage + m * kChunkPieces * upr;
+            const bool have = row0 + m < a.rows;
+            for (int L = tid; L < pieces; L += T)
+                xm[L + (L >> 4)] = have ? xg[m * pieces + L] : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
     }
     if constexpr (Q::kGridWords > 0)
         for (int i = tid; i < Q::kGridWords; i += T) grid[i] = Q::grid_table()[i];
     __syncthreads();
-    typename Q::X xr = Q::load_x(xstage, owner ? c : 0);
+    typename Q::X xr{};
+    if constexpr (MR == 1) xr = Q::load_x(xstage, owner ? c : 0);
 
     // Row results are collected in LDS and stored to memory in bursts (when the buffer is full, and at the end), so
     // the steady state has no vector-memory traffic besides the weight stream.
@@ -675,10 +692,11 @@ void matvec_rowstep_kernel(MatvecArgs a, const float* __restrict__ bias)
     int first_held = step;        // step number of ybuf[0 .. rs)
     auto flush = [&]() {
         __syncthreads();
-        for (int i = tid; i < held * rs; i += T) {
-            const int j = i / rs;
-            const int row = (first_held + j * stride) * rs + (i - j * rs);
-            if (row < a.out_w) {
+        for (int i = tid; i < held * rs * MR; i += T) {
+            const int j = i / (rs * MR), rem = i - j * rs * MR;
+            const int m = MR == 1 ? 0 : rem / rs;
+            const int row = (first_held + j * stride) * rs + (rem - m * rs);
+            if (row < a.out_w && (MR == 1 || row0 + m < a.rows)) {
                 float v = ybuf[i];
                 if (a.lora_rank > 0) {      // the branch of q35l_*_sg16_lora (NNtrain.Arc/Kernels/qwen35_linear_fast.cl:262-268)
                     const float* br = a.lora_b + static_cast<size_t>(row) * a.lora_rank;
@@ -686,24 +704,35 @@ void matvec_rowstep_kernel(MatvecArgs a, const float* __restrict__ bias)
                     for (int r = 0; r < a.lora_rank; ++r) sum = fmaf(a.lora_z[r], br[r], sum);
                     v = v + a.lora_scale * sum;
                 }
-                y[row] = a.addend ? a.addend[row] + v : v;
+                y[static_cast<size_t>(m) * a.out_w + row] = a.addend ? a.addend[row] + v : v;
             }
         }
         held = 0;
     };
     auto finish = [&](const typename Q::Regs& r, int st) {
-        part[buf][tid] = Q::dot(r, xr, c, grid);
+        if constexpr (MR == 1) {
+            part[buf][tid] = Q::dot(r, xr, c, grid);
+        } else {
+#pragma unroll 1
+            for (int m = 0; m < MR; ++m) {
+                if (row0 + m < a.rows) {          // (workgroup-uniform)
+                    const typename Q::X xm = Q::load_x(xstage + m * kChunkPieces * upr, owner ? c : 0);
+                    part[buf][m * kMaxWG + tid] = Q::dot(r, xm, c, grid);
+                }
+            }
+        }
         __syncthreads();
-        for (int rr = wave; rr < rs; rr += waves) {
-            const int row = st * rs + rr;
-            if (row < a.out_w) {
+        for (int rr = wave; rr < rs * MR; rr += waves) {
+            const int m = MR == 1 ? 0 : rr / rs, r0 = rr - m * rs;
+            const int row = st * rs + r0;
+            if (row < a.out_w && (MR == 1 || row0 + m < a.rows)) {
                 float t = 0.0f;
-                for (int u = lane; u < upr; u += 64) t += part[buf][rr * upr + u];
+                for (int u = lane; u < upr; u += 64) t += part[buf][m * kMaxWG + r0 * upr + u];
                 t = wave_sum(t);
                 // the row index is wave-uniform: the bias comes through the scalar cache and does not wait on the
                 // vector-memory counter that the prefetched weights are tracked by
                 const int urow = __builtin_amdgcn_readfirstlane(row);
-                if (lane == 0) ybuf[held * rs + rr] = (bias ? bias[urow] : 0.0f) + t;
+                if (lane == 0) ybuf[(held * MR + m) * rs + r0] = (bias ? bias[urow] : 0.0f) + t;
             }
         }
         buf ^= 1;
@@ -720,7 +749,7 @@ void matvec_rowstep_kernel(MatvecArgs a, const float* __restrict__ bias)
             finish(regs[d], step);
             step += stride;
         }
-        if ((held + kDepth) * rs > kYBuf) {         // rare: only matrices with very many rows per workgroup get here
+        if ((held + kDepth) * rs * MR > kYBuf) {         // rare: only matrices with very many rows per workgroup get here
             flush();
             __builtin_amdgcn_s_waitcnt(kWaitVm0);
             __syncthreads();
@@ -990,6 +1019,24 @@ bool plan(int in_w, int out_w, int compute_units, int max_t, Geometry* g)
     return true;
 }
 
+// Dynamic LDS a row-tiled launch may use: every further input row of the tile costs 8 KB of static partial sums.
+constexpr int max_dynamic_lds(int mr) { return kMaxDynamicLds - (mr - 1) * 2 * kMaxWG * static_cast<int>(sizeof(float)); }
+
+template <class Q, int PRE, int MR>
+hipError_t launch_rowstep_tiled(Lane* lane, const MatvecArgs& args, const Geometry& g, int rows, size_t lds)
+{
+    static bool big_lds_enabled = false;
+    if (lds > 32 * 1024 && !big_lds_enabled) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&matvec_rowstep_kernel<Q, PRE, MR>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, max_dynamic_lds(MR));
+        if (e != hipSuccess) return e;
+        big_lds_enabled = true;
+    }
+    hipLaunchKernelGGL((matvec_rowstep_kernel<Q, PRE, MR>), dim3(g.groups, (rows + MR - 1) / MR), dim3(g.threads), lds,
+                       lane->stream, args, args.bias);
+    return hipGetLastError();
+}
+
 template <class Q, int PRE = kPreNone>
 hipError_t launch_rowstep(Lane* lane, MatvecArgs args, int rows)
 {
@@ -998,16 +1045,16 @@ hipError_t launch_rowstep(Lane* lane, MatvecArgs args, int rows)
     if (PRE == kPreRmsNorm && g.threads < 128) g.threads = 128;     // the norm's partial sums take 128 lanes
     args.rows_per_step = g.rows_per_step;
     args.steps = g.steps;
+    args.rows = rows;
     const size_t lds = static_cast<size_t>(kChunkPieces) * args.units_per_row * sizeof(float4);
-    static bool big_lds_enabled = false;
-    if (lds > 48 * 1024 && !big_lds_enabled) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&matvec_rowstep_kernel<Q, PRE>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, kMaxDynamicLds);
-        if (e != hipSuccess) return e;
-        big_lds_enabled = true;
+    // Several input rows: four (or two) per pass over the weights when their staging areas fit LDS.  Only for the formats
+    // whose single-row kernel waits on memory: measured on 21504x5376 Q8_0, 4 rows take 50 us instead of 75 us; the K-quants,
+    // bound by their arithmetic, got slower (17408x5120 Q4_K, 4 rows: 50 us against 45 us), so they keep one row per pass.
+    if constexpr (PRE == kPreNone && (std::is_same<Q, Q8_0Unit>::value || std::is_same<Q, BF16Unit>::value)) {
+        if (rows >= 3 && 4 * lds <= static_cast<size_t>(max_dynamic_lds(4))) return launch_rowstep_tiled<Q, PRE, 4>(lane, args, g, rows, 4 * lds);
+        if (rows >= 2 && 2 * lds <= static_cast<size_t>(max_dynamic_lds(2))) return launch_rowstep_tiled<Q, PRE, 2>(lane, args, g, rows, 2 * lds);
     }
-    hipLaunchKernelGGL((matvec_rowstep_kernel<Q, PRE>), dim3(g.groups, rows), dim3(g.threads), lds, lane->stream, args, args.bias);
-    return hipGetLastError();
+    return launch_rowstep_tiled<Q, PRE, 1>(lane, args, g, rows, lds);
 }
 
 

@@ -181,6 +181,25 @@ def test_matvec_rows_equal_stacked_single_rows_bitwise(lane, typ):
     _check_against_f64(y, ref, asum)
 
 
+@pytest.mark.parametrize("in_w,out_w", [(5376, 70), (21504, 11), (7168, 33)])
+@pytest.mark.parametrize("rows", [2, 3, 4, 7])
+def test_matvec_row_tiles_equal_single_rows_bitwise(lane, rows, in_w, out_w):
+    """Q8_0 and bfloat16 launches with several input rows share one pass over the weights between up to four rows (two
+    when only two staging areas fit LDS, one for the widest vectors); a row's bits must not depend on the grouping."""
+    from nntrain_amd import GGML_BF16
+    x = synth.activations(rows, in_w, seed=rows + in_w)
+    bias = np.random.default_rng(8).standard_normal(out_w).astype(np.float32)
+    rng = np.random.default_rng(in_w + out_w)
+    bf16 = synth.to_bf16_bits(rng.standard_normal((out_w, in_w), dtype=np.float32) * np.float32(0.02)).view(np.uint8).reshape(-1)
+    for typ, payload in ((GGML_Q8_0, _random_payload(GGML_Q8_0, out_w, in_w, seed=31)), (GGML_BF16, bf16)):
+        y = _run_matvec(lane, typ, payload, x, bias, rows, in_w, out_w)
+        for r in range(rows):
+            y1 = _run_matvec(lane, typ, payload, x[r:r + 1], bias, 1, in_w, out_w)
+            assert np.array_equal(_bits(y[r]), _bits(y1[0])), (typ, r)
+    ref, asum = oracle.linear_f64(GGML_Q8_0, _random_payload(GGML_Q8_0, out_w, in_w, seed=31), x, bias, rows, in_w, out_w)
+    _check_against_f64(_run_matvec(lane, GGML_Q8_0, _random_payload(GGML_Q8_0, out_w, in_w, seed=31), x, bias, rows, in_w, out_w), ref, asum)
+
+
 def test_matvec_q8_0_odd_block_count_rows(lane):
     in_w, out_w = 32 * 5, 19
     payload = _random_payload(GGML_Q8_0, out_w, in_w, seed=77)
