@@ -312,6 +312,28 @@ def run_gemv(args, lane, nn, oracle):
         log(f"[gemv] {name}: single launch {us_ring:.2f} us ({algo / us_ring / 1e3:.0f} GB/s, "
             f"{100 * algo / us_ring / 1e3 / HBM_PEAK_GBS:.1f}% of 8 TB/s) HBM, {us_same:.2f} us cache-resident; batched "
             f"{us_batch:.2f} us/mat-vec ({100 * algo / us_batch / 1e3 / HBM_PEAK_GBS:.1f}%); rel-L2 {rel:.2e}")
+        if tname == "GGML_Q8_0":
+            # several input rows in one call (weights rotated as above): microseconds per call
+            per_rows = {}
+            for rows in (2, 4, 8):
+                xr = lane.upload_raw(synth.activations(rows, in_w, xseed + rows))
+                yr = lane.allocate(rows * out_w)
+
+                def launch_rows(w):
+                    nn.native.check(lib.nnhip_quant_matvec(h, typ, c_void_p(xr.ptr), c_void_p(w.ptr), None, c_void_p(yr.ptr),
+                                                           rows, in_w, out_w), "quant_matvec")
+
+                for w in ring:
+                    launch_rows(w)
+                samples = []
+                for _ in range(5):
+                    ms, _ = timed(lane, lambda: [launch_rows(w) for w in ring], 1)
+                    samples.append(ms * 1e3 / len(ring))
+                per_rows[f"rows={rows}"] = round(float(np.median(samples)), 2)
+                xr.dispose()
+                yr.dispose()
+            out[name]["us_per_call_with_several_input_rows"] = per_rows
+            log(f"[gemv] {name}: " + ", ".join(f"{k} {v:.1f} us" for k, v in per_rows.items()))
         for b in ring + ys + [x, y]:
             b.dispose()
     return out
