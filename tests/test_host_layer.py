@@ -231,3 +231,21 @@ def test_gguf_ranged_reads(tmp_path):
         assert r.read_tensor_range(t, 2304, 0) == b""
         with pytest.raises(ValueError):
             r.read_tensor_range(t, 2300, 5)
+
+
+def test_headers_compile_as_c_and_cpp(tmp_path):
+    """The ABI headers are what a binding is written from: they must be plain C (and valid C++) on their own."""
+    import shutil
+    import subprocess
+    from pathlib import Path
+    root = Path(__file__).resolve().parent.parent
+    src = tmp_path / "use_headers.c"
+    src.write_text('#include "nnhip.h"\n#include "nnhip_synth.h"\n'
+                   'int main(void) { nnhip_error_info e; nnhip_fused_matvec_desc d; (void)e; (void)d; return (int)sizeof(nnhip_matvec_desc) == 0; }\n')
+    for compiler, std in (("gcc", "-std=c99"), ("g++", "-std=c++17")):
+        if shutil.which(compiler) is None:
+            pytest.skip(f"{compiler} not installed")
+        lang = ["-x", "c++"] if compiler == "g++" else []
+        res = subprocess.run([compiler, std, "-Wall", "-Wextra", "-Werror", "-pedantic", "-fsyntax-only", f"-I{root / 'include'}", *lang, str(src)],
+                             capture_output=True, text=True)
+        assert res.returncode == 0, res.stderr
