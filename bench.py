@@ -38,46 +38,8 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def decode27b_tensors():
-    """(name, out_w, in_w) of every mat-vec of one token: Gemma-3-27B shapes (hidden 5376, 32 q heads, 16 kv heads,
-    head_dim 128, ffn 21504, vocab 262144)."""
-    hidden, q_out, kv_out, ffn, vocab, layers = 5376, 32 * 128, 16 * 128, 21504, 262144, 62
-    per_layer = [("attn_q", q_out, hidden), ("attn_k", kv_out, hidden), ("attn_v", kv_out, hidden),
-                 ("attn_o", hidden, q_out), ("ffn_gate", ffn, hidden), ("ffn_up", ffn, hidden),
-                 ("ffn_down", hidden, ffn)]
-    out = []
-    for layer in range(layers):
-        out += [(f"blk.{layer}.{n}", o, i) for n, o, i in per_layer]
-    out.append(("output", vocab, hidden))
-    return out
-
-
 def q8_bytes(out_w, in_w):
     return out_w * (in_w // 32) * 34
-
-
-class Synth:
-    def __init__(self):
-        path = ROOT / "nntrain_amd" / "csrc" / "libnnhip_synth.so"
-        if not path.exists():
-            raise FileNotFoundError(f"{path} is missing: run __graft_entry__.build()")
-        self.lib = ctypes.CDLL(str(path))
-        self.lib.nnhip_synth_q8_0.argtypes = [c_void_p, c_void_p, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_float]
-        self.lib.nnhip_synth_normal_f32.argtypes = [c_void_p, c_void_p, ctypes.c_uint64, ctypes.c_uint64]
-
-    def q8_0(self, lane, buf, blocks, seed, sigma=0.02):
-        s = c_void_p()
-        lane._lib.nnhip_lane_stream(lane._handle, ctypes.byref(s))
-        rc = self.lib.nnhip_synth_q8_0(s, c_void_p(buf.ptr), blocks, seed, sigma)
-        if rc:
-            raise RuntimeError(f"nnhip_synth_q8_0 failed ({rc})")
-
-    def normal(self, lane, buf, count, seed):
-        s = c_void_p()
-        lane._lib.nnhip_lane_stream(lane._handle, ctypes.byref(s))
-        rc = self.lib.nnhip_synth_normal_f32(s, c_void_p(buf.ptr), count, seed)
-        if rc:
-            raise RuntimeError(f"nnhip_synth_normal_f32 failed ({rc})")
 
 
 def timed(lane, fn, reps):
@@ -99,10 +61,11 @@ def timed(lane, fn, reps):
 
 def run_decode27b(args, lane, nn, oracle):
     from nntrain_amd.native import MatvecDesc
+    from nntrain_amd.synth import DeviceSynth, decode27b_tensors
     tensors = decode27b_tensors()
     total_bytes = sum(q8_bytes(o, i) for _, o, i in tensors)
     assert total_bytes == 28_695_625_728, total_bytes
-    synth = Synth()
+    synth = DeviceSynth()
     log(f"[decode27b] generating {len(tensors)} Q8_0 tensors, {total_bytes / 1e9:.2f} GB, on the device")
     weights, xs, ys = [], [], []
     for t, (name, out_w, in_w) in enumerate(tensors):

@@ -33,7 +33,16 @@ public sealed class HipQuantizedMatrix : IDisposable
     public int InputWidth { get; }
     public long StorageBytes { get; }
 
-    /// <summary>y[rows, out] = bias + x[rows, in] . W^T, FP32 activations; the caller disposes the result.</summary>
+    /// <summary>Rows at or above which Forward uses the matrix-core mat-mul (Qwen35QuantizedModel.cs:1249).</summary>
+    public const int PrefillMinRows = 16;
+
+    /// <summary>Whether Forward sends this many input rows to the matrix-core mat-mul.</summary>
+    public bool UsesPrefill(int rows) => rows >= PrefillMinRows && InputWidth % 256 == 0;
+
+    /// <summary>y[rows, out] = bias + x[rows, in] . W^T, FP32 activations; the caller disposes the result.
+    /// rows >= 16 go to the bf16 matrix-core mat-mul (activations rounded to bfloat16 on the device), fewer rows to the
+    /// dequantization-fused mat-vec, as Matrix.Forward routes them (Qwen35QuantizedModel.cs:1249-1369).  Allocating the
+    /// output per call is cheap: the lane hands out the block a previous Dispose returned.</summary>
     public HipBuffer Forward(HipExecutionLane lane, HipBuffer input, HipBuffer? bias, int rows = 1)
     {
         ArgumentNullException.ThrowIfNull(lane);
@@ -45,9 +54,13 @@ public sealed class HipQuantizedMatrix : IDisposable
             throw new ArgumentException("Quantized linear bias width mismatch.", nameof(bias));
         HipBuffer encoded = DevicePayload(lane);
         HipBuffer output = lane.Allocate(checked(rows * OutputWidth));
-        int status = lane.Locked(h => NnHipNative.nnhip_quant_matvec(h, GgmlType, input.Pointer, encoded.Pointer,
-            bias?.Pointer ?? 0, output.Pointer, rows, InputWidth, OutputWidth));
-        if (status != 0) { output.Dispose(); NnHipNative.Check(status, "quantized mat-vec"); }
+        bool prefill = UsesPrefill(rows);
+        int status = lane.Locked(h => prefill
+            ? NnHipNative.nnhip_quant_matmul(h, GgmlType, input.Pointer, encoded.Pointer, bias?.Pointer ?? 0, output.Pointer,
+                rows, InputWidth, OutputWidth)
+            : NnHipNative.nnhip_quant_matvec(h, GgmlType, input.Pointer, encoded.Pointer, bias?.Pointer ?? 0, output.Pointer,
+                rows, InputWidth, OutputWidth));
+        if (status != 0) { output.Dispose(); NnHipNative.Check(status, prefill ? "quantized mat-mul" : "quantized mat-vec"); }
         return output;
     }
 

@@ -1,7 +1,8 @@
 // Source-generated P/Invoke (LibraryImport) declarations for libnnhip.so - one per entry point of include/nnhip.h.
 // Drop into an NNtrain project that may reference NNtrain.Runtime (same layer as NNtrain.Arc / NNtrain.Cuda).
 // Not compiled in this repository (no .NET toolchain in the build image); the C header is the source of truth and
-// tests/test_host_layer.py checks that every symbol declared there is exported.
+// tests/test_host_layer.py checks that every symbol declared there is exported and that every declaration below
+// matches it in name, arity and argument widths (and the structure sizes).
 using System.Runtime.InteropServices;
 
 namespace NNtrain.Hip;
@@ -34,6 +35,14 @@ internal static unsafe partial class NnHipNative
         internal uint GgmlType; internal int Rows; internal int InW; internal int OutW;
     }
 
+    [StructLayout(LayoutKind.Sequential)]
+    internal struct MatvecPlanInfo
+    {
+        internal uint StructSize; internal int Kernel; internal int Threads; internal int RowsPerStep; internal int Steps;
+        internal int Groups; internal int RowTile; internal int RingDepth; internal int ResultBufferFloats;
+        internal int DynamicLdsBytes;
+    }
+
     internal const uint PreNone = 0, PreRmsNorm = 1, PreSiluMultiply = 2;
 
     [StructLayout(LayoutKind.Sequential)]
@@ -58,6 +67,7 @@ internal static unsafe partial class NnHipNative
     [LibraryImport(Library)] internal static partial int nnhip_lane_destroy(nint lane);
     [LibraryImport(Library)] internal static partial int nnhip_alloc(nint lane, nuint bytes, out nint dptr);
     [LibraryImport(Library)] internal static partial int nnhip_free(nint lane, nint dptr);
+    [LibraryImport(Library)] internal static partial int nnhip_lane_trim(nint lane);
     [LibraryImport(Library)] internal static partial int nnhip_upload(nint lane, nint dptr, nuint offset, void* host, nuint bytes);
     [LibraryImport(Library)] internal static partial int nnhip_download(nint lane, nint dptr, nuint offset, void* host, nuint bytes);
     [LibraryImport(Library)] internal static partial int nnhip_copy(nint lane, nint dst, nuint dstOffset, nint src, nuint srcOffset, nuint bytes);
@@ -67,8 +77,10 @@ internal static unsafe partial class NnHipNative
     [LibraryImport(Library)] internal static partial int nnhip_lane_stream(nint lane, out nint stream);
     [LibraryImport(Library)] internal static partial int nnhip_dequantize(nint lane, uint ggmlType, nint w, nint output, long elements);
     [LibraryImport(Library)] internal static partial int nnhip_quant_matvec(nint lane, uint ggmlType, nint x, nint w, nint bias, nint y, int rows, int inW, int outW);
+    [LibraryImport(Library)] internal static partial int nnhip_matvec_plan(uint ggmlType, int rows, int inW, int outW, int computeUnits, MatvecPlanInfo* info);
     [LibraryImport(Library)] internal static partial int nnhip_quant_matvec_batch(nint lane, MatvecDesc* descs, int count);
     [LibraryImport(Library)] internal static partial int nnhip_quant_matvec_fused(nint lane, FusedMatvecDesc* desc);
+    [LibraryImport(Library)] internal static partial int nnhip_quant_matmul(nint lane, uint ggmlType, nint x, nint w, nint bias, nint y, int rows, int inW, int outW);
     [LibraryImport(Library)] internal static partial int nnhip_quant_matmul_bf16(nint lane, uint ggmlType, nint xBf16, nint w, nint bias, nint y, int rows, int inW, int outW);
     [LibraryImport(Library)] internal static partial int nnhip_rms_norm(nint lane, nint input, nint weight, nint output, int rows, int width, int inputStride, float epsilon);
     [LibraryImport(Library)] internal static partial int nnhip_add_rms_norm(nint lane, nint destination, nint residual, nint weight, nint output, int rows, int width, int inputStride, float epsilon);

@@ -68,7 +68,7 @@ enum {
     NNHIP_OP_UPLOAD, NNHIP_OP_DOWNLOAD, NNHIP_OP_COPY, NNHIP_OP_SYNCHRONIZE, NNHIP_OP_DEQUANTIZE,
     NNHIP_OP_MATVEC, NNHIP_OP_MATVEC_BATCH, NNHIP_OP_MATMUL_BF16, NNHIP_OP_EVENT, NNHIP_OP_GRAPH,
     NNHIP_OP_DEVICE_QUERY, NNHIP_OP_FILL, NNHIP_OP_RMS_NORM, NNHIP_OP_SILU_MULTIPLY, NNHIP_OP_ADD_IN_PLACE,
-    NNHIP_OP_MATVEC_FUSED, NNHIP_OP_LORA, NNHIP_OP_ATTENTION
+    NNHIP_OP_MATVEC_FUSED, NNHIP_OP_LORA, NNHIP_OP_ATTENTION, NNHIP_OP_MATMUL
 };
 
 /* Same field order as the reference's NativeErrorInfo (CudaNativeGateway.cs:1360-1371). */
@@ -139,9 +139,16 @@ NNHIP_API int nnhip_lane_create(int device, void** lane);
 NNHIP_API int nnhip_lane_destroy(void* lane);
 
 /* Replaces ArcExecutionLane.Allocate / AllocateBytes (:241,:271) and ArcBuffer.Dispose (:917-931).
- * Memory is not cleared. */
+ * Memory is not cleared.  nnhip_free does not wait for the device: blocks of up to 64 MiB (at most 1 GiB in all) are
+ * kept by the lane and handed out again by the next nnhip_alloc of that size (rounded up to 256 bytes) - safe because
+ * all work of a lane is ordered on its one stream - so the reference's pattern of allocating each projection's output
+ * and disposing it after use (Qwen35QuantizedModel.cs:488-491) costs no synchronisation.  Larger blocks are returned
+ * to the driver after the stream has drained.  While a graph is being captured nnhip_alloc can only hand out kept
+ * blocks.  nnhip_lane_trim drains the stream and returns every kept block to the driver; it has no counterpart in the
+ * reference, whose OpenCL runtime defers releases itself. */
 NNHIP_API int nnhip_alloc(void* lane, size_t bytes, void** dptr);
 NNHIP_API int nnhip_free(void* lane, void* dptr);
+NNHIP_API int nnhip_lane_trim(void* lane);
 
 /* Blocking raw transfers.  Replace UploadRaw (:322-327) and Read / ReadRaw (:277,:334).  The bytes are not
  * interpreted: GGUF blocks go up exactly as they sit in the file. */
@@ -182,9 +189,36 @@ NNHIP_API int nnhip_dequantize(void* lane, uint32_t ggml_type, const void* w, fl
 NNHIP_API int nnhip_quant_matvec(void* lane, uint32_t ggml_type, const float* x, const void* w, const float* bias,
                                  float* y, int rows, int in_w, int out_w);
 
+/* The launch shape nnhip_quant_matvec picks for a call, computed on the host without touching a device: for
+ * reporting (the reference prints its kernel choice per matrix, Qwen35QuantizedModel.cs:1335-1344 selects by rows) and
+ * for checking the kernels' capacity assumptions in tests.  compute_units is the workgroup count to plan for (256 on
+ * MI355X).  Returns NNHIP_ERR_TOO_LARGE when no kernel takes the shape.  struct_size = sizeof of the structure. */
+enum { NNHIP_MATVEC_KERNEL_ROWSTEP = 0, NNHIP_MATVEC_KERNEL_Q8_0_ODD_BLOCKS = 1 };
+
+typedef struct nnhip_matvec_plan_info {
+    uint32_t struct_size;
+    int32_t kernel;                 /* NNHIP_MATVEC_KERNEL_*                                                   */
+    int32_t threads;                /* lanes per workgroup                                                     */
+    int32_t rows_per_step;          /* whole matrix rows a workgroup reduces per step                          */
+    int32_t steps;                  /* ceil(out_w / rows_per_step)                                             */
+    int32_t groups;                 /* workgroups along the matrix                                             */
+    int32_t row_tile;               /* input rows that share one pass over the weights                         */
+    int32_t ring_depth;             /* steps whose results are parked in LDS before a flush is possible        */
+    int32_t result_buffer_floats;   /* capacity of that LDS buffer: ring_depth * rows_per_step * row_tile fits */
+    int32_t dynamic_lds_bytes;
+} nnhip_matvec_plan_info;
+
+NNHIP_API int nnhip_matvec_plan(uint32_t ggml_type, int rows, int in_w, int out_w, int compute_units,
+                                nnhip_matvec_plan_info* info);
+
 /* `count` independent mat-vecs enqueued as one unit of work (a single launch per group of equal type), for the
  * per-token projection sets that ForwardTokenDevice issues back to back (Qwen35QuantizedModel.cs:451-513).
- * `descs` is a host array.  Results are identical to `count` nnhip_quant_matvec calls.  Asynchronous. */
+ * `descs` is a host array, read before the call returns.  Results are identical to `count` nnhip_quant_matvec calls.
+ * The descriptors reach the device as a table in lane-owned memory, written by a small kernel on the lane's stream
+ * (skipped when the table already holds them), so the call never waits for the device.  Under graph capture the write
+ * is recorded with the launch and a replay restores the table it needs; the table cannot grow during a capture
+ * (NNHIP_ERR_INVALID_ARGUMENT: issue a batch at least as large once before capturing), and tables a graph may name are
+ * kept until the lane is destroyed.  Asynchronous. */
 NNHIP_API int nnhip_quant_matvec_batch(void* lane, const nnhip_matvec_desc* descs, int count);
 
 /* Prefill: y[r, o] = bias[o] + sum_k x[r, k] * w[o, k] with x given as bfloat16 bit patterns [rows, in_w];
@@ -195,6 +229,16 @@ NNHIP_API int nnhip_quant_matvec_batch(void* lane, const nnhip_matvec_desc* desc
  * otherwise).  Asynchronous. */
 NNHIP_API int nnhip_quant_matmul_bf16(void* lane, uint32_t ggml_type, const uint16_t* x_bf16, const void* w,
                                       const float* bias, float* y, int rows, int in_w, int out_w);
+
+/* Prefill with FP32 activations, the form Matrix.Forward takes them in: x [rows, in_w] is rounded to bfloat16 on the
+ * device (round to nearest even) into a block owned by the lane, then multiplied as nnhip_quant_matmul_bf16 does.
+ * Replaces the input conversion + XMX launch pair of Matrix.Forward for rows >= 16 (Qwen35QuantizedModel.cs:1249-1317:
+ * q35l_prefill_xmx_input_f16x2 followed by q35l_prefill_xmx_<format>_f16x2, NNtrain.Arc/Kernels/
+ * qwen35_prefill_xmx.cl:35-47,112-184).  The result equals nnhip_quant_matmul_bf16 on the rounded activations bit for
+ * bit.  Same type and width rules.  The staging block comes from the lane's kept blocks when one of that size was
+ * freed before (always, from the second call of a shape on; required while a graph is being captured).  Asynchronous. */
+NNHIP_API int nnhip_quant_matmul(void* lane, uint32_t ggml_type, const float* x, const void* w, const float* bias,
+                                 float* y, int rows, int in_w, int out_w);
 
 /* --- FP32 row operations around the mat-vec ------------------------------------------------------------------ */
 

@@ -742,12 +742,11 @@ hipError_t launch_gemm(Lane* lane, const GemmArgs& a, dim3 grid)
 {
     constexpr int BM = (8 / WN) * RW, BN = 16 * CT;
     constexpr size_t lds = static_cast<size_t>(kStages) * 2 * (BM + BN) * kRowBytes;
-    static bool configured = false;
-    if (lds > 48 * 1024 && !configured) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&matmul_bf16_kernel<F, RW, CT, WN>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+    static LdsLimit big_lds;
+    if (lds > 48 * 1024) {
+        const hipError_t e = big_lds.ensure(lane->device, reinterpret_cast<const void*>(&matmul_bf16_kernel<F, RW, CT, WN>),
+                                            static_cast<int>(lds));
         if (e != hipSuccess) return e;
-        configured = true;
     }
     hipLaunchKernelGGL((matmul_bf16_kernel<F, RW, CT, WN>), grid, dim3(kGemmAll), lds, lane->stream, a);
     return hipGetLastError();
@@ -783,6 +782,29 @@ hipError_t launch_matmul_of(Lane* lane, const uint16_t* x, const void* w, const 
 }
 
 }  // namespace
+
+namespace {
+
+// FP32 -> bfloat16 (round to nearest even), eight values per thread; the last thread group handles the ragged end.
+__global__ __launch_bounds__(256) void to_bf16_kernel(const float* __restrict__ x, uint16_t* __restrict__ out, size_t count)
+{
+    const size_t i = (static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x) * 8;
+    if (i + 8 <= count) {
+        const float4 a = *reinterpret_cast<const float4*>(x + i), b = *reinterpret_cast<const float4*>(x + i + 4);
+        *reinterpret_cast<u32x4*>(out + i) = u32x4{pack_bf16(a.x, a.y), pack_bf16(a.z, a.w), pack_bf16(b.x, b.y), pack_bf16(b.z, b.w)};
+    } else {
+        for (size_t j = i; j < count; ++j) out[j] = static_cast<uint16_t>(pack_bf16(x[j], 0.0f) & 0xffffu);
+    }
+}
+
+}  // namespace
+
+hipError_t launch_to_bf16(Lane* lane, const float* x, uint16_t* out, size_t count)
+{
+    const size_t groups = (count + 2047) / 2048;
+    hipLaunchKernelGGL(to_bf16_kernel, dim3(static_cast<unsigned>(groups)), dim3(256), 0, lane->stream, x, out, count);
+    return hipGetLastError();
+}
 
 bool matmul_bf16_supported(uint32_t type, int in_w)
 {

@@ -993,12 +993,16 @@ struct Geometry {
 
 // Picks RS (whole rows per step) and from it the workgroup size.  Every workgroup runs ceil(steps / groups) rounds of
 // RS rows, so the launch lasts about rounds * RS row-times.  The largest RS that fits max_t lanes keeps the most
-// bytes in flight; a smaller one is taken only if it saves at least 2 % of rounds * RS.
-bool plan(int in_w, int out_w, int compute_units, int max_t, Geometry* g)
+// bytes in flight; a smaller one is taken only if it saves at least 2 % of rounds * RS.  `rs_cap` bounds RS from above:
+// a workgroup parks the results of a whole turn of the register ring (depth steps of RS rows for each of the MR input
+// rows of the tile) in its result buffer before it can flush, so depth * RS * MR must fit kYBuf.  The cap only binds
+// for rows of one to five units; a row's bits do not depend on RS.
+bool plan(int in_w, int out_w, int compute_units, int max_t, int rs_cap, Geometry* g)
 {
     const int upr = in_w / kUnitW;
-    if (upr < 1 || upr > max_t) return false;
-    const int rs_max = max_t / upr;
+    if (upr < 1 || upr > max_t || rs_cap < 1) return false;
+    int rs_max = max_t / upr;
+    if (rs_max > rs_cap) rs_max = rs_cap;
     const int rs_min = (3 * rs_max + 3) / 4;     // never give up more than a quarter of the lanes
     int best_rs = 0;
     long best_cost = 0;
@@ -1022,15 +1026,43 @@ bool plan(int in_w, int out_w, int compute_units, int max_t, Geometry* g)
 // Dynamic LDS a row-tiled launch may use: every further input row of the tile costs 8 KB of static partial sums.
 constexpr int max_dynamic_lds(int mr) { return kMaxDynamicLds - (mr - 1) * 2 * kMaxWG * static_cast<int>(sizeof(float)); }
 
+// Input rows that share one pass over the weights.  Four (or two) when their staging areas fit LDS, and only for the
+// formats whose single-row kernel waits on memory: measured on 21504x5376 Q8_0, 4 rows take 50 us instead of 75 us; the
+// K-quants, bound by their arithmetic, got slower (17408x5120 Q4_K, 4 rows: 50 us against 45 us), so they keep one row
+// per pass.
+template <class Q, int PRE>
+int row_tile_of(int rows, size_t lds_one_row)
+{
+    if constexpr (PRE == kPreNone && (std::is_same<Q, Q8_0Unit>::value || std::is_same<Q, BF16Unit>::value)) {
+        if (rows >= 3 && 4 * lds_one_row <= static_cast<size_t>(max_dynamic_lds(4))) return 4;
+        if (rows >= 2 && 2 * lds_one_row <= static_cast<size_t>(max_dynamic_lds(2))) return 2;
+    }
+    return 1;
+}
+
+// The whole launch shape of matvec_rowstep_kernel<Q, PRE, MR> for one call; false if a row does not fit a workgroup.
+template <class Q, int PRE>
+bool rowstep_shape(int rows, int in_w, int out_w, int compute_units, int* mr, Geometry* g)
+{
+    const size_t lds = static_cast<size_t>(kChunkPieces) * (in_w / kUnitW) * sizeof(float4);
+    *mr = row_tile_of<Q, PRE>(rows, lds);
+    if (!plan(in_w, out_w, compute_units, Shape<Q>::kMaxT, kYBuf / (Shape<Q>::kDepth * *mr), g)) return false;
+    if (PRE == kPreRmsNorm && g->threads < 128) g->threads = 128;     // the norm's partial sums take 128 lanes
+    return true;
+}
+
 template <class Q, int PRE, int MR>
 hipError_t launch_rowstep_tiled(Lane* lane, const MatvecArgs& args, const Geometry& g, int rows, size_t lds)
 {
-    static bool big_lds_enabled = false;
-    if (lds > 32 * 1024 && !big_lds_enabled) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&matvec_rowstep_kernel<Q, PRE, MR>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, max_dynamic_lds(MR));
+    // what the kernel's result buffer and partial-sum arrays assume (see plan)
+    if (Shape<Q>::kDepth * g.rows_per_step * MR > kYBuf || g.threads > Shape<Q>::kMaxT ||
+        g.rows_per_step * args.units_per_row > g.threads)
+        return hipErrorInvalidConfiguration;
+    static LdsLimit big_lds;
+    if (lds > 32 * 1024) {
+        const hipError_t e = big_lds.ensure(lane->device, reinterpret_cast<const void*>(&matvec_rowstep_kernel<Q, PRE, MR>),
+                                            max_dynamic_lds(MR));
         if (e != hipSuccess) return e;
-        big_lds_enabled = true;
     }
     hipLaunchKernelGGL((matvec_rowstep_kernel<Q, PRE, MR>), dim3(g.groups, (rows + MR - 1) / MR), dim3(g.threads), lds,
                        lane->stream, args, args.bias);
@@ -1041,39 +1073,67 @@ template <class Q, int PRE = kPreNone>
 hipError_t launch_rowstep(Lane* lane, MatvecArgs args, int rows)
 {
     Geometry g;
-    if (!plan(args.in_w, args.out_w, lane->compute_units, Shape<Q>::kMaxT, &g)) return hipErrorInvalidValue;
-    if (PRE == kPreRmsNorm && g.threads < 128) g.threads = 128;     // the norm's partial sums take 128 lanes
+    int mr = 1;
+    if (!rowstep_shape<Q, PRE>(rows, args.in_w, args.out_w, lane->compute_units, &mr, &g)) return hipErrorInvalidValue;
     args.rows_per_step = g.rows_per_step;
     args.steps = g.steps;
     args.rows = rows;
     const size_t lds = static_cast<size_t>(kChunkPieces) * args.units_per_row * sizeof(float4);
-    // Several input rows: four (or two) per pass over the weights when their staging areas fit LDS.  Only for the formats
-    // whose single-row kernel waits on memory: measured on 21504x5376 Q8_0, 4 rows take 50 us instead of 75 us; the K-quants,
-    // bound by their arithmetic, got slower (17408x5120 Q4_K, 4 rows: 50 us against 45 us), so they keep one row per pass.
     if constexpr (PRE == kPreNone && (std::is_same<Q, Q8_0Unit>::value || std::is_same<Q, BF16Unit>::value)) {
-        if (rows >= 3 && 4 * lds <= static_cast<size_t>(max_dynamic_lds(4))) return launch_rowstep_tiled<Q, PRE, 4>(lane, args, g, rows, 4 * lds);
-        if (rows >= 2 && 2 * lds <= static_cast<size_t>(max_dynamic_lds(2))) return launch_rowstep_tiled<Q, PRE, 2>(lane, args, g, rows, 2 * lds);
+        if (mr == 4) return launch_rowstep_tiled<Q, PRE, 4>(lane, args, g, rows, 4 * lds);
+        if (mr == 2) return launch_rowstep_tiled<Q, PRE, 2>(lane, args, g, rows, 2 * lds);
     }
     return launch_rowstep_tiled<Q, PRE, 1>(lane, args, g, rows, lds);
 }
 
 
-// Builds the device table for the entries of one block format and launches the persistent kernel.
+// Launches the persistent kernel over the entries of one block format; `table` is their slice of the device table.
 template <class Q>
-hipError_t launch_batch_of(Lane* lane, int total_chunks, int max_in_w, size_t table_offset)
+hipError_t launch_batch_of(Lane* lane, const BatchEntry* table, int total_chunks, int max_in_w)
 {
     const size_t lds = static_cast<size_t>(kChunkPieces) * (max_in_w / kUnitW) * sizeof(float4);
-    static bool big_lds_enabled = false;
-    if (lds > 48 * 1024 && !big_lds_enabled) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&matvec_batch_kernel<Q>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, kMaxDynamicLds);
+    static LdsLimit big_lds;
+    if (lds > 48 * 1024) {
+        const hipError_t e = big_lds.ensure(lane->device, reinterpret_cast<const void*>(&matvec_batch_kernel<Q>), kMaxDynamicLds);
         if (e != hipSuccess) return e;
-        big_lds_enabled = true;
     }
-    const BatchEntry* table = reinterpret_cast<const BatchEntry*>(static_cast<const char*>(lane->batch_table) + table_offset);
     const int groups = total_chunks < lane->compute_units ? total_chunks : lane->compute_units;
     hipLaunchKernelGGL(matvec_batch_kernel<Q>, dim3(groups), dim3(Shape<Q>::kMaxT), lds, lane->stream, table, total_chunks);
     return hipGetLastError();
+}
+
+// The descriptor table reaches the device as kernel arguments: a chunk of entries is passed by value to a one-workgroup
+// kernel that stores it.  The write is ordered on the lane's stream like the launches that read the table, so a table
+// can be rewritten without waiting for the host or the device, nothing is staged in host memory that would have to
+// outlive the call, and a captured graph carries the table's contents with it.
+constexpr int kEntryWords = static_cast<int>(sizeof(BatchEntry) / sizeof(uint32_t));
+constexpr int kWriteEntries = 48;                  // 48 * 80 bytes + 12 stay below the 4 KB of kernel arguments
+struct TableChunk {
+    uint32_t words[kWriteEntries * kEntryWords];
+};
+
+__global__ __launch_bounds__(1024) void table_write_kernel(uint32_t* __restrict__ dst, TableChunk chunk, int words)
+{
+    const int i = threadIdx.x;
+    if (i < words) dst[i] = chunk.words[i];
+}
+static_assert(kWriteEntries * kEntryWords <= 1024, "one workgroup writes a chunk");
+static_assert(sizeof(BatchEntry) == 80 && sizeof(TableChunk) + 12 <= 4096, "a chunk must fit the kernel arguments");
+
+hipError_t write_table(Lane* lane, void* device_table, const BatchEntry* entries, size_t count)
+{
+    TableChunk chunk;
+    for (size_t done = 0; done < count; done += kWriteEntries) {
+        const size_t n = count - done < static_cast<size_t>(kWriteEntries) ? count - done : kWriteEntries;
+        memcpy(chunk.words, entries + done, n * sizeof(BatchEntry));
+        hipLaunchKernelGGL(table_write_kernel, dim3(1), dim3(1024), 0, lane->stream,
+                           reinterpret_cast<uint32_t*>(static_cast<char*>(device_table) + done * sizeof(BatchEntry)), chunk,
+                           static_cast<int>(n * kEntryWords));
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+        lane->counters.kernel_launches += 1;
+    }
+    return hipSuccess;
 }
 
 void shape_of(uint32_t type, int* max_t, int* depth)
@@ -1097,6 +1157,54 @@ int matvec_max_in_w(uint32_t type)
     // one row must fit the workgroup: 768 lanes for the narrowest block-format shape, 512 for bfloat16 rows
     const int by_lanes = (type == NNHIP_TYPE_BF16 ? Shape<BF16Unit>::kMaxT : 768) * kUnitW;
     return by_lds < by_lanes ? by_lds : by_lanes;
+}
+
+namespace {
+
+template <class Q>
+bool describe_rowstep(int rows, int in_w, int out_w, int compute_units, nnhip_matvec_plan_info* info)
+{
+    Geometry g;
+    int mr = 1;
+    if (!rowstep_shape<Q, kPreNone>(rows, in_w, out_w, compute_units, &mr, &g)) return false;
+    info->kernel = NNHIP_MATVEC_KERNEL_ROWSTEP;
+    info->threads = g.threads;
+    info->rows_per_step = g.rows_per_step;
+    info->steps = g.steps;
+    info->groups = g.groups;
+    info->row_tile = mr;
+    info->ring_depth = Shape<Q>::kDepth;
+    info->result_buffer_floats = kYBuf;
+    info->dynamic_lds_bytes = static_cast<int32_t>(static_cast<size_t>(mr) * kChunkPieces * (in_w / kUnitW) * sizeof(float4));
+    return true;
+}
+
+}  // namespace
+
+bool describe_matvec(uint32_t type, int rows, int in_w, int out_w, int compute_units, nnhip_matvec_plan_info* info)
+{
+    if (type == NNHIP_TYPE_Q8_0 && ((in_w / 32) & 1)) {
+        info->kernel = NNHIP_MATVEC_KERNEL_Q8_0_ODD_BLOCKS;
+        info->threads = 256;
+        info->rows_per_step = 4;
+        info->steps = (out_w + 3) / 4;
+        info->groups = info->steps;
+        info->row_tile = 1;
+        info->ring_depth = 0;
+        info->result_buffer_floats = 0;
+        info->dynamic_lds_bytes = 0;
+        return true;
+    }
+    switch (type) {
+    case NNHIP_TYPE_Q8_0: return describe_rowstep<Q8_0Unit>(rows, in_w, out_w, compute_units, info);
+    case NNHIP_TYPE_Q4_K: return describe_rowstep<Q4KUnit>(rows, in_w, out_w, compute_units, info);
+    case NNHIP_TYPE_Q5_K: return describe_rowstep<Q5KUnit>(rows, in_w, out_w, compute_units, info);
+    case NNHIP_TYPE_Q6_K: return describe_rowstep<Q6KUnit>(rows, in_w, out_w, compute_units, info);
+    case NNHIP_TYPE_IQ3_S: return describe_rowstep<IQ3SUnit>(rows, in_w, out_w, compute_units, info);
+    case NNHIP_TYPE_BF16: return describe_rowstep<BF16Unit>(rows, in_w, out_w, compute_units, info);
+    case NNHIP_TYPE_IQ2_S: return describe_rowstep<IQ2SUnit>(rows, in_w, out_w, compute_units, info);
+    default: return false;
+    }
 }
 
 hipError_t launch_matvec(Lane* lane, uint32_t type, const float* x, const void* w, const float* bias, float* y,
@@ -1185,27 +1293,39 @@ hipError_t launch_matvec_fused(Lane* lane, const nnhip_fused_matvec_desc& d)
     }
 }
 
-hipError_t launch_matvec_batch(Lane* lane, const nnhip_matvec_desc* descs, int count)
+namespace {
+
+struct BatchGroup {
+    uint32_t type;
+    size_t begin, end;       // entries [begin, end) of the table
+    int total_chunks, max_in_w;
+};
+constexpr int kBatchTypes = 7;
+const uint32_t kBatchTypeOrder[kBatchTypes] = {NNHIP_TYPE_Q8_0, NNHIP_TYPE_Q4_K, NNHIP_TYPE_Q5_K, NNHIP_TYPE_Q6_K,
+                                               NNHIP_TYPE_IQ3_S, NNHIP_TYPE_IQ2_S, NNHIP_TYPE_BF16};
+
+// Entries of the batch, grouped by block format (one persistent launch per format); one entry per input row of a
+// descriptor.  Returns the number of entries, or -1 if they exceed `cap`.  Q8_0 rows with an odd number of blocks get no
+// entry: they are launched one by one.
+long build_batch(const nnhip_matvec_desc* descs, int count, BatchEntry* out, size_t cap, BatchGroup* groups, int* ngroups)
 {
-    static const uint32_t kTypes[7] = {NNHIP_TYPE_Q8_0, NNHIP_TYPE_Q4_K, NNHIP_TYPE_Q5_K, NNHIP_TYPE_Q6_K, NNHIP_TYPE_IQ3_S,
-                                       NNHIP_TYPE_IQ2_S, NNHIP_TYPE_BF16};
-    std::vector<BatchEntry> all;
-    struct Group { uint32_t type; size_t begin, end; int total_chunks, max_in_w; };
-    std::vector<Group> groups;
-    for (uint32_t type : kTypes) {
-        Group g{type, all.size(), all.size(), 0, 0};
+    size_t n = 0;
+    *ngroups = 0;
+    for (uint32_t type : kBatchTypeOrder) {
+        BatchGroup g{type, n, n, 0, 0};
         int max_t = 0, depth = 0;
         shape_of(type, &max_t, &depth);
+        int elems = 0, bytes = 0;
+        type_block(type, &elems, &bytes);
         for (int i = 0; i < count; ++i) {
             const nnhip_matvec_desc& d = descs[i];
             if (d.ggml_type != type) continue;
-            if (type == NNHIP_TYPE_Q8_0 && ((d.in_w / 32) & 1)) continue;   // launched one by one below
-            int elems = 0, bytes = 0;
-            type_block(type, &elems, &bytes);
+            if (type == NNHIP_TYPE_Q8_0 && ((d.in_w / 32) & 1)) continue;
             const int upr = d.in_w / kUnitW;
             int rs = max_t / upr;
             if (rs > d.out_w) rs = d.out_w;
             for (int r = 0; r < d.rows; ++r) {
+                if (n >= cap) return -1;
                 BatchEntry e{};
                 e.x = (decltype(e.x))(d.x + static_cast<size_t>(r) * d.in_w);
                 e.w = (decltype(e.w))(d.w);
@@ -1222,54 +1342,30 @@ hipError_t launch_matvec_batch(Lane* lane, const nnhip_matvec_desc* descs, int c
                 e.chunks = (e.steps + depth - 1) / depth;
                 g.total_chunks += e.chunks;
                 if (d.in_w > g.max_in_w) g.max_in_w = d.in_w;
-                all.push_back(e);
+                out[n++] = e;
             }
         }
-        g.end = all.size();
-        if (g.end > g.begin) groups.push_back(g);
+        g.end = n;
+        if (g.end > g.begin) groups[(*ngroups)++] = g;
     }
+    return static_cast<long>(n);
+}
 
-    // Upload the table unless it is the one already on the device.  The staging copy is pinned; a pending launch that
-    // still reads the old table is waited for before it is overwritten.
-    const size_t bytes = all.size() * sizeof(BatchEntry);
-    if (bytes) {
-        const bool same = lane->batch_table && bytes == lane->batch_table_used &&
-                          memcmp(lane->batch_table_host, all.data(), bytes) == 0;
-        if (!same) {
-            if (lane->capturing) return hipErrorStreamCaptureUnsupported;
-            hipError_t e = hipStreamSynchronize(lane->stream);
-            if (e != hipSuccess) return e;
-            if (bytes > lane->batch_table_bytes) {
-                if (lane->batch_table) (void)hipFree(lane->batch_table);
-                if (lane->batch_table_host) (void)hipHostFree(lane->batch_table_host);
-                lane->batch_table = nullptr;
-                lane->batch_table_host = nullptr;
-                lane->batch_table_bytes = 0;
-                const size_t cap = bytes * 2;
-                e = hipMalloc(&lane->batch_table, cap);
-                if (e != hipSuccess) return e;
-                e = hipHostMalloc(&lane->batch_table_host, cap, hipHostMallocDefault);
-                if (e != hipSuccess) return e;
-                lane->batch_table_bytes = cap;
-            }
-            memcpy(lane->batch_table_host, all.data(), bytes);
-            lane->batch_table_used = bytes;
-            e = hipMemcpyAsync(lane->batch_table, lane->batch_table_host, bytes, hipMemcpyHostToDevice, lane->stream);
-            if (e != hipSuccess) return e;
-        }
-    }
-
-    for (const Group& g : groups) {
+hipError_t launch_batch_groups(Lane* lane, const void* device_table, const BatchGroup* groups, int ngroups,
+                               const nnhip_matvec_desc* descs, int count)
+{
+    for (int i = 0; i < ngroups; ++i) {
+        const BatchGroup& g = groups[i];
+        const BatchEntry* t = reinterpret_cast<const BatchEntry*>(device_table) + g.begin;
         hipError_t e = hipSuccess;
-        const size_t off = g.begin * sizeof(BatchEntry);
         switch (g.type) {
-        case NNHIP_TYPE_Q8_0: e = launch_batch_of<Q8_0Unit>(lane, g.total_chunks, g.max_in_w, off); break;
-        case NNHIP_TYPE_Q4_K: e = launch_batch_of<Q4KUnit>(lane, g.total_chunks, g.max_in_w, off); break;
-        case NNHIP_TYPE_Q5_K: e = launch_batch_of<Q5KUnit>(lane, g.total_chunks, g.max_in_w, off); break;
-        case NNHIP_TYPE_Q6_K: e = launch_batch_of<Q6KUnit>(lane, g.total_chunks, g.max_in_w, off); break;
-        case NNHIP_TYPE_IQ3_S: e = launch_batch_of<IQ3SUnit>(lane, g.total_chunks, g.max_in_w, off); break;
-        case NNHIP_TYPE_BF16: e = launch_batch_of<BF16Unit>(lane, g.total_chunks, g.max_in_w, off); break;
-        default: e = launch_batch_of<IQ2SUnit>(lane, g.total_chunks, g.max_in_w, off); break;
+        case NNHIP_TYPE_Q8_0: e = launch_batch_of<Q8_0Unit>(lane, t, g.total_chunks, g.max_in_w); break;
+        case NNHIP_TYPE_Q4_K: e = launch_batch_of<Q4KUnit>(lane, t, g.total_chunks, g.max_in_w); break;
+        case NNHIP_TYPE_Q5_K: e = launch_batch_of<Q5KUnit>(lane, t, g.total_chunks, g.max_in_w); break;
+        case NNHIP_TYPE_Q6_K: e = launch_batch_of<Q6KUnit>(lane, t, g.total_chunks, g.max_in_w); break;
+        case NNHIP_TYPE_IQ3_S: e = launch_batch_of<IQ3SUnit>(lane, t, g.total_chunks, g.max_in_w); break;
+        case NNHIP_TYPE_BF16: e = launch_batch_of<BF16Unit>(lane, t, g.total_chunks, g.max_in_w); break;
+        default: e = launch_batch_of<IQ2SUnit>(lane, t, g.total_chunks, g.max_in_w); break;
         }
         if (e != hipSuccess) return e;
         lane->counters.kernel_launches += 1;
@@ -1283,6 +1379,49 @@ hipError_t launch_matvec_batch(Lane* lane, const nnhip_matvec_desc* descs, int c
         }
     }
     return hipSuccess;
+}
+
+}  // namespace
+
+// The lane's table grows by allocating a larger one; the old one is kept until the lane is destroyed, because a
+// captured graph may still name it.  Outside a capture the write is skipped when the device already holds these entries
+// (the common case of a decode loop that repeats one batch).
+hipError_t launch_matvec_batch(Lane* lane, const nnhip_matvec_desc* descs, int count)
+{
+    size_t cap = 0;
+    for (int i = 0; i < count; ++i) cap += static_cast<size_t>(descs[i].rows);
+    std::vector<BatchEntry> all(cap);
+    BatchGroup groups[kBatchTypes];
+    int ngroups = 0;
+    const long n = build_batch(descs, count, all.data(), cap, groups, &ngroups);
+    if (n < 0) return hipErrorInvalidValue;
+    const size_t bytes = static_cast<size_t>(n) * sizeof(BatchEntry);
+    if (bytes) {
+        if (bytes > lane->batch_table_bytes) {
+            if (lane->capturing) return hipErrorStreamCaptureUnsupported;     // the table cannot grow inside a capture
+            const size_t want = bytes * 2 < 65536 ? 65536 : bytes * 2;
+            void* fresh = nullptr;
+            const hipError_t e = hipMalloc(&fresh, want);
+            if (e != hipSuccess) return e;
+            if (lane->batch_table) lane->retired_tables.push_back(lane->batch_table);
+            lane->batch_table = fresh;
+            lane->batch_table_bytes = want;
+            lane->batch_shadow.clear();
+        }
+        const bool same = !lane->capturing && lane->batch_shadow.size() == bytes &&
+                          memcmp(lane->batch_shadow.data(), all.data(), bytes) == 0;
+        if (!same) {
+            const hipError_t e = write_table(lane, lane->batch_table, all.data(), static_cast<size_t>(n));
+            if (e != hipSuccess) return e;
+            if (lane->capturing) {
+                lane->batch_shadow.clear();     // recorded, not executed: the device contents are unknown until replay
+            } else {
+                lane->batch_shadow.assign(reinterpret_cast<const char*>(all.data()),
+                                          reinterpret_cast<const char*>(all.data()) + bytes);
+            }
+        }
+    }
+    return launch_batch_groups(lane, lane->batch_table, groups, ngroups, descs, count);
 }
 
 }  // namespace nnhip

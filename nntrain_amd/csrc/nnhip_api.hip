@@ -210,8 +210,14 @@ int nnhip_lane_destroy(void* handle)
         if (first == hipSuccess) first = e;
     }
     lane->buffers.clear();
+    for (auto& kv : lane->free_blocks)
+        for (void* p : kv.second) {
+            hipError_t e = hipFree(p);
+            if (first == hipSuccess) first = e;
+        }
+    lane->free_blocks.clear();
     if (lane->batch_table) (void)hipFree(lane->batch_table);
-    if (lane->batch_table_host) (void)hipHostFree(lane->batch_table_host);
+    for (void* t : lane->retired_tables) (void)hipFree(t);
     hipError_t e = hipStreamDestroy(lane->stream);
     if (first == hipSuccess) first = e;
     const int device = lane->device;
@@ -221,20 +227,40 @@ int nnhip_lane_destroy(void* handle)
     return NNHIP_OK;
 }
 
+// Allocation sizes are rounded up to 256 bytes and freed blocks of up to kCacheBlockMax are kept by the lane for the
+// next request of that size: the operator pattern of the reference allocates the output of every projection and
+// disposes it after use (Qwen35QuantizedModel.cs:488-491), which must not cost a device synchronisation per call.
 int nnhip_alloc(void* handle, size_t bytes, void** dptr)
 {
     NNHIP_LANE(handle, NNHIP_OP_ALLOC)
     if (!dptr || bytes == 0) return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_ALLOC, lane->device, 0, "allocation size must be positive and dptr non-null");
-    if (lane->capturing) return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_ALLOC, lane->device, 0, "no allocation while a graph is being captured");
+    const size_t capacity = (bytes + 255u) & ~static_cast<size_t>(255u);
     void* p = nullptr;
-    hipError_t e = hipMalloc(&p, bytes);
-    if (e == hipErrorOutOfMemory) {
-        (void)hipGetLastError();
-        return fail(NNHIP_ERR_OUT_OF_MEMORY, NNHIP_OP_ALLOC, lane->device, static_cast<uint32_t>(e), "device allocation of %zu bytes failed", bytes);
+    {
+        std::lock_guard<std::mutex> guard(lane->mutex);
+        auto it = lane->free_blocks.find(capacity);
+        if (it != lane->free_blocks.end() && !it->second.empty()) {
+            p = it->second.back();
+            it->second.pop_back();
+            lane->cached_bytes -= capacity;
+        }
     }
-    if (e != hipSuccess) return hip_fail(e, NNHIP_OP_ALLOC, lane->device, "hipMalloc");
+    if (!p) {
+        if (lane->capturing) return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_ALLOC, lane->device, 0, "no new device allocation while a graph is being captured (only blocks freed earlier can be handed out)");
+        hipError_t e = hipMalloc(&p, capacity);
+        if (e == hipErrorOutOfMemory) {
+            (void)hipGetLastError();
+            // give the cached blocks back and try once more
+            if (nnhip_lane_trim(handle) == NNHIP_OK) e = hipMalloc(&p, capacity);
+            if (e != hipSuccess) {
+                (void)hipGetLastError();
+                return fail(NNHIP_ERR_OUT_OF_MEMORY, NNHIP_OP_ALLOC, lane->device, static_cast<uint32_t>(e), "device allocation of %zu bytes failed", bytes);
+            }
+        }
+        if (e != hipSuccess) return hip_fail(e, NNHIP_OP_ALLOC, lane->device, "hipMalloc");
+    }
     std::lock_guard<std::mutex> guard(lane->mutex);
-    lane->buffers.emplace(p, bytes);
+    lane->buffers.emplace(p, Lane::Block{bytes, capacity});
     lane->counters.allocated_bytes += bytes;
     if (lane->counters.allocated_bytes > lane->counters.peak_allocated_bytes)
         lane->counters.peak_allocated_bytes = lane->counters.allocated_bytes;
@@ -246,21 +272,50 @@ int nnhip_free(void* handle, void* dptr)
 {
     NNHIP_LANE(handle, NNHIP_OP_FREE)
     if (!dptr) return NNHIP_OK;
-    if (lane->capturing) return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_FREE, lane->device, 0, "no free while a graph is being captured");
+    size_t capacity = 0;
     {
         std::lock_guard<std::mutex> guard(lane->mutex);
         auto it = lane->buffers.find(dptr);
         if (it == lane->buffers.end())
             return fail(NNHIP_ERR_BAD_HANDLE, NNHIP_OP_FREE, lane->device, 0, "pointer was not allocated by this lane");
-        lane->counters.allocated_bytes -= it->second;
+        capacity = it->second.capacity;
+        const bool keep = capacity <= kCacheBlockMax && lane->cached_bytes + capacity <= kCacheTotalMax;
+        if (!keep && lane->capturing)
+            return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_FREE, lane->device, 0, "a block this large cannot be freed while a graph is being captured");
+        lane->counters.allocated_bytes -= it->second.bytes;
         lane->buffers.erase(it);
+        if (keep) {
+            lane->free_blocks[capacity].push_back(dptr);
+            lane->cached_bytes += capacity;
+            return NNHIP_OK;
+        }
     }
-    // Work already enqueued may still read the buffer: drain the lane's stream first (hipFree itself only waits for
-    // the null stream, which a non-blocking stream does not join).
+    // Returned to the driver.  Work already enqueued may still read the buffer: drain the lane's stream first (hipFree
+    // itself only waits for the null stream, which a non-blocking stream does not join).
     hipError_t e = hipStreamSynchronize(lane->stream);
     if (e != hipSuccess) return hip_fail(e, NNHIP_OP_FREE, lane->device, "hipStreamSynchronize");
     e = hipFree(dptr);
     if (e != hipSuccess) return hip_fail(e, NNHIP_OP_FREE, lane->device, "hipFree");
+    return NNHIP_OK;
+}
+
+int nnhip_lane_trim(void* handle)
+{
+    NNHIP_LANE(handle, NNHIP_OP_FREE)
+    if (lane->capturing) return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_FREE, lane->device, 0, "no trim while a graph is being captured");
+    std::unordered_map<size_t, std::vector<void*>> blocks;
+    {
+        std::lock_guard<std::mutex> guard(lane->mutex);
+        blocks.swap(lane->free_blocks);
+        lane->cached_bytes = 0;
+    }
+    hipError_t first = hipStreamSynchronize(lane->stream);
+    for (auto& kv : blocks)
+        for (void* p : kv.second) {
+            const hipError_t e = hipFree(p);
+            if (first == hipSuccess) first = e;
+        }
+    if (first != hipSuccess) return hip_fail(first, NNHIP_OP_FREE, lane->device, "trim");
     return NNHIP_OK;
 }
 
@@ -372,6 +427,22 @@ int nnhip_quant_matvec(void* handle, uint32_t ggml_type, const float* x, const v
     hipError_t e = launch_matvec(lane, ggml_type, x, w, bias, y, rows, in_w, out_w);
     if (e != hipSuccess) return hip_fail(e, NNHIP_OP_MATVEC, lane->device, "mat-vec launch");
     lane->counters.kernel_launches += 1;
+    return NNHIP_OK;
+}
+
+int nnhip_matvec_plan(uint32_t ggml_type, int rows, int in_w, int out_w, int compute_units, nnhip_matvec_plan_info* info)
+{
+    int elems = 0;
+    if (!type_block(ggml_type, &elems, nullptr))
+        return fail(NNHIP_ERR_UNSUPPORTED_TYPE, NNHIP_OP_MATVEC, -1, 0, "GGML type %u is not a supported quantized matrix type", ggml_type);
+    if (!info || info->struct_size != sizeof(nnhip_matvec_plan_info))
+        return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_MATVEC, -1, 0, "info is null or has the wrong struct_size");
+    if (rows < 1 || in_w < 1 || out_w < 1 || compute_units < 1)
+        return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_MATVEC, -1, 0, "rows, in_w, out_w and compute_units must be positive");
+    if (in_w % elems != 0 || (ggml_type == NNHIP_TYPE_BF16 && in_w % 64 != 0))
+        return fail(NNHIP_ERR_INCOMPLETE_BLOCKS, NNHIP_OP_MATVEC, -1, 0, "quantized rows must contain complete blocks (in_w = %d)", in_w);
+    if (in_w > matvec_max_in_w(ggml_type) || !describe_matvec(ggml_type, rows, in_w, out_w, compute_units, info))
+        return fail(NNHIP_ERR_TOO_LARGE, NNHIP_OP_MATVEC, -1, 0, "in_w %d exceeds the %d values one workgroup can stage", in_w, matvec_max_in_w(ggml_type));
     return NNHIP_OK;
 }
 
@@ -543,6 +614,10 @@ int nnhip_quant_matvec_batch(void* handle, const nnhip_matvec_desc* descs, int c
     }
     if (count == 0) return NNHIP_OK;
     hipError_t e = launch_matvec_batch(lane, descs, count);
+    if (e == hipErrorStreamCaptureUnsupported)
+        return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_MATVEC_BATCH, lane->device, static_cast<uint32_t>(e),
+                    "the batch needs a larger descriptor table than the lane holds, and a table cannot grow while a graph is "
+                    "being captured: issue a batch of this size once before the capture");
     if (e != hipSuccess) return hip_fail(e, NNHIP_OP_MATVEC_BATCH, lane->device, "batched mat-vec launch");
     return NNHIP_OK;
 }
@@ -560,6 +635,31 @@ int nnhip_quant_matmul_bf16(void* handle, uint32_t ggml_type, const uint16_t* x_
         return fail(NNHIP_ERR_UNSUPPORTED_TYPE, NNHIP_OP_MATMUL_BF16, lane->device, 0, "bf16 prefill mat-mul does not support GGML type %u", ggml_type);
     if (e != hipSuccess) return hip_fail(e, NNHIP_OP_MATMUL_BF16, lane->device, "mat-mul launch");
     lane->counters.kernel_launches += 1;
+    return NNHIP_OK;
+}
+
+int nnhip_quant_matmul(void* handle, uint32_t ggml_type, const float* x, const void* w, const float* bias, float* y,
+                       int rows, int in_w, int out_w)
+{
+    NNHIP_LANE(handle, NNHIP_OP_MATMUL)
+    int rc = check_linear(NNHIP_OP_MATMUL, lane, ggml_type, x, w, y, rows, in_w, out_w);
+    if (rc != NNHIP_OK) return rc;
+    if (in_w % 256 != 0 && matmul_bf16_supported(ggml_type, 256))
+        return fail(NNHIP_ERR_INCOMPLETE_BLOCKS, NNHIP_OP_MATMUL, lane->device, 0, "the prefill mat-mul needs in_w to be a multiple of 256 (got %d)", in_w);
+    if (!matmul_bf16_supported(ggml_type, in_w))
+        return fail(NNHIP_ERR_UNSUPPORTED_TYPE, NNHIP_OP_MATMUL, lane->device, 0, "the prefill mat-mul does not support GGML type %u", ggml_type);
+    // the bfloat16 copy of the activations lives in a lane block for the duration of the two launches; freeing it hands
+    // it to the next call of the same size without touching the driver
+    const size_t count = static_cast<size_t>(rows) * static_cast<size_t>(in_w);
+    void* staged = nullptr;
+    rc = nnhip_alloc(handle, count * sizeof(uint16_t), &staged);
+    if (rc != NNHIP_OK) return rc;
+    hipError_t e = launch_to_bf16(lane, x, static_cast<uint16_t*>(staged), count);
+    if (e == hipSuccess) e = launch_matmul_bf16(lane, ggml_type, static_cast<const uint16_t*>(staged), w, bias, y, rows, in_w, out_w);
+    const int freed = nnhip_free(handle, staged);
+    if (e != hipSuccess) return hip_fail(e, NNHIP_OP_MATMUL, lane->device, "mat-mul launch");
+    if (freed != NNHIP_OK) return freed;
+    lane->counters.kernel_launches += 2;
     return NNHIP_OK;
 }
 
@@ -628,6 +728,7 @@ int nnhip_graph_end(void* handle, void** graph)
     NNHIP_LANE(handle, NNHIP_OP_GRAPH)
     if (!lane->capturing) return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_GRAPH, lane->device, 0, "no capture in progress");
     lane->capturing = false;
+    lane->batch_shadow.clear();
     hipGraph_t g = nullptr;
     hipError_t e = hipStreamEndCapture(lane->stream, &g);
     if (e != hipSuccess) return hip_fail(e, NNHIP_OP_GRAPH, lane->device, "hipStreamEndCapture");
@@ -658,6 +759,7 @@ int nnhip_graph_launch(void* handle, void* graph)
     if (!gr || gr->magic != kGraphMagic) return fail(NNHIP_ERR_BAD_HANDLE, NNHIP_OP_GRAPH, lane->device, 0, "not a graph handle");
     hipError_t e = hipGraphLaunch(gr->exec, lane->stream);
     if (e != hipSuccess) return hip_fail(e, NNHIP_OP_GRAPH, lane->device, "hipGraphLaunch");
+    lane->batch_shadow.clear();         // a replayed batch rewrites the lane's descriptor table
     return NNHIP_OK;
 }
 

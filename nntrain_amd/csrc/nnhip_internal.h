@@ -4,8 +4,10 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
 #include <mutex>
 #include <unordered_map>
+#include <vector>
 
 #include "../../include/nnhip.h"
 
@@ -15,6 +17,9 @@ constexpr uint32_t kLaneMagic = 0x4e4c414eu;   // "NLAN"
 constexpr uint32_t kEventMagic = 0x4e45564eu;  // "NEVN"
 constexpr uint32_t kGraphMagic = 0x4e475248u;  // "NGRH"
 
+constexpr size_t kCacheBlockMax = 64u << 20;   // larger blocks (weights) are returned to the driver when freed
+constexpr size_t kCacheTotalMax = 1u << 30;    // most bytes a lane keeps for reuse
+
 struct Lane {
     uint32_t magic = kLaneMagic;
     int device = 0;
@@ -22,12 +27,17 @@ struct Lane {
     hipStream_t stream = nullptr;
     bool capturing = false;
     nnhip_lane_counters counters{};
-    std::unordered_map<void*, size_t> buffers;  // device allocations still owned by the lane
+    struct Block { size_t bytes, capacity; };   // bytes asked for; bytes the allocation really has
+    std::unordered_map<void*, Block> buffers;   // device allocations handed out and still owned by the lane
+    // Freed blocks wait here, by capacity, to be handed out again.  All work of a lane runs on one in-order stream, so
+    // a block can be reused at once: whatever still reads it was enqueued before whatever the next owner enqueues.
+    std::unordered_map<size_t, std::vector<void*>> free_blocks;
+    size_t cached_bytes = 0;
     std::mutex mutex;                           // guards buffers + counters (uploads may come from loader threads)
-    void* batch_table = nullptr;                // device copy of the descriptor table of the last batch launch
-    size_t batch_table_bytes = 0;               // capacity of both copies
-    size_t batch_table_used = 0;                // bytes of the table that is on the device now
-    void* batch_table_host = nullptr;           // pinned staging for the table
+    void* batch_table = nullptr;                // device table of the batched mat-vec (written by a kernel on the stream)
+    size_t batch_table_bytes = 0;               // its capacity
+    std::vector<void*> retired_tables;          // outgrown tables: freed with the lane, a captured graph may name them
+    std::vector<char> batch_shadow;             // the entries the device table holds now (empty: unknown)
 };
 
 struct Event {
@@ -39,6 +49,20 @@ struct Graph {
     uint32_t magic = kGraphMagic;
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
+};
+
+// Raises the dynamic-LDS limit of one kernel, once per device (the attribute belongs to a function on a device).  Lanes
+// of several threads may get here together: setting it twice is harmless, so a lock-free "done" bit per device is enough.
+struct LdsLimit {
+    std::atomic<uint64_t> done{0};
+    hipError_t ensure(int device, const void* kernel, int bytes)
+    {
+        const uint64_t bit = 1ull << (device & 63);
+        if (done.load(std::memory_order_acquire) & bit) return hipSuccess;
+        const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+        if (e == hipSuccess) done.fetch_or(bit, std::memory_order_release);
+        return e;
+    }
 };
 
 // Block geometry; returns false for an unsupported type.
@@ -57,6 +81,7 @@ hipError_t launch_matvec_fused(Lane* lane, const nnhip_fused_matvec_desc& d);
 hipError_t launch_matvec_batch(Lane* lane, const nnhip_matvec_desc* descs, int count);
 hipError_t launch_matmul_bf16(Lane* lane, uint32_t type, const uint16_t* x, const void* w, const float* bias,
                               float* y, int rows, int in_w, int out_w);
+hipError_t launch_to_bf16(Lane* lane, const float* x, uint16_t* out, size_t count);
 // FP32 row operations (rowop_kernels.hip).  residual == nullptr: plain RMSNorm of io (not modified).
 hipError_t launch_rms_norm(Lane* lane, float* io, const float* residual, const float* weight, float* output, int rows,
                            int width, int input_stride, float epsilon);
@@ -68,6 +93,9 @@ hipError_t launch_lora_b(Lane* lane, const float* z, const float* b, float* y, i
 // Storage types and widths the bf16 prefill mat-mul covers.
 bool matmul_bf16_supported(uint32_t type, int in_w);
 hipError_t launch_fill_u32(Lane* lane, uint32_t* p, uint32_t value, size_t count);
+
+// Launch shape nnhip_quant_matvec would use (no device needed); false if no kernel takes the shape.
+bool describe_matvec(uint32_t type, int rows, int in_w, int out_w, int compute_units, nnhip_matvec_plan_info* info);
 
 // Largest in_w the mat-vec kernels can stage in LDS.
 int matvec_max_in_w(uint32_t type);

@@ -195,16 +195,13 @@ hipError_t launch_rms_norm(Lane* lane, float* io, const float* residual, const f
 {
     if (width >= 2 * kWideLanes && width <= kWideMaxWidth) {
         const size_t lds = static_cast<size_t>(width) * sizeof(float);
-        static bool big_lds_enabled = false;
-        if (!big_lds_enabled) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&rms_norm_wide_kernel<true>),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, kWideMaxWidth * sizeof(float));
-            if (e == hipSuccess)
-                e = hipFuncSetAttribute(reinterpret_cast<const void*>(&rms_norm_wide_kernel<false>),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, kWideMaxWidth * sizeof(float));
-            if (e != hipSuccess) return e;
-            big_lds_enabled = true;
-        }
+        static LdsLimit big_lds_add, big_lds_plain;
+        hipError_t e = big_lds_add.ensure(lane->device, reinterpret_cast<const void*>(&rms_norm_wide_kernel<true>),
+                                          static_cast<int>(kWideMaxWidth * sizeof(float)));
+        if (e == hipSuccess)
+            e = big_lds_plain.ensure(lane->device, reinterpret_cast<const void*>(&rms_norm_wide_kernel<false>),
+                                     static_cast<int>(kWideMaxWidth * sizeof(float)));
+        if (e != hipSuccess) return e;
         if (residual)
             hipLaunchKernelGGL(rms_norm_wide_kernel<true>, dim3(rows), dim3(kWideLanes), lds, lane->stream, io, residual, weight,
                                output, width, input_stride, epsilon);

@@ -134,6 +134,10 @@ class HipExecutionLane:
         check(self._lib.nnhip_alloc(self._handle, nbytes, byref(p)), "alloc")
         return HipBuffer(self, p.value, nbytes)
 
+    def trim(self) -> None:
+        """Drain the stream and return the blocks kept for reuse to the driver."""
+        check(self._lib.nnhip_lane_trim(self._handle), "lane_trim")
+
     def allocate(self, elements: int) -> HipBuffer:
         """FP32 elements, as ArcExecutionLane.Allocate."""
         return self.allocate_bytes(4 * elements)

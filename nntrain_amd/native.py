@@ -51,6 +51,12 @@ class FusedMatvecDesc(Structure):
                 ("lora_scale", c_float)]
 
 
+class MatvecPlanInfo(Structure):
+    _fields_ = [("struct_size", c_uint32), ("kernel", c_int32), ("threads", c_int32), ("rows_per_step", c_int32),
+                ("steps", c_int32), ("groups", c_int32), ("row_tile", c_int32), ("ring_depth", c_int32),
+                ("result_buffer_floats", c_int32), ("dynamic_lds_bytes", c_int32)]
+
+
 PRE_NONE, PRE_RMS_NORM, PRE_SILU_MULTIPLY = 0, 1, 2
 
 # name -> (restype, argtypes); exactly the prototypes of include/nnhip.h
@@ -67,6 +73,7 @@ PROTOTYPES = {
     "nnhip_lane_destroy": (c_int, [c_void_p]),
     "nnhip_alloc": (c_int, [c_void_p, c_size_t, POINTER(c_void_p)]),
     "nnhip_free": (c_int, [c_void_p, c_void_p]),
+    "nnhip_lane_trim": (c_int, [c_void_p]),
     "nnhip_upload": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p, c_size_t]),
     "nnhip_download": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p, c_size_t]),
     "nnhip_copy": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p, c_size_t, c_size_t]),
@@ -76,8 +83,10 @@ PROTOTYPES = {
     "nnhip_lane_stream": (c_int, [c_void_p, POINTER(c_void_p)]),
     "nnhip_dequantize": (c_int, [c_void_p, c_uint32, c_void_p, c_void_p, c_int64]),
     "nnhip_quant_matvec": (c_int, [c_void_p, c_uint32, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int]),
+    "nnhip_matvec_plan": (c_int, [c_uint32, c_int, c_int, c_int, c_int, POINTER(MatvecPlanInfo)]),
     "nnhip_quant_matvec_batch": (c_int, [c_void_p, POINTER(MatvecDesc), c_int]),
     "nnhip_quant_matvec_fused": (c_int, [c_void_p, POINTER(FusedMatvecDesc)]),
+    "nnhip_quant_matmul": (c_int, [c_void_p, c_uint32, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int]),
     "nnhip_quant_matmul_bf16": (c_int, [c_void_p, c_uint32, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int]),
     "nnhip_rms_norm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float]),
     "nnhip_add_rms_norm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float]),

@@ -124,9 +124,16 @@ class HipQuantizedMatrix:
         self._storage_bytes = int(self._payload.size)
         self._payload = None
 
+    def uses_prefill(self, rows: int) -> bool:
+        """Whether forward() sends `rows` input rows to the matrix-core mat-mul: rows >= 16 as in Matrix.Forward
+        (Qwen35QuantizedModel.cs:1249), when the rows are whole 256-weight blocks; the mat-vec kernels otherwise."""
+        return rows >= PREFILL_MIN_ROWS and self.input_width % 256 == 0
+
     def forward(self, lane: HipExecutionLane, x: HipBuffer, bias: HipBuffer | None, rows: int = 1,
                 out: HipBuffer | None = None) -> HipBuffer:
-        """y[rows, out] = bias + x[rows, in] . W^T on the device; x is FP32.  The caller disposes the result."""
+        """y[rows, out] = bias + x[rows, in] . W^T on the device; x is FP32.  The caller disposes the result.
+        rows >= 16 go to the bf16 matrix-core mat-mul (the activations are rounded to bfloat16 on the device), fewer
+        rows to the dequantization-fused mat-vec, as Matrix.Forward routes them (Qwen35QuantizedModel.cs:1249-1369)."""
         if rows < 1:
             raise ValueError("rows must be positive.")
         if x.nbytes < 4 * rows * self.input_width:
@@ -134,13 +141,20 @@ class HipQuantizedMatrix:
         if bias is not None and bias.nbytes < 4 * self.output_width:
             raise ValueError("Quantized linear bias width mismatch.")
         w = self.device_payload(lane)
-        y = out if out is not None else lane.allocate(rows * self.output_width)
-        if y.nbytes < 4 * rows * self.output_width:
+        if out is not None and out.nbytes < 4 * rows * self.output_width:
             raise ValueError("output buffer too small")
-        with lane.kernel("quant_matvec"):
-            check(lane._lib.nnhip_quant_matvec(lane._handle, self.ggml_type, c_void_p(x._require()), c_void_p(w._require()),
-                                               c_void_p(bias._require()) if bias is not None else None,
-                                               c_void_p(y._require()), rows, self.input_width, self.output_width), "quant_matvec")
+        y = out if out is not None else lane.allocate(rows * self.output_width)
+        entry, fn = (("quant_matmul", lane._lib.nnhip_quant_matmul) if self.uses_prefill(rows)
+                     else ("quant_matvec", lane._lib.nnhip_quant_matvec))
+        try:
+            with lane.kernel(entry):
+                check(fn(lane._handle, self.ggml_type, c_void_p(x._require()), c_void_p(w._require()),
+                         c_void_p(bias._require()) if bias is not None else None, c_void_p(y._require()), rows,
+                         self.input_width, self.output_width), entry)
+        except BaseException:
+            if out is None:
+                y.dispose()
+            raise
         return y
 
     def forward_fused(self, lane: HipExecutionLane, x: HipBuffer, *, pre_op: int = PRE_NONE, x2: HipBuffer | None = None,
@@ -191,13 +205,20 @@ class HipQuantizedMatrix:
         if bias is not None and bias.nbytes < 4 * self.output_width:
             raise ValueError("Quantized linear bias width mismatch.")
         w = self.device_payload(lane)
+        if out is not None and out.nbytes < 4 * rows * self.output_width:
+            raise ValueError("output buffer too small")
         y = out if out is not None else lane.allocate(rows * self.output_width)
-        with lane.kernel("quant_matmul_bf16"):
-            check(lane._lib.nnhip_quant_matmul_bf16(lane._handle, self.ggml_type, c_void_p(x_bf16._require()),
-                                                    c_void_p(w._require()),
-                                                    c_void_p(bias._require()) if bias is not None else None,
-                                                    c_void_p(y._require()), rows, self.input_width, self.output_width),
-                  "quant_matmul_bf16")
+        try:
+            with lane.kernel("quant_matmul_bf16"):
+                check(lane._lib.nnhip_quant_matmul_bf16(lane._handle, self.ggml_type, c_void_p(x_bf16._require()),
+                                                        c_void_p(w._require()),
+                                                        c_void_p(bias._require()) if bias is not None else None,
+                                                        c_void_p(y._require()), rows, self.input_width, self.output_width),
+                      "quant_matmul_bf16")
+        except BaseException:
+            if out is None:
+                y.dispose()
+            raise
         return y
 
     def dequantize(self, lane: HipExecutionLane, row: int | None = None, out: HipBuffer | None = None) -> HipBuffer:

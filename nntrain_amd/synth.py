@@ -7,6 +7,10 @@ sees the same bytes.
 """
 from __future__ import annotations
 
+import ctypes
+from ctypes import c_void_p
+from pathlib import Path
+
 import numpy as np
 
 from .quantized_matrix import (BLOCK_BYTES, BLOCK_ELEMS, GGML_BF16, GGML_IQ2_S, GGML_IQ3_S, GGML_Q4_K, GGML_Q5_K,
@@ -87,3 +91,46 @@ def to_bf16_bits(x: np.ndarray) -> np.ndarray:
     u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
     r = ((u >> 16) & 1) + np.uint32(0x7FFF)
     return ((u + r) >> 16).astype(np.uint16)
+
+
+class DeviceSynth:
+    """Draws synthetic Q8_0 blocks and N(0, 1) activations on the device (libnnhip_synth.so): the 27B-shape decode set
+    is 28.7 GB of random-init weights, far quicker to generate in HBM than to upload."""
+
+    def __init__(self):
+        path = Path(__file__).resolve().parent / "csrc" / "libnnhip_synth.so"
+        if not path.exists():
+            raise FileNotFoundError(f"{path} is missing: build it with `make -C nntrain_amd/csrc`")
+        self.lib = ctypes.CDLL(str(path))
+        self.lib.nnhip_synth_q8_0.argtypes = [c_void_p, c_void_p, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_float]
+        self.lib.nnhip_synth_normal_f32.argtypes = [c_void_p, c_void_p, ctypes.c_uint64, ctypes.c_uint64]
+
+    @staticmethod
+    def _stream(lane) -> c_void_p:
+        s = c_void_p()
+        lane._lib.nnhip_lane_stream(lane._handle, ctypes.byref(s))
+        return s
+
+    def q8_0(self, lane, buf, blocks: int, seed: int, sigma: float = 0.02) -> None:
+        rc = self.lib.nnhip_synth_q8_0(self._stream(lane), c_void_p(buf.ptr), blocks, seed, sigma)
+        if rc:
+            raise RuntimeError(f"nnhip_synth_q8_0 failed ({rc})")
+
+    def normal(self, lane, buf, count: int, seed: int) -> None:
+        rc = self.lib.nnhip_synth_normal_f32(self._stream(lane), c_void_p(buf.ptr), count, seed)
+        if rc:
+            raise RuntimeError(f"nnhip_synth_normal_f32 failed ({rc})")
+
+
+def decode27b_tensors():
+    """(name, out_w, in_w) of every mat-vec of one token of a Gemma-3-27B-shaped stack: hidden 5376, 32 query and 16
+    key/value heads of 128, feed-forward 21504, vocabulary 262144, 62 layers: 435 matrices, 28,695,625,728 Q8_0 bytes."""
+    hidden, q_out, kv_out, ffn, vocab, layers = 5376, 32 * 128, 16 * 128, 21504, 262144, 62
+    per_layer = [("attn_q", q_out, hidden), ("attn_k", kv_out, hidden), ("attn_v", kv_out, hidden),
+                 ("attn_o", hidden, q_out), ("ffn_gate", ffn, hidden), ("ffn_up", ffn, hidden),
+                 ("ffn_down", hidden, ffn)]
+    out = []
+    for layer in range(layers):
+        out += [(f"blk.{layer}.{n}", o, i) for n, o, i in per_layer]
+    out.append(("output", vocab, hidden))
+    return out

@@ -1,0 +1,334 @@
+"""GPU tests of the benchmark configurations at their full sizes and of the operator-level behaviour around them:
+the 435-matrix Q8_0 decode set as one batched launch, the 17408 x 5120 Q4_K prefill at every row count of the sweep,
+rows-based routing of HipQuantizedMatrix.forward, the allocate / forward / dispose pattern, and graph replay of a batch.
+Everything goes through the C ABI; the CPU oracle is the checker.
+"""
+import time
+from ctypes import c_void_p
+
+import numpy as np
+import pytest
+
+import oracle
+from nntrain_amd import GGML_Q4_K, GGML_Q5_K, GGML_Q8_0, HipExecutionLane, HipQuantizedMatrix, synth
+from nntrain_amd.native import MatvecDesc, check
+
+pytestmark = pytest.mark.gpu
+
+NAN_BITS = 0x7FC00000
+MATVEC_BAR = 1e-5
+PREFILL_BAR = 2e-3          # against the float64 oracle fed the same bf16 activation bits
+PREFILL_TIGHT_BAR = 5e-6    # against the float64 product taken with the oracle's weights rounded to bfloat16
+
+
+@pytest.fixture(scope="module")
+def lane():
+    with HipExecutionLane(0) as ln:
+        yield ln
+
+
+def _bits(a):
+    return np.ascontiguousarray(a, dtype=np.float32).view(np.uint32)
+
+
+# ------------------------------------------------------------------------------- the 27B-shape decode set, whole
+
+def test_decode27b_full_set_as_one_batched_launch(lane):
+    """All 435 Q8_0 matrices of the Gemma-3-27B-shaped token (28,695,625,728 bytes resident) through one
+    nnhip_quant_matvec_batch call; first and last 256 rows of ten matrices of every shape, the vocabulary head among
+    them, against the float64 oracle on the bytes that are in HBM."""
+    tensors = synth.decode27b_tensors()
+    assert len(tensors) == 435
+    dev = synth.DeviceSynth()
+    weights, xs, ys = [], [], []
+    total = 0
+    for t, (_, out_w, in_w) in enumerate(tensors):
+        nbytes = out_w * (in_w // 32) * 34
+        total += nbytes
+        w = lane.allocate_bytes(nbytes)
+        dev.q8_0(lane, w, out_w * (in_w // 32), 3000 + t)
+        x = lane.allocate(in_w)
+        dev.normal(lane, x, in_w, 3_999_000 + t)
+        y = lane.allocate(out_w + 2)
+        lane.fill_u32(y, NAN_BITS, out_w + 2)
+        weights.append(w)
+        xs.append(x)
+        ys.append(y)
+    assert total == 28_695_625_728
+    descs = (MatvecDesc * len(tensors))()
+    for t, (_, out_w, in_w) in enumerate(tensors):
+        descs[t] = MatvecDesc(xs[t].ptr, weights[t].ptr, None, ys[t].ptr, GGML_Q8_0, 1, in_w, out_w)
+    before = lane.counters()
+    check(lane._lib.nnhip_quant_matvec_batch(lane._handle, descs, len(tensors)), "quant_matvec_batch")
+    lane.synchronize()
+    after = lane.counters()
+    assert after["h2d_bytes"] == before["h2d_bytes"] and after["d2h_bytes"] == before["d2h_bytes"]
+    worst = 0.0
+    # layer 0 and layer 61 in full (q k v o gate up down), one mid-stack feed-forward pair, and the head
+    for t in list(range(0, 7)) + [7 * 30 + 4, 7 * 30 + 6] + list(range(7 * 61, 7 * 62)) + [434]:
+        _, out_w, in_w = tensors[t]
+        row_bytes = (in_w // 32) * 34
+        x = lane.read(xs[t], np.float32)
+        y = lane.read(ys[t], np.float32)
+        assert np.isnan(y[-1]) and np.isnan(y[-2]), tensors[t][0]
+        assert np.all(np.isfinite(y[:-2])), tensors[t][0]
+        for r0 in (0, out_w - 256):
+            raw = lane.read(weights[t], np.uint8, 256 * row_bytes, r0 * row_bytes)
+            ref, asum = oracle.linear_f64(GGML_Q8_0, raw, x, None, 1, in_w, 256)
+            got = y[r0:r0 + 256]
+            worst = max(worst, oracle.rel_l2(got, ref[0]))
+            assert np.all(np.abs(got.astype(np.float64) - ref[0]) <= 2e-6 + 3e-6 * asum[0]), tensors[t][0]
+    print(f"decode27b full set: worst sampled rel-L2 = {worst:.3e}")
+    assert worst <= MATVEC_BAR
+    # no output of the set stayed unwritten
+    for t in range(0, 435, 29):
+        assert np.all(np.isfinite(lane.read(ys[t], np.float32)[:-2]))
+    for b in weights + xs + ys:
+        b.dispose()
+    lane.trim()
+
+
+# ------------------------------------------------------------------------------- prefill, full shape, every M
+
+@pytest.fixture(scope="module")
+def q4k_full():
+    in_w, out_w = 5120, 17408
+    payload = synth.matrix(GGML_Q4_K, out_w, in_w, 2001)
+    w = oracle.dequantize(GGML_Q4_K, payload).reshape(out_w, in_w)
+    w_bf16 = oracle.bf16_widen(oracle.bf16_round(w)).astype(np.float64)
+    return payload, w_bf16
+
+
+@pytest.mark.parametrize("rows", [256, 512, 2048])
+def test_prefill_full_shape_sampled_rows(lane, q4k_full, rows):
+    """BASELINE's prefill matrix (Q4_K 17408 x 5120) at M = 256, 512 and 2048 (the 32-row and the 64-row wave tiles over
+    256 and 128 strips): every output of every 16th input row, both bars, through the FP32-activation entry point."""
+    in_w, out_w = 5120, 17408
+    payload, w_bf16 = q4k_full
+    x = synth.activations(rows, in_w, 4000)
+    xb = synth.to_bf16_bits(x)
+    mat = HipQuantizedMatrix(payload, GGML_Q4_K, out_w, in_w)
+    xd = lane.upload_raw(x)
+    yd = lane.allocate(rows * out_w + 2)
+    lane.fill_u32(yd, NAN_BITS, rows * out_w + 2)
+    assert mat.uses_prefill(rows)
+    mat.forward(lane, xd, None, rows, out=yd)
+    lane.synchronize()
+    got = lane.read(yd)
+    assert np.isnan(got[-1]) and np.isnan(got[-2])
+    got = got[:-2].reshape(rows, out_w)
+    pick = np.arange(0, rows, 16)
+    tight = oracle.bf16_widen(xb[pick]).astype(np.float64) @ w_bf16.T
+    assert oracle.rel_l2(got[pick], tight) <= PREFILL_TIGHT_BAR
+    ref, _ = oracle.linear_f64(GGML_Q4_K, payload, xb[pick], None, len(pick), in_w, out_w, x_is_bf16=True)
+    rel = oracle.rel_l2(got[pick], ref)
+    print(f"prefill {rows}x5120x17408 rel-L2 = {rel:.3e}")
+    assert rel <= PREFILL_BAR
+    assert np.all(np.isfinite(got))
+    for b in (xd, yd):
+        b.dispose()
+    mat.dispose()
+
+
+# ------------------------------------------------------------------------------- operator routing by rows
+
+@pytest.mark.parametrize("typ", [GGML_Q4_K, GGML_Q8_0])
+def test_forward_routes_sixteen_rows_and_more_to_the_matrix_cores(lane, typ):
+    """Matrix.Forward takes FP32 rows and sends rows >= 16 to the matrix-core kernel after converting them on the
+    device (Qwen35QuantizedModel.cs:1249-1262); fewer rows, and widths that are not whole 256-blocks, to the mat-vec."""
+    in_w, out_w = 1024, 300
+    payload = synth.matrix(typ, out_w, in_w, seed=71)
+    mat = HipQuantizedMatrix(payload, typ, out_w, in_w)
+    bias = np.random.default_rng(1).standard_normal(out_w).astype(np.float32)
+    bd = lane.upload_raw(bias)
+    for rows in (15, 16, 128):
+        x = synth.activations(rows, in_w, seed=rows)
+        xd = lane.upload_raw(x)
+        launches = lane.counters()["kernel_launches"]
+        y = lane.read(mat.forward(lane, xd, bd, rows)).reshape(rows, out_w)
+        if rows < 16:
+            assert not mat.uses_prefill(rows)
+            ref, asum = oracle.linear_f64(typ, payload, x, bias, rows, in_w, out_w)
+            assert oracle.rel_l2(y, ref) <= MATVEC_BAR
+            one = lane.read(mat.forward(lane, xd, bd, 1))[:out_w]
+            assert np.array_equal(_bits(y[0]), _bits(one))
+        else:
+            assert mat.uses_prefill(rows)
+            assert lane.counters()["kernel_launches"] - launches == 2        # conversion + mat-mul
+            xb = synth.to_bf16_bits(x)
+            xbd = lane.upload_raw(xb)
+            same = lane.read(mat.forward_bf16(lane, xbd, bd, rows)).reshape(rows, out_w)
+            assert np.array_equal(_bits(y), _bits(same))          # the device rounding is round-to-nearest-even
+            ref, _ = oracle.linear_f64(typ, payload, xb, bias, rows, in_w, out_w, x_is_bf16=True)
+            assert oracle.rel_l2(y, ref) <= PREFILL_BAR
+            w = oracle.bf16_widen(oracle.bf16_round(oracle.dequantize(typ, payload).reshape(out_w, in_w))).astype(np.float64)
+            tight = oracle.bf16_widen(xb).astype(np.float64) @ w.T + bias.astype(np.float64)
+            assert oracle.rel_l2(y, tight) <= PREFILL_TIGHT_BAR
+            xbd.dispose()
+        xd.dispose()
+    mat.dispose()
+    # rows of 32-weight blocks that are no whole 256-blocks stay on the mat-vec kernels whatever the row count
+    narrow = HipQuantizedMatrix(synth.matrix(GGML_Q8_0, 40, 320, seed=3), GGML_Q8_0, 40, 320)
+    assert not narrow.uses_prefill(64)
+    x = synth.activations(20, 320, seed=2)
+    xd = lane.upload_raw(x)
+    y = lane.read(narrow.forward(lane, xd, None, 20)).reshape(20, 40)
+    ref, _ = oracle.linear_f64(GGML_Q8_0, synth.matrix(GGML_Q8_0, 40, 320, seed=3), x, None, 20, 320, 40)
+    assert oracle.rel_l2(y, ref) <= MATVEC_BAR
+    for b in (xd, bd):
+        b.dispose()
+    narrow.dispose()
+
+
+def test_forward_with_many_rows_beats_one_weight_pass_per_row(lane):
+    in_w, out_w, rows = 5120, 4096, 128
+    mat = HipQuantizedMatrix(synth.matrix(GGML_Q5_K, out_w, in_w, seed=9), GGML_Q5_K, out_w, in_w)
+    xd = lane.upload_raw(synth.activations(rows, in_w, seed=1))
+    yd = lane.allocate(rows * out_w)
+    mat.forward(lane, xd, None, rows, out=yd)             # warm-up (staging block, LDS attribute)
+    e0, e1, e2 = lane.event(), lane.event(), lane.event()
+    lane.synchronize()
+    e0.record()
+    mat.forward(lane, xd, None, rows, out=yd)
+    e1.record()
+    check(lane._lib.nnhip_quant_matvec(lane._handle, GGML_Q5_K, c_void_p(xd.ptr), c_void_p(mat.device_payload(lane).ptr), None,
+                                       c_void_p(yd.ptr), rows, in_w, out_w), "quant_matvec")
+    e2.record()
+    prefill_ms, matvec_ms = lane.elapsed_ms(e0, e1), lane.elapsed_ms(e1, e2)
+    print(f"128 rows x 4096 x 5120 Q5_K: routed forward {prefill_ms * 1e3:.0f} us, mat-vec passes {matvec_ms * 1e3:.0f} us")
+    assert prefill_ms < matvec_ms / 4
+    for e in (e0, e1, e2):
+        e.dispose()
+    for b in (xd, yd):
+        b.dispose()
+    mat.dispose()
+
+
+# ------------------------------------------------------------------------------- allocate / forward / dispose
+
+def test_allocate_forward_dispose_pattern_does_not_wait_for_the_device(lane):
+    """The reference allocates each projection's output and disposes it after use (Qwen35QuantizedModel.cs:488-491).
+    A thousand such rounds must enqueue as fast as a loop over preallocated outputs: no synchronisation per free."""
+    in_w, out_w = 5120, 5120
+    mats = [HipQuantizedMatrix(synth.matrix(GGML_Q4_K, out_w, in_w, seed=s), GGML_Q4_K, out_w, in_w) for s in (1, 2)]
+    for m in mats:
+        m.device_payload(lane)
+    x = lane.upload_raw(synth.activations(1, in_w, seed=3))
+    keep = lane.allocate(out_w)
+    rounds = 1000
+
+    def preallocated():
+        for i in range(rounds):
+            mats[i & 1].forward(lane, x, None, 1, out=keep)
+
+    def allocating():
+        for i in range(rounds):
+            y = mats[i & 1].forward(lane, x, None, 1)
+            y.dispose()
+
+    def wall(fn):
+        lane.synchronize()
+        t0 = time.perf_counter()
+        fn()
+        enqueue = time.perf_counter() - t0
+        lane.synchronize()
+        return enqueue, time.perf_counter() - t0
+
+    wall(allocating)                                    # first round trip: the block enters the lane's cache
+    launches = lane.counters()["kernel_launches"]
+    alloc_enqueue, alloc_total = wall(allocating)
+    assert lane.counters()["kernel_launches"] - launches == rounds
+    pre_enqueue, pre_total = wall(preallocated)
+    print(f"1000 projections: preallocated {pre_total * 1e3:.1f} ms (enqueue {pre_enqueue * 1e3:.1f}), "
+          f"allocate+dispose {alloc_total * 1e3:.1f} ms (enqueue {alloc_enqueue * 1e3:.1f})")
+    assert alloc_total <= 1.2 * pre_total + 2e-3
+    peak = lane.counters()["peak_allocated_bytes"]
+    wall(allocating)
+    assert lane.counters()["peak_allocated_bytes"] == peak       # the same block is handed out again and again
+    # results are those of the preallocated call
+    y = mats[0].forward(lane, x, None, 1)
+    mats[0].forward(lane, x, None, 1, out=keep)
+    assert np.array_equal(_bits(lane.read(y)), _bits(lane.read(keep)))
+    for b in (y, keep, x):
+        b.dispose()
+    for m in mats:
+        m.dispose()
+
+
+# ------------------------------------------------------------------------------- a captured batch, replayed
+
+def test_captured_batch_replays_after_other_batches(lane):
+    """A batch captured into a graph carries its descriptor table: batches with other descriptors issued between the
+    replays (which rewrite the lane's table, and here also outgrow it) must not change what a replay computes."""
+    lib, h = lane._lib, lane._handle
+    rng = np.random.default_rng(77)
+
+    def make(shapes, seed):
+        items = []
+        for i, (typ, in_w, out_w) in enumerate(shapes):
+            payload = synth.matrix(typ, out_w, in_w, seed=seed + i)
+            x = rng.standard_normal((1, in_w)).astype(np.float32)
+            items.append((typ, in_w, out_w, payload, x, lane.upload_raw(payload), lane.upload_raw(x), lane.allocate(out_w)))
+        descs = (MatvecDesc * len(items))()
+        for i, (typ, in_w, out_w, payload, x, wb, xb, yb) in enumerate(items):
+            descs[i] = MatvecDesc(xb.ptr, wb.ptr, None, yb.ptr, typ, 1, in_w, out_w)
+        return items, descs
+
+    small, small_descs = make([(GGML_Q8_0, 1024, 200), (GGML_Q4_K, 512, 90), (GGML_Q8_0, 2048, 33)], 100)
+    other, other_descs = make([(GGML_Q4_K, 1024, 70), (GGML_Q8_0, 512, 64)], 200)
+    # 1500 one-row entries need more than the 64 KB table the lane starts with: the table is replaced
+    many_x = lane.upload_raw(rng.standard_normal((1500, 256)).astype(np.float32))
+    many_w = lane.upload_raw(synth.matrix(GGML_Q8_0, 3, 256, seed=5))
+    many_y = lane.allocate(1500 * 3)
+    many_descs = (MatvecDesc * 1)()
+    many_descs[0] = MatvecDesc(many_x.ptr, many_w.ptr, None, many_y.ptr, GGML_Q8_0, 1500, 256, 3)
+
+    def expect(items):
+        return [oracle.linear_f64(t, p, x, None, 1, i, o)[0][0] for t, i, o, p, x, *_ in items]
+
+    def clear(items):
+        for *_, yb in items:
+            lane.fill_u32(yb, NAN_BITS, yb.nbytes // 4)
+
+    def check_items(items, want):
+        for (typ, in_w, out_w, *_rest), ref in zip(items, want):
+            got = lane.read(_rest[-1])
+            assert oracle.rel_l2(got, ref) <= MATVEC_BAR, (typ, in_w, out_w)
+
+    want_small, want_other = expect(small), expect(other)
+    check(lib.nnhip_quant_matvec_batch(h, small_descs, len(small)), "quant_matvec_batch")     # eager, sizes the table
+    lane.synchronize()
+    check_items(small, want_small)
+    eager = [lane.read(it[-1]) for it in small]
+
+    lane.graph_begin()
+    check(lib.nnhip_quant_matvec_batch(h, small_descs, len(small)), "quant_matvec_batch")
+    graph = lane.graph_end()
+    for between in (None, (other_descs, len(other)), (many_descs, 1), (other_descs, len(other))):
+        if between is not None:
+            clear(other)
+            check(lib.nnhip_quant_matvec_batch(h, between[0], between[1]), "quant_matvec_batch")
+            lane.synchronize()
+            if between[0] is other_descs:
+                check_items(other, want_other)
+        clear(small)
+        lane.synchronize()
+        lane.graph_launch(graph)
+        lane.synchronize()
+        for it, first in zip(small, eager):
+            assert np.array_equal(_bits(lane.read(it[-1])), _bits(first))
+    # the eager path after replays: the lane must not believe its table still holds the last eager batch
+    clear(other)
+    check(lib.nnhip_quant_matvec_batch(h, other_descs, len(other)), "quant_matvec_batch")
+    lane.synchronize()
+    check_items(other, want_other)
+    ref_many, _ = oracle.linear_f64(GGML_Q8_0, synth.matrix(GGML_Q8_0, 3, 256, seed=5),
+                                    np.frombuffer(lane.read(many_x, np.float32), np.float32).reshape(1500, 256), None, 1500, 256, 3)
+    assert oracle.rel_l2(lane.read(many_y).reshape(1500, 3), ref_many) <= MATVEC_BAR
+    lane.graph_destroy(graph)
+    for items in (small, other):
+        for it in items:
+            for b in it[5:]:
+                b.dispose()
+    for b in (many_x, many_w, many_y):
+        b.dispose()

@@ -200,6 +200,44 @@ def test_matvec_row_tiles_equal_single_rows_bitwise(lane, rows, in_w, out_w):
     _check_against_f64(_run_matvec(lane, GGML_Q8_0, _random_payload(GGML_Q8_0, out_w, in_w, seed=31), x, bias, rows, in_w, out_w), ref, asum)
 
 
+@pytest.mark.parametrize("in_w", [64, 128, 192, 256])
+@pytest.mark.parametrize("out_w", [300, 1000, 5000])
+def test_matvec_narrow_rows_several_input_rows(lane, in_w, out_w):
+    """Rows of one to four units with several input rows: a workgroup then holds hundreds of matrix rows per step, and
+    the results of a whole ring turn (times the input rows of the tile) must still fit its LDS result buffer.  Compared
+    with the oracle and, bit for bit, with single-row launches (NaN guards past the output checked by the helper).
+    Odd shapes and guard elements follow NNtrain.Core.Tests/Qwen35GpuLinearTests.cs:24-86."""
+    from nntrain_amd import GGML_BF16
+    rng = np.random.default_rng(in_w * 7 + out_w)
+    bias = rng.standard_normal(out_w).astype(np.float32)
+    bf16 = synth.to_bf16_bits(rng.standard_normal((out_w, in_w), dtype=np.float32) * np.float32(0.02)).view(np.uint8).reshape(-1)
+    q8 = _random_payload(GGML_Q8_0, out_w, in_w, seed=in_w + out_w)
+    singles = {}
+    for rows in (1, 2, 3, 4, 7):
+        x = synth.activations(7, in_w, seed=in_w)[:rows]
+        for typ, payload in ((GGML_Q8_0, q8), (GGML_BF16, bf16)):
+            y = _run_matvec(lane, typ, payload, x, bias, rows, in_w, out_w)
+            if rows == 1:
+                for r in range(7):
+                    xr = synth.activations(7, in_w, seed=in_w)[r:r + 1]
+                    singles[(typ, r)] = _run_matvec(lane, typ, payload, xr, bias, 1, in_w, out_w)[0]
+            for r in range(rows):
+                assert np.array_equal(_bits(y[r]), _bits(singles[(typ, r)])), (typ, rows, r)
+            if typ == GGML_Q8_0:
+                ref, asum = oracle.linear_f64(typ, payload, x, bias, rows, in_w, out_w)
+                _check_against_f64(y, ref, asum)
+
+
+def test_matvec_narrow_rows_very_tall_matrix(lane):
+    """in_w = 64 with more rows than one ring turn of every workgroup holds: the flush in the middle of the loop."""
+    in_w, out_w = 64, 400_000
+    payload = _random_payload(GGML_Q8_0, out_w, in_w, seed=5)
+    x = synth.activations(1, in_w, seed=6)
+    y = _run_matvec(lane, GGML_Q8_0, payload, x, None, 1, in_w, out_w)
+    ref, asum = oracle.linear_f64(GGML_Q8_0, payload, x, None, 1, in_w, out_w)
+    _check_against_f64(y, ref, asum)
+
+
 def test_matvec_q8_0_odd_block_count_rows(lane):
     in_w, out_w = 32 * 5, 19
     payload = _random_payload(GGML_Q8_0, out_w, in_w, seed=77)

@@ -23,11 +23,84 @@ def test_library_exports_every_declared_symbol():
     assert declared == set(native.PROTOTYPES), declared ^ set(native.PROTOTYPES)
 
 
+def _c_prototypes(header: str) -> dict:
+    """name -> list of argument classes from nnhip.h: 'p' (pointer, size_t, uint64_t: one unsigned 64-bit register),
+    'i32', 'u32', 'i64', 'f32'."""
+    protos = {}
+    for m in re.finditer(r"NNHIP_API\s+(?:int|uint32_t)\s+(nnhip_\w+)\s*\(([^;]*?)\)\s*;", header, re.S):
+        args = []
+        body = " ".join(m.group(2).split())
+        if body != "void":
+            for a in body.split(","):
+                a = a.strip()
+                if "*" in a or a.startswith("size_t"):
+                    args.append("p")
+                elif a.startswith("uint32_t"):
+                    args.append("u32")
+                elif a.startswith("int64_t"):
+                    args.append("i64")
+                elif a.startswith("uint64_t"):
+                    args.append("p")
+                elif a.startswith("float"):
+                    args.append("f32")
+                elif a.startswith("int"):
+                    args.append("i32")
+                else:
+                    raise AssertionError(f"unclassified C argument {a!r} of {m.group(1)}")
+        protos[m.group(1)] = args
+    return protos
+
+
+def test_csharp_declarations_match_the_header():
+    """bindings/csharp/NnHipNative.cs is not compiled here, so every LibraryImport is checked against include/nnhip.h
+    mechanically: same set of names, same arity, same 32/64-bit width and kind per argument, and the structures both
+    bindings pass by pointer have the sizes the C compiler gives them."""
+    root = native.library_path().parent.parent.parent
+    protos = _c_prototypes((root / "include" / "nnhip.h").read_text())
+    assert set(protos) == set(native.PROTOTYPES)
+    cs = (root / "bindings" / "csharp" / "NnHipNative.cs").read_text()
+    width = {"nint": "p", "nuint": "p", "int": "i32", "uint": "u32", "long": "i64", "ulong": "p", "float": "f32"}
+    seen = {}
+    for m in re.finditer(r"\[LibraryImport\(Library\)\]\s+internal static partial (\w+) (nnhip_\w+)\(([^)]*)\);", cs):
+        ret, name, body = m.groups()
+        args = []
+        for a in filter(None, (x.strip() for x in body.split(","))):
+            parts = a.split()
+            if parts[0] == "out" or parts[-2].endswith("*"):
+                args.append("p")
+            else:
+                args.append(width[parts[-2]])
+        seen[name] = args
+        assert ret == ("uint" if name == "nnhip_abi_version" else "int"), name
+    assert set(seen) == set(protos), set(seen) ^ set(protos)
+    for name, args in protos.items():
+        assert seen[name] == args, (name, seen[name], args)
+    # ctypes prototypes agree with the header as well
+    kinds = {ctypes.c_int: "i32", ctypes.c_uint32: "u32", ctypes.c_int64: "i64", ctypes.c_float: "f32"}
+    for name, (_, argtypes) in native.PROTOTYPES.items():
+        got = [kinds.get(t, "p") for t in argtypes]
+        assert got == protos[name], (name, got, protos[name])
+    # structure sizes: C# field lists (4-byte scalars, 8-byte nint / ulong) against the ctypes structures
+    sizes = {"uint": 4, "int": 4, "float": 4, "nint": 8, "ulong": 8}
+    for cs_name, ct in (("ErrorInfo", native.ErrorInfo), ("LaneCounters", native.LaneCounters), ("MatvecDesc", native.MatvecDesc),
+                        ("FusedMatvecDesc", native.FusedMatvecDesc), ("MatvecPlanInfo", native.MatvecPlanInfo)):
+        body = re.search(r"internal struct %s\s*\{(.*?)\n    \}" % cs_name, cs, re.S).group(1)
+        fields = re.findall(r"internal (\w+) \w+;", body)
+        offset = 0
+        for f in fields:
+            offset = (offset + sizes[f] - 1) // sizes[f] * sizes[f] + sizes[f]
+        assert (offset + 7) // 8 * 8 == ctypes.sizeof(ct), (cs_name, offset, ctypes.sizeof(ct))
+        assert len(fields) == len(ct._fields_), cs_name
+    assert ctypes.sizeof(native.FusedMatvecDesc) == 120
+
+
 def test_abi_version_and_struct_layouts():
     assert native.abi_version() == (1, 0)
     assert ctypes.sizeof(native.ErrorInfo) == 32      # the reference's NativeErrorInfo layout
     assert ctypes.sizeof(native.MatvecDesc) == 48
     assert ctypes.sizeof(native.LaneCounters) == 48
+    assert ctypes.sizeof(native.MatvecPlanInfo) == 40
+    assert ctypes.sizeof(native.FusedMatvecDesc) == 120
 
 
 def test_geometry_queries_without_a_gpu():
@@ -46,6 +119,38 @@ def test_geometry_queries_without_a_gpu():
     assert lib.nnhip_matrix_bytes(12, 5000, 10, byref(n)) == 3
     info, msg = native.last_error()
     assert info.status == 3 and "256" in msg and info.struct_size == 32
+
+
+def test_matvec_plan_keeps_a_ring_turn_inside_the_result_buffer():
+    """A workgroup of the row-step kernel parks ring_depth * rows_per_step * row_tile results in LDS before it can
+    flush; the plan must keep that inside the buffer for every accepted shape (narrow rows with several input rows are
+    the ones that would overrun)."""
+    lib = native.load_library()
+    info = native.MatvecPlanInfo(struct_size=ctypes.sizeof(native.MatvecPlanInfo))
+    seen_tiles = set()
+    for typ, widths in ((8, (64, 128, 192, 256, 320, 640, 1024, 5376, 21504)), (30, (64, 128, 256, 4096)),
+                        (12, (256, 512, 5120, 17408)), (13, (256, 5120)), (14, (256, 5120)), (21, (256, 5120)),
+                        (22, (256, 17408))):
+        for in_w in widths:
+            for out_w in (1, 2, 63, 300, 1000, 5000, 200_000, 1_000_000):
+                for rows in (1, 2, 3, 4, 7, 16):
+                    assert lib.nnhip_matvec_plan(typ, rows, in_w, out_w, 256, byref(info)) == 0, (typ, in_w, out_w, rows)
+                    if info.kernel != 0:
+                        continue
+                    assert info.ring_depth * info.rows_per_step * info.row_tile <= info.result_buffer_floats, \
+                        (typ, in_w, out_w, rows, info.rows_per_step, info.row_tile)
+                    assert info.rows_per_step * (in_w // 64) <= info.threads <= 1024
+                    assert info.threads % 64 == 0 and 1 <= info.rows_per_step <= out_w
+                    assert info.steps == -(-out_w // info.rows_per_step) and info.groups == min(info.steps, 256)
+                    assert info.dynamic_lds_bytes <= 140 * 1024
+                    seen_tiles.add((typ, info.row_tile))
+    assert {(8, 1), (8, 2), (8, 4), (30, 4), (12, 1)} <= seen_tiles
+    assert lib.nnhip_matvec_plan(8, 1, 32 * 5, 19, 256, byref(info)) == 0 and info.kernel == 1   # odd block count
+    assert lib.nnhip_matvec_plan(12, 1, 255, 19, 256, byref(info)) == 3
+    assert lib.nnhip_matvec_plan(12, 1, 256 * 300, 19, 256, byref(info)) == 8
+    assert lib.nnhip_matvec_plan(99, 1, 256, 19, 256, byref(info)) == 2
+    info.struct_size = 8
+    assert lib.nnhip_matvec_plan(12, 1, 256, 19, 256, byref(info)) == 1
 
 
 def test_bad_handles_are_reported_not_dereferenced():
