@@ -221,6 +221,17 @@ NNHIP_API int nnhip_matvec_plan(uint32_t ggml_type, int rows, int in_w, int out_
  * kept until the lane is destroyed.  Asynchronous. */
 NNHIP_API int nnhip_quant_matvec_batch(void* lane, const nnhip_matvec_desc* descs, int count);
 
+/* nnhip_quant_matvec_batch for callers that cannot allocate device memory: code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same arguments and bit-identical
+ * results; the descriptor table lives in a fixed array inside the library's device image (80 bytes per mat-vec row,
+ * NNHIP_STATIC_BATCH_MAX_ENTRIES rows = 80 KiB, held on every device the library is loaded on until the process ends)
+ * instead of lane-owned memory, and the call makes no device or host allocation.  A batch with more rows (the sum of
+ * `rows` over the descriptors) is rejected with NNHIP_ERR_TOO_LARGE.  All lanes of a device share the one array: a
+ * call rewrites the entries it uses, and calls whose work overlaps on one device (two lanes, or one lane whose earlier
+ * static batch is still running while another lane issues one) race on it - serialise them.  Asynchronous. */
+#define NNHIP_STATIC_BATCH_MAX_ENTRIES 1024
+NNHIP_API int nnhip_quant_matvec_batch_static(void* lane, const nnhip_matvec_desc* descs, int count);
+
 /* Prefill: y[r, o] = bias[o] + sum_k x[r, k] * w[o, k] with x given as bfloat16 bit patterns [rows, in_w];
  * weight tiles are dequantized to bfloat16 in LDS and contracted on MFMA with FP32 accumulators.  Replaces the
  * XMX prefill launch of Matrix.Forward for rows >= 16 (Qwen35QuantizedModel.cs:1249-1317, kernels

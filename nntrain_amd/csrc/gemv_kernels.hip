@@ -1136,6 +1136,12 @@ hipError_t write_table(Lane* lane, void* device_table, const BatchEntry* entries
     return hipSuccess;
 }
 
+// Fixed device workspace of nnhip_quant_matvec_batch_static: the descriptor table of a batch, in a file-scope device
+// array so that the entry point never allocates.  Every device holds its own copy at its own address; host code uses
+// the address hipGetSymbolAddress returns for the current device (kept in the lane), never the array's name.
+constexpr int kStaticTableEntries = NNHIP_STATIC_BATCH_MAX_ENTRIES;
+static __device__ __align__(256) unsigned char scratch[kStaticTableEntries * sizeof(BatchEntry)];
+
 void shape_of(uint32_t type, int* max_t, int* depth)
 {
     switch (type) {
@@ -1422,6 +1428,28 @@ hipError_t launch_matvec_batch(Lane* lane, const nnhip_matvec_desc* descs, int c
         }
     }
     return launch_batch_groups(lane, lane->batch_table, groups, ngroups, descs, count);
+}
+
+hipError_t static_table_address(void** address)
+{
+    return hipGetSymbolAddress(address, HIP_SYMBOL(scratch));
+}
+
+// As launch_matvec_batch with the table in the device's fixed workspace: no device or host allocation on this path.
+// hipErrorInvalidValue: more entries than the workspace holds.
+hipError_t launch_matvec_batch_static(Lane* lane, const nnhip_matvec_desc* descs, int count)
+{
+    if (!lane->static_table) return hipErrorNotInitialized;
+    BatchEntry entries[kStaticTableEntries];
+    BatchGroup groups[kBatchTypes];
+    int ngroups = 0;
+    const long n = build_batch(descs, count, entries, kStaticTableEntries, groups, &ngroups);
+    if (n < 0) return hipErrorInvalidValue;
+    if (n > 0) {
+        const hipError_t e = write_table(lane, lane->static_table, entries, static_cast<size_t>(n));
+        if (e != hipSuccess) return e;
+    }
+    return launch_batch_groups(lane, lane->static_table, groups, ngroups, descs, count);
 }
 
 }  // namespace nnhip

@@ -197,6 +197,13 @@ int nnhip_lane_create(int device, void** out)
         delete lane;
         return hip_fail(e, NNHIP_OP_LANE_CREATE, device, "hipStreamCreateWithFlags");
     }
+    // the fixed batch workspace: every device has its own copy of the array, at its own address
+    e = static_table_address(&lane->static_table);
+    if (e != hipSuccess || !lane->static_table) {
+        (void)hipStreamDestroy(lane->stream);
+        delete lane;
+        return hip_fail(e, NNHIP_OP_LANE_CREATE, device, "hipGetSymbolAddress of the fixed batch workspace");
+    }
     *out = lane;
     return NNHIP_OK;
 }
@@ -619,6 +626,30 @@ int nnhip_quant_matvec_batch(void* handle, const nnhip_matvec_desc* descs, int c
                     "the batch needs a larger descriptor table than the lane holds, and a table cannot grow while a graph is "
                     "being captured: issue a batch of this size once before the capture");
     if (e != hipSuccess) return hip_fail(e, NNHIP_OP_MATVEC_BATCH, lane->device, "batched mat-vec launch");
+    return NNHIP_OK;
+}
+
+int nnhip_quant_matvec_batch_static(void* handle, const nnhip_matvec_desc* descs, int count)
+{
+    NNHIP_LANE(handle, NNHIP_OP_MATVEC_BATCH)
+    if (count < 0 || (count > 0 && !descs))
+        return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_MATVEC_BATCH, lane->device, 0, "descriptor array is null or count negative");
+    long entries = 0;
+    for (int i = 0; i < count; ++i) {
+        const nnhip_matvec_desc& d = descs[i];
+        int rc = check_linear(NNHIP_OP_MATVEC_BATCH, lane, d.ggml_type, d.x, d.w, d.y, d.rows, d.in_w, d.out_w);
+        if (rc != NNHIP_OK) return rc;
+        if (d.in_w > matvec_max_in_w(d.ggml_type))
+            return fail(NNHIP_ERR_TOO_LARGE, NNHIP_OP_MATVEC_BATCH, lane->device, 0, "descriptor %d: in_w %d exceeds the %d values one workgroup can stage", i, d.in_w, matvec_max_in_w(d.ggml_type));
+        entries += d.rows;
+    }
+    if (entries > NNHIP_STATIC_BATCH_MAX_ENTRIES)
+        return fail(NNHIP_ERR_TOO_LARGE, NNHIP_OP_MATVEC_BATCH, lane->device, 0,
+                    "the batch has %ld mat-vec rows; the fixed workspace holds %d (use nnhip_quant_matvec_batch, or split the batch)",
+                    entries, NNHIP_STATIC_BATCH_MAX_ENTRIES);
+    if (count == 0) return NNHIP_OK;
+    hipError_t e = launch_matvec_batch_static(lane, descs, count);
+    if (e != hipSuccess) return hip_fail(e, NNHIP_OP_MATVEC_BATCH, lane->device, "batched mat-vec launch (fixed workspace)");
     return NNHIP_OK;
 }
 

@@ -38,6 +38,7 @@ struct Lane {
     size_t batch_table_bytes = 0;               // its capacity
     std::vector<void*> retired_tables;          // outgrown tables: freed with the lane, a captured graph may name them
     std::vector<char> batch_shadow;             // the entries the device table holds now (empty: unknown)
+    void* static_table = nullptr;               // this device's address of the library's fixed batch workspace
 };
 
 struct Event {
@@ -79,6 +80,9 @@ hipError_t launch_matvec(Lane* lane, uint32_t type, const float* x, const void* 
 bool matvec_fused_supported(uint32_t type, int in_w);
 hipError_t launch_matvec_fused(Lane* lane, const nnhip_fused_matvec_desc& d);
 hipError_t launch_matvec_batch(Lane* lane, const nnhip_matvec_desc* descs, int count);
+// The fixed device workspace: its address on the current device, and the batched launch that uses it.
+hipError_t static_table_address(void** address);
+hipError_t launch_matvec_batch_static(Lane* lane, const nnhip_matvec_desc* descs, int count);
 hipError_t launch_matmul_bf16(Lane* lane, uint32_t type, const uint16_t* x, const void* w, const float* bias,
                               float* y, int rows, int in_w, int out_w);
 hipError_t launch_to_bf16(Lane* lane, const float* x, uint16_t* out, size_t count);
