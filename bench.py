@@ -258,7 +258,13 @@ def run_gemv(args, lane, nn, oracle):
             descs[i] = MatvecDesc(x.ptr, w.ptr, None, ys[i].ptr, typ, 1, in_w, out_w)
         nn.native.check(lib.nnhip_quant_matvec_batch(h, descs, len(ring)), "quant_matvec_batch")
         lane.synchronize()
-        if not np.array_equal(lane.read(ys[-1], np.uint32), lane.read(y, np.uint32)):
+        # large Q4_K / Q5_K groups run on the matrix-core kernel (fixed-point activations): same bar against the oracle,
+        # not the single launch's bits; the other formats share the single launch's kernel and must match bitwise
+        y_batch = lane.read(ys[-1], np.float32)
+        rel_batch = oracle.rel_l2(y_batch, ref[0])
+        if not rel_batch <= 1e-5:
+            raise SystemExit(f"{name}: batched launch parity failure, rel-L2 {rel_batch:.3e}")
+        if tname not in ("GGML_Q4_K", "GGML_Q5_K") and not np.array_equal(y_batch.view(np.uint32), lane.read(y, np.uint32)):
             raise SystemExit(f"{name}: batched launch differs bitwise from the single launch")
         samples_batch = []
         for _ in range(7):
@@ -271,7 +277,8 @@ def run_gemv(args, lane, nn, oracle):
                      "sustained_us_per_matvec_batched": round(us_batch, 2),
                      "sustained_gb_per_s_batched": round(algo / us_batch / 1e3, 1),
                      "sustained_frac_of_8TBs": round(algo / us_batch / 1e3 / HBM_PEAK_GBS, 4),
-                     "algorithmic_bytes": algo, "rel_l2_vs_f64_oracle": rel, "weight_copies_rotated": len(ring)}
+                     "algorithmic_bytes": algo, "rel_l2_vs_f64_oracle": rel, "rel_l2_batched_vs_f64_oracle": rel_batch,
+                     "weight_copies_rotated": len(ring)}
         log(f"[gemv] {name}: single launch {us_ring:.2f} us ({algo / us_ring / 1e3:.0f} GB/s, "
             f"{100 * algo / us_ring / 1e3 / HBM_PEAK_GBS:.1f}% of 8 TB/s) HBM, {us_same:.2f} us cache-resident; batched "
             f"{us_batch:.2f} us/mat-vec ({100 * algo / us_batch / 1e3 / HBM_PEAK_GBS:.1f}%); rel-L2 {rel:.2e}")

@@ -213,7 +213,12 @@ NNHIP_API int nnhip_matvec_plan(uint32_t ggml_type, int rows, int in_w, int out_
 
 /* `count` independent mat-vecs enqueued as one unit of work (a single launch per group of equal type), for the
  * per-token projection sets that ForwardTokenDevice issues back to back (Qwen35QuantizedModel.cs:451-513).
- * `descs` is a host array, read before the call returns.  Results are identical to `count` nnhip_quant_matvec calls.
+ * `descs` is a host array, read before the call returns.  Results are identical to `count` nnhip_quant_matvec calls,
+ * with one exception: Q4_K and Q5_K matrices of one in_w whose 16-row tiles add up to 2048 or more within a call (in_w
+ * a multiple of 256 that the matrix-core mat-vec can split: 5120 and 2560 among others) are multiplied on the matrix
+ * cores with the activations in 32-bit fixed point.  Those results are deterministic, depend on the weights, in_w and
+ * the activations only (not on out_w, the other matrices of the call or the order), agree with the single launch to
+ * FP32 summation accuracy (relative L2 difference below 1e-6) and are closer to the exact product than it.
  * The descriptors reach the device as a table in lane-owned memory, written by a small kernel on the lane's stream
  * (skipped when the table already holds them), so the call never waits for the device.  Under graph capture the write
  * is recorded with the launch and a replay restores the table it needs; the table cannot grow during a capture
@@ -223,7 +228,7 @@ NNHIP_API int nnhip_quant_matvec_batch(void* lane, const nnhip_matvec_desc* desc
 
 /* nnhip_quant_matvec_batch for callers that cannot allocate device memory: code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same arguments and bit-identical
- * results; the descriptor table lives in a fixed array inside the library's device image (80 bytes per mat-vec row,
+ * results to nnhip_quant_matvec_batch; the descriptor table lives in a fixed array inside the library's device image (80 bytes per mat-vec row,
  * NNHIP_STATIC_BATCH_MAX_ENTRIES rows = 80 KiB, held on every device the library is loaded on until the process ends)
  * instead of lane-owned memory, and the call makes no device or host allocation.  A batch with more rows (the sum of
  * `rows` over the descriptors) is rejected with NNHIP_ERR_TOO_LARGE.  All lanes of a device share the one array: a

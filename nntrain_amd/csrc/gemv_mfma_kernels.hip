@@ -1,0 +1,693 @@
+// Decode mat-vec on the matrix cores for the super-block formats whose unpacking is too much vector-ALU work for the
+// lane-per-unit kernels (gemv_kernels.hip): Q4_K and Q5_K here.  Used for the large groups of a batched launch, where
+// it streams faster than the row-step kernels; it takes longer to start, so single launches stay with those.
+//
+// y[r, o] = bias[o] + sum_k x[r, k] * w[o, k]     (NNtrain.Arc/Kernels/qwen.cl:374-406 defines the operator)
+//
+// Arithmetic.  The activation vector is turned into 32-bit fixed point relative to its largest magnitude
+// (v = rint(x * 2^e), |v| <= 2^30) and split into four balanced base-256 digits (each in [-128, 127]).
+// v_mfma_i32_16x16x32_i8 then takes the exact integer sums sum_k digit_p(x_k) * q_k of one 32-weight sub-block for 16
+// matrix rows at a time (operand B = the sub-block's quants as bytes, two masks away from the raw block; operand A = digit
+// planes).  The four K groups of an instruction carry four different 64-weight quarters of a super-block and operand A is
+// block-diagonal to match (rows 4P .. 4P+3 = the four digit planes of quarter P in K group P, zeros elsewhere), so the 64
+// lanes of the result hold the plane sums of (quarter lane / 16, matrix row lane % 16).  They are recombined
+// (sum_p 256^p S_p), scaled by d * scale and accumulated per lane in FP32; minima use FP32 sums of x per sub-block:
+// sum x (s q - m) = s sum(q x) - m sum(x).  The error of the fixed-point form is at most 2^-31 of the largest |x| per
+// element, below the rounding of one FP32 product.
+//
+// Data movement.  A stage is 16 matrix rows x C super-blocks, copied verbatim: every wave requests its 1 KB pieces of a
+// stage (consecutive memory, non-temporal 16-byte buffer loads) into one of two register sets and parks the set in one of
+// two LDS stage buffers a whole stage later, so two stages are always on their way while one is multiplied; one
+// workgroup barrier per stage publishes the parked stage and frees the other buffer.  The LDS row stride is an odd
+// number of 16-byte pieces, so the 16 rows an operand read touches fall into different bank groups.
+//
+// Work split.  Wave w of W owns super-block columns w (+ W) of every stage (a task = 16 rows x one super-block: eight
+// MFMAs) and keeps its part of operand A for those columns in registers for as long as the activations stay the same;
+// when they change, the digit planes pass once through the free stage buffer.  At the end of a 16-row tile the four
+// quarters are added across lanes, the W wave partials go through LDS and 16 lanes add them in wave order.  W and C depend
+// on the storage type and in_w only, and a launch is a table of matrices that share both, worked through as one sequence
+// of tiles dealt round-robin to the workgroups: a row's bits depend on its weights, in_w and the activation vector, never
+// on out_w, on the other matrices of the launch or on its place in it.
+#include <cstring>
+#include <type_traits>
+
+#include "nnhip_internal.h"
+#include "quant_device.h"
+
+namespace nnhip {
+
+namespace {
+
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kTileRows = 16;            // matrix rows per stage = the N of the MFMA
+constexpr int kMaxWaves = 12;            // three waves per SIMD: 170 vector registers each
+
+
+constexpr int kLdsBudget = 156 * 1024;   // dynamic LDS a workgroup may take (the static arrays take 2.1 KB of the 160 KB)
+constexpr uint32_t kNoPiece = 0x80000000u;       // added to the offset of a piece that is not to be fetched: beyond any matrix
+
+#define NNHIP_LDS_PTR __attribute__((address_space(3)))
+// address-space qualifiers only mean something to the device pass
+#if defined(__HIP_DEVICE_COMPILE__)
+#define NNHIP_CONST_PTR __attribute__((address_space(4)))
+#else
+#define NNHIP_CONST_PTR
+#endif
+
+// Launch geometry of the matrix-core mat-vec: a function of the storage type and in_w alone.
+struct MfmaGeom {
+    int waves;            // W
+    int cols;             // C: super-block columns per stage (a multiple of W)
+    int kchunks;          // stages per 16-row tile = ceil(nblocks / C)
+    int row_pieces;       // LDS row stride of a stage in 16-byte pieces (odd)
+    int stage_bytes;      // bytes of one stage (multiple of 1 KB)
+    int stage_loads;      // 1 KB load instructions that fill a stage
+    int loads_per_wave;   // ceil(stage_loads / W)
+    int stages;           // LDS stage buffers (2)
+    int tasks;            // M: super-block columns a wave owns per stage
+    size_t lds_bytes;     // the stage buffers
+};
+
+using MfmaEntry = MfmaTableEntry;     // one matrix of a launch (nnhip_internal.h)
+
+struct MfmaArgs {
+    const MfmaEntry* table;        // device table, one entry per matrix and input row
+    int entries;
+    int total_tiles;
+    int in_w;
+    int nblocks;                   // super-blocks per row
+    uint32_t row_bytes;
+    uint32_t row_pieces_magic;     // ceil(2^32 / row_pieces)
+    MfmaGeom g;
+};
+
+__device__ __forceinline__ uint32_t umax_u(uint32_t a, uint32_t b) { return a > b ? a : b; }
+
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_mov_u(uint32_t v)
+{
+    return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), CTRL, 0xf, 0xf, true));
+}
+
+__device__ __forceinline__ uint32_t wave_umax(uint32_t v)
+{
+    v = umax_u(v, dpp_mov_u<0xB1>(v));
+    v = umax_u(v, dpp_mov_u<0x4E>(v));
+    v = umax_u(v, dpp_mov_u<0x141>(v));
+    v = umax_u(v, dpp_mov_u<0x140>(v));
+    const uint32_t a = __builtin_amdgcn_readlane(v, 0), b = __builtin_amdgcn_readlane(v, 16);
+    const uint32_t c = __builtin_amdgcn_readlane(v, 32), d = __builtin_amdgcn_readlane(v, 48);
+    return umax_u(umax_u(a, b), umax_u(c, d));
+}
+
+// p[l] + p[l+16] + p[l+32] + p[l+48] as (p0 + p1) + (p2 + p3), in every lane (v_permlane16_swap exchanges the odd
+// 16-lane rows of its first operand with the even rows of its second, v_permlane32_swap the upper half of the first
+// with the lower half of the second).
+__device__ __forceinline__ float quarter_sum(float p)
+{
+    const uint32_t u = __float_as_uint(p);
+    auto s16 = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    const float t = __uint_as_float(s16[0]) + __uint_as_float(s16[1]);
+    const uint32_t v = __float_as_uint(t);
+    auto s32 = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+    return __uint_as_float(s32[0]) + __uint_as_float(s32[1]);
+}
+
+// Four fixed-point values -> the four digit planes of those values (byte i of plane p = digit p of value i).
+__device__ __forceinline__ void digit_planes(int v0, int v1, int v2, int v3, uint32_t out[4])
+{
+    // balanced digits: add 128 to the three low digits with carry, then flip their top bits
+    const uint32_t d0 = (static_cast<uint32_t>(v0) + 0x00808080u) ^ 0x00808080u;
+    const uint32_t d1 = (static_cast<uint32_t>(v1) + 0x00808080u) ^ 0x00808080u;
+    const uint32_t d2 = (static_cast<uint32_t>(v2) + 0x00808080u) ^ 0x00808080u;
+    const uint32_t d3 = (static_cast<uint32_t>(v3) + 0x00808080u) ^ 0x00808080u;
+    // 4 x 4 byte transpose (v_perm_b32: selector bytes 0-3 pick from the second operand, 4-7 from the first)
+    const uint32_t t0 = __builtin_amdgcn_perm(d1, d0, 0x05010400u);   // d0.b0 d1.b0 d0.b1 d1.b1
+    const uint32_t t1 = __builtin_amdgcn_perm(d1, d0, 0x07030602u);   // d0.b2 d1.b2 d0.b3 d1.b3
+    const uint32_t t2 = __builtin_amdgcn_perm(d3, d2, 0x05010400u);
+    const uint32_t t3 = __builtin_amdgcn_perm(d3, d2, 0x07030602u);
+    out[0] = __builtin_amdgcn_perm(t2, t0, 0x05040100u);
+    out[1] = __builtin_amdgcn_perm(t2, t0, 0x07060302u);
+    out[2] = __builtin_amdgcn_perm(t3, t1, 0x05040100u);
+    out[3] = __builtin_amdgcn_perm(t3, t1, 0x07060302u);
+}
+
+// sum_p 256^p S_p of the four digit-plane sums.  |S_p| <= 32 * 31 * 128 < 2^17, so S_0 + 256 S_1 and S_2 + 256 S_3 are
+// exact in int32 and below 2^25... their conversions to FP32 round at most once each (below 2^24: exact), and one fused
+// multiply-add joins them.
+__device__ __forceinline__ float recombine(i32x4 s)
+{
+    const int lo = s[0] + (s[1] << 8), hi = s[2] + (s[3] << 8);
+    return fmaf(static_cast<float>(hi), 65536.0f, static_cast<float>(lo));
+}
+
+__device__ __forceinline__ i32x4 mfma_i8(uint32_t a0, uint32_t a1, uint32_t b0, uint32_t b1, i32x4 c)
+{
+    return __builtin_amdgcn_mfma_i32_16x16x32_i8(__builtin_bit_cast(long, u32x2{a0, a1}), __builtin_bit_cast(long, u32x2{b0, b1}),
+                                                 c, 0, 0, 0);
+}
+
+__device__ __forceinline__ u32x4 lds128(const uint8_t* p) { return *reinterpret_cast<const u32x4*>(p); }
+
+// The activation loads are written as inline assembly so that the compiler's counter bookkeeping does not see them: it
+// would otherwise wait for every load in flight, the weight stream included, before their first use.  The wait is placed
+// by hand (wait_vm_imm) and the registers are tied to it with an empty asm statement.
+//
+// 16 bytes per lane into registers; valid only after a wait_vm that covers it.
+__device__ __forceinline__ float4 gload16(const float* base, uint32_t voff)
+{
+    float4 r;
+    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(r) : "v"(voff), "s"(base) : "memory");
+    return r;
+}
+
+// This lane's part of operand A for one super-block column: 64 bytes (its digit plane of its quarter's 64 activations;
+// zeros in the lanes outside the block diagonal) and the FP32 sums of x over the quarter's two 32-weight sub-blocks.
+struct XSet {
+    u32x4 a[4];
+    float2 sx;
+};
+
+// One task of a storage format: 16 rows x one super-block.  `blk` is this lane's row of the stage at the task's block
+// column (LDS).  Adds this lane's share (quarter lane / 16 of row lane % 16) to accq (the quant part, still in
+// fixed-point units) and accm (the minimum part).
+struct Q4KTask {
+    static constexpr int kBlockBytes = kQ4KBytes;     // 144 = 9 pieces; blocks and rows are 16-byte aligned
+    struct Raw { u32x4 h, q1, q2; };
+
+    static __device__ __forceinline__ Raw load(const uint8_t* blk, int quarter)
+    {
+        Raw r;
+        r.q1 = lds128(blk + 16 + 32 * quarter);
+        r.q2 = lds128(blk + 32 + 32 * quarter);
+        r.h = lds128(blk);
+        return r;
+    }
+
+    static __device__ __forceinline__ void run(const Raw& r, const XSet& xs, int quarter, float& accq, float& accm)
+    {
+        constexpr uint32_t kLow = 0x0f0f0f0fu;
+        const u32x4 q1 = r.q1, q2 = r.q2, h = r.h;
+        const u32x4 a0 = xs.a[0], a1 = xs.a[1], a2 = xs.a[2], a3 = xs.a[3];
+        i32x4 s_lo = {0, 0, 0, 0}, s_hi = {0, 0, 0, 0};
+        // low nibbles: weights 0-31 of the quarter (sub-block 2 * quarter), high nibbles: weights 32-63
+        s_lo = mfma_i8(a0[0], a0[1], q1[0] & kLow, q1[1] & kLow, s_lo);
+        s_hi = mfma_i8(a2[0], a2[1], (q1[0] >> 4) & kLow, (q1[1] >> 4) & kLow, s_hi);
+        s_lo = mfma_i8(a0[2], a0[3], q1[2] & kLow, q1[3] & kLow, s_lo);
+        s_hi = mfma_i8(a2[2], a2[3], (q1[2] >> 4) & kLow, (q1[3] >> 4) & kLow, s_hi);
+        s_lo = mfma_i8(a1[0], a1[1], q2[0] & kLow, q2[1] & kLow, s_lo);
+        s_hi = mfma_i8(a3[0], a3[1], (q2[0] >> 4) & kLow, (q2[1] >> 4) & kLow, s_hi);
+        s_lo = mfma_i8(a1[2], a1[3], q2[2] & kLow, q2[3] & kLow, s_lo);
+        s_hi = mfma_i8(a3[2], a3[3], (q2[2] >> 4) & kLow, (q2[3] >> 4) & kLow, s_hi);
+        const float d = half_bits_to_float(h[0]), dmin = half_bits_to_float(h[0] >> 16);
+        uint32_t sc, mn;
+        k4_scale_pair(h[1], h[2], h[3], quarter, sc, mn);
+        accq = fmaf(d * ubyte0(sc), recombine(s_lo), accq);
+        accq = fmaf(d * ubyte1(sc), recombine(s_hi), accq);
+        accm = fmaf(dmin * ubyte0(mn), xs.sx.x, accm);
+        accm = fmaf(dmin * ubyte1(mn), xs.sx.y, accm);
+    }
+};
+
+// Q5_K: as Q4_K plus one high bit per weight; bit g of qh[i] belongs to weight i of sub-block g (header, 32 bytes of
+// qh, 128 nibble bytes: 176 = 11 pieces).
+struct Q5KTask {
+    static constexpr int kBlockBytes = kQ5KBytes;
+    struct Raw { u32x4 h, ha, hb, q1, q2; };
+
+    static __device__ __forceinline__ Raw load(const uint8_t* blk, int quarter)
+    {
+        Raw r;
+        r.q1 = lds128(blk + 48 + 32 * quarter);
+        r.ha = lds128(blk + 16);
+        r.q2 = lds128(blk + 64 + 32 * quarter);
+        r.hb = lds128(blk + 32);
+        r.h = lds128(blk);
+        return r;
+    }
+
+    static __device__ __forceinline__ void run(const Raw& r, const XSet& xs, int quarter, float& accq, float& accm)
+    {
+        constexpr uint32_t kLow = 0x0f0f0f0fu, kBit4 = 0x10101010u;
+        const u32x4 h = r.h, ha = r.ha, hb = r.hb, q1 = r.q1, q2 = r.q2;
+        const u32x4 a0 = xs.a[0], a1 = xs.a[1], a2 = xs.a[2], a3 = xs.a[3];
+        const int sh = 2 * quarter;
+        i32x4 s_lo = {0, 0, 0, 0}, s_hi = {0, 0, 0, 0};
+        auto lo5 = [&](uint32_t q, uint32_t hq) { return (q & kLow) | (((hq >> sh) << 4) & kBit4); };
+        auto hi5 = [&](uint32_t q, uint32_t hq) { return ((q >> 4) & kLow) | (((hq >> sh) << 3) & kBit4); };
+        s_lo = mfma_i8(a0[0], a0[1], lo5(q1[0], ha[0]), lo5(q1[1], ha[1]), s_lo);
+        s_hi = mfma_i8(a2[0], a2[1], hi5(q1[0], ha[0]), hi5(q1[1], ha[1]), s_hi);
+        s_lo = mfma_i8(a0[2], a0[3], lo5(q1[2], ha[2]), lo5(q1[3], ha[3]), s_lo);
+        s_hi = mfma_i8(a2[2], a2[3], hi5(q1[2], ha[2]), hi5(q1[3], ha[3]), s_hi);
+        s_lo = mfma_i8(a1[0], a1[1], lo5(q2[0], hb[0]), lo5(q2[1], hb[1]), s_lo);
+        s_hi = mfma_i8(a3[0], a3[1], hi5(q2[0], hb[0]), hi5(q2[1], hb[1]), s_hi);
+        s_lo = mfma_i8(a1[2], a1[3], lo5(q2[2], hb[2]), lo5(q2[3], hb[3]), s_lo);
+        s_hi = mfma_i8(a3[2], a3[3], hi5(q2[2], hb[2]), hi5(q2[3], hb[3]), s_hi);
+        const float d = half_bits_to_float(h[0]), dmin = half_bits_to_float(h[0] >> 16);
+        uint32_t sc, mn;
+        k4_scale_pair(h[1], h[2], h[3], quarter, sc, mn);
+        accq = fmaf(d * ubyte0(sc), recombine(s_lo), accq);
+        accq = fmaf(d * ubyte1(sc), recombine(s_hi), accq);
+        accm = fmaf(dmin * ubyte0(mn), xs.sx.x, accm);
+        accm = fmaf(dmin * ubyte1(mn), xs.sx.y, accm);
+    }
+};
+
+// s_waitcnt vmcnt(N): at most N vector-memory loads of this wave still in flight.  The immediate is
+// 0x0F70 | (N & 15) | ((N >> 4) << 14).
+template <int N>
+__device__ __forceinline__ void wait_vm_imm() { __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14)); }
+
+// Loads of the weight stream: 16 bytes per lane through a buffer descriptor that spans the matrix, non-temporal.  An
+// offset beyond the buffer returns zeros without touching memory.
+__device__ __forceinline__ u32x4 stream16(__amdgpu_buffer_rsrc_t matrix, uint32_t off)
+{
+    return __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(matrix, static_cast<int>(off), 0, 2));
+}
+
+// grid.x = workgroups striding over the launch's 16-row tiles, blockDim.x = 64 * W.  KC = stages per tile (1 or 2),
+// M = super-block columns a wave owns per stage, LPW = 1 KB pieces of a stage a wave moves.  A lane keeps operand A of its KC * M columns in registers for as long as the activations stay
+// the same.
+template <class F, int KC, int M, int LPW>
+__global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_kernel(MfmaArgs a)
+{
+    static_assert(KC == 1 || KC == 2, "a turn of the two register sets is one or two tiles");
+    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+    __shared__ float part[2][kMaxWaves][kTileRows];
+    __shared__ uint32_t red[kMaxWaves];
+
+    const MfmaGeom& g = a.g;
+    const int tid = threadIdx.x, lane = tid & 63, T = blockDim.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int W = g.waves;
+    const int row_l = lane & 15, quarter = lane >> 4;
+
+    // The table is read-only for the whole launch and indexed with workgroup-uniform values: through the constant
+    // address space those reads are scalar loads, which do not touch the vector-memory counter.
+    const NNHIP_CONST_PTR MfmaEntry* table = (const NNHIP_CONST_PTR MfmaEntry*)a.table;
+    auto entry_at = [&](int m) {
+        const NNHIP_CONST_PTR MfmaEntry& t = table[m];
+        MfmaEntry e;
+        e.x = t.x;
+        e.w = t.w;
+        e.bias = t.bias;
+        e.y = t.y;
+        e.out_w = t.out_w;
+        e.w_bytes = t.w_bytes;
+        e.tiles = t.tiles;
+        e.first_tile = t.first_tile;
+        return e;
+    };
+
+    // ---- this lane's pieces of a stage: piece I = wave + W * i is slots 64 I .. 64 I + 63 of the stage; slot s is
+    // 16-byte piece s % row_pieces of stage row s / row_pieces (the last piece of a row is padding when the row has an
+    // even number of pieces).  rel[i] is the piece's byte offset from the stage's first byte in the matrix; pieces that do
+    // not exist get an offset beyond any matrix and read as zeros.
+    const int pieces_used = g.cols * (F::kBlockBytes / 16);
+    uint32_t rel[LPW];
+#pragma unroll
+    for (int i = 0; i < LPW; ++i) {
+        const uint32_t slot = static_cast<uint32_t>(64 * (wave + W * i) + lane);
+        const uint32_t r = __umulhi(slot, a.row_pieces_magic);
+        const uint32_t q = slot - r * static_cast<uint32_t>(g.row_pieces);
+        const bool real = r < static_cast<uint32_t>(kTileRows) && q < static_cast<uint32_t>(pieces_used);
+        rel[i] = real ? r * a.row_bytes + q * 16u : kNoPiece;
+    }
+
+    // ---- the stage sequence of this workgroup: tiles blockIdx.x, blockIdx.x + G, ... of the launch's tile sequence,
+    // KC stages per tile
+    const int G = gridDim.x;
+    const int my_tiles = (a.total_tiles - static_cast<int>(blockIdx.x) + G - 1) / G;
+    const int total = my_tiles * KC;
+    const uint32_t chunk_bytes = static_cast<uint32_t>(g.cols) * F::kBlockBytes;
+    const int n4 = a.in_w >> 2;
+
+    // ---- prefetch side: the stage it requests next, the matrix that stage belongs to
+    constexpr int kXRegs = 4;              // float4 per lane that hold the next matrix' activations on their way in
+    float4 xv[kXRegs];
+    int xv_m = -1;                         // the table entry whose activations are in xv (or on their way)
+    const bool x_fits = n4 <= kXRegs * T;
+    int f_t = blockIdx.x, f_k = 0, f_m = 0;
+    MfmaEntry fe = entry_at(0);
+    const float* f_x = nullptr;            // vector of the matrix the prefetch side was in last
+    __amdgpu_buffer_rsrc_t f_matrix;
+    // (written as assembly so that the wait for it can be placed by hand: the compiler would wait for every load in
+    // flight, the weight stream included, before the first use)
+    auto request_x = [&](const float* x, int m) {
+#pragma unroll
+        for (int j = 0; j < kXRegs; ++j) {
+            const int i = tid + j * T;
+            xv[j] = gload16(x, static_cast<uint32_t>(i < n4 ? i : 0) * 16u);
+        }
+        xv_m = m;
+    };
+    auto fetch_enter = [&]() {             // f_t moved: find its matrix; ask for its activations if they are new
+        while (f_t >= fe.first_tile + fe.tiles && f_m + 1 < a.entries) fe = entry_at(++f_m);
+        f_matrix = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(fe.w), 0, static_cast<int>(fe.w_bytes), 0x00020000);
+        if (fe.x != f_x) {
+            // only one vector can be on its way; a second change before the first was consumed is fetched at the switch
+            if (x_fits && xv_m < 0) request_x(fe.x, f_m);
+            f_x = fe.x;
+        }
+    };
+    // Requests this wave's pieces of the next stage into a register set.  Pieces that are padding, rows past the matrix
+    // and stages past the end lie beyond the buffer: zeros, no memory traffic.
+    auto fetch = [&](u32x4 (&set)[LPW]) {
+        const uint32_t base = f_t < a.total_tiles
+            ? static_cast<uint32_t>(f_t - fe.first_tile) * kTileRows * a.row_bytes + static_cast<uint32_t>(f_k) * chunk_bytes
+            : kNoPiece;
+#pragma unroll
+        for (int i = 0; i < LPW; ++i) set[i] = stream16(f_matrix, base + rel[i]);
+        if (++f_k == KC) {
+            f_k = 0;
+            f_t += G;
+            if (f_t < a.total_tiles && f_t >= fe.first_tile + fe.tiles) fetch_enter();
+        }
+    };
+    // Copies a register set to its place in an LDS stage buffer.
+    auto park = [&](uint8_t* buf, const u32x4 (&set)[LPW]) {
+        // (a buffer has room for all W * LPW pieces; those past the stage's last are zeros nobody reads)
+        uint8_t* dst = buf + wave * 1024 + lane * 16;
+#pragma unroll
+        for (int i = 0; i < LPW; ++i) *reinterpret_cast<u32x4*>(dst + W * i * 1024) = set[i];
+    };
+
+    // ---- consume side
+    int c_t = blockIdx.x, c_m = -1;
+    MfmaEntry ce{};
+    float inv = 0.0f;
+    const float* regs_x = nullptr;         // the vector operand A in the registers below was made from
+    XSet xs[KC * M];
+    // Operand A of this lane: A row lane % 16 = plane (lane % 4) of quarter (lane % 16) / 4, K group lane / 16; it is
+    // non-zero only where the K group carries that quarter.
+    const bool diag = (row_l >> 2) == quarter;
+
+    // Turns matrix c_m's activations into this lane's operand-A registers (all waves; three barriers inside).  The digit
+    // planes and sub-block sums pass through the stage buffer `scratch`, which is free at that point.  The vector is in xv
+    // when the prefetch side asked for it; otherwise it is fetched here.
+    auto prepare_x = [&](uint8_t* scratch) {
+        if (xv_m != c_m) {
+            request_x(ce.x, c_m);
+            wait_vm_imm<0>();
+        } else {
+            wait_vm_imm<2 * LPW>();     // older than the two register sets that are still on their way
+        }
+        xv_m = -1;
+#pragma unroll
+        for (int j = 0; j < kXRegs; ++j) asm volatile("" : "+v"(xv[j].x), "+v"(xv[j].y), "+v"(xv[j].z), "+v"(xv[j].w));
+        constexpr float4 kZero4 = {0.0f, 0.0f, 0.0f, 0.0f};
+        const float4* x4 = reinterpret_cast<const float4*>(ce.x);
+        const int plane_stride = a.in_w + 16;
+        float* sumx = reinterpret_cast<float*>(scratch + 4 * plane_stride);
+        auto umax4 = [](uint32_t m, const float4& v) {
+            m = umax_u(m, __float_as_uint(v.x) & 0x7fffffffu);
+            m = umax_u(m, __float_as_uint(v.y) & 0x7fffffffu);
+            m = umax_u(m, __float_as_uint(v.z) & 0x7fffffffu);
+            return umax_u(m, __float_as_uint(v.w) & 0x7fffffffu);
+        };
+        uint32_t mx = 0;
+#pragma unroll
+        for (int j = 0; j < kXRegs; ++j) {
+            if (tid + j * T >= n4) xv[j] = kZero4;
+            mx = umax4(mx, xv[j]);
+        }
+        for (int i = tid + kXRegs * T; i < n4; i += T) mx = umax4(mx, x4[i]);      // (vectors too long for xv: re-read)
+        mx = wave_umax(mx);
+        if (lane == 0) red[wave] = mx;
+        __syncthreads();
+        mx = 0;
+        for (int i = 0; i < W; ++i) mx = umax_u(mx, red[i]);
+        // |x| < 2^(E - 126) for the biased exponent E of the largest magnitude; e = 156 - E puts it below 2^30
+        const int E = static_cast<int>(mx >> 23);
+        int e = 156 - E;
+        e = e > 126 ? 126 : e;
+        const float scale = __uint_as_float(static_cast<uint32_t>(e + 127) << 23);
+        // a NaN or an infinity among the activations makes every output NaN
+        inv = E == 255 ? __uint_as_float(0x7fc00000u) : __uint_as_float(static_cast<uint32_t>(127 - e) << 23);
+        auto to_planes = [&](int i, const float4& v) {
+            uint32_t pl[4];
+            digit_planes(__float2int_rn(v.x * scale), __float2int_rn(v.y * scale), __float2int_rn(v.z * scale),
+                         __float2int_rn(v.w * scale), pl);
+#pragma unroll
+            for (int p = 0; p < 4; ++p) *reinterpret_cast<uint32_t*>(scratch + p * plane_stride + 4 * i) = pl[p];
+            const float s = oct_sum((v.x + v.y) + (v.z + v.w));      // 32 consecutive activations: one sub-block
+            if ((i & 7) == 0) sumx[i >> 3] = s;
+        };
+#pragma unroll
+        for (int j = 0; j < kXRegs; ++j) {
+            const int i = tid + j * T;                               // (whole groups of eight lanes are in or out: n4 % 8 == 0)
+            if (i < n4) to_planes(i, xv[j]);
+        }
+        for (int i = tid + kXRegs * T; i < n4; i += T) to_planes(i, x4[i]);
+        __syncthreads();
+        // set k * M + t = super-block column k * cols + t * W + wave of a row
+#pragma unroll
+        for (int k = 0; k < KC; ++k) {
+#pragma unroll
+            for (int t = 0; t < M; ++t) {
+                const int b = k * g.cols + t * W + wave;
+                XSet& set = xs[k * M + t];
+                const uint8_t* src = scratch + (row_l & 3) * plane_stride + 256 * b + 64 * quarter;
+#pragma unroll
+                for (int u = 0; u < 4; ++u) set.a[u] = diag ? lds128(src + 16 * u) : u32x4{0u, 0u, 0u, 0u};
+                set.sx = *reinterpret_cast<const float2*>(sumx + 8 * b + 2 * quarter);
+            }
+        }
+        regs_x = ce.x;
+        __syncthreads();
+    };
+
+    // ---- start: the first matrix' activations are requested ahead of the weight stream, then two stages
+    uint8_t* const buf0 = smem;
+    uint8_t* const buf1 = smem + g.stage_bytes;
+    u32x4 regs[2][LPW];
+    fetch_enter();
+    fetch(regs[0]);
+    fetch(regs[1]);
+
+    const uint32_t row_off = static_cast<uint32_t>(row_l) * (static_cast<uint32_t>(g.row_pieces) * 16u) +
+                             static_cast<uint32_t>(wave) * F::kBlockBytes;
+    int pbuf = 0;
+    // the tile whose wave partials sit in part[pbuf ^ 1]: added up and stored after the next barrier
+    bool done = false;
+    float* done_y = nullptr;
+    const float* done_bias = nullptr;
+    int done_row0 = 0, done_rows = 0;
+    auto finalize = [&]() {
+        if (tid < kTileRows) {
+            float t = 0.0f;
+            for (int w2 = 0; w2 < W; ++w2) t += part[pbuf ^ 1][w2][tid];
+            if (done_bias) {
+                // the 16 bias values come through the scalar cache (wave-uniform addresses) and are dealt to the lanes
+                const NNHIP_CONST_PTR float* cb = (const NNHIP_CONST_PTR float*)done_bias + done_row0;
+                float bv = 0.0f;
+#pragma unroll
+                for (int j = 0; j < kTileRows; ++j) {
+                    const float v = cb[j < done_rows ? j : 0];
+                    bv = tid == j ? v : bv;
+                }
+                t += bv;
+            }
+            if (tid < done_rows) done_y[done_row0 + tid] = t;
+        }
+        done = false;
+    };
+
+    float accq = 0.0f, accm = 0.0f;
+    // One stage: buffer `cur` holds it; `nxt` receives the stage after it from `landing`, whose loads have been in
+    // flight for a whole stage; `refill` (free since it was parked a stage ago) takes the requests of the stage after that.
+    auto stage_step = [&](auto k_tag, uint8_t* cur, uint8_t* nxt, u32x4 (&refill)[LPW], const u32x4 (&landing)[LPW]) {
+        constexpr int k = decltype(k_tag)::value;
+        bool new_x = false;
+        if (k == 0) {
+            if (c_t >= ce.first_tile + ce.tiles) {              // (always at the first tile: ce.tiles == 0)
+                while (c_t >= ce.first_tile + ce.tiles) ce = entry_at(++c_m);
+                new_x = ce.x != regs_x;
+            }
+        }
+        fetch(refill);                  // (before the activations are dealt with: the stream must not pause for them)
+        if (k == 0 && new_x) prepare_x(nxt);
+        if (done) finalize();
+        const uint8_t* stage = cur + row_off;
+        typename F::Raw raw[M];
+#pragma unroll
+        for (int t = 0; t < M; ++t) raw[t] = F::load(stage + t * W * F::kBlockBytes, quarter);
+#pragma unroll
+        for (int t = 0; t < M; ++t) F::run(raw[t], xs[k * M + t], quarter, accq, accm);
+        if (k == KC - 1) {
+            float p = fmaf(accq, inv, -accm);
+            p = quarter_sum(p);
+            if (lane < kTileRows) part[pbuf][wave][lane] = p;
+            accq = 0.0f;
+            accm = 0.0f;
+            done = true;
+            done_y = ce.y;
+            done_bias = ce.bias;
+            done_row0 = (c_t - ce.first_tile) * kTileRows;
+            done_rows = ce.out_w - done_row0 < kTileRows ? ce.out_w - done_row0 : kTileRows;
+            pbuf ^= 1;
+            c_t += G;
+        }
+        park(nxt, landing);
+        __syncthreads();                // publishes `nxt`, frees `cur`
+    };
+
+    park(buf0, regs[0]);
+    __syncthreads();
+    using std::integral_constant;
+    for (int n = 0; n < total; n += 2) {
+        stage_step(integral_constant<int, 0>{}, buf0, buf1, regs[0], regs[1]);
+        if (n + 1 < total) stage_step(integral_constant<int, KC - 1>{}, buf1, buf0, regs[1], regs[0]);
+    }
+    if (done) finalize();
+}
+
+// The (KC, M, LPW) combinations the kernel is instantiated for.
+struct Variant { int kc, m, lpw; };
+constexpr Variant kVariants[] = {{1, 2, 5}, {1, 2, 6}, {2, 1, 3}, {1, 1, 3}, {2, 2, 5}, {2, 2, 6}, {1, 1, 2}, {2, 1, 2}};
+
+// Picks W and C for (block bytes, in_w).  C = W * M columns per stage must divide the row's super-blocks into KC whole
+// stages, two stage buffers must fit LDS (one of them doubles as scratch for the digit planes when the activations
+// change), (KC, M, LPW) must be an instantiated variant, and among those the choice maximises the bytes a stage holds,
+// then the waves.
+bool plan_mfma(int block_bytes, int in_w, MfmaGeom* out)
+{
+    const int nblocks = in_w / 256;
+    const int bp = block_bytes / 16;
+    if (nblocks < 1 || block_bytes % 16 != 0) return false;
+    const int planes_bytes = 4 * (in_w + 16) + (in_w / 32) * 4;
+    double best_score = -1.0;
+    MfmaGeom best{};
+    for (int W = 6; W <= kMaxWaves; ++W) {
+        for (int m = 1; m <= 2; ++m) {
+            MfmaGeom g{};
+            g.waves = W;
+            g.cols = W * m;
+            if (nblocks % g.cols != 0) continue;
+            g.kchunks = nblocks / g.cols;
+            g.tasks = m;
+            g.row_pieces = (g.cols * bp) | 1;
+            g.stage_loads = (kTileRows * g.row_pieces + 63) / 64;
+            g.loads_per_wave = (g.stage_loads + W - 1) / W;
+            g.stage_bytes = g.loads_per_wave * W * 1024;          // every wave parks loads_per_wave pieces
+            if (g.stage_bytes < planes_bytes || 2 * g.stage_bytes > kLdsBudget) continue;
+            bool ok = false;
+            for (const Variant& v : kVariants) ok = ok || (v.kc == g.kchunks && v.m == m && v.lpw == g.loads_per_wave);
+            if (!ok) continue;
+            g.stages = 2;
+            g.lds_bytes = 2 * static_cast<size_t>(g.stage_bytes);
+            // one column per wave keeps the register sets small (no spills); then the larger stage, then the waves
+            const double score = (m == 1 ? 1.0 : 0.0) + static_cast<double>(g.stage_bytes) / (256.0 * 1024) + 1e-3 * W;
+            if (score > best_score) {
+                best_score = score;
+                best = g;
+            }
+        }
+    }
+    if (best_score < 0) return false;
+    *out = best;
+    return true;
+}
+
+template <class F, int KC, int M, int LPW>
+hipError_t launch_mfma_variant(Lane* lane, const MfmaArgs& a, dim3 grid)
+{
+    static LdsLimit big_lds;
+    const hipError_t e = big_lds.ensure(lane->device, reinterpret_cast<const void*>(&matvec_mfma_kernel<F, KC, M, LPW>), kLdsBudget);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL((matvec_mfma_kernel<F, KC, M, LPW>), grid, dim3(64 * a.g.waves), a.g.lds_bytes, lane->stream, a);
+    return hipGetLastError();
+}
+
+template <class F>
+hipError_t launch_mfma(Lane* lane, const MfmaArgs& a)
+{
+    const int groups = a.total_tiles < lane->compute_units ? a.total_tiles : lane->compute_units;
+    const dim3 grid(groups);
+    const int kc = a.g.kchunks, m = a.g.tasks, lpw = a.g.loads_per_wave;
+#define NNHIP_VARIANT(K, MM, L) if (kc == K && m == MM && lpw == L) return launch_mfma_variant<F, K, MM, L>(lane, a, grid);
+    NNHIP_VARIANT(1, 2, 5) NNHIP_VARIANT(1, 2, 6) NNHIP_VARIANT(2, 1, 3) NNHIP_VARIANT(1, 1, 3) NNHIP_VARIANT(2, 2, 5)
+    NNHIP_VARIANT(2, 2, 6) NNHIP_VARIANT(1, 1, 2) NNHIP_VARIANT(2, 1, 2)
+#undef NNHIP_VARIANT
+    return hipErrorInvalidConfiguration;
+}
+
+int block_bytes_of(uint32_t type)
+{
+    switch (type) {
+    case NNHIP_TYPE_Q4_K: return Q4KTask::kBlockBytes;
+    case NNHIP_TYPE_Q5_K: return Q5KTask::kBlockBytes;
+    default: return 0;
+    }
+}
+
+bool entry_ok(uint32_t type, int in_w, int out_w, const void* w)
+{
+    const int bb = block_bytes_of(type);
+    if (!bb || in_w % 256 != 0 || (reinterpret_cast<uintptr_t>(w) & 15u)) return false;
+    const uint64_t bytes = static_cast<uint64_t>(out_w) * (in_w / 256) * bb;
+    return bytes < 0x7fffffffull;            // piece offsets are 32-bit and "no piece" is bit 31
+}
+
+void fill_args(uint32_t type, int in_w, const MfmaGeom& g, MfmaArgs* a)
+{
+    a->g = g;
+    a->in_w = in_w;
+    a->nblocks = in_w / 256;
+    a->row_bytes = static_cast<uint32_t>(a->nblocks) * static_cast<uint32_t>(block_bytes_of(type));
+    a->row_pieces_magic = static_cast<uint32_t>((0x100000000ull + g.row_pieces - 1) / g.row_pieces);
+}
+
+}  // namespace
+
+MfmaTableEntry matvec_mfma_entry(uint32_t type, const float* x, const void* w, const float* bias, float* y, int in_w,
+                                 int out_w, int first_tile)
+{
+    MfmaTableEntry e{};
+    e.x = x;
+    e.w = static_cast<const uint8_t*>(w);
+    e.bias = bias;
+    e.y = y;
+    e.out_w = out_w;
+    e.w_bytes = static_cast<uint32_t>(out_w) * static_cast<uint32_t>(in_w / 256) * static_cast<uint32_t>(block_bytes_of(type));
+    e.tiles = (out_w + kTileRows - 1) / kTileRows;
+    e.first_tile = first_tile;
+    return e;
+}
+
+bool matvec_mfma_geometry(uint32_t type, int in_w, int out_w, const void* w, MfmaPlan* plan)
+{
+    if (!entry_ok(type, in_w, out_w, w)) return false;
+    MfmaGeom g;
+    if (!plan_mfma(block_bytes_of(type), in_w, &g)) return false;
+    if (plan) {
+        plan->waves = g.waves;
+        plan->cols = g.cols;
+        plan->kchunks = g.kchunks;
+        plan->stages = g.stages;
+        plan->stage_bytes = g.stage_bytes;
+        plan->loads_per_wave = g.loads_per_wave;
+        plan->lds_bytes = static_cast<int>(g.lds_bytes);
+    }
+    return true;
+}
+
+hipError_t launch_matvec_mfma_table(Lane* lane, uint32_t type, int in_w, const MfmaTableEntry* device_entries, int entries,
+                                    int total_tiles)
+{
+    MfmaArgs a{};
+    MfmaGeom g;
+    if (!plan_mfma(block_bytes_of(type), in_w, &g)) return hipErrorInvalidValue;
+    fill_args(type, in_w, g, &a);
+    a.table = device_entries;
+    a.entries = entries;
+    a.total_tiles = total_tiles;
+    switch (type) {
+    case NNHIP_TYPE_Q4_K: return launch_mfma<Q4KTask>(lane, a);
+    case NNHIP_TYPE_Q5_K: return launch_mfma<Q5KTask>(lane, a);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace nnhip

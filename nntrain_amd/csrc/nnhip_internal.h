@@ -80,6 +80,29 @@ hipError_t launch_matvec(Lane* lane, uint32_t type, const float* x, const void* 
 bool matvec_fused_supported(uint32_t type, int in_w);
 hipError_t launch_matvec_fused(Lane* lane, const nnhip_fused_matvec_desc& d);
 hipError_t launch_matvec_batch(Lane* lane, const nnhip_matvec_desc* descs, int count);
+// Matrix-core form of the mat-vec (gemv_mfma_kernels.hip): whether it takes a shape (and with which geometry), and its launch.
+struct MfmaPlan {
+    int waves, cols, kchunks, stages, stage_bytes, loads_per_wave, lds_bytes;
+};
+bool matvec_mfma_geometry(uint32_t type, int in_w, int out_w, const void* w, MfmaPlan* plan);
+// One matrix (one input row of it) of a table-driven launch of the matrix-core mat-vec: all entries of a launch share
+// the storage type and in_w.  80 bytes, the slot size of a lane's descriptor table.
+struct MfmaTableEntry {
+    const float* x;
+    const uint8_t* w;
+    const float* bias;
+    float* y;
+    int out_w;
+    uint32_t w_bytes;       // whole matrix (< 2 GB)
+    int tiles;              // ceil(out_w / 16)
+    int first_tile;         // position of the matrix' first tile in the launch's tile sequence
+    uint32_t pad_[8];
+};
+static_assert(sizeof(MfmaTableEntry) == 80, "table slots are 80 bytes");
+MfmaTableEntry matvec_mfma_entry(uint32_t type, const float* x, const void* w, const float* bias, float* y, int in_w,
+                                 int out_w, int first_tile);
+hipError_t launch_matvec_mfma_table(Lane* lane, uint32_t type, int in_w, const MfmaTableEntry* device_entries, int entries,
+                                    int total_tiles);
 // The fixed device workspace: its address on the current device, and the batched launch that uses it.
 hipError_t static_table_address(void** address);
 hipError_t launch_matvec_batch_static(Lane* lane, const nnhip_matvec_desc* descs, int count);

@@ -332,3 +332,104 @@ def test_captured_batch_replays_after_other_batches(lane):
                 b.dispose()
     for b in (many_x, many_w, many_y):
         b.dispose()
+
+
+# ------------------------------------------------------------------------------- large batched groups (matrix cores)
+
+def _batch_run(lane, items):
+    descs = (MatvecDesc * len(items))()
+    for i, it in enumerate(items):
+        descs[i] = MatvecDesc(it["xd"].ptr, it["wd"].ptr, it["bd"].ptr if it["bd"] else None, it["yd"].ptr, it["typ"],
+                              it["rows"], it["in_w"], it["out_w"])
+    for it in items:
+        lane.fill_u32(it["yd"], NAN_BITS, it["rows"] * it["out_w"] + 2)
+    check(lane._lib.nnhip_quant_matvec_batch(lane._handle, descs, len(items)), "quant_matvec_batch")
+    lane.synchronize()
+    out = []
+    for it in items:
+        y = lane.read(it["yd"])
+        assert np.isnan(y[-1]) and np.isnan(y[-2]), "guard elements past the output were overwritten"
+        out.append(y[:-2].reshape(it["rows"], it["out_w"]).copy())
+    return out
+
+
+@pytest.mark.parametrize("typ", [GGML_Q4_K, GGML_Q5_K])
+def test_large_batched_groups_on_the_matrix_cores(lane, typ):
+    """Groups of Q4_K / Q5_K matrices with at least 2048 sixteen-row tiles go to the matrix-core mat-vec: against the
+    float64 oracle at both bars, with bias, ragged row counts, several input rows, activations that change and repeat
+    from matrix to matrix, and two widths in one call (two launches).  A row's bits must not depend on the other
+    matrices of the call or on its place in it."""
+    rng = np.random.default_rng(typ)
+    shapes = [(5120, 17408, 1, True), (5120, 5000 + 3, 1, False), (5120, 17, 2, True), (5120, 17408, 1, False),
+              (2560, 9000 + 5, 1, True), (2560, 40000, 1, False), (5120, 1, 1, False), (5120, 4096, 3, False)]
+    items = []
+    shared_x = {}
+    for i, (in_w, out_w, rows, bias) in enumerate(shapes):
+        payload = synth.matrix(typ, out_w, in_w, seed=100 * typ + i)
+        # matrices 0 and 1 share their activations, as q / k / v or gate / up do
+        key = (in_w, rows, 0 if i < 2 else i)
+        if key not in shared_x:
+            xh = rng.standard_normal((rows, in_w)).astype(np.float32)
+            shared_x[key] = (xh, lane.upload_raw(xh))
+        xh, xd = shared_x[key]
+        bh = rng.standard_normal(out_w).astype(np.float32) if bias else None
+        items.append(dict(typ=typ, in_w=in_w, out_w=out_w, rows=rows, payload=payload, x=xh, xd=xd, bias=bh,
+                          wd=lane.upload_raw(payload), bd=lane.upload_raw(bh) if bias else None,
+                          yd=lane.allocate(rows * out_w + 2)))
+    before = lane.counters()
+    got = _batch_run(lane, items)
+    after = lane.counters()
+    assert after["h2d_bytes"] == before["h2d_bytes"] and after["allocated_bytes"] == before["allocated_bytes"]
+    for it, y in zip(items, got):
+        assert np.all(np.isfinite(y))
+        ref, asum = oracle.linear_f64(typ, it["payload"], it["x"], it["bias"], it["rows"], it["in_w"], it["out_w"])
+        assert oracle.rel_l2(y, ref) <= MATVEC_BAR, (it["in_w"], it["out_w"])
+        assert np.all(np.abs(y.astype(np.float64) - ref) <= 2e-6 + 3e-6 * asum), (it["in_w"], it["out_w"])
+    # another composition and order of the same matrices: identical bits per row
+    order = [3, 0, 7, 1, 5, 2]
+    again = _batch_run(lane, [items[i] for i in order])
+    for i, y in zip(order, again):
+        assert np.array_equal(_bits(y), _bits(got[i])), shapes[i]
+    # and the single launch agrees to FP32 summation accuracy (another kernel, another summation order)
+    it = items[0]
+    single = lane.allocate(it["out_w"])
+    check(lane._lib.nnhip_quant_matvec(lane._handle, typ, c_void_p(it["xd"].ptr), c_void_p(it["wd"].ptr), c_void_p(it["bd"].ptr),
+                                       c_void_p(single.ptr), 1, it["in_w"], it["out_w"]), "quant_matvec")
+    assert oracle.rel_l2(lane.read(single), got[0][0]) <= 1e-6
+    single.dispose()
+    for it in items:
+        for key in ("wd", "bd", "yd"):
+            if it[key] is not None:
+                it[key].dispose()
+    for _, xd in shared_x.values():
+        xd.dispose()
+    lane.trim()
+
+
+def test_large_batched_group_special_activations(lane):
+    """All-zero activations give the bias; one NaN or infinity makes every output of that matrix NaN, as a floating-point
+    dot product would; a huge outlier among the activations must not cost the small ones their accuracy."""
+    typ, in_w, out_w = GGML_Q4_K, 5120, 17408
+    payload = synth.matrix(typ, out_w, in_w, seed=77)
+    wd = lane.upload_raw(payload)
+    bias = np.random.default_rng(3).standard_normal(out_w).astype(np.float32)
+    bd = lane.upload_raw(bias)
+    xs = [np.zeros((1, in_w), np.float32), synth.activations(1, in_w, seed=5), synth.activations(1, in_w, seed=6),
+          synth.activations(1, in_w, seed=7)]
+    xs[1][0, 1234] = np.nan
+    xs[2][0, 77] = np.inf
+    xs[3][0, 4000] = 3.0e4
+    items = [dict(typ=typ, in_w=in_w, out_w=out_w, rows=1, x=x, xd=lane.upload_raw(x), wd=wd, bd=bd, bias=bias,
+                  yd=lane.allocate(out_w + 2)) for x in xs]
+    got = _batch_run(lane, items)
+    assert np.array_equal(_bits(got[0][0]), _bits(bias))
+    assert np.all(np.isnan(got[1])) and np.all(np.isnan(got[2]))
+    ref, asum = oracle.linear_f64(typ, payload, xs[3], bias, 1, in_w, out_w)
+    assert oracle.rel_l2(got[3], ref) <= MATVEC_BAR
+    assert np.all(np.abs(got[3].astype(np.float64) - ref) <= 2e-6 + 3e-6 * asum)
+    for it in items:
+        it["xd"].dispose()
+        it["yd"].dispose()
+    wd.dispose()
+    bd.dispose()
+    lane.trim()

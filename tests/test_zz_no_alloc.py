@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 
 import oracle
-from nntrain_amd import GGML_IQ2_S, GGML_Q4_K, GGML_Q6_K, GGML_Q8_0, HipExecutionLane, synth
+from nntrain_amd import GGML_IQ2_S, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_Q8_0, HipExecutionLane, synth
 from nntrain_amd.native import MatvecDesc, check, last_error
 
 pytestmark = pytest.mark.gpu
@@ -61,7 +61,8 @@ def test_static_workspace_batch_matches_the_allocating_entry_point():
         lib, h = lane._lib, lane._handle
         first = _batch(lane, [(GGML_Q8_0, 5376, 300, 1), (GGML_Q4_K, 5120, 260, 1), (GGML_Q8_0, 64, 5, 2),
                               (GGML_Q6_K, 1024, 130, 3), (GGML_IQ2_S, 2048, 40, 1), (GGML_Q8_0, 160, 9, 1),
-                              (GGML_Q8_0, 21504, 90, 1), (GGML_Q4_K, 256, 3, 60)], seed=400)
+                              (GGML_Q8_0, 21504, 90, 1), (GGML_Q4_K, 256, 3, 60),
+                              (GGML_Q5_K, 2560, 33000, 1)], seed=400)         # the last one: a matrix-core group
         second = _batch(lane, [(GGML_Q4_K, 1024, 70, 1), (GGML_Q8_0, 512, 64, 2)], seed=500)
         for items in (first, second):           # the second call is smaller: stale entries of the first stay behind it
             for it in items:
@@ -108,7 +109,7 @@ def test_static_workspace_batch_inside_a_captured_graph():
     """The caller this entry point is for: a graph captured without any allocation, replayed between eager work."""
     with HipExecutionLane(0) as lane:
         lib, h = lane._lib, lane._handle
-        items = _batch(lane, [(GGML_Q8_0, 1024, 200, 1), (GGML_Q4_K, 512, 90, 1)], seed=600)
+        items = _batch(lane, [(GGML_Q8_0, 1024, 200, 1), (GGML_Q4_K, 512, 90, 1), (GGML_Q4_K, 2560, 33000, 1)], seed=600)
         other = _batch(lane, [(GGML_Q6_K, 256, 31, 1)], seed=700)
         check(lib.nnhip_quant_matvec_batch(h, _descs(items, "y_ref"), len(items)), "quant_matvec_batch")
         lane.synchronize()
