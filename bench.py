@@ -258,13 +258,13 @@ def run_gemv(args, lane, nn, oracle):
             descs[i] = MatvecDesc(x.ptr, w.ptr, None, ys[i].ptr, typ, 1, in_w, out_w)
         nn.native.check(lib.nnhip_quant_matvec_batch(h, descs, len(ring)), "quant_matvec_batch")
         lane.synchronize()
-        # large Q4_K / Q5_K groups run on the matrix-core kernel (fixed-point activations): same bar against the oracle,
+        # large Q4_K / Q5_K / Q6_K groups run on the matrix-core kernel (fixed-point activations): same bar against the oracle,
         # not the single launch's bits; the other formats share the single launch's kernel and must match bitwise
         y_batch = lane.read(ys[-1], np.float32)
         rel_batch = oracle.rel_l2(y_batch, ref[0])
         if not rel_batch <= 1e-5:
             raise SystemExit(f"{name}: batched launch parity failure, rel-L2 {rel_batch:.3e}")
-        if tname not in ("GGML_Q4_K", "GGML_Q5_K") and not np.array_equal(y_batch.view(np.uint32), lane.read(y, np.uint32)):
+        if tname not in ("GGML_Q4_K", "GGML_Q5_K", "GGML_Q6_K") and not np.array_equal(y_batch.view(np.uint32), lane.read(y, np.uint32)):
             raise SystemExit(f"{name}: batched launch differs bitwise from the single launch")
         samples_batch = []
         for _ in range(7):

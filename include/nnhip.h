@@ -214,7 +214,7 @@ NNHIP_API int nnhip_matvec_plan(uint32_t ggml_type, int rows, int in_w, int out_
 /* `count` independent mat-vecs enqueued as one unit of work (a single launch per group of equal type), for the
  * per-token projection sets that ForwardTokenDevice issues back to back (Qwen35QuantizedModel.cs:451-513).
  * `descs` is a host array, read before the call returns.  Results are identical to `count` nnhip_quant_matvec calls,
- * with one exception: Q4_K and Q5_K matrices of one in_w whose 16-row tiles add up to 2048 or more within a call (in_w
+ * with one exception: Q4_K, Q5_K and Q6_K matrices of one in_w whose 16-row tiles add up to 2048 or more within a call (in_w
  * a multiple of 256 that the matrix-core mat-vec can split: 5120 and 2560 among others) are multiplied on the matrix
  * cores with the activations in 32-bit fixed point.  Those results are deterministic, depend on the weights, in_w and
  * the activations only (not on out_w, the other matrices of the call or the order), agree with the single launch to

@@ -1,5 +1,5 @@
 // Decode mat-vec on the matrix cores for the super-block formats whose unpacking is too much vector-ALU work for the
-// lane-per-unit kernels (gemv_kernels.hip): Q4_K and Q5_K here.  Used for the large groups of a batched launch, where
+// lane-per-unit kernels (gemv_kernels.hip): Q4_K, Q5_K and Q6_K here.  Used for the large groups of a batched launch, where
 // it streams faster than the row-step kernels; it takes longer to start, so single launches stay with those.
 //
 // y[r, o] = bias[o] + sum_k x[r, k] * w[o, k]     (NNtrain.Arc/Kernels/qwen.cl:374-406 defines the operator)
@@ -7,17 +7,19 @@
 // Arithmetic.  The activation vector is turned into 32-bit fixed point relative to its largest magnitude
 // (v = rint(x * 2^e), |v| <= 2^30) and split into four balanced base-256 digits (each in [-128, 127]).
 // v_mfma_i32_16x16x32_i8 then takes the exact integer sums sum_k digit_p(x_k) * q_k of one 32-weight sub-block for 16
-// matrix rows at a time (operand B = the sub-block's quants as bytes, two masks away from the raw block; operand A = digit
-// planes).  The four K groups of an instruction carry four different 64-weight quarters of a super-block and operand A is
+// matrix rows at a time (operand B = the sub-block's quants as bytes, a few masks away from the raw block; operand A =
+// digit planes).  The four K groups of an instruction carry four different 64-weight quarters of a super-block and operand A is
 // block-diagonal to match (rows 4P .. 4P+3 = the four digit planes of quarter P in K group P, zeros elsewhere), so the 64
 // lanes of the result hold the plane sums of (quarter lane / 16, matrix row lane % 16).  They are recombined
 // (sum_p 256^p S_p), scaled by d * scale and accumulated per lane in FP32; minima use FP32 sums of x per sub-block:
 // sum x (s q - m) = s sum(q x) - m sum(x).  The error of the fixed-point form is at most 2^-31 of the largest |x| per
 // element, below the rounding of one FP32 product.
 //
-// Data movement.  A stage is 16 matrix rows x C super-blocks, copied verbatim: every wave requests its 1 KB pieces of a
+// Data movement.  A stage is 16 matrix rows x C super-blocks, copied block by block in 16-byte pieces (verbatim for the
+// formats whose blocks are whole pieces; a 210-byte Q6_K block takes 14 pieces so that it starts on a piece boundary in
+// LDS, the last piece overlapping the one before it): every wave requests its 1 KB pieces of a
 // stage (consecutive memory, non-temporal 16-byte buffer loads) into one of two register sets and parks the set in one of
-// two LDS stage buffers a whole stage later, so two stages are always on their way while one is multiplied; one
+// two LDS stage buffers a whole stage later, so up to two stages are on their way while one is multiplied; one
 // workgroup barrier per stage publishes the parked stage and frees the other buffer.  The LDS row stride is an odd
 // number of 16-byte pieces, so the 16 rows an operand read touches fall into different bank groups.
 //
@@ -150,23 +152,12 @@ __device__ __forceinline__ i32x4 mfma_i8(uint32_t a0, uint32_t a1, uint32_t b0, 
 
 __device__ __forceinline__ u32x4 lds128(const uint8_t* p) { return *reinterpret_cast<const u32x4*>(p); }
 
-// The activation loads are written as inline assembly so that the compiler's counter bookkeeping does not see them: it
-// would otherwise wait for every load in flight, the weight stream included, before their first use.  The wait is placed
-// by hand (wait_vm_imm) and the registers are tied to it with an empty asm statement.
-//
-// 16 bytes per lane into registers; valid only after a wait_vm that covers it.
-__device__ __forceinline__ float4 gload16(const float* base, uint32_t voff)
-{
-    float4 r;
-    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(r) : "v"(voff), "s"(base) : "memory");
-    return r;
-}
-
 // This lane's part of operand A for one super-block column: 64 bytes (its digit plane of its quarter's 64 activations;
-// zeros in the lanes outside the block diagonal) and the FP32 sums of x over the quarter's two 32-weight sub-blocks.
+// zeros in the lanes outside the block diagonal) and the FP32 sums of x over the quarter's NS scale groups.
+template <int NS>
 struct XSet {
     u32x4 a[4];
-    float2 sx;
+    float sx[NS];
 };
 
 // One task of a storage format: 16 rows x one super-block.  `blk` is this lane's row of the stage at the task's block
@@ -174,7 +165,23 @@ struct XSet {
 // fixed-point units) and accm (the minimum part).
 struct Q4KTask {
     static constexpr int kBlockBytes = kQ4KBytes;     // 144 = 9 pieces; blocks and rows are 16-byte aligned
+    static constexpr int kPieces = 9;                 // 16-byte pieces a block takes in a stage
+    static constexpr int kSumRun = 32;                // activations per FP32 sum (one sub-block)
+    using X = XSet<2>;
     struct Raw { u32x4 h, q1, q2; };
+
+    static __device__ __forceinline__ uint32_t piece_src(uint32_t q) { return 16u * q; }
+
+    // plane = this lane's digit plane of the whole vector, sums = the per-sub-block sums of x; b = super-block column
+    static __device__ __forceinline__ void load_x(X& xs, const uint8_t* plane, const float* sums, int b, int quarter, bool diag)
+    {
+        const uint8_t* src = plane + 256 * b + 64 * quarter;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) xs.a[u] = diag ? lds128(src + 16 * u) : u32x4{0u, 0u, 0u, 0u};
+        const float2 v = *reinterpret_cast<const float2*>(sums + 8 * b + 2 * quarter);
+        xs.sx[0] = v.x;
+        xs.sx[1] = v.y;
+    }
 
     static __device__ __forceinline__ Raw load(const uint8_t* blk, int quarter)
     {
@@ -185,7 +192,7 @@ struct Q4KTask {
         return r;
     }
 
-    static __device__ __forceinline__ void run(const Raw& r, const XSet& xs, int quarter, float& accq, float& accm)
+    static __device__ __forceinline__ void run(const Raw& r, const X& xs, int quarter, float& accq, float& accm)
     {
         constexpr uint32_t kLow = 0x0f0f0f0fu;
         const u32x4 q1 = r.q1, q2 = r.q2, h = r.h;
@@ -205,8 +212,8 @@ struct Q4KTask {
         k4_scale_pair(h[1], h[2], h[3], quarter, sc, mn);
         accq = fmaf(d * ubyte0(sc), recombine(s_lo), accq);
         accq = fmaf(d * ubyte1(sc), recombine(s_hi), accq);
-        accm = fmaf(dmin * ubyte0(mn), xs.sx.x, accm);
-        accm = fmaf(dmin * ubyte1(mn), xs.sx.y, accm);
+        accm = fmaf(dmin * ubyte0(mn), xs.sx[0], accm);
+        accm = fmaf(dmin * ubyte1(mn), xs.sx[1], accm);
     }
 };
 
@@ -214,7 +221,17 @@ struct Q4KTask {
 // qh, 128 nibble bytes: 176 = 11 pieces).
 struct Q5KTask {
     static constexpr int kBlockBytes = kQ5KBytes;
+    static constexpr int kPieces = 11;
+    static constexpr int kSumRun = 32;
+    using X = XSet<2>;
     struct Raw { u32x4 h, ha, hb, q1, q2; };
+
+    static __device__ __forceinline__ uint32_t piece_src(uint32_t q) { return 16u * q; }
+
+    static __device__ __forceinline__ void load_x(X& xs, const uint8_t* plane, const float* sums, int b, int quarter, bool diag)
+    {
+        Q4KTask::load_x(xs, plane, sums, b, quarter, diag);
+    }
 
     static __device__ __forceinline__ Raw load(const uint8_t* blk, int quarter)
     {
@@ -227,7 +244,7 @@ struct Q5KTask {
         return r;
     }
 
-    static __device__ __forceinline__ void run(const Raw& r, const XSet& xs, int quarter, float& accq, float& accm)
+    static __device__ __forceinline__ void run(const Raw& r, const X& xs, int quarter, float& accq, float& accm)
     {
         constexpr uint32_t kLow = 0x0f0f0f0fu, kBit4 = 0x10101010u;
         const u32x4 h = r.h, ha = r.ha, hb = r.hb, q1 = r.q1, q2 = r.q2;
@@ -249,15 +266,84 @@ struct Q5KTask {
         k4_scale_pair(h[1], h[2], h[3], quarter, sc, mn);
         accq = fmaf(d * ubyte0(sc), recombine(s_lo), accq);
         accq = fmaf(d * ubyte1(sc), recombine(s_hi), accq);
-        accm = fmaf(dmin * ubyte0(mn), xs.sx.x, accm);
-        accm = fmaf(dmin * ubyte1(mn), xs.sx.y, accm);
+        accm = fmaf(dmin * ubyte0(mn), xs.sx[0], accm);
+        accm = fmaf(dmin * ubyte1(mn), xs.sx[1], accm);
     }
 };
 
-// s_waitcnt vmcnt(N): at most N vector-memory loads of this wave still in flight.  The immediate is
-// 0x0F70 | (N & 15) | ((N >> 4) << 14).
-template <int N>
-__device__ __forceinline__ void wait_vm_imm() { __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14)); }
+// Q6_K (GgufQ6K.cs:9-54): 210 bytes = ql[128] qh[64] scales[16] (int8) d (fp16); w = d * scale * (q - 32).  In half h,
+// byte l of ql[64h ..] and ql[64h + 32 ..] carries weights l / l + 64 and l + 32 / l + 96 of the half in its nibbles, byte l
+// of qh[32h ..] their four 2-bit tops, and the 16-weight group of weight i has scale 8h + i / 16.  Quarter (h, e) is
+// the 32 ql bytes at 64h + 32e: low nibbles = weights 32e + l, high nibbles = weights 64 + 32e + l, four scale groups.
+// The -32 is taken through sums of x: sum x s (q - 32) = s sum(q x) - 32 s sum(x).
+// A block is 2-byte aligned in memory; a stage gives it 14 pieces (224 bytes) so that it starts 16-byte aligned in LDS.
+// Pieces 0-12 are its bytes 0-207; piece 13 is bytes 194-209 (d lands at 222), which never reaches past the block.
+struct Q6KTask {
+    static constexpr int kBlockBytes = kQ6KBytes;
+    static constexpr int kPieces = 14;
+    static constexpr int kSumRun = 16;
+    using X = XSet<4>;
+    struct Raw { u32x4 la, lb, ha, hb; u32x2 sc; uint32_t d; };
+
+    static __device__ __forceinline__ uint32_t piece_src(uint32_t q) { return q < 13u ? 16u * q : 194u; }
+
+    static __device__ __forceinline__ void load_x(X& xs, const uint8_t* plane, const float* sums, int b, int quarter, bool diag)
+    {
+        const int h = quarter >> 1, e = quarter & 1;
+        const uint8_t* src = plane + 256 * b + 128 * h + 32 * e;
+        xs.a[0] = diag ? lds128(src) : u32x4{0u, 0u, 0u, 0u};
+        xs.a[1] = diag ? lds128(src + 16) : u32x4{0u, 0u, 0u, 0u};
+        xs.a[2] = diag ? lds128(src + 64) : u32x4{0u, 0u, 0u, 0u};
+        xs.a[3] = diag ? lds128(src + 80) : u32x4{0u, 0u, 0u, 0u};
+        const float* sp = sums + 16 * b + 8 * h + 2 * e;
+        const float2 lo = *reinterpret_cast<const float2*>(sp), hi = *reinterpret_cast<const float2*>(sp + 4);
+        xs.sx[0] = lo.x;
+        xs.sx[1] = lo.y;
+        xs.sx[2] = hi.x;
+        xs.sx[3] = hi.y;
+    }
+
+    static __device__ __forceinline__ Raw load(const uint8_t* blk, int quarter)
+    {
+        const int h = quarter >> 1, e = quarter & 1;
+        Raw r;
+        r.la = lds128(blk + 64 * h + 32 * e);
+        r.ha = lds128(blk + 128 + 32 * h);
+        r.lb = lds128(blk + 64 * h + 32 * e + 16);
+        r.hb = lds128(blk + 128 + 32 * h + 16);
+        r.sc = *reinterpret_cast<const u32x2*>(blk + 192 + 8 * h);
+        r.d = *reinterpret_cast<const uint32_t*>(blk + 220) >> 16;
+        return r;
+    }
+
+    static __device__ __forceinline__ void run(const Raw& r, const X& xs, int quarter, float& accq, float& accm)
+    {
+        constexpr uint32_t kLow = 0x0f0f0f0fu, kTop = 0x30303030u;
+        const int sh = 2 * (quarter & 1);
+        const u32x4 a0 = xs.a[0], a1 = xs.a[1], a2 = xs.a[2], a3 = xs.a[3];
+        auto lo6 = [&](uint32_t q, uint32_t t) { return (q & kLow) | (((t >> sh) << 4) & kTop); };
+        auto hi6 = [&](uint32_t q, uint32_t t) { return ((q >> 4) & kLow) | ((t >> sh) & kTop); };
+        i32x4 s0 = {0, 0, 0, 0}, s1 = {0, 0, 0, 0}, s2 = {0, 0, 0, 0}, s3 = {0, 0, 0, 0};
+        s0 = mfma_i8(a0[0], a0[1], lo6(r.la[0], r.ha[0]), lo6(r.la[1], r.ha[1]), s0);
+        s2 = mfma_i8(a2[0], a2[1], hi6(r.la[0], r.ha[0]), hi6(r.la[1], r.ha[1]), s2);
+        s0 = mfma_i8(a0[2], a0[3], lo6(r.la[2], r.ha[2]), lo6(r.la[3], r.ha[3]), s0);
+        s2 = mfma_i8(a2[2], a2[3], hi6(r.la[2], r.ha[2]), hi6(r.la[3], r.ha[3]), s2);
+        s1 = mfma_i8(a1[0], a1[1], lo6(r.lb[0], r.hb[0]), lo6(r.lb[1], r.hb[1]), s1);
+        s3 = mfma_i8(a3[0], a3[1], hi6(r.lb[0], r.hb[0]), hi6(r.lb[1], r.hb[1]), s3);
+        s1 = mfma_i8(a1[2], a1[3], lo6(r.lb[2], r.hb[2]), lo6(r.lb[3], r.hb[3]), s1);
+        s3 = mfma_i8(a3[2], a3[3], hi6(r.lb[2], r.hb[2]), hi6(r.lb[3], r.hb[3]), s3);
+        // scales 8h + 2e + {0, 1} and 8h + 4 + 2e + {0, 1}: bytes 2e, 2e + 1 of the two dwords read for half h
+        const uint32_t w0 = r.sc[0] >> (8 * sh), w1 = r.sc[1] >> (8 * sh);
+        const float d = half_bits_to_float(r.d);
+        const float c0 = sbyte0(w0), c1 = sbyte1(w0), c2 = sbyte0(w1), c3 = sbyte1(w1);
+        accq = fmaf(d * c0, recombine(s0), accq);
+        accq = fmaf(d * c1, recombine(s1), accq);
+        accq = fmaf(d * c2, recombine(s2), accq);
+        accq = fmaf(d * c3, recombine(s3), accq);
+        const float t = fmaf(c0, xs.sx[0], fmaf(c1, xs.sx[1], fmaf(c2, xs.sx[2], c3 * xs.sx[3])));
+        accm = fmaf(32.0f * d, t, accm);
+    }
+};
 
 // Loads of the weight stream: 16 bytes per lane through a buffer descriptor that spans the matrix, non-temporal.  An
 // offset beyond the buffer returns zeros without touching memory.
@@ -301,18 +387,19 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_kernel(MfmaArgs a)
     };
 
     // ---- this lane's pieces of a stage: piece I = wave + W * i is slots 64 I .. 64 I + 63 of the stage; slot s is
-    // 16-byte piece s % row_pieces of stage row s / row_pieces (the last piece of a row is padding when the row has an
-    // even number of pieces).  rel[i] is the piece's byte offset from the stage's first byte in the matrix; pieces that do
+    // 16-byte piece s % row_pieces of stage row s / row_pieces: piece q % kPieces of block q / kPieces (the last piece of
+    // a row is padding when the blocks take an even number of pieces).  rel[i] is the piece's byte offset from the stage's first byte in the matrix; pieces that do
     // not exist get an offset beyond any matrix and read as zeros.
-    const int pieces_used = g.cols * (F::kBlockBytes / 16);
+    const int pieces_used = g.cols * F::kPieces;
     uint32_t rel[LPW];
 #pragma unroll
     for (int i = 0; i < LPW; ++i) {
         const uint32_t slot = static_cast<uint32_t>(64 * (wave + W * i) + lane);
         const uint32_t r = __umulhi(slot, a.row_pieces_magic);
         const uint32_t q = slot - r * static_cast<uint32_t>(g.row_pieces);
+        const uint32_t c = q / static_cast<uint32_t>(F::kPieces);
         const bool real = r < static_cast<uint32_t>(kTileRows) && q < static_cast<uint32_t>(pieces_used);
-        rel[i] = real ? r * a.row_bytes + q * 16u : kNoPiece;
+        rel[i] = real ? r * a.row_bytes + c * F::kBlockBytes + F::piece_src(q - c * F::kPieces) : kNoPiece;
     }
 
     // ---- the stage sequence of this workgroup: tiles blockIdx.x, blockIdx.x + G, ... of the launch's tile sequence,
@@ -332,13 +419,12 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_kernel(MfmaArgs a)
     MfmaEntry fe = entry_at(0);
     const float* f_x = nullptr;            // vector of the matrix the prefetch side was in last
     __amdgpu_buffer_rsrc_t f_matrix;
-    // (written as assembly so that the wait for it can be placed by hand: the compiler would wait for every load in
-    // flight, the weight stream included, before the first use)
     auto request_x = [&](const float* x, int m) {
+        const float4* x4 = reinterpret_cast<const float4*>(x);
 #pragma unroll
         for (int j = 0; j < kXRegs; ++j) {
             const int i = tid + j * T;
-            xv[j] = gload16(x, static_cast<uint32_t>(i < n4 ? i : 0) * 16u);
+            xv[j] = x4[i < n4 ? i : 0];
         }
         xv_m = m;
     };
@@ -378,7 +464,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_kernel(MfmaArgs a)
     MfmaEntry ce{};
     float inv = 0.0f;
     const float* regs_x = nullptr;         // the vector operand A in the registers below was made from
-    XSet xs[KC * M];
+    typename F::X xs[KC * M];
     // Operand A of this lane: A row lane % 16 = plane (lane % 4) of quarter (lane % 16) / 4, K group lane / 16; it is
     // non-zero only where the K group carries that quarter.
     const bool diag = (row_l >> 2) == quarter;
@@ -387,15 +473,8 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_kernel(MfmaArgs a)
     // planes and sub-block sums pass through the stage buffer `scratch`, which is free at that point.  The vector is in xv
     // when the prefetch side asked for it; otherwise it is fetched here.
     auto prepare_x = [&](uint8_t* scratch) {
-        if (xv_m != c_m) {
-            request_x(ce.x, c_m);
-            wait_vm_imm<0>();
-        } else {
-            wait_vm_imm<2 * LPW>();     // older than the two register sets that are still on their way
-        }
+        if (xv_m != c_m) request_x(ce.x, c_m);
         xv_m = -1;
-#pragma unroll
-        for (int j = 0; j < kXRegs; ++j) asm volatile("" : "+v"(xv[j].x), "+v"(xv[j].y), "+v"(xv[j].z), "+v"(xv[j].w));
         constexpr float4 kZero4 = {0.0f, 0.0f, 0.0f, 0.0f};
         const float4* x4 = reinterpret_cast<const float4*>(ce.x);
         const int plane_stride = a.in_w + 16;
@@ -431,8 +510,15 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_kernel(MfmaArgs a)
                          __float2int_rn(v.w * scale), pl);
 #pragma unroll
             for (int p = 0; p < 4; ++p) *reinterpret_cast<uint32_t*>(scratch + p * plane_stride + 4 * i) = pl[p];
-            const float s = oct_sum((v.x + v.y) + (v.z + v.w));      // 32 consecutive activations: one sub-block
-            if ((i & 7) == 0) sumx[i >> 3] = s;
+            float s = (v.x + v.y) + (v.z + v.w);
+            if (F::kSumRun == 32) {                                  // 32 consecutive activations: one sub-block
+                s = oct_sum(s);
+                if ((i & 7) == 0) sumx[i >> 3] = s;
+            } else {                                                 // 16 consecutive activations
+                s += dpp_mov<0xB1>(s);
+                s += dpp_mov<0x4E>(s);
+                if ((i & 3) == 0) sumx[i >> 2] = s;
+            }
         };
 #pragma unroll
         for (int j = 0; j < kXRegs; ++j) {
@@ -447,11 +533,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_kernel(MfmaArgs a)
 #pragma unroll
             for (int t = 0; t < M; ++t) {
                 const int b = k * g.cols + t * W + wave;
-                XSet& set = xs[k * M + t];
-                const uint8_t* src = scratch + (row_l & 3) * plane_stride + 256 * b + 64 * quarter;
-#pragma unroll
-                for (int u = 0; u < 4; ++u) set.a[u] = diag ? lds128(src + 16 * u) : u32x4{0u, 0u, 0u, 0u};
-                set.sx = *reinterpret_cast<const float2*>(sumx + 8 * b + 2 * quarter);
+                F::load_x(xs[k * M + t], scratch + (row_l & 3) * plane_stride, sumx, b, quarter, diag);
             }
         }
         regs_x = ce.x;
@@ -467,7 +549,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_kernel(MfmaArgs a)
     fetch(regs[1]);
 
     const uint32_t row_off = static_cast<uint32_t>(row_l) * (static_cast<uint32_t>(g.row_pieces) * 16u) +
-                             static_cast<uint32_t>(wave) * F::kBlockBytes;
+                             static_cast<uint32_t>(wave) * (16u * F::kPieces);
     int pbuf = 0;
     // the tile whose wave partials sit in part[pbuf ^ 1]: added up and stored after the next barrier
     bool done = false;
@@ -512,7 +594,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_kernel(MfmaArgs a)
         const uint8_t* stage = cur + row_off;
         typename F::Raw raw[M];
 #pragma unroll
-        for (int t = 0; t < M; ++t) raw[t] = F::load(stage + t * W * F::kBlockBytes, quarter);
+        for (int t = 0; t < M; ++t) raw[t] = F::load(stage + t * W * (16 * F::kPieces), quarter);
 #pragma unroll
         for (int t = 0; t < M; ++t) F::run(raw[t], xs[k * M + t], quarter, accq, accm);
         if (k == KC - 1) {
@@ -545,18 +627,19 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_kernel(MfmaArgs a)
 
 // The (KC, M, LPW) combinations the kernel is instantiated for.
 struct Variant { int kc, m, lpw; };
-constexpr Variant kVariants[] = {{1, 2, 5}, {1, 2, 6}, {2, 1, 3}, {1, 1, 3}, {2, 2, 5}, {2, 2, 6}, {1, 1, 2}, {2, 1, 2}};
+constexpr Variant kVariants[] = {{1, 2, 5}, {1, 2, 6}, {2, 1, 3}, {1, 1, 3}, {2, 2, 5}, {2, 2, 6}, {1, 1, 2}, {2, 1, 2},
+                                 {1, 1, 4}, {2, 1, 4}};
 
 // Picks W and C for (block bytes, in_w).  C = W * M columns per stage must divide the row's super-blocks into KC whole
 // stages, two stage buffers must fit LDS (one of them doubles as scratch for the digit planes when the activations
 // change), (KC, M, LPW) must be an instantiated variant, and among those the choice maximises the bytes a stage holds,
 // then the waves.
-bool plan_mfma(int block_bytes, int in_w, MfmaGeom* out)
+bool plan_mfma(int block_pieces, int in_w, MfmaGeom* out)
 {
     const int nblocks = in_w / 256;
-    const int bp = block_bytes / 16;
-    if (nblocks < 1 || block_bytes % 16 != 0) return false;
-    const int planes_bytes = 4 * (in_w + 16) + (in_w / 32) * 4;
+    const int bp = block_pieces;
+    if (nblocks < 1 || bp < 1) return false;
+    const int planes_bytes = 4 * (in_w + 16) + (in_w / 16) * 4;
     double best_score = -1.0;
     MfmaGeom best{};
     for (int W = 6; W <= kMaxWaves; ++W) {
@@ -608,7 +691,7 @@ hipError_t launch_mfma(Lane* lane, const MfmaArgs& a)
     const int kc = a.g.kchunks, m = a.g.tasks, lpw = a.g.loads_per_wave;
 #define NNHIP_VARIANT(K, MM, L) if (kc == K && m == MM && lpw == L) return launch_mfma_variant<F, K, MM, L>(lane, a, grid);
     NNHIP_VARIANT(1, 2, 5) NNHIP_VARIANT(1, 2, 6) NNHIP_VARIANT(2, 1, 3) NNHIP_VARIANT(1, 1, 3) NNHIP_VARIANT(2, 2, 5)
-    NNHIP_VARIANT(2, 2, 6) NNHIP_VARIANT(1, 1, 2) NNHIP_VARIANT(2, 1, 2)
+    NNHIP_VARIANT(2, 2, 6) NNHIP_VARIANT(1, 1, 2) NNHIP_VARIANT(2, 1, 2) NNHIP_VARIANT(1, 1, 4) NNHIP_VARIANT(2, 1, 4)
 #undef NNHIP_VARIANT
     return hipErrorInvalidConfiguration;
 }
@@ -618,6 +701,17 @@ int block_bytes_of(uint32_t type)
     switch (type) {
     case NNHIP_TYPE_Q4_K: return Q4KTask::kBlockBytes;
     case NNHIP_TYPE_Q5_K: return Q5KTask::kBlockBytes;
+    case NNHIP_TYPE_Q6_K: return Q6KTask::kBlockBytes;
+    default: return 0;
+    }
+}
+
+int block_pieces_of(uint32_t type)
+{
+    switch (type) {
+    case NNHIP_TYPE_Q4_K: return Q4KTask::kPieces;
+    case NNHIP_TYPE_Q5_K: return Q5KTask::kPieces;
+    case NNHIP_TYPE_Q6_K: return Q6KTask::kPieces;
     default: return 0;
     }
 }
@@ -660,7 +754,7 @@ bool matvec_mfma_geometry(uint32_t type, int in_w, int out_w, const void* w, Mfm
 {
     if (!entry_ok(type, in_w, out_w, w)) return false;
     MfmaGeom g;
-    if (!plan_mfma(block_bytes_of(type), in_w, &g)) return false;
+    if (!plan_mfma(block_pieces_of(type), in_w, &g)) return false;
     if (plan) {
         plan->waves = g.waves;
         plan->cols = g.cols;
@@ -678,7 +772,7 @@ hipError_t launch_matvec_mfma_table(Lane* lane, uint32_t type, int in_w, const M
 {
     MfmaArgs a{};
     MfmaGeom g;
-    if (!plan_mfma(block_bytes_of(type), in_w, &g)) return hipErrorInvalidValue;
+    if (!plan_mfma(block_pieces_of(type), in_w, &g)) return hipErrorInvalidValue;
     fill_args(type, in_w, g, &a);
     a.table = device_entries;
     a.entries = entries;
@@ -686,6 +780,7 @@ hipError_t launch_matvec_mfma_table(Lane* lane, uint32_t type, int in_w, const M
     switch (type) {
     case NNHIP_TYPE_Q4_K: return launch_mfma<Q4KTask>(lane, a);
     case NNHIP_TYPE_Q5_K: return launch_mfma<Q5KTask>(lane, a);
+    case NNHIP_TYPE_Q6_K: return launch_mfma<Q6KTask>(lane, a);
     default: return hipErrorInvalidValue;
     }
 }

@@ -10,7 +10,7 @@ import numpy as np
 import pytest
 
 import oracle
-from nntrain_amd import GGML_Q4_K, GGML_Q5_K, GGML_Q8_0, HipExecutionLane, HipQuantizedMatrix, synth
+from nntrain_amd import GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_Q8_0, HipExecutionLane, HipQuantizedMatrix, synth
 from nntrain_amd.native import MatvecDesc, check
 
 pytestmark = pytest.mark.gpu
@@ -353,9 +353,9 @@ def _batch_run(lane, items):
     return out
 
 
-@pytest.mark.parametrize("typ", [GGML_Q4_K, GGML_Q5_K])
+@pytest.mark.parametrize("typ", [GGML_Q4_K, GGML_Q5_K, GGML_Q6_K])
 def test_large_batched_groups_on_the_matrix_cores(lane, typ):
-    """Groups of Q4_K / Q5_K matrices with at least 2048 sixteen-row tiles go to the matrix-core mat-vec: against the
+    """Groups of Q4_K / Q5_K / Q6_K matrices with at least 2048 sixteen-row tiles go to the matrix-core mat-vec: against the
     float64 oracle at both bars, with bias, ragged row counts, several input rows, activations that change and repeat
     from matrix to matrix, and two widths in one call (two launches).  A row's bits must not depend on the other
     matrices of the call or on its place in it."""
