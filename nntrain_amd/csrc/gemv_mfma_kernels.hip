@@ -170,7 +170,7 @@ struct Q4KTask {
     using X = XSet<2>;
     struct Raw { u32x4 h, q1, q2; };
 
-    static __device__ __forceinline__ uint32_t piece_src(uint32_t q) { return 16u * q; }
+    static __device__ __forceinline__ uint32_t piece_src(uint32_t q, bool) { return 16u * q; }
 
     // plane = this lane's digit plane of the whole vector, sums = the per-sub-block sums of x; b = super-block column
     static __device__ __forceinline__ void load_x(X& xs, const uint8_t* plane, const float* sums, int b, int quarter, bool diag)
@@ -183,7 +183,7 @@ struct Q4KTask {
         xs.sx[1] = v.y;
     }
 
-    static __device__ __forceinline__ Raw load(const uint8_t* blk, int quarter)
+    static __device__ __forceinline__ Raw load(const uint8_t* blk, int quarter, bool)
     {
         Raw r;
         r.q1 = lds128(blk + 16 + 32 * quarter);
@@ -226,14 +226,14 @@ struct Q5KTask {
     using X = XSet<2>;
     struct Raw { u32x4 h, ha, hb, q1, q2; };
 
-    static __device__ __forceinline__ uint32_t piece_src(uint32_t q) { return 16u * q; }
+    static __device__ __forceinline__ uint32_t piece_src(uint32_t q, bool) { return 16u * q; }
 
     static __device__ __forceinline__ void load_x(X& xs, const uint8_t* plane, const float* sums, int b, int quarter, bool diag)
     {
         Q4KTask::load_x(xs, plane, sums, b, quarter, diag);
     }
 
-    static __device__ __forceinline__ Raw load(const uint8_t* blk, int quarter)
+    static __device__ __forceinline__ Raw load(const uint8_t* blk, int quarter, bool)
     {
         Raw r;
         r.q1 = lds128(blk + 48 + 32 * quarter);
@@ -277,7 +277,6 @@ struct Q5KTask {
 // the 32 ql bytes at 64h + 32e: low nibbles = weights 32e + l, high nibbles = weights 64 + 32e + l, four scale groups.
 // The -32 is taken through sums of x: sum x s (q - 32) = s sum(q x) - 32 s sum(x).
 // A block is 2-byte aligned in memory; a stage gives it 14 pieces (224 bytes) so that it starts 16-byte aligned in LDS.
-// Pieces 0-12 are its bytes 0-207; piece 13 is bytes 194-209 (d lands at 222), which never reaches past the block.
 struct Q6KTask {
     static constexpr int kBlockBytes = kQ6KBytes;
     static constexpr int kPieces = 14;
@@ -285,7 +284,11 @@ struct Q6KTask {
     using X = XSet<4>;
     struct Raw { u32x4 la, lb, ha, hb; u32x2 sc; uint32_t d; };
 
-    static __device__ __forceinline__ uint32_t piece_src(uint32_t q) { return q < 13u ? 16u * q : 194u; }
+    // Blocks with an even index start on a 4-byte boundary of their row and are fetched from there; the others start 2
+    // bytes past one and are fetched from it, so every 16-byte request is dword-aligned and an odd block sits 2 bytes
+    // into its 14 pieces.  (The last two bytes of an even block share a dword with the next block, an odd one: rows hold
+    // an even number of blocks here, so that dword never reaches past the matrix.)
+    static __device__ __forceinline__ uint32_t piece_src(uint32_t q, bool odd) { return 16u * q - (odd ? 2u : 0u); }
 
     static __device__ __forceinline__ void load_x(X& xs, const uint8_t* plane, const float* sums, int b, int quarter, bool diag)
     {
@@ -303,16 +306,39 @@ struct Q6KTask {
         xs.sx[3] = hi.y;
     }
 
-    static __device__ __forceinline__ Raw load(const uint8_t* blk, int quarter)
+    // `odd` (uniform over the wave): the block's bytes sit 2 bytes into its pieces; whole dwords are read and shifted
+    static __device__ __forceinline__ Raw load(const uint8_t* blk, int quarter, bool odd)
     {
         const int h = quarter >> 1, e = quarter & 1;
+        const uint8_t* ql = blk + 64 * h + 32 * e;
+        const uint8_t* qh = blk + 128 + 32 * h;
+        const uint8_t* sc = blk + 192 + 8 * h;
         Raw r;
-        r.la = lds128(blk + 64 * h + 32 * e);
-        r.ha = lds128(blk + 128 + 32 * h);
-        r.lb = lds128(blk + 64 * h + 32 * e + 16);
-        r.hb = lds128(blk + 128 + 32 * h + 16);
-        r.sc = *reinterpret_cast<const u32x2*>(blk + 192 + 8 * h);
-        r.d = *reinterpret_cast<const uint32_t*>(blk + 220) >> 16;
+        r.la = lds128(ql);
+        r.ha = lds128(qh);
+        r.lb = lds128(ql + 16);
+        r.hb = lds128(qh + 16);
+        r.sc = *reinterpret_cast<const u32x2*>(sc);
+        const uint32_t dword = *reinterpret_cast<const uint32_t*>(blk + 208);
+        r.d = odd ? dword >> 16 : dword & 0xffffu;
+        if (odd) {
+            const uint32_t lt = *reinterpret_cast<const uint32_t*>(ql + 32), ht = *reinterpret_cast<const uint32_t*>(qh + 32);
+            const uint32_t st = *reinterpret_cast<const uint32_t*>(sc + 8);
+            auto shift8 = [](u32x4& a, u32x4& b, uint32_t tail) {
+                a[0] = __builtin_amdgcn_alignbyte(a[1], a[0], 2);
+                a[1] = __builtin_amdgcn_alignbyte(a[2], a[1], 2);
+                a[2] = __builtin_amdgcn_alignbyte(a[3], a[2], 2);
+                a[3] = __builtin_amdgcn_alignbyte(b[0], a[3], 2);
+                b[0] = __builtin_amdgcn_alignbyte(b[1], b[0], 2);
+                b[1] = __builtin_amdgcn_alignbyte(b[2], b[1], 2);
+                b[2] = __builtin_amdgcn_alignbyte(b[3], b[2], 2);
+                b[3] = __builtin_amdgcn_alignbyte(tail, b[3], 2);
+            };
+            shift8(r.la, r.lb, lt);
+            shift8(r.ha, r.hb, ht);
+            r.sc[0] = __builtin_amdgcn_alignbyte(r.sc[1], r.sc[0], 2);
+            r.sc[1] = __builtin_amdgcn_alignbyte(st, r.sc[1], 2);
+        }
         return r;
     }
 
@@ -399,7 +425,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_kernel(MfmaArgs a)
         const uint32_t q = slot - r * static_cast<uint32_t>(g.row_pieces);
         const uint32_t c = q / static_cast<uint32_t>(F::kPieces);
         const bool real = r < static_cast<uint32_t>(kTileRows) && q < static_cast<uint32_t>(pieces_used);
-        rel[i] = real ? r * a.row_bytes + c * F::kBlockBytes + F::piece_src(q - c * F::kPieces) : kNoPiece;
+        rel[i] = real ? r * a.row_bytes + c * F::kBlockBytes + F::piece_src(q - c * F::kPieces, c & 1u) : kNoPiece;
     }
 
     // ---- the stage sequence of this workgroup: tiles blockIdx.x, blockIdx.x + G, ... of the launch's tile sequence,
@@ -594,7 +620,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_kernel(MfmaArgs a)
         const uint8_t* stage = cur + row_off;
         typename F::Raw raw[M];
 #pragma unroll
-        for (int t = 0; t < M; ++t) raw[t] = F::load(stage + t * W * (16 * F::kPieces), quarter);
+        for (int t = 0; t < M; ++t) raw[t] = F::load(stage + t * W * (16 * F::kPieces), quarter, (wave & 1) != 0);
 #pragma unroll
         for (int t = 0; t < M; ++t) F::run(raw[t], xs[k * M + t], quarter, accq, accm);
         if (k == KC - 1) {
@@ -634,7 +660,7 @@ constexpr Variant kVariants[] = {{1, 2, 5}, {1, 2, 6}, {2, 1, 3}, {1, 1, 3}, {2,
 // stages, two stage buffers must fit LDS (one of them doubles as scratch for the digit planes when the activations
 // change), (KC, M, LPW) must be an instantiated variant, and among those the choice maximises the bytes a stage holds,
 // then the waves.
-bool plan_mfma(int block_pieces, int in_w, MfmaGeom* out)
+bool plan_mfma(int block_pieces, int in_w, bool even_waves, MfmaGeom* out)
 {
     const int nblocks = in_w / 256;
     const int bp = block_pieces;
@@ -645,6 +671,7 @@ bool plan_mfma(int block_pieces, int in_w, MfmaGeom* out)
     for (int W = 6; W <= kMaxWaves; ++W) {
         for (int m = 1; m <= 2; ++m) {
             MfmaGeom g{};
+            if (even_waves && (W & 1)) continue;       // block parity must be wave parity (Q6_K)
             g.waves = W;
             g.cols = W * m;
             if (nblocks % g.cols != 0) continue;
@@ -754,7 +781,7 @@ bool matvec_mfma_geometry(uint32_t type, int in_w, int out_w, const void* w, Mfm
 {
     if (!entry_ok(type, in_w, out_w, w)) return false;
     MfmaGeom g;
-    if (!plan_mfma(block_pieces_of(type), in_w, &g)) return false;
+    if (!plan_mfma(block_pieces_of(type), in_w, block_bytes_of(type) % 16 != 0, &g)) return false;
     if (plan) {
         plan->waves = g.waves;
         plan->cols = g.cols;
@@ -772,7 +799,7 @@ hipError_t launch_matvec_mfma_table(Lane* lane, uint32_t type, int in_w, const M
 {
     MfmaArgs a{};
     MfmaGeom g;
-    if (!plan_mfma(block_pieces_of(type), in_w, &g)) return hipErrorInvalidValue;
+    if (!plan_mfma(block_pieces_of(type), in_w, block_bytes_of(type) % 16 != 0, &g)) return hipErrorInvalidValue;
     fill_args(type, in_w, g, &a);
     a.table = device_entries;
     a.entries = entries;
