@@ -437,10 +437,10 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_kernel(MfmaArgs a)
     const int n4 = a.in_w >> 2;
 
     // ---- prefetch side: the stage it requests next, the matrix that stage belongs to
-    constexpr int kXRegs = 4;              // float4 per lane that hold the next matrix' activations on their way in
+    // float4 per lane that hold the next matrix' activations on their way in: in_w = KC * M * W * 256 floats over 64 W lanes
+    constexpr int kXRegs = KC * M;
     float4 xv[kXRegs];
     int xv_m = -1;                         // the table entry whose activations are in xv (or on their way)
-    const bool x_fits = n4 <= kXRegs * T;
     int f_t = blockIdx.x, f_k = 0, f_m = 0;
     MfmaEntry fe = entry_at(0);
     const float* f_x = nullptr;            // vector of the matrix the prefetch side was in last
@@ -459,7 +459,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_kernel(MfmaArgs a)
         f_matrix = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(fe.w), 0, static_cast<int>(fe.w_bytes), 0x00020000);
         if (fe.x != f_x) {
             // only one vector can be on its way; a second change before the first was consumed is fetched at the switch
-            if (x_fits && xv_m < 0) request_x(fe.x, f_m);
+            if (xv_m < 0) request_x(fe.x, f_m);
             f_x = fe.x;
         }
     };
@@ -502,7 +502,6 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_kernel(MfmaArgs a)
         if (xv_m != c_m) request_x(ce.x, c_m);
         xv_m = -1;
         constexpr float4 kZero4 = {0.0f, 0.0f, 0.0f, 0.0f};
-        const float4* x4 = reinterpret_cast<const float4*>(ce.x);
         const int plane_stride = a.in_w + 16;
         float* sumx = reinterpret_cast<float*>(scratch + 4 * plane_stride);
         auto umax4 = [](uint32_t m, const float4& v) {
@@ -517,7 +516,6 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_kernel(MfmaArgs a)
             if (tid + j * T >= n4) xv[j] = kZero4;
             mx = umax4(mx, xv[j]);
         }
-        for (int i = tid + kXRegs * T; i < n4; i += T) mx = umax4(mx, x4[i]);      // (vectors too long for xv: re-read)
         mx = wave_umax(mx);
         if (lane == 0) red[wave] = mx;
         __syncthreads();
@@ -551,7 +549,6 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_kernel(MfmaArgs a)
             const int i = tid + j * T;                               // (whole groups of eight lanes are in or out: n4 % 8 == 0)
             if (i < n4) to_planes(i, xv[j]);
         }
-        for (int i = tid + kXRegs * T; i < n4; i += T) to_planes(i, x4[i]);
         __syncthreads();
         // set k * M + t = super-block column k * cols + t * W + wave of a row
 #pragma unroll
@@ -569,6 +566,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_kernel(MfmaArgs a)
     // ---- start: the first matrix' activations are requested ahead of the weight stream, then two stages
     uint8_t* const buf0 = smem;
     uint8_t* const buf1 = smem + g.stage_bytes;
+    // (a third register set, three stages on their way, was measured without gain)
     u32x4 regs[2][LPW];
     fetch_enter();
     fetch(regs[0]);
