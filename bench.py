@@ -6,7 +6,8 @@ random-init, resident in HBM (62 layers x {q,k,v,o,gate,up,down} + lm_head = 435
 per token).  A "step" is one token: every mat-vec of the set once, fresh N(0,1) FP32 activations, batch 1.
 `value` is tokens/s; `roofline` is the Q8_0 mat-vec kernel's achieved HBM rate over the same timed region.
 
-Other workloads (`--workload gemv|prefill|all`) time the single-matrix configurations and are reported under "also".
+Other workloads (`--workload gemv|prefill|ffn|decode_loop|decode27b_chained|all`) time the single-matrix configurations,
+the fused layer half, the GGUF decode loop and the 27B-shape token in dependency order; they are reported under "also".
 
 One JSON line on stdout; progress on stderr.
 """
@@ -28,10 +29,37 @@ sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 BF16_PEAK_TFLOPS = 2500.0      # MI355X dense bf16 MFMA, published
-# HBM bytes one batched launch of the decode27b set moves, from two rocprofv3 --pmc runs (FETCH_SIZE x 2.000 and
-# WRITE_SIZE x 1.000, the factors a plain copy kernel of known size gives); summary in
-# profiles/matvec_batch_q8_0_decode27b_hbm_traffic.md.  Only valid for --mode batch.
-DECODE27B_BATCH_TRAFFIC_BYTES = 29_074_665_059
+COPY_KERNEL = "__amd_rocclr_copyBuffer"      # the runtime's device-to-device copy, whose true traffic is its size
+
+
+def traffic_from_counters(fetch_csv, write_csv, kernel_substring, copy_bytes):
+    """HBM bytes per launch of the kernel named `kernel_substring`, from two `rocprofv3 --pmc` runs of this same command
+    with --copy-calibration (FETCH_SIZE in one, WRITE_SIZE in the other; both count KiB per dispatch).  Each counter is
+    scaled by what it reads for the calibration copy of `copy_bytes` bytes.  Returns (bytes, details)."""
+    import csv
+
+    def per_kernel(path, counter):
+        kernel, copy = [], []
+        with open(path, newline="") as f:
+            for row in csv.DictReader(f):
+                if row["Counter_Name"] != counter:
+                    continue
+                if kernel_substring in row["Kernel_Name"]:
+                    kernel.append(float(row["Counter_Value"]))
+                elif COPY_KERNEL in row["Kernel_Name"]:
+                    copy.append(float(row["Counter_Value"]))
+        if not kernel or not copy:
+            raise SystemExit(f"{path}: no {counter} rows for '{kernel_substring}' and the calibration copy")
+        # the calibration copy is the largest copy of the run
+        return sum(kernel) / len(kernel), max(copy)
+
+    true_kib = copy_bytes / 1024.0
+    fetch, fetch_copy = per_kernel(fetch_csv, "FETCH_SIZE")
+    write, write_copy = per_kernel(write_csv, "WRITE_SIZE")
+    f_scale, w_scale = true_kib / fetch_copy, true_kib / write_copy
+    total = int(round((fetch * f_scale + write * w_scale) * 1024.0))
+    return total, {"fetch_kib_per_dispatch": fetch, "write_kib_per_dispatch": write, "fetch_scale": round(f_scale, 4),
+                   "write_scale": round(w_scale, 4), "calibration_copy_bytes": copy_bytes}
 
 
 def log(*a):
@@ -126,6 +154,7 @@ def run_decode27b(args, lane, nn, oracle):
             raise SystemExit(f"parity failure ({tag}): rel-L2 {worst:.3e} > 1e-5")
         return worst
 
+    calibration_bytes = weights[-1].nbytes
     if args.copy_calibration:
         # a plain device-to-device copy of known size, so that a counter run (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)
         # of this same command can scale the counters by what they read for it
@@ -155,6 +184,12 @@ def run_decode27b(args, lane, nn, oracle):
     for b in weights + xs + ys:
         b.dispose()
     n_launch = len(tensors) if args.mode != "batch" else 1
+    traffic = None
+    if args.traffic_from:
+        if args.mode != "batch":
+            raise SystemExit("--traffic-from applies to --mode batch (one launch per token)")
+        traffic, detail = traffic_from_counters(args.traffic_from[0], args.traffic_from[1], "matvec_batch_kernel", calibration_bytes)
+        log(f"[decode27b] HBM traffic per launch from counters: {traffic} bytes ({detail})")
     return {
         "metric": "27B-shape Q8_0 decode tokens/sec", "value": round(tok_s, 2), "unit": "tokens/s",
         "ms_per_step": round(ms_per_step, 4),
@@ -163,7 +198,7 @@ def run_decode27b(args, lane, nn, oracle):
                    "launch": args.mode, "launches_per_token": n_launch},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4),
-                     "traffic": DECODE27B_BATCH_TRAFFIC_BYTES if args.mode == "batch" else None,
+                     "traffic": traffic,
                      "kernel": "matvec_batch_kernel<Q8_0Unit>" if args.mode == "batch" else "matvec_rowstep_kernel<Q8_0Unit>",
                      "bytes_per_launch": total_bytes // n_launch},
         "cpu_baseline": cpu,
@@ -171,32 +206,51 @@ def run_decode27b(args, lane, nn, oracle):
     }
 
 
-def cpu_baseline_decode(lane, nn, oracle, tensors, weights, xs):
-    """The CPU restatement of the reference's operator (dequantize row + sequential FP32 FMA) on one layer's seven
-    matrices, all host threads; the token rate is extrapolated by bytes to the whole set."""
+def cpu_leg(oracle, typ, w_host, x_host, in_w, out_w, budget_s):
+    """The CPU restatement of the reference's operator (dequantize row + sequential FP32 FMA, Tensor.QwenQuantized.cs:
+    113-165) on one matrix, compiled for this host: all threads for about budget_s seconds, then one thread on the
+    first rows.  Returns seconds per pass (all threads), seconds per pass extrapolated from one thread, thread count."""
     threads = oracle.max_threads()
-    sample = list(range(7))
-    host = []
-    for t in sample:
-        name, out_w, in_w = tensors[t]
-        host.append((lane.read(weights[t], np.uint8), lane.read(xs[t], np.float32), in_w, out_w))
-    sample_bytes = sum(w.size for w, _, _, _ in host)
-    total_bytes = sum(q8_bytes(o, i) for _, o, i in tensors)
     reps, spent = 0, 0.0
     t_begin = time.perf_counter()
-    while spent < 10.0 or reps < 2:
-        for w, x, in_w, out_w in host:
-            oracle.cpu_linear(nn.GGML_Q8_0, w, x, None, 1, in_w, out_w, threads)
+    while spent < budget_s or reps < 2:
+        oracle.cpu_linear(typ, w_host, x_host, None, 1, in_w, out_w, threads, native=True)
         reps += 1
         spent = time.perf_counter() - t_begin
-    per_layer = spent / reps
+    per_pass = spent / reps
+    rows1 = max(1, min(out_w, int(out_w * min(1.0, 0.5 / max(per_pass * threads, 1e-9)))))
+    row_bytes = w_host.size // out_w
+    t_begin = time.perf_counter()
+    oracle.cpu_linear(typ, w_host[:rows1 * row_bytes], x_host, None, 1, in_w, rows1, 1, native=True)
+    one = (time.perf_counter() - t_begin) * out_w / rows1
+    return per_pass, one, threads, reps
+
+
+def cpu_baseline_decode(lane, nn, oracle, tensors, weights, xs):
+    """One layer's seven matrices through cpu_leg; the token rate is extrapolated by bytes to the whole set."""
+    sample = list(range(7))
+    sample_bytes = sum(q8_bytes(tensors[t][1], tensors[t][2]) for t in sample)
+    total_bytes = sum(q8_bytes(o, i) for _, o, i in tensors)
+    per_layer = one_layer = 0.0
+    passes = []
+    for t in sample:
+        name, out_w, in_w = tensors[t]
+        per_pass, one, threads, reps = cpu_leg(oracle, nn.GGML_Q8_0, lane.read(weights[t], np.uint8), lane.read(xs[t], np.float32),
+                                               in_w, out_w, 1.5)
+        per_layer += per_pass
+        one_layer += one
+        passes.append(reps)
     tok_s = 1.0 / (per_layer * total_bytes / sample_bytes)
+    tok_s_one = 1.0 / (one_layer * total_bytes / sample_bytes)
     log(f"[cpu_baseline] {threads} threads: layer sample {per_layer * 1e3:.1f} ms ({sample_bytes / per_layer / 1e9:.1f} GB/s)"
-        f" -> {tok_s:.3f} tok/s extrapolated")
+        f" -> {tok_s:.3f} tok/s extrapolated; one thread {tok_s_one:.4f} tok/s")
     return {"value": round(tok_s, 4), "unit": "tokens/s", "cores": threads, "kind": "port",
-            "sample": f"layer 0's seven Q8_0 matrices ({sample_bytes} bytes) x {reps} passes, {spent:.1f} s; token rate "
-                      f"extrapolated by weight bytes to the 435-matrix set",
-            "gb_per_s": round(sample_bytes / per_layer / 1e9, 2)}
+            "sample": f"layer 0's seven Q8_0 matrices ({sample_bytes} bytes), {min(passes)}-{max(passes)} passes each; token "
+                      f"rate extrapolated by weight bytes to the 435-matrix set",
+            "gb_per_s": round(sample_bytes / per_layer / 1e9, 2),
+            "one_thread": {"value": round(tok_s_one, 5), "gb_per_s": round(sample_bytes / one_layer / 1e9, 3),
+                           "sample": "the first rows of the same matrices, extrapolated by rows"},
+            "cpu_model": oracle.cpu_model(), "host_threads_available": os.cpu_count(), "build": oracle.native_lib()[1]}
 
 
 GEMV_CONFIGS = [
@@ -282,6 +336,11 @@ def run_gemv(args, lane, nn, oracle):
         log(f"[gemv] {name}: single launch {us_ring:.2f} us ({algo / us_ring / 1e3:.0f} GB/s, "
             f"{100 * algo / us_ring / 1e3 / HBM_PEAK_GBS:.1f}% of 8 TB/s) HBM, {us_same:.2f} us cache-resident; batched "
             f"{us_batch:.2f} us/mat-vec ({100 * algo / us_batch / 1e3 / HBM_PEAK_GBS:.1f}%); rel-L2 {rel:.2e}")
+        if not args.no_cpu_baseline:
+            per_pass, one, threads, _ = cpu_leg(oracle, typ, payload, x_host, in_w, out_w, 1.0)
+            out[name]["cpu_baseline"] = {"gb_per_s": round(nbytes / per_pass / 1e9, 2), "us_per_matvec": round(per_pass * 1e6, 1),
+                                         "cores": threads, "one_thread_gb_per_s": round(nbytes / one / 1e9, 3), "kind": "port"}
+            log(f"[gemv] {name}: CPU port {nbytes / per_pass / 1e9:.1f} GB/s on {threads} threads, {nbytes / one / 1e9:.2f} GB/s on one")
         if tname == "GGML_Q8_0":
             # several input rows in one call (weights rotated as above): microseconds per call
             per_rows = {}
@@ -521,6 +580,92 @@ def run_decode_loop(args, lane, nn, oracle):
     return out
 
 
+def run_decode27b_chained(args, lane, nn, oracle):
+    """The 27B-shape Q8_0 token in its real dependency order: the decode loop of nntrain_amd.decoder (norm -> q|k|v ->
+    first-token attention -> o -> norm -> gate|up -> SiLU product -> down -> ... -> head, NNtrain.Core/Modules/
+    Qwen35QuantizedModel.cs:451-513) over the same 435 matrix shapes as the headline set, weights drawn on the device,
+    the head tied to the embedding.  Every mat-vec consumes what the one before it produced, so nothing overlaps across
+    launches: one launch per operation (the reference's sequence), the fused launches, and those replayed from a HIP
+    graph.  All three end in the same logits bit for bit."""
+    from nntrain_amd.decoder import DecoderDescriptor, QuantizedDecoder
+    from nntrain_amd.synth import DeviceSynth
+    d = DecoderDescriptor("gemma3-27b-shape", 62, 5376, 21504, 32, 16, 128, 1e-6, 262144)
+    synth = DeviceSynth()
+    def weights():
+        seeds = iter(range(7000, 9000))
+
+        def matrix(name, in_w, out_w):
+            w = lane.allocate_bytes(q8_bytes(out_w, in_w))
+            synth.q8_0(lane, w, out_w * (in_w // 32), next(seeds))
+            return nn.HipQuantizedMatrix.from_device(lane, w, nn.GGML_Q8_0, out_w, in_w)
+
+        def dense(name, width):
+            import zlib
+            return lane.upload_raw(np.random.default_rng(zlib.crc32(name.encode())).uniform(0.5, 1.5, width).astype(np.float32))
+
+        return matrix, dense
+
+    log("[decode27b_chained] generating two copies of the weights (one launch per operation / fused)")
+    m1, d1 = weights()
+    plain = QuantizedDecoder.from_weights(lane, d, m1, d1, has_output=False, fused=False)
+    m2, d2 = weights()
+    fused = QuantizedDecoder.from_weights(lane, d, m2, d2, has_output=False, fused=True)
+    lane.synchronize()
+    vocab = d.vocabulary
+    weight_bytes = plain.quantized_bytes          # every matrix is streamed whole: the head is the tied embedding
+    tokens = [3, 1000, 262143, 17]
+    for t in tokens[:2]:
+        a = lane.read(plain.forward_token(t), np.uint32, count=vocab)
+        b = lane.read(fused.forward_token(t), np.uint32, count=vocab)
+        if not np.array_equal(a, b):
+            raise SystemExit("decode27b_chained: fused and unfused logits differ bitwise")
+    # the head against the float64 oracle, from the hidden state the chain ended in
+    hidden = lane.read(plain._hidden[plain._cur], np.float32).astype(np.float64)
+    gamma = lane.read(plain.output_norm, np.float32).astype(np.float64)
+    normed = (hidden / np.sqrt(np.mean(hidden * hidden) + d.rms_epsilon) * gamma).astype(np.float32)
+    row_bytes = (d.embedding_length // 32) * 34
+    raw = lane.read(plain.embedding.device_payload(lane), np.uint8, 256 * row_bytes, 0)
+    ref, _ = oracle.linear_f64(nn.GGML_Q8_0, raw, normed, None, 1, d.embedding_length, 256)
+    logits = lane.read(plain.logits, np.float32, count=256)
+    rel = oracle.rel_l2(logits, ref[0])
+    log(f"[decode27b_chained] head logits (first 256) vs float64 oracle from the final hidden state: rel-L2 {rel:.3e}")
+    if not (np.all(np.isfinite(logits)) and rel <= 1e-4):       # the norm is recomputed here in float64: looser than 1e-5
+        raise SystemExit(f"decode27b_chained: parity failure, rel-L2 {rel:.3e}")
+
+    def per_token(dec):
+        samples = []
+        for _ in range(5):
+            ms, _ = timed(lane, lambda: [dec.forward_token(t) for t in tokens], 1)
+            samples.append(ms / len(tokens))
+        return float(np.median(samples))
+
+    ms_plain, ms_fused = per_token(plain), per_token(fused)
+    fused.capture_graph()
+    if not np.array_equal(lane.read(fused.forward_token(tokens[1]), np.uint32, count=vocab),
+                          lane.read(plain.forward_token(tokens[1]), np.uint32, count=vocab)):
+        raise SystemExit("decode27b_chained: graph replay differs bitwise")
+    ms_graph = per_token(fused)
+
+    def entry(ms):
+        return {"ms_per_token": round(ms, 4), "tokens_per_s": round(1e3 / ms, 2), "gb_per_s": round(weight_bytes / ms / 1e6, 1),
+                "frac_of_8TBs": round(weight_bytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+
+    layers = d.layer_count
+    out = {"config": "62 layers, hidden 5376, feed-forward 21504, heads 32/16 x 128, vocabulary 262144 (head tied to the "
+                     "embedding), Q8_0, first-token attention (no cache)",
+           "weight_bytes_streamed_per_token": weight_bytes,
+           "one_launch_per_operation": entry(ms_plain), "fused_launches": entry(ms_fused),
+           "fused_launches_hip_graph": entry(ms_graph),
+           "launches_per_token": {"one_launch_per_operation": 1 + 12 * layers + 2, "fused_launches": 1 + 5 * layers + 1},
+           "rel_l2_head_vs_f64_oracle": rel, "bitwise_equal": True}
+    log(f"[decode27b_chained] per token: {ms_plain:.3f} ms one launch per operation, {ms_fused:.3f} ms fused, "
+        f"{ms_graph:.3f} ms fused + graph ({weight_bytes / ms_graph / 1e6:.0f} GB/s, {1e3 / ms_graph:.1f} tok/s)")
+    plain.dispose()
+    fused.dispose()
+    lane.trim()
+    return out
+
+
 def run_prefill(args, lane, nn, oracle):
     """Q4_K 17408x5120 bf16-MFMA prefill mat-mul at M = 128, 256, 512, 2048 (BASELINE configs[3]); the other formats
     the kernel decodes (Q5_K, Q6_K, Q8_0, IQ2_S, IQ3_S) at M = 512 under "other_formats"."""
@@ -581,10 +726,13 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", choices=["decode27b", "gemv", "prefill", "ffn", "decode_loop", "all"], default="all")
+    ap.add_argument("--workload", choices=["decode27b", "decode27b_chained", "gemv", "prefill", "ffn", "decode_loop", "all"], default="all")
     ap.add_argument("--mode", choices=["forward", "graph", "batch"], default="batch",
                     help="decode27b: one launch per matrix, the same captured in a HIP graph, or the batched entry point")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--traffic-from", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
+                    help="decode27b --mode batch: counter_collection.csv files of two rocprofv3 --pmc runs of this command "
+                         "with --copy-calibration (FETCH_SIZE, WRITE_SIZE); fills roofline.traffic, which is null otherwise")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="decode27b: also run one device-to-device copy of the lm_head weights (for counter runs)")
     args = ap.parse_args()
@@ -606,6 +754,8 @@ def main():
         also["ffn_layer_half_fused_epilogues"] = run_ffn(args, lane, nn, oracle)
     if args.workload in ("decode_loop", "all"):
         also["decode_loop_gguf_file"] = run_decode_loop(args, lane, nn, oracle)
+    if args.workload in ("decode27b_chained", "all"):
+        also["decode27b_chained"] = run_decode27b_chained(args, lane, nn, oracle)
     if args.workload in ("decode27b", "all"):
         res = run_decode27b(args, lane, nn, oracle)
     else:

@@ -94,57 +94,76 @@ class QuantizedDecoder:
     """Weights of one GGUF file resident on one lane, and the per-token loop over them."""
 
     def __init__(self, lane: HipExecutionLane, reader: GgufReader, fused: bool = True, chunk_bytes: int = 64 << 20):
-        self.lane = lane
-        self.fused = fused
-        self.descriptor = d = DecoderDescriptor.inspect(reader)
+        descriptor = DecoderDescriptor.inspect(reader)
         directory = GgufTensorDirectory(reader)
         loader = HipGgufLoader(lane, reader, chunk_bytes)
+        self._build(lane, descriptor, fused,
+                    matrix=lambda name, in_w, out_w: loader.load_matrix(directory.matrix(name, in_w, out_w)),
+                    dense=lambda name, width: loader.load_dense(directory.dense(name, width)),
+                    has_output="output.weight" in directory, finish=directory.reject_unexpected)
+        self.quantized_bytes, self.dense_bytes = loader.quantized_bytes, loader.dense_bytes
+
+    @classmethod
+    def from_weights(cls, lane: HipExecutionLane, descriptor: DecoderDescriptor, matrix, dense, has_output: bool,
+                     fused: bool = True) -> "QuantizedDecoder":
+        """The same loop over weights that are already on the lane: matrix(name, in_w, out_w) returns a
+        HipQuantizedMatrix whose payload is resident, dense(name, width) an FP32 HipBuffer; the decoder owns both."""
+        self = cls.__new__(cls)
+        self._build(lane, descriptor, fused, matrix, dense, has_output, finish=lambda: None)
+        self.quantized_bytes = sum(m.storage_bytes for m in self._owned if isinstance(m, HipQuantizedMatrix))
+        self.dense_bytes = sum(b.nbytes for b in self._owned if isinstance(b, HipBuffer))
+        return self
+
+    def _build(self, lane, descriptor, fused, matrix, dense, has_output, finish) -> None:
+        self.lane = lane
+        self.fused = fused
+        self.descriptor = d = descriptor
         q_width, kv_width = d.head_count * d.head_width, d.kv_head_count * d.head_width
         self._owned: list = []
 
-        def matrix(name, in_w, out_w):
-            m = loader.load_matrix(directory.matrix(name, in_w, out_w))
-            self._owned.append(m)
-            return m
+        def own(item):
+            self._owned.append(item)
+            return item
 
-        def dense(name, width):
-            b = loader.load_dense(directory.dense(name, width))
-            self._owned.append(b)
-            return b
+        def stack(parts):
+            """One matrix from projections of the same vector; the parts are freed, the stack replaces them."""
+            whole = own(HipQuantizedMatrix.stacked(lane, parts))
+            for m in parts:
+                self._owned.remove(m)
+                m.dispose()
+            return whole
 
         try:
-            self.embedding = matrix("token_embd.weight", d.embedding_length, d.vocabulary)
+            self.embedding = own(matrix("token_embd.weight", d.embedding_length, d.vocabulary))
             self.layers: list[_Layer] = []
             for i in range(d.layer_count):
                 p, L = f"blk.{i}.", _Layer()
-                L.attn_norm = dense(p + "attn_norm.weight", d.embedding_length)
-                L.q = matrix(p + "attn_q.weight", d.embedding_length, q_width)
-                L.k = matrix(p + "attn_k.weight", d.embedding_length, kv_width)
-                L.v = matrix(p + "attn_v.weight", d.embedding_length, kv_width)
-                L.o = matrix(p + "attn_output.weight", q_width, d.embedding_length)
-                L.ffn_norm = dense(p + "ffn_norm.weight", d.embedding_length)
-                L.gate = matrix(p + "ffn_gate.weight", d.embedding_length, d.feed_forward_length)
-                L.up = matrix(p + "ffn_up.weight", d.embedding_length, d.feed_forward_length)
-                L.down = matrix(p + "ffn_down.weight", d.feed_forward_length, d.embedding_length)
+                L.attn_norm = own(dense(p + "attn_norm.weight", d.embedding_length))
+                L.q = own(matrix(p + "attn_q.weight", d.embedding_length, q_width))
+                L.k = own(matrix(p + "attn_k.weight", d.embedding_length, kv_width))
+                L.v = own(matrix(p + "attn_v.weight", d.embedding_length, kv_width))
+                L.o = own(matrix(p + "attn_output.weight", q_width, d.embedding_length))
+                L.ffn_norm = own(dense(p + "ffn_norm.weight", d.embedding_length))
+                L.gate = own(matrix(p + "ffn_gate.weight", d.embedding_length, d.feed_forward_length))
+                L.up = own(matrix(p + "ffn_up.weight", d.embedding_length, d.feed_forward_length))
+                L.down = own(matrix(p + "ffn_down.weight", d.feed_forward_length, d.embedding_length))
                 L.qkv = L.gate_up = None
                 if fused:
                     # projections of the same vector become one launch when their storage types agree
                     if L.q.ggml_type == L.k.ggml_type == L.v.ggml_type:
-                        L.qkv = HipQuantizedMatrix.stacked(lane, [L.q, L.k, L.v])
-                        self._owned.append(L.qkv)
+                        L.qkv = stack([L.q, L.k, L.v])
+                        L.q = L.k = L.v = None
                     if L.gate.ggml_type == L.up.ggml_type:
-                        L.gate_up = HipQuantizedMatrix.stacked(lane, [L.gate, L.up])
-                        self._owned.append(L.gate_up)
+                        L.gate_up = stack([L.gate, L.up])
+                        L.gate = L.up = None
                 self.layers.append(L)
-            self.output_norm = dense("output_norm.weight", d.embedding_length)
+            self.output_norm = own(dense("output_norm.weight", d.embedding_length))
             # a file without output.weight ties the head to the embedding, as llama.cpp does
-            self.output = matrix("output.weight", d.embedding_length, d.vocabulary) if "output.weight" in directory \
-                else self.embedding
-            directory.reject_unexpected()
+            self.output = own(matrix("output.weight", d.embedding_length, d.vocabulary)) if has_output else self.embedding
+            finish()
         except BaseException:
             self.dispose()
             raise
-        self.quantized_bytes, self.dense_bytes = loader.quantized_bytes, loader.dense_bytes
 
         # activations: allocated once, so a token step allocates nothing (and can be captured in a graph)
         alloc = lane.allocate

@@ -15,6 +15,7 @@ from __future__ import annotations
 
 import ctypes
 import re
+import os
 import subprocess
 from pathlib import Path
 
@@ -66,6 +67,42 @@ def lib() -> ctypes.CDLL:
     return _lib
 
 
+_native = None
+
+
+def native_lib():
+    """The same sources compiled for the host this process runs on (-march=native), for timing the CPU path where it
+    runs; the committed library is built for x86-64-v3 so that it loads anywhere.  Returns (library, build flags);
+    falls back to the committed library when no compiler is at hand."""
+    global _native
+    if _native is None:
+        import tempfile
+        flags = "-O3 -march=native -ffp-contract=off -fno-fast-math -fopenmp -fPIC"
+        out = Path(tempfile.gettempdir()) / f"libquant_oracle_native_{os.getpid()}.so"
+        try:
+            subprocess.run(["gcc", *flags.split(), "-shared", "-o", str(out), str(HERE / "quant_oracle.c"),
+                            str(HERE / "norm_oracle.c"), "-lm"], check=True, capture_output=True)
+            L = ctypes.CDLL(str(out))
+            L.oracle_cpu_linear.argtypes = lib().oracle_cpu_linear.argtypes
+            _native = (L, "gcc " + flags)
+        except (OSError, subprocess.CalledProcessError):
+            _native = (lib(), "committed build (x86-64-v3)")
+        finally:
+            if out.exists():
+                out.unlink()
+    return _native
+
+
+def cpu_model() -> str:
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def _ptr(a):
     return None if a is None else a.ctypes.data_as(ctypes.c_void_p)
 
@@ -95,15 +132,17 @@ def dequantize(ggml_type: int, raw, elements: int | None = None) -> np.ndarray:
 
 
 def cpu_linear(ggml_type: int, raw, x: np.ndarray, bias, rows: int, in_w: int, out_w: int,
-               threads: int = 0) -> np.ndarray:
-    """C oracle: the reference's CpuLinear (FP32 sequential FMA from bias)."""
+               threads: int = 0, native: bool = False) -> np.ndarray:
+    """C oracle: the reference's CpuLinear (FP32 sequential FMA from bias).  native=True runs the build made for this
+    host (native_lib), for timing."""
     raw = _raw(raw)
     x = np.ascontiguousarray(x, dtype=np.float32)
     assert x.size == rows * in_w
     assert raw.size == out_w * (in_w // BLOCK_ELEMS[ggml_type]) * BLOCK_BYTES[ggml_type]
     b = None if bias is None else np.ascontiguousarray(bias, dtype=np.float32)
     y = np.empty((rows, out_w), dtype=np.float32)
-    rc = lib().oracle_cpu_linear(ggml_type, _ptr(raw), _ptr(x), _ptr(b), _ptr(y), rows, in_w, out_w, threads)
+    L = native_lib()[0] if native else lib()
+    rc = L.oracle_cpu_linear(ggml_type, _ptr(raw), _ptr(x), _ptr(b), _ptr(y), rows, in_w, out_w, threads)
     if rc != 0:
         raise ValueError(f"oracle_cpu_linear failed ({rc})")
     return y
