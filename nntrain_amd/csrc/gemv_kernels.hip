@@ -1305,7 +1305,7 @@ struct BatchGroup {
     uint32_t type;
     size_t begin, end;       // entries [begin, end) of the table
     int total_chunks, max_in_w;
-    bool mfma;               // a launch of the matrix-core kernel: entries are MfmaTableEntry, total_chunks counts tiles
+    int mfma;                // 0, or the form of the matrix-core kernel (1 - 3): entries are MfmaTableEntry, total_chunks counts tiles
 };
 constexpr int kBatchTypes = 7;
 constexpr int kBatchGroupsMax = kBatchTypes + 8;      // row-step groups plus matrix-core groups (one per type and in_w)
@@ -1325,32 +1325,43 @@ long build_batch(const nnhip_matvec_desc* descs, int count, BatchEntry* out, siz
 {
     size_t n = 0;
     *ngroups = 0;
-    // matrix-core groups first: per (type, in_w) with enough tiles
-    auto mfma_ok = [&](const nnhip_matvec_desc& d) { return matvec_mfma_geometry(d.ggml_type, d.in_w, d.out_w, d.w, nullptr); };
-    auto in_mfma_group = [&](const nnhip_matvec_desc& d) {
-        if (!mfma_ok(d)) return false;
+    // matrix-core groups first: per (type, in_w, form) with enough tiles.  Forms: 1 = operand A in registers (in_w splits
+    // into one or two whole stages), 2 = the wide form with one input row per entry, 3 = the wide form with up to four
+    // input rows of a descriptor sharing a pass (descriptors with rows >= 2).
+    auto form_of = [&](const nnhip_matvec_desc& d) {
+        if (d.rows >= 2 && matvec_mfma_wide_geometry(d.ggml_type, d.in_w, d.out_w, d.w, 4)) return 3;
+        if (matvec_mfma_geometry(d.ggml_type, d.in_w, d.out_w, d.w, nullptr)) return 1;
+        if (matvec_mfma_wide_geometry(d.ggml_type, d.in_w, d.out_w, d.w, 1)) return 2;
+        return 0;
+    };
+    auto same_group = [&](const nnhip_matvec_desc& p, int form, const nnhip_matvec_desc& d) {
+        return d.ggml_type == p.ggml_type && d.in_w == p.in_w && form_of(d) == form;
+    };
+    auto in_mfma_group = [&](const nnhip_matvec_desc& d, int form) {
+        if (!form) return false;
         long tiles = 0;
         for (int j = 0; j < count; ++j)
-            if (descs[j].ggml_type == d.ggml_type && descs[j].in_w == d.in_w && mfma_ok(descs[j]))
-                tiles += static_cast<long>(descs[j].rows) * ((descs[j].out_w + 15) / 16);
+            if (same_group(d, form, descs[j])) tiles += static_cast<long>(descs[j].rows) * ((descs[j].out_w + 15) / 16);
         return tiles >= kMfmaBatchMinTiles;
     };
     for (int i = 0; i < count; ++i) {
         const nnhip_matvec_desc& lead = descs[i];
-        if (!in_mfma_group(lead)) continue;
+        const int form = form_of(lead);
+        if (!in_mfma_group(lead, form)) continue;
         bool seen = false;
-        for (int j = 0; j < i; ++j)
-            seen = seen || (descs[j].ggml_type == lead.ggml_type && descs[j].in_w == lead.in_w && mfma_ok(descs[j]));
+        for (int j = 0; j < i; ++j) seen = seen || same_group(lead, form, descs[j]);
         if (seen) continue;
         if (*ngroups >= kBatchGroupsMax - kBatchTypes) break;      // (further groups stay with the row-step kernel)
-        BatchGroup g{lead.ggml_type, n, n, 0, lead.in_w, true};
+        BatchGroup g{lead.ggml_type, n, n, 0, lead.in_w, form};
         for (int j = i; j < count; ++j) {
             const nnhip_matvec_desc& d = descs[j];
-            if (d.ggml_type != lead.ggml_type || d.in_w != lead.in_w || !mfma_ok(d)) continue;
-            for (int r = 0; r < d.rows; ++r) {
+            if (!same_group(lead, form, d)) continue;
+            const int share = form == 3 ? 4 : 1;
+            for (int r = 0; r < d.rows; r += share) {
                 if (n >= cap) return -1;
-                const MfmaTableEntry e = matvec_mfma_entry(d.ggml_type, d.x + static_cast<size_t>(r) * d.in_w, d.w, d.bias,
-                                                           d.y + static_cast<size_t>(r) * d.out_w, d.in_w, d.out_w, g.total_chunks);
+                MfmaTableEntry e = matvec_mfma_entry(d.ggml_type, d.x + static_cast<size_t>(r) * d.in_w, d.w, d.bias,
+                                                     d.y + static_cast<size_t>(r) * d.out_w, d.in_w, d.out_w, g.total_chunks);
+                e.rows = d.rows - r < share ? d.rows - r : share;
                 memcpy(&out[n++], &e, sizeof(e));
                 g.total_chunks += e.tiles;
             }
@@ -1359,13 +1370,14 @@ long build_batch(const nnhip_matvec_desc* descs, int count, BatchEntry* out, siz
         groups[(*ngroups)++] = g;
     }
     auto taken = [&](const nnhip_matvec_desc& d) {
+        const int form = form_of(d);
         for (int k = 0; k < *ngroups; ++k)
-            if (groups[k].mfma && groups[k].type == d.ggml_type && groups[k].max_in_w == d.in_w && mfma_ok(d)) return true;
+            if (groups[k].mfma && groups[k].mfma == form && groups[k].type == d.ggml_type && groups[k].max_in_w == d.in_w) return true;
         return false;
     };
     const int mfma_groups = *ngroups;
     for (uint32_t type : kBatchTypeOrder) {
-        BatchGroup g{type, n, n, 0, 0, false};
+        BatchGroup g{type, n, n, 0, 0, 0};
         int max_t = 0, depth = 0;
         shape_of(type, &max_t, &depth);
         int elems = 0, bytes = 0;
@@ -1413,8 +1425,10 @@ hipError_t launch_batch_groups(Lane* lane, const void* device_table, const Batch
         const BatchEntry* t = reinterpret_cast<const BatchEntry*>(device_table) + g.begin;
         hipError_t e = hipSuccess;
         if (g.mfma) {
-            e = launch_matvec_mfma_table(lane, g.type, g.max_in_w, reinterpret_cast<const MfmaTableEntry*>(t),
-                                         static_cast<int>(g.end - g.begin), g.total_chunks);
+            const MfmaTableEntry* mt = reinterpret_cast<const MfmaTableEntry*>(t);
+            const int entries = static_cast<int>(g.end - g.begin);
+            e = g.mfma == 1 ? launch_matvec_mfma_table(lane, g.type, g.max_in_w, mt, entries, g.total_chunks)
+                            : launch_matvec_mfma_wide_table(lane, g.type, g.max_in_w, g.mfma == 3 ? 4 : 1, mt, entries, g.total_chunks);
             if (e != hipSuccess) return e;
             lane->counters.kernel_launches += 1;
             continue;
@@ -1483,6 +1497,12 @@ hipError_t launch_matvec_batch(Lane* lane, const nnhip_matvec_desc* descs, int c
         }
     }
     return launch_batch_groups(lane, lane->batch_table, groups, ngroups, descs, count);
+}
+
+bool matvec_rows_share_pass(uint32_t type, int rows, int in_w, int out_w, const void* w)
+{
+    return rows >= 2 && rows <= 16 && static_cast<long>(rows) * ((out_w + 15) / 16) >= kMfmaBatchMinTiles &&
+           matvec_mfma_wide_geometry(type, in_w, out_w, w, 4);
 }
 
 hipError_t static_table_address(void** address)

@@ -30,6 +30,7 @@
 // on the storage type and in_w only, and a launch is a table of matrices that share both, worked through as one sequence
 // of tiles dealt round-robin to the workgroups: a row's bits depend on its weights, in_w and the activation vector, never
 // on out_w, on the other matrices of the launch or on its place in it.
+#include <cstddef>
 #include <cstring>
 #include <type_traits>
 
@@ -167,6 +168,7 @@ struct Q4KTask {
     static constexpr int kBlockBytes = kQ4KBytes;     // 144 = 9 pieces; blocks and rows are 16-byte aligned
     static constexpr int kPieces = 9;                 // 16-byte pieces a block takes in a stage
     static constexpr int kSumRun = 32;                // activations per FP32 sum (one sub-block)
+    static constexpr int kWideLpw = 3;                // 1 KB pieces per wave and stage in the wide form (W <= 12)
     using X = XSet<2>;
     struct Raw { u32x4 h, q1, q2; };
 
@@ -223,6 +225,7 @@ struct Q5KTask {
     static constexpr int kBlockBytes = kQ5KBytes;
     static constexpr int kPieces = 11;
     static constexpr int kSumRun = 32;
+    static constexpr int kWideLpw = 3;
     using X = XSet<2>;
     struct Raw { u32x4 h, ha, hb, q1, q2; };
 
@@ -281,6 +284,7 @@ struct Q6KTask {
     static constexpr int kBlockBytes = kQ6KBytes;
     static constexpr int kPieces = 14;
     static constexpr int kSumRun = 16;
+    static constexpr int kWideLpw = 4;
     using X = XSet<4>;
     struct Raw { u32x4 la, lb, ha, hb; u32x2 sc; uint32_t d; };
 
@@ -649,6 +653,330 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_kernel(MfmaArgs a)
     if (done) finalize();
 }
 
+
+// ---------------------------------------------------------------------------------------------------- the wide form
+// The same mat-vec for rows that do not split into one or two whole stages (17408 = 68 super-blocks) and for calls
+// with 2 - 4 input rows that share one pass over the weights: the digit planes of the activations stay in LDS for as
+// long as the vector is the same and a lane reads its 64 bytes of operand A for every task (instead of keeping them in
+// registers), a tile takes ceil(nblocks / W) stages of W block columns, the last one partly empty, and a task multiplies
+// the unpacked quants with the operand A of every input row of the entry.  Rows, planes and results of input row r of
+// an entry are x + r * in_w, the r-th plane set and y + r * out_w.
+struct WideGeom {
+    int waves;            // W (even: block parity is wave parity)
+    int kchunks;          // stages per tile = ceil(nblocks / W)
+    int tail_cols;        // block columns of a tile's last stage
+    int row_pieces;       // LDS row stride of a stage in 16-byte pieces (odd)
+    int stage_bytes;
+    int plane_stride;     // bytes of one digit plane (in_w + 16)
+    int set_bytes;        // four planes and the sums of one input row
+    size_t lds_bytes;     // two stage buffers and R plane sets
+};
+
+struct WideArgs {
+    const MfmaEntry* table;        // device table, or null: the entries are `inline_entries` below
+    int entries;
+    int total_tiles;
+    int in_w;
+    int nblocks;
+    uint32_t row_bytes;
+    uint32_t row_pieces_magic;
+    WideGeom g;
+    MfmaEntry inline_entries[4];   // a call with up to 16 input rows needs no table in device memory
+};
+
+template <class F, int LPW, int R>
+__global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideArgs a)
+{
+    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+    __shared__ float part[2][R][kMaxWaves][kTileRows];
+    __shared__ uint32_t red[R][kMaxWaves];
+
+    const WideGeom& g = a.g;
+    const int tid = threadIdx.x, lane = tid & 63, T = blockDim.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int W = g.waves, KC = g.kchunks;
+    const int row_l = lane & 15, quarter = lane >> 4;
+
+    // (the kernel's only argument starts the kernel-argument segment, which is constant memory like the table)
+    const NNHIP_CONST_PTR MfmaEntry* table =
+        a.table ? (const NNHIP_CONST_PTR MfmaEntry*)a.table
+                : (const NNHIP_CONST_PTR MfmaEntry*)((const NNHIP_CONST_PTR char*)__builtin_amdgcn_kernarg_segment_ptr() +
+                                                     offsetof(WideArgs, inline_entries));
+    auto entry_at = [&](int m) {
+        const NNHIP_CONST_PTR MfmaEntry& t = table[m];
+        MfmaEntry e;
+        e.x = t.x;
+        e.w = t.w;
+        e.bias = t.bias;
+        e.y = t.y;
+        e.out_w = t.out_w;
+        e.w_bytes = t.w_bytes;
+        e.tiles = t.tiles;
+        e.first_tile = t.first_tile;
+        e.rows = t.rows;
+        return e;
+    };
+
+    // this lane's pieces of a stage, as in the kernel above; rel_tail: the same for a tile's last stage, where the block
+    // columns past the row's end fetch nothing
+    uint32_t rel[LPW], rel_tail[LPW];
+#pragma unroll
+    for (int i = 0; i < LPW; ++i) {
+        const uint32_t slot = static_cast<uint32_t>(64 * (wave + W * i) + lane);
+        const uint32_t r = __umulhi(slot, a.row_pieces_magic);
+        const uint32_t q = slot - r * static_cast<uint32_t>(g.row_pieces);
+        const uint32_t c = q / static_cast<uint32_t>(F::kPieces);
+        const bool real = r < static_cast<uint32_t>(kTileRows) && c < static_cast<uint32_t>(W);
+        rel[i] = real ? r * a.row_bytes + c * F::kBlockBytes + F::piece_src(q - c * F::kPieces, c & 1u) : kNoPiece;
+        rel_tail[i] = c < static_cast<uint32_t>(g.tail_cols) ? rel[i] : kNoPiece;
+    }
+
+    const int G = gridDim.x;
+    const int my_tiles = (a.total_tiles - static_cast<int>(blockIdx.x) + G - 1) / G;
+    const int total = my_tiles * KC;
+    const uint32_t chunk_bytes = static_cast<uint32_t>(W) * F::kBlockBytes;
+    const int n4 = a.in_w >> 2;
+
+    // ---- prefetch side
+    int f_t = blockIdx.x, f_k = 0, f_m = 0;
+    MfmaEntry fe = entry_at(0);
+    __amdgpu_buffer_rsrc_t f_matrix;
+    auto fetch_enter = [&]() {
+        while (f_t >= fe.first_tile + fe.tiles && f_m + 1 < a.entries) fe = entry_at(++f_m);
+        f_matrix = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(fe.w), 0, static_cast<int>(fe.w_bytes), 0x00020000);
+    };
+    auto fetch = [&](u32x4 (&set)[LPW]) {
+        const uint32_t base = f_t < a.total_tiles
+            ? static_cast<uint32_t>(f_t - fe.first_tile) * kTileRows * a.row_bytes + static_cast<uint32_t>(f_k) * chunk_bytes
+            : kNoPiece;
+        const bool tail = f_k == KC - 1;
+#pragma unroll
+        for (int i = 0; i < LPW; ++i) set[i] = stream16(f_matrix, base + (tail ? rel_tail[i] : rel[i]));
+        if (++f_k == KC) {
+            f_k = 0;
+            f_t += G;
+            if (f_t < a.total_tiles && f_t >= fe.first_tile + fe.tiles) fetch_enter();
+        }
+    };
+    auto park = [&](uint8_t* buf, const u32x4 (&set)[LPW]) {
+        uint8_t* dst = buf + wave * 1024 + lane * 16;
+#pragma unroll
+        for (int i = 0; i < LPW; ++i) *reinterpret_cast<u32x4*>(dst + W * i * 1024) = set[i];
+    };
+
+    // ---- consume side
+    uint8_t* const buf0 = smem;
+    uint8_t* const buf1 = smem + g.stage_bytes;
+    uint8_t* const planes = smem + 2 * g.stage_bytes;
+    int c_t = blockIdx.x, c_k = 0, c_m = -1;
+    MfmaEntry ce{};
+    float inv[R] = {};
+    const float* planes_x = nullptr;       // the vector(s) the planes in LDS were made from
+    int planes_rows = 0;
+    const bool diag = (row_l >> 2) == quarter;
+
+    // Turns the activations of matrix c_m (its `rows` input rows) into digit planes and sums in LDS; two barriers.
+    // Every wave has left the stage that last read the planes when this runs.  When the rows fit kPrep float4 per lane
+    // they are all requested at once (one trip to memory); longer ones are read twice, row by row.
+    constexpr int kPrep = (LPW > 3 && R > 1) ? 4 : 8;     // (the Q6_K form with shared passes has the fewest registers to spare)
+    auto prepare_x = [&]() {
+        auto umax4 = [](uint32_t m, const float4& v) {
+            m = umax_u(m, __float_as_uint(v.x) & 0x7fffffffu);
+            m = umax_u(m, __float_as_uint(v.y) & 0x7fffffffu);
+            m = umax_u(m, __float_as_uint(v.z) & 0x7fffffffu);
+            return umax_u(m, __float_as_uint(v.w) & 0x7fffffffu);
+        };
+        auto scale_of = [&](int r, float& scale) {          // after the barrier that publishes red[r][]
+            uint32_t mx = 0;
+            for (int i = 0; i < W; ++i) mx = umax_u(mx, red[r][i]);
+            // |x| < 2^(E - 126) for the biased exponent E of the largest magnitude; e = 156 - E puts it below 2^30
+            const int E = static_cast<int>(mx >> 23);
+            int e = 156 - E;
+            e = e > 126 ? 126 : e;
+            scale = __uint_as_float(static_cast<uint32_t>(e + 127) << 23);
+            // a NaN or an infinity among the activations makes every output of the row NaN
+            inv[r] = E == 255 ? __uint_as_float(0x7fc00000u) : __uint_as_float(static_cast<uint32_t>(127 - e) << 23);
+        };
+        auto to_planes = [&](int r, int i, const float4& v, float scale) {
+            uint8_t* set = planes + r * g.set_bytes;
+            float* sumx = reinterpret_cast<float*>(set + 4 * g.plane_stride);
+            uint32_t pl[4];
+            digit_planes(__float2int_rn(v.x * scale), __float2int_rn(v.y * scale), __float2int_rn(v.z * scale),
+                         __float2int_rn(v.w * scale), pl);
+#pragma unroll
+            for (int p = 0; p < 4; ++p) *reinterpret_cast<uint32_t*>(set + p * g.plane_stride + 4 * i) = pl[p];
+            float s = (v.x + v.y) + (v.z + v.w);
+            if (F::kSumRun == 32) {
+                s = oct_sum(s);
+                if ((i & 7) == 0) sumx[i >> 3] = s;
+            } else {
+                s += dpp_mov<0xB1>(s);
+                s += dpp_mov<0x4E>(s);
+                if ((i & 3) == 0) sumx[i >> 2] = s;
+            }
+        };
+        const int rows = ce.rows;
+        if (rows * n4 <= kPrep * T) {
+            // flat index f = r * n4 + i over the rows; a wave's 64 values of one round belong to one row (n4 % 64 == 0)
+            float4 xr[kPrep];
+            const float4* x4 = reinterpret_cast<const float4*>(ce.x);      // the rows are consecutive: x4[f]
+            auto row_of = [&](int j) {                                      // wave-uniform; -1 past the last row
+                const int f0 = (tid & ~63) + j * T;
+                const int r = R > 1 ? (f0 >= n4) + (f0 >= 2 * n4) + (f0 >= 3 * n4) : 0;
+                return f0 >= rows * n4 ? -1 : __builtin_amdgcn_readfirstlane(r);
+            };
+#pragma unroll
+            for (int j = 0; j < kPrep; ++j) xr[j] = x4[row_of(j) >= 0 ? tid + j * T : 0];
+            uint32_t mx[R] = {};
+#pragma unroll
+            for (int j = 0; j < kPrep; ++j) {
+                const int rj = row_of(j);
+                const uint32_t m = umax4(0u, xr[j]);
+#pragma unroll
+                for (int r = 0; r < R; ++r) mx[r] = rj == r ? umax_u(mx[r], m) : mx[r];
+            }
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                if (r < rows) {
+                    const uint32_t m = wave_umax(mx[r]);
+                    if (lane == 0) red[r][wave] = m;
+                }
+            }
+            __syncthreads();
+            float scale[R] = {};
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+                if (r < rows) scale_of(r, scale[r]);
+#pragma unroll
+            for (int j = 0; j < kPrep; ++j) {
+                const int rj = row_of(j);
+                if (rj >= 0) {
+                    float sc = scale[0];
+#pragma unroll
+                    for (int r = 1; r < R; ++r) sc = rj == r ? scale[r] : sc;
+                    to_planes(rj, tid + j * T - rj * n4, xr[j], sc);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                if (r < rows) {
+                    const float4* x4 = reinterpret_cast<const float4*>(ce.x + static_cast<size_t>(r) * a.in_w);
+                    uint32_t mx = 0;
+                    for (int i = tid; i < n4; i += T) mx = umax4(mx, x4[i]);
+                    mx = wave_umax(mx);
+                    if (lane == 0) red[r][wave] = mx;
+                }
+            }
+            __syncthreads();
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                if (r < rows) {
+                    float scale;
+                    scale_of(r, scale);
+                    const float4* x4 = reinterpret_cast<const float4*>(ce.x + static_cast<size_t>(r) * a.in_w);
+                    for (int i = tid; i < n4; i += T) to_planes(r, i, x4[i], scale);
+                }
+            }
+        }
+        planes_x = ce.x;
+        planes_rows = rows;
+        __syncthreads();
+    };
+
+    u32x4 regs[2][LPW];
+    fetch_enter();
+    fetch(regs[0]);
+    fetch(regs[1]);
+
+    const uint32_t row_off = static_cast<uint32_t>(row_l) * (static_cast<uint32_t>(g.row_pieces) * 16u) +
+                             static_cast<uint32_t>(wave) * (16u * F::kPieces);
+    int pbuf = 0;
+    bool done = false;
+    float* done_y = nullptr;
+    const float* done_bias = nullptr;
+    int done_row0 = 0, done_rows = 0, done_out_w = 0, done_inputs = 0;
+    auto finalize = [&]() {
+        if (tid < kTileRows * R) {
+            const int r = tid >> 4, j0 = tid & 15;
+            if (r < done_inputs) {
+                float t = 0.0f;
+                for (int w2 = 0; w2 < W; ++w2) t += part[pbuf ^ 1][r][w2][j0];
+                if (done_bias) {
+                    const NNHIP_CONST_PTR float* cb = (const NNHIP_CONST_PTR float*)done_bias + done_row0;
+                    float bv = 0.0f;
+#pragma unroll
+                    for (int j = 0; j < kTileRows; ++j) {
+                        const float v = cb[j < done_rows ? j : 0];
+                        bv = j0 == j ? v : bv;
+                    }
+                    t += bv;
+                }
+                if (j0 < done_rows) done_y[static_cast<size_t>(r) * done_out_w + done_row0 + j0] = t;
+            }
+        }
+        done = false;
+    };
+
+    float accq[R], accm[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) accq[r] = accm[r] = 0.0f;
+    auto stage_step = [&](uint8_t* cur, uint8_t* nxt, u32x4 (&refill)[LPW], const u32x4 (&landing)[LPW]) {
+        bool new_x = false;
+        if (c_k == 0 && c_t >= ce.first_tile + ce.tiles) {
+            while (c_t >= ce.first_tile + ce.tiles) ce = entry_at(++c_m);
+            new_x = ce.x != planes_x || ce.rows != planes_rows;
+        }
+        fetch(refill);
+        if (new_x) prepare_x();
+        if (done) finalize();
+        const int b = c_k * W + wave;                    // this wave's block column of the row
+        if (b < a.nblocks) {
+            const typename F::Raw raw = F::load(cur + row_off, quarter, (wave & 1) != 0);
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                if (r < ce.rows) {
+                    const uint8_t* set = planes + r * g.set_bytes;
+                    typename F::X xs;
+                    F::load_x(xs, set + (row_l & 3) * g.plane_stride, reinterpret_cast<const float*>(set + 4 * g.plane_stride), b,
+                              quarter, diag);
+                    F::run(raw, xs, quarter, accq[r], accm[r]);
+                }
+            }
+        }
+        if (++c_k == KC) {
+            c_k = 0;
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                float p = fmaf(accq[r], inv[r], -accm[r]);
+                p = quarter_sum(p);
+                if (lane < kTileRows) part[pbuf][r][wave][lane] = p;
+                accq[r] = 0.0f;
+                accm[r] = 0.0f;
+            }
+            done = true;
+            done_y = ce.y;
+            done_bias = ce.bias;
+            done_out_w = ce.out_w;
+            done_inputs = ce.rows;
+            done_row0 = (c_t - ce.first_tile) * kTileRows;
+            done_rows = ce.out_w - done_row0 < kTileRows ? ce.out_w - done_row0 : kTileRows;
+            pbuf ^= 1;
+            c_t += G;
+        }
+        park(nxt, landing);
+        __syncthreads();
+    };
+
+    park(buf0, regs[0]);
+    __syncthreads();
+    for (int n = 0; n < total; n += 2) {
+        stage_step(buf0, buf1, regs[0], regs[1]);
+        if (n + 1 < total) stage_step(buf1, buf0, regs[1], regs[0]);
+    }
+    if (done) finalize();
+}
+
 // The (KC, M, LPW) combinations the kernel is instantiated for.
 struct Variant { int kc, m, lpw; };
 constexpr Variant kVariants[] = {{1, 2, 5}, {1, 2, 6}, {2, 1, 3}, {1, 1, 3}, {2, 2, 5}, {2, 2, 6}, {1, 1, 2}, {2, 1, 2},
@@ -741,10 +1069,76 @@ int block_pieces_of(uint32_t type)
     }
 }
 
+
+int wide_lpw_of(uint32_t type)
+{
+    switch (type) {
+    case NNHIP_TYPE_Q4_K: return Q4KTask::kWideLpw;
+    case NNHIP_TYPE_Q5_K: return Q5KTask::kWideLpw;
+    case NNHIP_TYPE_Q6_K: return Q6KTask::kWideLpw;
+    default: return 0;
+    }
+}
+
+// W for the wide form: even, as many of the row's blocks per stage as two stage buffers beside the plane sets of
+// `inputs` rows leave room for: the most waves, weighted by the share of block slots a tile fills and by an even
+// split over the four SIMDs.
+bool plan_wide(uint32_t type, int in_w, int inputs, WideGeom* out)
+{
+    const int nblocks = in_w / 256, bp = block_pieces_of(type), lpw = wide_lpw_of(type);
+    if (!bp || nblocks < 4) return false;
+    WideGeom best{};
+    double best_score = -1.0;
+    for (int W = 12; W >= 4; W -= 2) {
+        if (W > nblocks + 1) continue;
+        WideGeom g{};
+        g.waves = W;
+        g.kchunks = (nblocks + W - 1) / W;
+        g.tail_cols = nblocks - (g.kchunks - 1) * W;
+        g.row_pieces = (W * bp) | 1;
+        const int loads = (kTileRows * g.row_pieces + 63) / 64;
+        if ((loads + W - 1) / W > lpw) continue;
+        g.stage_bytes = lpw * W * 1024;
+        g.plane_stride = in_w + 16;
+        g.set_bytes = (4 * g.plane_stride + (in_w / 16) * 4 + 15) / 16 * 16;
+        g.lds_bytes = 2 * static_cast<size_t>(g.stage_bytes) + static_cast<size_t>(inputs) * g.set_bytes;
+        if (g.lds_bytes + 8 * 1024 > static_cast<size_t>(160 * 1024)) continue;      // (8 KB: the static arrays)
+        const double fill = static_cast<double>(nblocks) / (g.kchunks * W);
+        // (throughput grows with the waves: a stage holds W blocks per row and W tasks run side by side)
+        const double score = fill * W / 12.0 * (W % 4 == 0 ? 1.0 : 0.95);
+        if (score > best_score) {
+            best_score = score;
+            best = g;
+        }
+    }
+    if (best_score < 0) return false;
+    *out = best;
+    return true;
+}
+
+template <class F, int R>
+hipError_t launch_wide_of(Lane* lane, const WideArgs& a)
+{
+    static LdsLimit big_lds;
+    const void* fn = reinterpret_cast<const void*>(&matvec_mfma_wide_kernel<F, F::kWideLpw, R>);
+    const hipError_t e = big_lds.ensure(lane->device, fn, 160 * 1024 - 8 * 1024);
+    if (e != hipSuccess) return e;
+    const int groups = a.total_tiles < lane->compute_units ? a.total_tiles : lane->compute_units;
+    hipLaunchKernelGGL((matvec_mfma_wide_kernel<F, F::kWideLpw, R>), dim3(groups), dim3(64 * a.g.waves), a.g.lds_bytes, lane->stream, a);
+    return hipGetLastError();
+}
+
+template <class F>
+hipError_t launch_wide(Lane* lane, const WideArgs& a, int inputs)
+{
+    return inputs == 1 ? launch_wide_of<F, 1>(lane, a) : launch_wide_of<F, 4>(lane, a);
+}
+
 bool entry_ok(uint32_t type, int in_w, int out_w, const void* w)
 {
     const int bb = block_bytes_of(type);
     if (!bb || in_w % 256 != 0 || (reinterpret_cast<uintptr_t>(w) & 15u)) return false;
+    if (bb % 16 != 0 && ((in_w / 256) & 1)) return false;      // (Q6_K: a row must end with an odd block, see piece_src)
     const uint64_t bytes = static_cast<uint64_t>(out_w) * (in_w / 256) * bb;
     return bytes < 0x7fffffffull;            // piece offsets are 32-bit and "no piece" is bit 31
 }
@@ -772,6 +1166,7 @@ MfmaTableEntry matvec_mfma_entry(uint32_t type, const float* x, const void* w, c
     e.w_bytes = static_cast<uint32_t>(out_w) * static_cast<uint32_t>(in_w / 256) * static_cast<uint32_t>(block_bytes_of(type));
     e.tiles = (out_w + kTileRows - 1) / kTileRows;
     e.first_tile = first_tile;
+    e.rows = 1;
     return e;
 }
 
@@ -808,6 +1203,57 @@ hipError_t launch_matvec_mfma_table(Lane* lane, uint32_t type, int in_w, const M
     case NNHIP_TYPE_Q6_K: return launch_mfma<Q6KTask>(lane, a);
     default: return hipErrorInvalidValue;
     }
+}
+
+bool matvec_mfma_wide_geometry(uint32_t type, int in_w, int out_w, const void* w, int inputs)
+{
+    WideGeom g;
+    return inputs >= 1 && inputs <= 4 && entry_ok(type, in_w, out_w, w) && plan_wide(type, in_w, inputs == 1 ? 1 : 4, &g);
+}
+
+namespace {
+
+hipError_t launch_wide_args(Lane* lane, uint32_t type, int in_w, int inputs, WideArgs& a)
+{
+    if (!plan_wide(type, in_w, inputs == 1 ? 1 : 4, &a.g)) return hipErrorInvalidValue;
+    a.in_w = in_w;
+    a.nblocks = in_w / 256;
+    a.row_bytes = static_cast<uint32_t>(a.nblocks) * static_cast<uint32_t>(block_bytes_of(type));
+    a.row_pieces_magic = static_cast<uint32_t>((0x100000000ull + a.g.row_pieces - 1) / a.g.row_pieces);
+    switch (type) {
+    case NNHIP_TYPE_Q4_K: return launch_wide<Q4KTask>(lane, a, inputs);
+    case NNHIP_TYPE_Q5_K: return launch_wide<Q5KTask>(lane, a, inputs);
+    case NNHIP_TYPE_Q6_K: return launch_wide<Q6KTask>(lane, a, inputs);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace
+
+hipError_t launch_matvec_mfma_wide_table(Lane* lane, uint32_t type, int in_w, int inputs, const MfmaTableEntry* device_entries,
+                                         int entries, int total_tiles)
+{
+    WideArgs a{};
+    a.table = device_entries;
+    a.entries = entries;
+    a.total_tiles = total_tiles;
+    return launch_wide_args(lane, type, in_w, inputs, a);
+}
+
+hipError_t launch_matvec_rows_shared(Lane* lane, uint32_t type, const float* x, const void* w, const float* bias, float* y,
+                                     int rows, int in_w, int out_w)
+{
+    if (rows < 2 || rows > 16) return hipErrorInvalidValue;
+    WideArgs a{};
+    a.table = nullptr;
+    for (int r = 0; r < rows; r += 4) {
+        MfmaTableEntry e = matvec_mfma_entry(type, x + static_cast<size_t>(r) * in_w, w, bias, y + static_cast<size_t>(r) * out_w,
+                                             in_w, out_w, a.total_tiles);
+        e.rows = rows - r < 4 ? rows - r : 4;
+        a.inline_entries[a.entries++] = e;
+        a.total_tiles += e.tiles;
+    }
+    return launch_wide_args(lane, type, in_w, 4, a);
 }
 
 }  // namespace nnhip

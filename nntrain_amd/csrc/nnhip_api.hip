@@ -204,6 +204,15 @@ int nnhip_lane_create(int device, void** out)
         delete lane;
         return hip_fail(e, NNHIP_OP_LANE_CREATE, device, "hipGetSymbolAddress of the fixed batch workspace");
     }
+    // the descriptor table of batched launches starts with room for 819 mat-vec rows, so that small batches (and calls
+    // with a few input rows, which use it) never have to grow it inside a graph capture
+    e = hipMalloc(&lane->batch_table, 65536);
+    if (e != hipSuccess) {
+        (void)hipStreamDestroy(lane->stream);
+        delete lane;
+        return hip_fail(e, NNHIP_OP_LANE_CREATE, device, "hipMalloc of the batch descriptor table");
+    }
+    lane->batch_table_bytes = 65536;
     *out = lane;
     return NNHIP_OK;
 }
@@ -431,6 +440,14 @@ int nnhip_quant_matvec(void* handle, uint32_t ggml_type, const float* x, const v
     if (in_w > matvec_max_in_w(ggml_type))
         return fail(NNHIP_ERR_TOO_LARGE, NNHIP_OP_MATVEC, lane->device, 0, "in_w %d exceeds the %d values one workgroup can stage", in_w, matvec_max_in_w(ggml_type));
     if (rows > 65535) return fail(NNHIP_ERR_TOO_LARGE, NNHIP_OP_MATVEC, lane->device, 0, "rows %d exceeds 65535", rows);
+    if (matvec_rows_share_pass(ggml_type, rows, in_w, out_w, w)) {
+        // 2 - 15 input rows of a K-quant matrix: up to four rows share a pass over the weights on the matrix cores
+        // (the reference routes such calls to row-tiled kernels, Qwen35QuantizedModel.cs:1335-1344)
+        const hipError_t e = launch_matvec_rows_shared(lane, ggml_type, x, w, bias, y, rows, in_w, out_w);
+        if (e != hipSuccess) return hip_fail(e, NNHIP_OP_MATVEC, lane->device, "mat-vec launch");
+        lane->counters.kernel_launches += 1;
+        return NNHIP_OK;
+    }
     hipError_t e = launch_matvec(lane, ggml_type, x, w, bias, y, rows, in_w, out_w);
     if (e != hipSuccess) return hip_fail(e, NNHIP_OP_MATVEC, lane->device, "mat-vec launch");
     lane->counters.kernel_launches += 1;

@@ -96,13 +96,25 @@ struct MfmaTableEntry {
     uint32_t w_bytes;       // whole matrix (< 2 GB)
     int tiles;              // ceil(out_w / 16)
     int first_tile;         // position of the matrix' first tile in the launch's tile sequence
-    uint32_t pad_[8];
+    int rows;               // input rows that share the pass (wide form: 1 - 4; x, y advance by in_w, out_w per row)
+    uint32_t pad_[7];
 };
 static_assert(sizeof(MfmaTableEntry) == 80, "table slots are 80 bytes");
 MfmaTableEntry matvec_mfma_entry(uint32_t type, const float* x, const void* w, const float* bias, float* y, int in_w,
                                  int out_w, int first_tile);
 hipError_t launch_matvec_mfma_table(Lane* lane, uint32_t type, int in_w, const MfmaTableEntry* device_entries, int entries,
                                     int total_tiles);
+// The wide form of the matrix-core mat-vec (activation planes in LDS): any in_w of at least four super-blocks, and
+// entries of up to four input rows that share a pass over the weights (`inputs` = 1: every entry has one row).
+bool matvec_mfma_wide_geometry(uint32_t type, int in_w, int out_w, const void* w, int inputs);
+// True when a single call with `rows` input rows is served by that form (as a one-descriptor batch) rather than by one
+// row-step pass per input row.
+bool matvec_rows_share_pass(uint32_t type, int rows, int in_w, int out_w, const void* w);
+// That call: 2 - 16 input rows, up to four per pass, the descriptors travelling in the kernel arguments.
+hipError_t launch_matvec_rows_shared(Lane* lane, uint32_t type, const float* x, const void* w, const float* bias, float* y,
+                                     int rows, int in_w, int out_w);
+hipError_t launch_matvec_mfma_wide_table(Lane* lane, uint32_t type, int in_w, int inputs, const MfmaTableEntry* device_entries,
+                                         int entries, int total_tiles);
 // The fixed device workspace: its address on the current device, and the batched launch that uses it.
 hipError_t static_table_address(void** address);
 hipError_t launch_matvec_batch_static(Lane* lane, const nnhip_matvec_desc* descs, int count);

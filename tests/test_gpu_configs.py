@@ -433,3 +433,106 @@ def test_large_batched_group_special_activations(lane):
     wd.dispose()
     bd.dispose()
     lane.trim()
+
+
+@pytest.mark.parametrize("typ", [GGML_Q4_K, GGML_Q5_K, GGML_Q6_K])
+def test_matrix_core_groups_with_long_rows_and_shared_passes(lane, typ):
+    """Rows that do not split into whole stages (17408 = 68 super-blocks, 3072 = 12, 1024 = 4) and descriptors with
+    2 - 5 input rows (up to four share a pass over the weights) take the form of the matrix-core mat-vec that keeps the
+    activation planes in LDS: both bars against the float64 oracle, bias, ragged row counts, guard elements, and per-row
+    bits that do not depend on how many input rows travel together."""
+    rng = np.random.default_rng(100 + typ)
+    shapes = [(17408, 5120, 1, True), (17408, 5120 + 7, 1, False), (17408, 30000, 1, False),      # wide, one row each
+              (3072, 40000, 1, True), (1024, 33000, 1, False),
+              (5120, 17408, 4, True), (5120, 9000 + 3, 5, False), (5120, 4096, 2, False),           # shared passes
+              (17408, 5120, 3, False)]
+    items = []
+    for i, (in_w, out_w, rows, bias) in enumerate(shapes):
+        payload = synth.matrix(typ, out_w, in_w, seed=300 * typ + i)
+        xh = rng.standard_normal((rows, in_w)).astype(np.float32)
+        xh[:, ::7] *= 0.01
+        if rows > 1:
+            xh[1] *= 300.0                       # every input row has its own fixed-point scale
+        bh = rng.standard_normal(out_w).astype(np.float32) if bias else None
+        items.append(dict(typ=typ, in_w=in_w, out_w=out_w, rows=rows, payload=payload, x=xh, xd=lane.upload_raw(xh), bias=bh,
+                          wd=lane.upload_raw(payload), bd=lane.upload_raw(bh) if bias else None,
+                          yd=lane.allocate(rows * out_w + 2)))
+    got = _batch_run(lane, items)
+    for it, y in zip(items, got):
+        assert np.all(np.isfinite(y)), (it["in_w"], it["out_w"], it["rows"])
+        ref, asum = oracle.linear_f64(typ, it["payload"], it["x"], it["bias"], it["rows"], it["in_w"], it["out_w"])
+        assert oracle.rel_l2(y, ref) <= MATVEC_BAR, (it["in_w"], it["out_w"], it["rows"])
+        assert np.all(np.abs(y.astype(np.float64) - ref) <= 2e-6 + 3e-6 * asum), (it["in_w"], it["out_w"], it["rows"])
+    # rows 0-3 of the five-row descriptor travelled together, row 4 alone: the same call with the rows as five descriptors
+    # of two rows (overlapping pairs) must give every row the same bits
+    it = items[6]
+    pairs = []
+    for r in range(4):
+        pairs.append(dict(typ=typ, in_w=it["in_w"], out_w=it["out_w"], rows=2, xd=it["xd"].view(4 * r * it["in_w"], 8 * it["in_w"]),
+                          wd=it["wd"], bd=None, yd=lane.allocate(2 * it["out_w"] + 2)))
+    again = _batch_run(lane, pairs + [items[5]])
+    for r in range(4):
+        assert np.array_equal(_bits(again[r][0]), _bits(got[6][r])), r
+        assert np.array_equal(_bits(again[r][1]), _bits(got[6][r + 1])), r
+    assert np.array_equal(_bits(again[4]), _bits(got[5]))
+    for p in pairs:
+        p["yd"].dispose()
+    for it in items:
+        for key in ("xd", "wd", "bd", "yd"):
+            if it[key] is not None:
+                it[key].dispose()
+    lane.trim()
+
+
+@pytest.mark.parametrize("typ", [GGML_Q4_K, GGML_Q6_K])
+def test_several_input_rows_share_a_pass_in_a_single_call(lane, typ):
+    """nnhip_quant_matvec with 2 - 9 input rows on a K-quant matrix large enough for the matrix cores (rows x 16-row
+    tiles >= 2048): up to four rows share a pass over the weights.  Both bars against the oracle, the guard elements,
+    no transfers, and a row's bits do not depend on the rows it travels with; the same call inside a captured graph
+    gives the same bits on every replay."""
+    in_w, out_w = 5120, 17408
+    payload = synth.matrix(typ, out_w, in_w, seed=900 + typ)
+    mat = HipQuantizedMatrix(payload, typ, out_w, in_w)
+    mat.device_payload(lane)
+    bias = np.random.default_rng(2).standard_normal(out_w).astype(np.float32)
+    bd = lane.upload_raw(bias)
+    x = synth.activations(9, in_w, seed=31)
+    x[2] *= 1e-3
+    x[5] *= 4e3
+    xd = lane.upload_raw(x)
+    results = {}
+    for rows in (2, 4, 9):
+        yd = lane.allocate(rows * out_w + 2)
+        lane.fill_u32(yd, NAN_BITS, rows * out_w + 2)
+        before = lane.counters()
+        mat.forward(lane, xd, bd, rows, out=yd)
+        lane.synchronize()
+        after = lane.counters()
+        assert after["h2d_bytes"] == before["h2d_bytes"] and after["allocated_bytes"] == before["allocated_bytes"]
+        y = lane.read(yd)
+        assert np.isnan(y[-1]) and np.isnan(y[-2])
+        y = y[:-2].reshape(rows, out_w)
+        ref, asum = oracle.linear_f64(typ, payload, x[:rows], bias, rows, in_w, out_w)
+        assert oracle.rel_l2(y, ref) <= MATVEC_BAR
+        assert np.all(np.abs(y.astype(np.float64) - ref) <= 2e-6 + 3e-6 * asum)
+        results[rows] = y
+        yd.dispose()
+    assert np.array_equal(_bits(results[9][:4]), _bits(results[4]))
+    assert np.array_equal(_bits(results[4][:2]), _bits(results[2]))
+    # captured: the descriptor table write is recorded with the launch
+    yd = lane.allocate(4 * out_w)
+    lane.graph_begin()
+    mat.forward(lane, xd, bd, 4, out=yd)
+    graph = lane.graph_end()
+    for _ in range(3):
+        lane.fill_u32(yd, NAN_BITS, 4 * out_w)
+        mat.forward(lane, xd, None, 2)              # eager work between the replays uses the same table
+        lane.synchronize()
+        lane.graph_launch(graph)
+        lane.synchronize()
+        assert np.array_equal(_bits(lane.read(yd).reshape(4, out_w)), _bits(results[4]))
+    lane.graph_destroy(graph)
+    for b in (xd, bd, yd):
+        b.dispose()
+    mat.dispose()
+    lane.trim()
