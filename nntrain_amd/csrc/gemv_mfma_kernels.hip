@@ -37,6 +37,8 @@
 #include "nnhip_internal.h"
 #include "quant_device.h"
 
+#include "iq_grids.inc"
+
 namespace nnhip {
 
 namespace {
@@ -168,7 +170,12 @@ struct Q4KTask {
     static constexpr int kBlockBytes = kQ4KBytes;     // 144 = 9 pieces; blocks and rows are 16-byte aligned
     static constexpr int kPieces = 9;                 // 16-byte pieces a block takes in a stage
     static constexpr int kSumRun = 32;                // activations per FP32 sum (one sub-block)
-    static constexpr int kWideLpw = 3;                // 1 KB pieces per wave and stage in the wide form (W <= 12)
+    static constexpr int kWideM = 1;                  // wide form: block columns per wave and stage,
+    static constexpr int kWideLpw = 3;                // and 1 KB pieces per wave and stage (W <= 12)
+    static constexpr bool kNeedsSums = true;
+    static constexpr bool kTightStage = false;
+    static constexpr int kSharedM = kWideM, kSharedLpw = kWideLpw;      // the same with four input rows per pass
+    static __device__ __forceinline__ void init_tables(uint8_t*, int, int) {}
     using X = XSet<2>;
     struct Raw { u32x4 h, q1, q2; };
 
@@ -194,7 +201,7 @@ struct Q4KTask {
         return r;
     }
 
-    static __device__ __forceinline__ void run(const Raw& r, const X& xs, int quarter, float& accq, float& accm)
+    static __device__ __forceinline__ void run(const Raw& r, const X& xs, int quarter, const uint8_t*, float& accq, float& accm)
     {
         constexpr uint32_t kLow = 0x0f0f0f0fu;
         const u32x4 q1 = r.q1, q2 = r.q2, h = r.h;
@@ -225,7 +232,12 @@ struct Q5KTask {
     static constexpr int kBlockBytes = kQ5KBytes;
     static constexpr int kPieces = 11;
     static constexpr int kSumRun = 32;
+    static constexpr int kWideM = 1;
     static constexpr int kWideLpw = 3;
+    static constexpr bool kNeedsSums = true;
+    static constexpr bool kTightStage = false;
+    static constexpr int kSharedM = kWideM, kSharedLpw = kWideLpw;      // the same with four input rows per pass
+    static __device__ __forceinline__ void init_tables(uint8_t*, int, int) {}
     using X = XSet<2>;
     struct Raw { u32x4 h, ha, hb, q1, q2; };
 
@@ -247,7 +259,7 @@ struct Q5KTask {
         return r;
     }
 
-    static __device__ __forceinline__ void run(const Raw& r, const X& xs, int quarter, float& accq, float& accm)
+    static __device__ __forceinline__ void run(const Raw& r, const X& xs, int quarter, const uint8_t*, float& accq, float& accm)
     {
         constexpr uint32_t kLow = 0x0f0f0f0fu, kBit4 = 0x10101010u;
         const u32x4 h = r.h, ha = r.ha, hb = r.hb, q1 = r.q1, q2 = r.q2;
@@ -284,7 +296,12 @@ struct Q6KTask {
     static constexpr int kBlockBytes = kQ6KBytes;
     static constexpr int kPieces = 14;
     static constexpr int kSumRun = 16;
+    static constexpr int kWideM = 1;
     static constexpr int kWideLpw = 4;
+    static constexpr bool kNeedsSums = true;
+    static constexpr bool kTightStage = false;
+    static constexpr int kSharedM = kWideM, kSharedLpw = kWideLpw;      // the same with four input rows per pass
+    static __device__ __forceinline__ void init_tables(uint8_t*, int, int) {}
     using X = XSet<4>;
     struct Raw { u32x4 la, lb, ha, hb; u32x2 sc; uint32_t d; };
 
@@ -346,7 +363,7 @@ struct Q6KTask {
         return r;
     }
 
-    static __device__ __forceinline__ void run(const Raw& r, const X& xs, int quarter, float& accq, float& accm)
+    static __device__ __forceinline__ void run(const Raw& r, const X& xs, int quarter, const uint8_t*, float& accq, float& accm)
     {
         constexpr uint32_t kLow = 0x0f0f0f0fu, kTop = 0x30303030u;
         const int sh = 2 * (quarter & 1);
@@ -372,6 +389,108 @@ struct Q6KTask {
         accq = fmaf(d * c3, recombine(s3), accq);
         const float t = fmaf(c0, xs.sx[0], fmaf(c1, xs.sx[1], fmaf(c2, xs.sx[2], c3 * xs.sx[3])));
         accm = fmaf(32.0f * d, t, accm);
+    }
+};
+
+// IQ2_S (NNtrain.Arc/Kernels/qwen35_iq.cl:411-419): 82 bytes = d (fp16), 32 index bytes, 32 sign bytes, 8 bytes of index
+// tops (two bits per eight weights), 8 bytes of 4-bit scales (one per 16 weights).  Eight weights are one entry of a
+// 1024-entry codebook of magnitude bytes (8, 25 or 43) with a sign bit each; w = d * (0.5 + scale) * 0.25 * magnitude *
+// sign.  A codebook entry is exactly the eight bytes of operand B that a lane supplies for one MFMA; the signs go in as
+// (magnitude ^ mask) + (mask & 1) per byte, with the two masks of a sign byte read from a 256-entry table.  Both tables
+// sit in LDS (12 KB).  Quarter P = weights 64P .. 64P + 63 = 32-weight groups 2P and 2P + 1; four scale groups.
+// Blocks are 2-byte aligned: fetched from the dword boundary at or below their start into six pieces, so an odd block
+// sits 2 bytes into its pieces (and its index and sign bytes on dword boundaries, while those of an even block need a
+// 2-byte shift).
+__device__ const uint64_t g_iq2s_grid_mv[1024] = { NNHIP_IQ2S_GRID_VALUES };
+
+struct IQ2STask {
+    static constexpr int kBlockBytes = kIQ2SBytes;
+    static constexpr int kPieces = 6;
+    static constexpr int kSumRun = 32;
+    static constexpr int kWideM = 2;                  // (the blocks are small: two per wave make a stage worth its barrier;
+    static constexpr int kWideLpw = 4;                //  one where four input rows share a pass: registers)
+    static constexpr int kSharedM = 1;
+    static constexpr int kSharedLpw = 2;
+    static constexpr bool kNeedsSums = false;         // no minimum or offset
+    static constexpr bool kTightStage = true;         // 17408-wide planes leave no room for whole 1 KB slots per wave
+    static constexpr int kGridBytes = 8192;
+    static constexpr int kTableBytes = kGridBytes + 64;       // the codebook and 16 byte selectors
+    using X = XSet<1>;
+    struct Raw { uint32_t q[2], s[2], tops, scales, d; };
+
+    static __device__ __forceinline__ uint32_t piece_src(uint32_t q, bool odd) { return 16u * q - (odd ? 2u : 0u); }
+
+    static __device__ __forceinline__ void init_tables(uint8_t* t, int tid, int threads)
+    {
+        for (int i = tid; i < 1024; i += threads) reinterpret_cast<uint64_t*>(t)[i] = g_iq2s_grid_mv[i];
+        if (tid < 16) {
+            // four sign bits -> a v_perm_b32 selector: byte k of the result comes from the magnitudes (selector byte k) or
+            // from their negation (selector byte 4 + k); the 64-byte table is read without bank conflicts
+            const uint32_t spread = (static_cast<uint32_t>(tid) * 0x00204081u) & 0x01010101u;
+            reinterpret_cast<uint32_t*>(t + kGridBytes)[tid] = 0x03020100u + (spread << 2);
+        }
+    }
+
+    static __device__ __forceinline__ void load_x(X& xs, const uint8_t* plane, const float*, int b, int quarter, bool diag)
+    {
+        const uint8_t* src = plane + 256 * b + 64 * quarter;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) xs.a[u] = diag ? lds128(src + 16 * u) : u32x4{0u, 0u, 0u, 0u};
+        xs.sx[0] = 0.0f;
+    }
+
+    static __device__ __forceinline__ Raw load(const uint8_t* blk, int quarter, bool odd)
+    {
+        // the block's byte k is at blk + k (+ 2 when odd); its index bytes 8P .. 8P + 7 start at 2 + 8P, the sign bytes 32 later
+        const uint32_t* base = reinterpret_cast<const uint32_t*>(blk + 8 * quarter + (odd ? 4 : 0));
+        const uint32_t sh = odd ? 0u : 2u;
+        const uint8_t* b0 = blk + (odd ? 2 : 0);
+        Raw r;
+        const uint32_t q0 = base[0], q1 = base[1], q2 = base[2];
+        const uint32_t s0 = base[8], s1 = base[9], s2 = base[10];
+        r.q[0] = __builtin_amdgcn_alignbyte(q1, q0, sh);
+        r.q[1] = __builtin_amdgcn_alignbyte(q2, q1, sh);
+        r.s[0] = __builtin_amdgcn_alignbyte(s1, s0, sh);
+        r.s[1] = __builtin_amdgcn_alignbyte(s2, s1, sh);
+        r.tops = *reinterpret_cast<const uint16_t*>(b0 + 66 + 2 * quarter);
+        r.scales = *reinterpret_cast<const uint16_t*>(b0 + 74 + 2 * quarter);
+        r.d = *reinterpret_cast<const uint16_t*>(b0);
+        return r;
+    }
+
+    static __device__ __forceinline__ void run(const Raw& r, const X& xs, int, const uint8_t* tables, float& accq, float&)
+    {
+        // every lookup of the task is requested before the first result is used (the scheduling barrier keeps the
+        // compiler from folding the reads back into a chain of eight round trips to LDS)
+        const uint32_t* selectors = reinterpret_cast<const uint32_t*>(tables + kGridBytes);
+        u32x2 mag[8];
+        uint32_t sel[8][2];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const int g = e >> 2, o = e & 3;                                  // 32-weight group of the quarter, entry in it
+            const uint32_t index = ((r.q[g] >> (8 * o)) & 0xffu) | (((r.tops >> (8 * g + 2 * o)) & 3u) << 8);
+            const uint32_t sign = r.s[g] >> (8 * o);
+            mag[e] = *reinterpret_cast<const u32x2*>(tables + 8u * index);
+            sel[e][0] = selectors[sign & 15u];
+            sel[e][1] = selectors[(sign >> 4) & 15u];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        i32x4 acc[4] = {{0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}};
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            // -m per byte = (m ^ 0xff) + 1: no carry leaves a byte because no magnitude is zero
+            const uint32_t neg0 = (mag[e][0] ^ 0xffffffffu) + 0x01010101u, neg1 = (mag[e][1] ^ 0xffffffffu) + 0x01010101u;
+            const uint32_t b0 = __builtin_amdgcn_perm(neg0, mag[e][0], sel[e][0]), b1 = __builtin_amdgcn_perm(neg1, mag[e][1], sel[e][1]);
+            const u32x4 av = xs.a[e >> 1];
+            acc[e >> 1] = mfma_i8(av[2 * (e & 1)], av[2 * (e & 1) + 1], b0, b1, acc[e >> 1]);
+        }
+        const float d = half_bits_to_float(r.d);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            // scale group k of the quarter: nibble (k & 1) of scale byte k >> 1
+            const float sc = static_cast<float>((r.scales >> (4 * k)) & 15u);
+            accq = fmaf((d * (0.5f + sc)) * 0.25f, recombine(acc[k]), accq);
+        }
     }
 };
 
@@ -624,7 +743,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_kernel(MfmaArgs a)
 #pragma unroll
         for (int t = 0; t < M; ++t) raw[t] = F::load(stage + t * W * (16 * F::kPieces), quarter, (wave & 1) != 0);
 #pragma unroll
-        for (int t = 0; t < M; ++t) F::run(raw[t], xs[k * M + t], quarter, accq, accm);
+        for (int t = 0; t < M; ++t) F::run(raw[t], xs[k * M + t], quarter, nullptr, accq, accm);
         if (k == KC - 1) {
             float p = fmaf(accq, inv, -accm);
             p = quarter_sum(p);
@@ -663,7 +782,8 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_kernel(MfmaArgs a)
 // an entry are x + r * in_w, the r-th plane set and y + r * out_w.
 struct WideGeom {
     int waves;            // W (even: block parity is wave parity)
-    int kchunks;          // stages per tile = ceil(nblocks / W)
+    int cols;             // block columns per stage = W * M
+    int kchunks;          // stages per tile = ceil(nblocks / cols)
     int tail_cols;        // block columns of a tile's last stage
     int row_pieces;       // LDS row stride of a stage in 16-byte pieces (odd)
     int stage_bytes;
@@ -684,7 +804,7 @@ struct WideArgs {
     MfmaEntry inline_entries[4];   // a call with up to 16 input rows needs no table in device memory
 };
 
-template <class F, int LPW, int R>
+template <class F, int M, int LPW, int R>
 __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideArgs a)
 {
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
@@ -720,21 +840,23 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
     // this lane's pieces of a stage, as in the kernel above; rel_tail: the same for a tile's last stage, where the block
     // columns past the row's end fetch nothing
     uint32_t rel[LPW], rel_tail[LPW];
+    uint32_t in_stage = 0;                 // bit i: this lane's piece i lies inside the stage buffer
 #pragma unroll
     for (int i = 0; i < LPW; ++i) {
         const uint32_t slot = static_cast<uint32_t>(64 * (wave + W * i) + lane);
         const uint32_t r = __umulhi(slot, a.row_pieces_magic);
         const uint32_t q = slot - r * static_cast<uint32_t>(g.row_pieces);
         const uint32_t c = q / static_cast<uint32_t>(F::kPieces);
-        const bool real = r < static_cast<uint32_t>(kTileRows) && c < static_cast<uint32_t>(W);
+        const bool real = r < static_cast<uint32_t>(kTileRows) && c < static_cast<uint32_t>(g.cols);
         rel[i] = real ? r * a.row_bytes + c * F::kBlockBytes + F::piece_src(q - c * F::kPieces, c & 1u) : kNoPiece;
         rel_tail[i] = c < static_cast<uint32_t>(g.tail_cols) ? rel[i] : kNoPiece;
+        in_stage |= (r < static_cast<uint32_t>(kTileRows) ? 1u : 0u) << i;
     }
 
     const int G = gridDim.x;
     const int my_tiles = (a.total_tiles - static_cast<int>(blockIdx.x) + G - 1) / G;
     const int total = my_tiles * KC;
-    const uint32_t chunk_bytes = static_cast<uint32_t>(W) * F::kBlockBytes;
+    const uint32_t chunk_bytes = static_cast<uint32_t>(g.cols) * F::kBlockBytes;
     const int n4 = a.in_w >> 2;
 
     // ---- prefetch side
@@ -759,15 +881,19 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
         }
     };
     auto park = [&](uint8_t* buf, const u32x4 (&set)[LPW]) {
+        // (where LDS is tight a stage buffer ends with the stage's last row and the slots behind it are not stored)
         uint8_t* dst = buf + wave * 1024 + lane * 16;
 #pragma unroll
-        for (int i = 0; i < LPW; ++i) *reinterpret_cast<u32x4*>(dst + W * i * 1024) = set[i];
+        for (int i = 0; i < LPW; ++i)
+            if (!F::kTightStage || ((in_stage >> i) & 1u)) *reinterpret_cast<u32x4*>(dst + W * i * 1024) = set[i];
     };
 
     // ---- consume side
     uint8_t* const buf0 = smem;
     uint8_t* const buf1 = smem + g.stage_bytes;
     uint8_t* const planes = smem + 2 * g.stage_bytes;
+    uint8_t* const tables = planes + R * g.set_bytes;      // the format's lookup tables (published by the first barrier)
+    F::init_tables(tables, tid, T);
     int c_t = blockIdx.x, c_k = 0, c_m = -1;
     MfmaEntry ce{};
     float inv[R] = {};
@@ -776,9 +902,9 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
     const bool diag = (row_l >> 2) == quarter;
 
     // Turns the activations of matrix c_m (its `rows` input rows) into digit planes and sums in LDS; two barriers.
-    // Every wave has left the stage that last read the planes when this runs.  When the rows fit kPrep float4 per lane
-    // they are all requested at once (one trip to memory); longer ones are read twice, row by row.
-    constexpr int kPrep = (LPW > 3 && R > 1) ? 4 : 8;     // (the Q6_K form with shared passes has the fewest registers to spare)
+    // Every wave has left the stage that last read the planes when this runs.  (A variant that requested all rows at once
+    // into registers, one trip to memory instead of two per row, made the compiler wait for every outstanding load
+    // before each parking write of the main loop: 12.6 instead of 8.6 us per 17408-wide Q4_K mat-vec.  Not kept.)
     auto prepare_x = [&]() {
         auto umax4 = [](uint32_t m, const float4& v) {
             m = umax_u(m, __float_as_uint(v.x) & 0x7fffffffu);
@@ -786,96 +912,51 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
             m = umax_u(m, __float_as_uint(v.z) & 0x7fffffffu);
             return umax_u(m, __float_as_uint(v.w) & 0x7fffffffu);
         };
-        auto scale_of = [&](int r, float& scale) {          // after the barrier that publishes red[r][]
-            uint32_t mx = 0;
-            for (int i = 0; i < W; ++i) mx = umax_u(mx, red[r][i]);
-            // |x| < 2^(E - 126) for the biased exponent E of the largest magnitude; e = 156 - E puts it below 2^30
-            const int E = static_cast<int>(mx >> 23);
-            int e = 156 - E;
-            e = e > 126 ? 126 : e;
-            scale = __uint_as_float(static_cast<uint32_t>(e + 127) << 23);
-            // a NaN or an infinity among the activations makes every output of the row NaN
-            inv[r] = E == 255 ? __uint_as_float(0x7fc00000u) : __uint_as_float(static_cast<uint32_t>(127 - e) << 23);
-        };
-        auto to_planes = [&](int r, int i, const float4& v, float scale) {
-            uint8_t* set = planes + r * g.set_bytes;
-            float* sumx = reinterpret_cast<float*>(set + 4 * g.plane_stride);
-            uint32_t pl[4];
-            digit_planes(__float2int_rn(v.x * scale), __float2int_rn(v.y * scale), __float2int_rn(v.z * scale),
-                         __float2int_rn(v.w * scale), pl);
-#pragma unroll
-            for (int p = 0; p < 4; ++p) *reinterpret_cast<uint32_t*>(set + p * g.plane_stride + 4 * i) = pl[p];
-            float s = (v.x + v.y) + (v.z + v.w);
-            if (F::kSumRun == 32) {
-                s = oct_sum(s);
-                if ((i & 7) == 0) sumx[i >> 3] = s;
-            } else {
-                s += dpp_mov<0xB1>(s);
-                s += dpp_mov<0x4E>(s);
-                if ((i & 3) == 0) sumx[i >> 2] = s;
-            }
-        };
         const int rows = ce.rows;
-        if (rows * n4 <= kPrep * T) {
-            // flat index f = r * n4 + i over the rows; a wave's 64 values of one round belong to one row (n4 % 64 == 0)
-            float4 xr[kPrep];
-            const float4* x4 = reinterpret_cast<const float4*>(ce.x);      // the rows are consecutive: x4[f]
-            auto row_of = [&](int j) {                                      // wave-uniform; -1 past the last row
-                const int f0 = (tid & ~63) + j * T;
-                const int r = R > 1 ? (f0 >= n4) + (f0 >= 2 * n4) + (f0 >= 3 * n4) : 0;
-                return f0 >= rows * n4 ? -1 : __builtin_amdgcn_readfirstlane(r);
-            };
 #pragma unroll
-            for (int j = 0; j < kPrep; ++j) xr[j] = x4[row_of(j) >= 0 ? tid + j * T : 0];
-            uint32_t mx[R] = {};
-#pragma unroll
-            for (int j = 0; j < kPrep; ++j) {
-                const int rj = row_of(j);
-                const uint32_t m = umax4(0u, xr[j]);
-#pragma unroll
-                for (int r = 0; r < R; ++r) mx[r] = rj == r ? umax_u(mx[r], m) : mx[r];
+        for (int r = 0; r < R; ++r) {
+            if (r < rows) {
+                const float4* x4 = reinterpret_cast<const float4*>(ce.x + static_cast<size_t>(r) * a.in_w);
+                uint32_t mx = 0;
+                for (int i = tid; i < n4; i += T) mx = umax4(mx, x4[i]);
+                mx = wave_umax(mx);
+                if (lane == 0) red[r][wave] = mx;
             }
+        }
+        __syncthreads();
 #pragma unroll
-            for (int r = 0; r < R; ++r) {
-                if (r < rows) {
-                    const uint32_t m = wave_umax(mx[r]);
-                    if (lane == 0) red[r][wave] = m;
-                }
-            }
-            __syncthreads();
-            float scale[R] = {};
+        for (int r = 0; r < R; ++r) {
+            if (r < rows) {
+                uint32_t mx = 0;
+                for (int i = 0; i < W; ++i) mx = umax_u(mx, red[r][i]);
+                // |x| < 2^(E - 126) for the biased exponent E of the largest magnitude; e = 156 - E puts it below 2^30
+                const int E = static_cast<int>(mx >> 23);
+                int e = 156 - E;
+                e = e > 126 ? 126 : e;
+                const float scale = __uint_as_float(static_cast<uint32_t>(e + 127) << 23);
+                // a NaN or an infinity among the activations makes every output of the row NaN
+                inv[r] = E == 255 ? __uint_as_float(0x7fc00000u) : __uint_as_float(static_cast<uint32_t>(127 - e) << 23);
+                uint8_t* set = planes + r * g.set_bytes;
+                float* sumx = reinterpret_cast<float*>(set + 4 * g.plane_stride);
+                const float4* x4 = reinterpret_cast<const float4*>(ce.x + static_cast<size_t>(r) * a.in_w);
+                for (int i = tid; i < n4; i += T) {       // (whole groups of eight lanes are in or out: n4 % 64 == 0)
+                    const float4 v = x4[i];
+                    uint32_t pl[4];
+                    digit_planes(__float2int_rn(v.x * scale), __float2int_rn(v.y * scale), __float2int_rn(v.z * scale),
+                                 __float2int_rn(v.w * scale), pl);
 #pragma unroll
-            for (int r = 0; r < R; ++r)
-                if (r < rows) scale_of(r, scale[r]);
-#pragma unroll
-            for (int j = 0; j < kPrep; ++j) {
-                const int rj = row_of(j);
-                if (rj >= 0) {
-                    float sc = scale[0];
-#pragma unroll
-                    for (int r = 1; r < R; ++r) sc = rj == r ? scale[r] : sc;
-                    to_planes(rj, tid + j * T - rj * n4, xr[j], sc);
-                }
-            }
-        } else {
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                if (r < rows) {
-                    const float4* x4 = reinterpret_cast<const float4*>(ce.x + static_cast<size_t>(r) * a.in_w);
-                    uint32_t mx = 0;
-                    for (int i = tid; i < n4; i += T) mx = umax4(mx, x4[i]);
-                    mx = wave_umax(mx);
-                    if (lane == 0) red[r][wave] = mx;
-                }
-            }
-            __syncthreads();
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                if (r < rows) {
-                    float scale;
-                    scale_of(r, scale);
-                    const float4* x4 = reinterpret_cast<const float4*>(ce.x + static_cast<size_t>(r) * a.in_w);
-                    for (int i = tid; i < n4; i += T) to_planes(r, i, x4[i], scale);
+                    for (int p = 0; p < 4; ++p) *reinterpret_cast<uint32_t*>(set + p * g.plane_stride + 4 * i) = pl[p];
+                    float s = (v.x + v.y) + (v.z + v.w);
+                    if (!F::kNeedsSums) {
+                        // (the format has neither minima nor an offset: no room is kept for the sums)
+                    } else if (F::kSumRun == 32) {
+                        s = oct_sum(s);
+                        if ((i & 7) == 0) sumx[i >> 3] = s;
+                    } else {
+                        s += dpp_mov<0xB1>(s);
+                        s += dpp_mov<0x4E>(s);
+                        if ((i & 3) == 0) sumx[i >> 2] = s;
+                    }
                 }
             }
         }
@@ -930,9 +1011,10 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
         fetch(refill);
         if (new_x) prepare_x();
         if (done) finalize();
-        const int b = c_k * W + wave;                    // this wave's block column of the row
-        if (b < a.nblocks) {
-            const typename F::Raw raw = F::load(cur + row_off, quarter, (wave & 1) != 0);
+        // task t of this wave: block column c_k * cols + t * W + wave of the row (W is even: the block's parity is the
+        // wave's).  Stages whose tasks all exist run them as one straight piece of code, so that the lookups and products
+        // of one task overlap the other's; a tile's last stage may hold fewer.
+        auto task = [&](const typename F::Raw& raw, int b) {
 #pragma unroll
             for (int r = 0; r < R; ++r) {
                 if (r < ce.rows) {
@@ -940,9 +1022,22 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
                     typename F::X xs;
                     F::load_x(xs, set + (row_l & 3) * g.plane_stride, reinterpret_cast<const float*>(set + 4 * g.plane_stride), b,
                               quarter, diag);
-                    F::run(raw, xs, quarter, accq[r], accm[r]);
+                    F::run(raw, xs, quarter, tables, accq[r], accm[r]);
                 }
             }
+        };
+        const int b0 = c_k * g.cols + wave;
+        const uint8_t* stage = cur + row_off;
+        if (b0 + (M - 1) * W < a.nblocks) {
+            typename F::Raw raw[M];
+#pragma unroll
+            for (int t = 0; t < M; ++t) raw[t] = F::load(stage + t * W * (16 * F::kPieces), quarter, (wave & 1) != 0);
+#pragma unroll
+            for (int t = 0; t < M; ++t) task(raw[t], b0 + t * W);
+        } else {
+#pragma unroll
+            for (int t = 0; t < M - 1; ++t)
+                if (b0 + t * W < a.nblocks) task(F::load(stage + t * W * (16 * F::kPieces), quarter, (wave & 1) != 0), b0 + t * W);
         }
         if (++c_k == KC) {
             c_k = 0;
@@ -1055,6 +1150,7 @@ int block_bytes_of(uint32_t type)
     case NNHIP_TYPE_Q4_K: return Q4KTask::kBlockBytes;
     case NNHIP_TYPE_Q5_K: return Q5KTask::kBlockBytes;
     case NNHIP_TYPE_Q6_K: return Q6KTask::kBlockBytes;
+    case NNHIP_TYPE_IQ2_S: return IQ2STask::kBlockBytes;
     default: return 0;
     }
 }
@@ -1065,46 +1161,64 @@ int block_pieces_of(uint32_t type)
     case NNHIP_TYPE_Q4_K: return Q4KTask::kPieces;
     case NNHIP_TYPE_Q5_K: return Q5KTask::kPieces;
     case NNHIP_TYPE_Q6_K: return Q6KTask::kPieces;
+    case NNHIP_TYPE_IQ2_S: return IQ2STask::kPieces;
     default: return 0;
     }
 }
 
 
-int wide_lpw_of(uint32_t type)
+struct WideTraits { int pieces, m, lpw, table_bytes; bool sums, tight; };
+
+template <class F>
+constexpr WideTraits wide_traits_of(bool shared)
+{
+    return {F::kPieces, shared ? F::kSharedM : F::kWideM, shared ? F::kSharedLpw : F::kWideLpw, 0, F::kNeedsSums, F::kTightStage};
+}
+
+WideTraits wide_traits(uint32_t type, bool shared)
 {
     switch (type) {
-    case NNHIP_TYPE_Q4_K: return Q4KTask::kWideLpw;
-    case NNHIP_TYPE_Q5_K: return Q5KTask::kWideLpw;
-    case NNHIP_TYPE_Q6_K: return Q6KTask::kWideLpw;
-    default: return 0;
+    case NNHIP_TYPE_Q4_K: return wide_traits_of<Q4KTask>(shared);
+    case NNHIP_TYPE_Q5_K: return wide_traits_of<Q5KTask>(shared);
+    case NNHIP_TYPE_Q6_K: return wide_traits_of<Q6KTask>(shared);
+    case NNHIP_TYPE_IQ2_S: {
+        WideTraits t = wide_traits_of<IQ2STask>(shared);
+        t.table_bytes = IQ2STask::kTableBytes;
+        return t;
+    }
+    default: return {0, 0, 0, 0, false, false};
     }
 }
+
+constexpr int kWideStaticLds = 8 * 1024;      // room left for the kernel's static arrays (partial sums, maxima)
 
 // W for the wide form: even, as many of the row's blocks per stage as two stage buffers beside the plane sets of
 // `inputs` rows leave room for: the most waves, weighted by the share of block slots a tile fills and by an even
 // split over the four SIMDs.
 bool plan_wide(uint32_t type, int in_w, int inputs, WideGeom* out)
 {
-    const int nblocks = in_w / 256, bp = block_pieces_of(type), lpw = wide_lpw_of(type);
-    if (!bp || nblocks < 4) return false;
+    const WideTraits tr = wide_traits(type, inputs > 1);
+    const int nblocks = in_w / 256;
+    if (!tr.pieces || nblocks < 4) return false;
     WideGeom best{};
     double best_score = -1.0;
     for (int W = 12; W >= 4; W -= 2) {
-        if (W > nblocks + 1) continue;
         WideGeom g{};
         g.waves = W;
-        g.kchunks = (nblocks + W - 1) / W;
-        g.tail_cols = nblocks - (g.kchunks - 1) * W;
-        g.row_pieces = (W * bp) | 1;
+        g.cols = W * tr.m;
+        if (g.cols > nblocks + tr.m) continue;
+        g.kchunks = (nblocks + g.cols - 1) / g.cols;
+        g.tail_cols = nblocks - (g.kchunks - 1) * g.cols;
+        g.row_pieces = (g.cols * tr.pieces) | 1;
         const int loads = (kTileRows * g.row_pieces + 63) / 64;
-        if ((loads + W - 1) / W > lpw) continue;
-        g.stage_bytes = lpw * W * 1024;
+        if ((loads + W - 1) / W > tr.lpw) continue;
+        g.stage_bytes = (tr.tight ? loads : tr.lpw * W) * 1024;      // to the last row's end, or every wave's slots
         g.plane_stride = in_w + 16;
-        g.set_bytes = (4 * g.plane_stride + (in_w / 16) * 4 + 15) / 16 * 16;
-        g.lds_bytes = 2 * static_cast<size_t>(g.stage_bytes) + static_cast<size_t>(inputs) * g.set_bytes;
-        if (g.lds_bytes + 8 * 1024 > static_cast<size_t>(160 * 1024)) continue;      // (8 KB: the static arrays)
-        const double fill = static_cast<double>(nblocks) / (g.kchunks * W);
-        // (throughput grows with the waves: a stage holds W blocks per row and W tasks run side by side)
+        g.set_bytes = (4 * g.plane_stride + (tr.sums ? (in_w / 16) * 4 : 0) + 15) / 16 * 16;
+        g.lds_bytes = 2 * static_cast<size_t>(g.stage_bytes) + static_cast<size_t>(inputs) * g.set_bytes + tr.table_bytes;
+        if (g.lds_bytes + kWideStaticLds > static_cast<size_t>(160 * 1024)) continue;
+        const double fill = static_cast<double>(nblocks) / (g.kchunks * g.cols);
+        // (throughput grows with the waves: a stage holds W * M blocks per row and W tasks run side by side)
         const double score = fill * W / 12.0 * (W % 4 == 0 ? 1.0 : 0.95);
         if (score > best_score) {
             best_score = score;
@@ -1119,12 +1233,13 @@ bool plan_wide(uint32_t type, int in_w, int inputs, WideGeom* out)
 template <class F, int R>
 hipError_t launch_wide_of(Lane* lane, const WideArgs& a)
 {
+    constexpr int M = R == 1 ? F::kWideM : F::kSharedM, LPW = R == 1 ? F::kWideLpw : F::kSharedLpw;
     static LdsLimit big_lds;
-    const void* fn = reinterpret_cast<const void*>(&matvec_mfma_wide_kernel<F, F::kWideLpw, R>);
-    const hipError_t e = big_lds.ensure(lane->device, fn, 160 * 1024 - 8 * 1024);
+    const void* fn = reinterpret_cast<const void*>(&matvec_mfma_wide_kernel<F, M, LPW, R>);
+    const hipError_t e = big_lds.ensure(lane->device, fn, 160 * 1024 - kWideStaticLds);
     if (e != hipSuccess) return e;
     const int groups = a.total_tiles < lane->compute_units ? a.total_tiles : lane->compute_units;
-    hipLaunchKernelGGL((matvec_mfma_wide_kernel<F, F::kWideLpw, R>), dim3(groups), dim3(64 * a.g.waves), a.g.lds_bytes, lane->stream, a);
+    hipLaunchKernelGGL((matvec_mfma_wide_kernel<F, M, LPW, R>), dim3(groups), dim3(64 * a.g.waves), a.g.lds_bytes, lane->stream, a);
     return hipGetLastError();
 }
 
@@ -1172,6 +1287,7 @@ MfmaTableEntry matvec_mfma_entry(uint32_t type, const float* x, const void* w, c
 
 bool matvec_mfma_geometry(uint32_t type, int in_w, int out_w, const void* w, MfmaPlan* plan)
 {
+    if (type == NNHIP_TYPE_IQ2_S) return false;            // (the codebook format has the wide form only)
     if (!entry_ok(type, in_w, out_w, w)) return false;
     MfmaGeom g;
     if (!plan_mfma(block_pieces_of(type), in_w, block_bytes_of(type) % 16 != 0, &g)) return false;
@@ -1224,6 +1340,7 @@ hipError_t launch_wide_args(Lane* lane, uint32_t type, int in_w, int inputs, Wid
     case NNHIP_TYPE_Q4_K: return launch_wide<Q4KTask>(lane, a, inputs);
     case NNHIP_TYPE_Q5_K: return launch_wide<Q5KTask>(lane, a, inputs);
     case NNHIP_TYPE_Q6_K: return launch_wide<Q6KTask>(lane, a, inputs);
+    case NNHIP_TYPE_IQ2_S: return launch_wide<IQ2STask>(lane, a, inputs);
     default: return hipErrorInvalidValue;
     }
 }

@@ -10,7 +10,7 @@ import numpy as np
 import pytest
 
 import oracle
-from nntrain_amd import GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_Q8_0, HipExecutionLane, HipQuantizedMatrix, synth
+from nntrain_amd import GGML_IQ2_S, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_Q8_0, HipExecutionLane, HipQuantizedMatrix, synth
 from nntrain_amd.native import MatvecDesc, check
 
 pytestmark = pytest.mark.gpu
@@ -435,7 +435,7 @@ def test_large_batched_group_special_activations(lane):
     lane.trim()
 
 
-@pytest.mark.parametrize("typ", [GGML_Q4_K, GGML_Q5_K, GGML_Q6_K])
+@pytest.mark.parametrize("typ", [GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_IQ2_S])
 def test_matrix_core_groups_with_long_rows_and_shared_passes(lane, typ):
     """Rows that do not split into whole stages (17408 = 68 super-blocks, 3072 = 12, 1024 = 4) and descriptors with
     2 - 5 input rows (up to four share a pass over the weights) take the form of the matrix-core mat-vec that keeps the
