@@ -147,6 +147,15 @@ __device__ __forceinline__ float recombine(i32x4 s)
     return fmaf(static_cast<float>(hi), 65536.0f, static_cast<float>(lo));
 }
 
+// The same for plane sums of up to 2^24 (scale factors already multiplied in): the pairs are joined in FP32, each join
+// rounding at 2^-24 of its value.
+__device__ __forceinline__ float recombine_wide(i32x4 s)
+{
+    const float lo = fmaf(static_cast<float>(s[1]), 256.0f, static_cast<float>(s[0]));
+    const float hi = fmaf(static_cast<float>(s[3]), 256.0f, static_cast<float>(s[2]));
+    return fmaf(hi, 65536.0f, lo);
+}
+
 __device__ __forceinline__ i32x4 mfma_i8(uint32_t a0, uint32_t a1, uint32_t b0, uint32_t b1, i32x4 c)
 {
     return __builtin_amdgcn_mfma_i32_16x16x32_i8(__builtin_bit_cast(long, u32x2{a0, a1}), __builtin_bit_cast(long, u32x2{b0, b1}),
@@ -181,12 +190,14 @@ struct Q4KTask {
 
     static __device__ __forceinline__ uint32_t piece_src(uint32_t q, bool) { return 16u * q; }
 
-    // plane = this lane's digit plane of the whole vector, sums = the per-sub-block sums of x; b = super-block column
-    static __device__ __forceinline__ void load_x(X& xs, const uint8_t* plane, const float* sums, int b, int quarter, bool diag)
+    // plane = this lane's digit plane of the whole vector, sums = the per-sub-block sums of x; b = super-block column;
+    // zeros = null in the lanes on the block diagonal of operand A, else 256 zero bytes in LDS (read in place of the
+    // plane: no branch, and the compiler may interleave the reads of two tasks)
+    static __device__ __forceinline__ void load_x(X& xs, const uint8_t* plane, const float* sums, int b, int quarter, const uint8_t* zeros)
     {
-        const uint8_t* src = plane + 256 * b + 64 * quarter;
+        const uint8_t* src = zeros ? zeros : plane + 256 * b + 64 * quarter;
 #pragma unroll
-        for (int u = 0; u < 4; ++u) xs.a[u] = diag ? lds128(src + 16 * u) : u32x4{0u, 0u, 0u, 0u};
+        for (int u = 0; u < 4; ++u) xs.a[u] = lds128(src + 16 * u);
         const float2 v = *reinterpret_cast<const float2*>(sums + 8 * b + 2 * quarter);
         xs.sx[0] = v.x;
         xs.sx[1] = v.y;
@@ -243,9 +254,9 @@ struct Q5KTask {
 
     static __device__ __forceinline__ uint32_t piece_src(uint32_t q, bool) { return 16u * q; }
 
-    static __device__ __forceinline__ void load_x(X& xs, const uint8_t* plane, const float* sums, int b, int quarter, bool diag)
+    static __device__ __forceinline__ void load_x(X& xs, const uint8_t* plane, const float* sums, int b, int quarter, const uint8_t* zeros)
     {
-        Q4KTask::load_x(xs, plane, sums, b, quarter, diag);
+        Q4KTask::load_x(xs, plane, sums, b, quarter, zeros);
     }
 
     static __device__ __forceinline__ Raw load(const uint8_t* blk, int quarter, bool)
@@ -311,14 +322,14 @@ struct Q6KTask {
     // an even number of blocks here, so that dword never reaches past the matrix.)
     static __device__ __forceinline__ uint32_t piece_src(uint32_t q, bool odd) { return 16u * q - (odd ? 2u : 0u); }
 
-    static __device__ __forceinline__ void load_x(X& xs, const uint8_t* plane, const float* sums, int b, int quarter, bool diag)
+    static __device__ __forceinline__ void load_x(X& xs, const uint8_t* plane, const float* sums, int b, int quarter, const uint8_t* zeros)
     {
         const int h = quarter >> 1, e = quarter & 1;
-        const uint8_t* src = plane + 256 * b + 128 * h + 32 * e;
-        xs.a[0] = diag ? lds128(src) : u32x4{0u, 0u, 0u, 0u};
-        xs.a[1] = diag ? lds128(src + 16) : u32x4{0u, 0u, 0u, 0u};
-        xs.a[2] = diag ? lds128(src + 64) : u32x4{0u, 0u, 0u, 0u};
-        xs.a[3] = diag ? lds128(src + 80) : u32x4{0u, 0u, 0u, 0u};
+        const uint8_t* src = zeros ? zeros : plane + 256 * b + 128 * h + 32 * e;
+        xs.a[0] = lds128(src);
+        xs.a[1] = lds128(src + 16);
+        xs.a[2] = lds128(src + 64);
+        xs.a[3] = lds128(src + 80);
         const float* sp = sums + 16 * b + 8 * h + 2 * e;
         const float2 lo = *reinterpret_cast<const float2*>(sp), hi = *reinterpret_cast<const float2*>(sp + 4);
         xs.sx[0] = lo.x;
@@ -414,7 +425,7 @@ struct IQ2STask {
     static constexpr bool kNeedsSums = false;         // no minimum or offset
     static constexpr bool kTightStage = true;         // 17408-wide planes leave no room for whole 1 KB slots per wave
     static constexpr int kGridBytes = 8192;
-    static constexpr int kTableBytes = kGridBytes + 64;       // the codebook and 16 byte selectors
+    static constexpr int kTableBytes = kGridBytes + 2048;     // the codebook and 256 selector pairs
     using X = XSet<1>;
     struct Raw { uint32_t q[2], s[2], tops, scales, d; };
 
@@ -423,19 +434,20 @@ struct IQ2STask {
     static __device__ __forceinline__ void init_tables(uint8_t* t, int tid, int threads)
     {
         for (int i = tid; i < 1024; i += threads) reinterpret_cast<uint64_t*>(t)[i] = g_iq2s_grid_mv[i];
-        if (tid < 16) {
-            // four sign bits -> a v_perm_b32 selector: byte k of the result comes from the magnitudes (selector byte k) or
-            // from their negation (selector byte 4 + k); the 64-byte table is read without bank conflicts
-            const uint32_t spread = (static_cast<uint32_t>(tid) * 0x00204081u) & 0x01010101u;
-            reinterpret_cast<uint32_t*>(t + kGridBytes)[tid] = 0x03020100u + (spread << 2);
+        for (int i = tid; i < 256; i += threads) {
+            // eight sign bits -> two v_perm_b32 selectors: byte k of a result comes from the magnitudes (selector byte k)
+            // or from their negation (selector byte 4 + k)
+            const uint32_t lo = ((static_cast<uint32_t>(i) & 15u) * 0x00204081u) & 0x01010101u;
+            const uint32_t hi = ((static_cast<uint32_t>(i) >> 4) * 0x00204081u) & 0x01010101u;
+            reinterpret_cast<u32x2*>(t + kGridBytes)[i] = u32x2{0x03020100u + (lo << 2), 0x03020100u + (hi << 2)};
         }
     }
 
-    static __device__ __forceinline__ void load_x(X& xs, const uint8_t* plane, const float*, int b, int quarter, bool diag)
+    static __device__ __forceinline__ void load_x(X& xs, const uint8_t* plane, const float*, int b, int quarter, const uint8_t* zeros)
     {
-        const uint8_t* src = plane + 256 * b + 64 * quarter;
+        const uint8_t* src = zeros ? zeros : plane + 256 * b + 64 * quarter;
 #pragma unroll
-        for (int u = 0; u < 4; ++u) xs.a[u] = diag ? lds128(src + 16 * u) : u32x4{0u, 0u, 0u, 0u};
+        for (int u = 0; u < 4; ++u) xs.a[u] = lds128(src + 16 * u);
         xs.sx[0] = 0.0f;
     }
 
@@ -462,17 +474,20 @@ struct IQ2STask {
     {
         // every lookup of the task is requested before the first result is used (the scheduling barrier keeps the
         // compiler from folding the reads back into a chain of eight round trips to LDS)
-        const uint32_t* selectors = reinterpret_cast<const uint32_t*>(tables + kGridBytes);
-        u32x2 mag[8];
-        uint32_t sel[8][2];
+        u32x2 mag[8], sel[8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const int g = e >> 2, o = e & 3;                                  // 32-weight group of the quarter, entry in it
-            const uint32_t index = ((r.q[g] >> (8 * o)) & 0xffu) | (((r.tops >> (8 * g + 2 * o)) & 3u) << 8);
-            const uint32_t sign = r.s[g] >> (8 * o);
-            mag[e] = *reinterpret_cast<const u32x2*>(tables + 8u * index);
-            sel[e][0] = selectors[sign & 15u];
-            sel[e][1] = selectors[(sign >> 4) & 15u];
+        for (int g = 0; g < 2; ++g) {
+            // the two top bits of entry o of the group as byte o, then index bytes and tops interleaved into 16-bit indices
+            const uint32_t t8 = (r.tops >> (8 * g)) & 0xffu;
+            const uint32_t tops = (t8 | (t8 << 6) | (t8 << 12) | (t8 << 18)) & 0x03030303u;
+            const uint32_t pair[2] = {__builtin_amdgcn_perm(tops, r.q[g], 0x05010400u), __builtin_amdgcn_perm(tops, r.q[g], 0x07030602u)};
+#pragma unroll
+            for (int o = 0; o < 4; ++o) {
+                const uint32_t index = (pair[o >> 1] >> (16 * (o & 1))) & 0xffffu;
+                const uint32_t sign = (r.s[g] >> (8 * o)) & 0xffu;
+                mag[4 * g + o] = *reinterpret_cast<const u32x2*>(tables + 8u * index);
+                sel[4 * g + o] = *reinterpret_cast<const u32x2*>(tables + kGridBytes + 8u * sign);
+            }
         }
         __builtin_amdgcn_sched_barrier(0);
         i32x4 acc[4] = {{0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}};
@@ -484,13 +499,16 @@ struct IQ2STask {
             const u32x4 av = xs.a[e >> 1];
             acc[e >> 1] = mfma_i8(av[2 * (e & 1)], av[2 * (e & 1) + 1], b0, b1, acc[e >> 1]);
         }
-        const float d = half_bits_to_float(r.d);
+        // d (0.5 + s) 0.25 = d / 8 * (2 s + 1): the plane sums of the four scale groups are added up with the integer
+        // factors 2 s + 1 (|sum| < 4 * 31 * 2^17 < 2^24: exact) and recombined once
+        i32x4 total = {0, 0, 0, 0};
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
-            // scale group k of the quarter: nibble (k & 1) of scale byte k >> 1
-            const float sc = static_cast<float>((r.scales >> (4 * k)) & 15u);
-            accq = fmaf((d * (0.5f + sc)) * 0.25f, recombine(acc[k]), accq);
+            const int factor = static_cast<int>(2u * ((r.scales >> (4 * k)) & 15u) + 1u);    // nibble k & 1 of scale byte k >> 1
+#pragma unroll
+            for (int p = 0; p < 4; ++p) total[p] += factor * acc[k][p];
         }
+        accq = fmaf(half_bits_to_float(r.d) * 0.125f, recombine_wide(total), accq);
     }
 };
 
@@ -511,6 +529,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_kernel(MfmaArgs a)
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
     __shared__ float part[2][kMaxWaves][kTileRows];
     __shared__ uint32_t red[kMaxWaves];
+    __shared__ __attribute__((aligned(16))) uint8_t zero_area[256];       // operand A outside the block diagonal
 
     const MfmaGeom& g = a.g;
     const int tid = threadIdx.x, lane = tid & 63, T = blockDim.x;
@@ -617,6 +636,8 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_kernel(MfmaArgs a)
     // Operand A of this lane: A row lane % 16 = plane (lane % 4) of quarter (lane % 16) / 4, K group lane / 16; it is
     // non-zero only where the K group carries that quarter.
     const bool diag = (row_l >> 2) == quarter;
+    if (tid < 64) reinterpret_cast<uint32_t*>(zero_area)[tid] = 0u;      // (published by the barrier after the first parking)
+    const uint8_t* const a_zeros = diag ? nullptr : zero_area;
 
     // Turns matrix c_m's activations into this lane's operand-A registers (all waves; three barriers inside).  The digit
     // planes and sub-block sums pass through the stage buffer `scratch`, which is free at that point.  The vector is in xv
@@ -679,7 +700,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_kernel(MfmaArgs a)
 #pragma unroll
             for (int t = 0; t < M; ++t) {
                 const int b = k * g.cols + t * W + wave;
-                F::load_x(xs[k * M + t], scratch + (row_l & 3) * plane_stride, sumx, b, quarter, diag);
+                F::load_x(xs[k * M + t], scratch + (row_l & 3) * plane_stride, sumx, b, quarter, a_zeros);
             }
         }
         regs_x = ce.x;
@@ -810,6 +831,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
     __shared__ float part[2][R][kMaxWaves][kTileRows];
     __shared__ uint32_t red[R][kMaxWaves];
+    __shared__ __attribute__((aligned(16))) uint8_t zero_area[256];       // operand A outside the block diagonal
 
     const WideGeom& g = a.g;
     const int tid = threadIdx.x, lane = tid & 63, T = blockDim.x;
@@ -900,6 +922,8 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
     const float* planes_x = nullptr;       // the vector(s) the planes in LDS were made from
     int planes_rows = 0;
     const bool diag = (row_l >> 2) == quarter;
+    if (tid < 64) reinterpret_cast<uint32_t*>(zero_area)[tid] = 0u;      // (published by the barrier after the first parking)
+    const uint8_t* const a_zeros = diag ? nullptr : zero_area;
 
     // Turns the activations of matrix c_m (its `rows` input rows) into digit planes and sums in LDS; two barriers.
     // Every wave has left the stage that last read the planes when this runs.  (A variant that requested all rows at once
@@ -1021,7 +1045,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
                     const uint8_t* set = planes + r * g.set_bytes;
                     typename F::X xs;
                     F::load_x(xs, set + (row_l & 3) * g.plane_stride, reinterpret_cast<const float*>(set + 4 * g.plane_stride), b,
-                              quarter, diag);
+                              quarter, a_zeros);
                     F::run(raw, xs, quarter, tables, accq[r], accm[r]);
                 }
             }
