@@ -259,7 +259,9 @@ GEMV_CONFIGS = [
     ("cfg2 Q5_K 17408x5120", "GGML_Q5_K", 5120, 17408, 2002, 2000),
     ("cfg2 Q6_K 17408x5120", "GGML_Q6_K", 5120, 17408, 2003, 2000),
     ("cfg5 IQ2_S 5120x17408", "GGML_IQ2_S", 17408, 5120, 5001, 5002),
+    ("down projection Q4_K 5120x17408", "GGML_Q4_K", 17408, 5120, 2004, 2005),
 ]
+MATRIX_CORE_TYPES = ("GGML_Q4_K", "GGML_Q5_K", "GGML_Q6_K", "GGML_IQ2_S")
 
 
 def run_gemv(args, lane, nn, oracle):
@@ -312,13 +314,13 @@ def run_gemv(args, lane, nn, oracle):
             descs[i] = MatvecDesc(x.ptr, w.ptr, None, ys[i].ptr, typ, 1, in_w, out_w)
         nn.native.check(lib.nnhip_quant_matvec_batch(h, descs, len(ring)), "quant_matvec_batch")
         lane.synchronize()
-        # large Q4_K / Q5_K / Q6_K groups run on the matrix-core kernel (fixed-point activations): same bar against the oracle,
-        # not the single launch's bits; the other formats share the single launch's kernel and must match bitwise
+        # large Q4_K / Q5_K / Q6_K / IQ2_S groups run on the matrix-core kernels (fixed-point activations): same bar against
+        # the oracle, not the single launch's bits; the other formats share the single launch's kernel and must match bitwise
         y_batch = lane.read(ys[-1], np.float32)
         rel_batch = oracle.rel_l2(y_batch, ref[0])
         if not rel_batch <= 1e-5:
             raise SystemExit(f"{name}: batched launch parity failure, rel-L2 {rel_batch:.3e}")
-        if tname not in ("GGML_Q4_K", "GGML_Q5_K", "GGML_Q6_K") and not np.array_equal(y_batch.view(np.uint32), lane.read(y, np.uint32)):
+        if tname not in MATRIX_CORE_TYPES and not np.array_equal(y_batch.view(np.uint32), lane.read(y, np.uint32)):
             raise SystemExit(f"{name}: batched launch differs bitwise from the single launch")
         samples_batch = []
         for _ in range(7):
@@ -341,8 +343,9 @@ def run_gemv(args, lane, nn, oracle):
             out[name]["cpu_baseline"] = {"gb_per_s": round(nbytes / per_pass / 1e9, 2), "us_per_matvec": round(per_pass * 1e6, 1),
                                          "cores": threads, "one_thread_gb_per_s": round(nbytes / one / 1e9, 3), "kind": "port"}
             log(f"[gemv] {name}: CPU port {nbytes / per_pass / 1e9:.1f} GB/s on {threads} threads, {nbytes / one / 1e9:.2f} GB/s on one")
-        if tname == "GGML_Q8_0":
-            # several input rows in one call (weights rotated as above): microseconds per call
+        if tname == "GGML_Q8_0" or name.startswith("cfg2 Q4_K"):
+            # several input rows in one call (weights rotated as above): microseconds per call.  Q8_0: four rows per pass
+            # of the row-step kernel; Q4_K: four rows per pass of the matrix-core kernel
             per_rows = {}
             for rows in (2, 4, 8):
                 xr = lane.upload_raw(synth.activations(rows, in_w, xseed + rows))

@@ -184,8 +184,10 @@ NNHIP_API int nnhip_dequantize(void* lane, uint32_t ggml_type, const void* w, fl
  * by Qwen35QuantizedModel.Matrix.Forward (Qwen35QuantizedModel.cs:1210-1369) and Tensor.ArcQwenQuantizedLinear
  * (NNtrain.Core/Tensors/Tensor.QwenQuantized.cs:29-96) for decode (rows == 1) and small row counts.  Each
  * output row of y is computed with the same operation order whatever `rows` is, so rows > 1 equals stacked
- * rows == 1 calls bit for bit (Qwen35InferencePrefillLinearTests.cs:64-77).  bias may be null (zero).
- * Asynchronous. */
+ * rows == 1 calls bit for bit (Qwen35InferencePrefillLinearTests.cs:64-77), except for calls with 2 - 16 input rows
+ * on Q4_K / Q5_K / Q6_K / IQ2_S matrices with rows x ceil(out_w / 16) >= 2048: those take the matrix-core path described
+ * at nnhip_quant_matvec_batch (up to four input rows per pass over the weights; a row's bits do not depend on the
+ * rows it travels with; 1e-6 from the rows == 1 result).  bias may be null (zero).  Asynchronous. */
 NNHIP_API int nnhip_quant_matvec(void* lane, uint32_t ggml_type, const float* x, const void* w, const float* bias,
                                  float* y, int rows, int in_w, int out_w);
 
@@ -193,13 +195,14 @@ NNHIP_API int nnhip_quant_matvec(void* lane, uint32_t ggml_type, const float* x,
  * reporting (the reference prints its kernel choice per matrix, Qwen35QuantizedModel.cs:1335-1344 selects by rows) and
  * for checking the kernels' capacity assumptions in tests.  compute_units is the workgroup count to plan for (256 on
  * MI355X).  Returns NNHIP_ERR_TOO_LARGE when no kernel takes the shape.  struct_size = sizeof of the structure. */
-enum { NNHIP_MATVEC_KERNEL_ROWSTEP = 0, NNHIP_MATVEC_KERNEL_Q8_0_ODD_BLOCKS = 1 };
+enum { NNHIP_MATVEC_KERNEL_ROWSTEP = 0, NNHIP_MATVEC_KERNEL_Q8_0_ODD_BLOCKS = 1,
+       NNHIP_MATVEC_KERNEL_MATRIX_CORE = 2 /* 16-row tiles over the workgroups, up to four input rows per pass */ };
 
 typedef struct nnhip_matvec_plan_info {
     uint32_t struct_size;
     int32_t kernel;                 /* NNHIP_MATVEC_KERNEL_*                                                   */
     int32_t threads;                /* lanes per workgroup                                                     */
-    int32_t rows_per_step;          /* whole matrix rows a workgroup reduces per step                          */
+    int32_t rows_per_step;          /* whole matrix rows a workgroup reduces per step (matrix core: 16 per tile)  */
     int32_t steps;                  /* ceil(out_w / rows_per_step)                                             */
     int32_t groups;                 /* workgroups along the matrix                                             */
     int32_t row_tile;               /* input rows that share one pass over the weights                         */
@@ -214,11 +217,13 @@ NNHIP_API int nnhip_matvec_plan(uint32_t ggml_type, int rows, int in_w, int out_
 /* `count` independent mat-vecs enqueued as one unit of work (a single launch per group of equal type), for the
  * per-token projection sets that ForwardTokenDevice issues back to back (Qwen35QuantizedModel.cs:451-513).
  * `descs` is a host array, read before the call returns.  Results are identical to `count` nnhip_quant_matvec calls,
- * with one exception: Q4_K, Q5_K and Q6_K matrices of one in_w whose 16-row tiles add up to 2048 or more within a call (in_w
- * a multiple of 256 that the matrix-core mat-vec can split: 5120 and 2560 among others) are multiplied on the matrix
- * cores with the activations in 32-bit fixed point.  Those results are deterministic, depend on the weights, in_w and
- * the activations only (not on out_w, the other matrices of the call or the order), agree with the single launch to
- * FP32 summation accuracy (relative L2 difference below 1e-6) and are closer to the exact product than it.
+ * with one exception: Q4_K, Q5_K, Q6_K and IQ2_S matrices of one in_w (at least 1024, a multiple of 256; an even
+ * number of 256-blocks for Q6_K and IQ2_S) whose 16-row tiles, counted once per input row, add up to 2048 or more
+ * within a call are multiplied on the matrix cores with the activations in 32-bit fixed point; descriptors with two or
+ * more input rows share one pass over the weights between up to four rows there.  Those results are deterministic,
+ * depend on the weights, in_w and the activations of the row only (not on out_w, the other matrices or input rows of
+ * the call, or the order), agree with the single launch to FP32 summation accuracy (relative L2 difference below 1e-6)
+ * and are closer to the exact product than it.
  * The descriptors reach the device as a table in lane-owned memory, written by a small kernel on the lane's stream
  * (skipped when the table already holds them), so the call never waits for the device.  Under graph capture the write
  * is recorded with the launch and a replay restores the table it needs; the table cannot grow during a capture

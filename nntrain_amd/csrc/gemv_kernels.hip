@@ -1189,6 +1189,9 @@ bool describe_rowstep(int rows, int in_w, int out_w, int compute_units, nnhip_ma
 
 bool describe_matvec(uint32_t type, int rows, int in_w, int out_w, int compute_units, nnhip_matvec_plan_info* info)
 {
+    // (the plan is made without the weight pointer: the matrix-core path also needs it 16-byte aligned)
+    if (matvec_rows_share_pass(type, rows, in_w, out_w, nullptr))
+        return describe_matvec_rows_shared(type, rows, in_w, out_w, compute_units, info);
     if (type == NNHIP_TYPE_Q8_0 && ((in_w / 32) & 1)) {
         info->kernel = NNHIP_MATVEC_KERNEL_Q8_0_ODD_BLOCKS;
         info->threads = 256;

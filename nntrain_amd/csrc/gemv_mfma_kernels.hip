@@ -1371,6 +1371,23 @@ hipError_t launch_wide_args(Lane* lane, uint32_t type, int in_w, int inputs, Wid
 
 }  // namespace
 
+bool describe_matvec_rows_shared(uint32_t type, int rows, int in_w, int out_w, int compute_units, nnhip_matvec_plan_info* info)
+{
+    WideGeom g;
+    if (!plan_wide(type, in_w, 4, &g)) return false;
+    const int tiles = (out_w + kTileRows - 1) / kTileRows * ((rows + 3) / 4);
+    info->kernel = NNHIP_MATVEC_KERNEL_MATRIX_CORE;
+    info->threads = 64 * g.waves;
+    info->rows_per_step = kTileRows;
+    info->steps = tiles;
+    info->groups = tiles < compute_units ? tiles : compute_units;
+    info->row_tile = rows < 4 ? rows : 4;
+    info->ring_depth = 2;                                   // stage buffers
+    info->result_buffer_floats = 2 * 4 * kMaxWaves * kTileRows;
+    info->dynamic_lds_bytes = static_cast<int32_t>(g.lds_bytes);
+    return true;
+}
+
 hipError_t launch_matvec_mfma_wide_table(Lane* lane, uint32_t type, int in_w, int inputs, const MfmaTableEntry* device_entries,
                                          int entries, int total_tiles)
 {

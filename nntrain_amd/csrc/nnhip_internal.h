@@ -111,6 +111,7 @@ bool matvec_mfma_wide_geometry(uint32_t type, int in_w, int out_w, const void* w
 // row-step pass per input row.
 bool matvec_rows_share_pass(uint32_t type, int rows, int in_w, int out_w, const void* w);
 // That call: 2 - 16 input rows, up to four per pass, the descriptors travelling in the kernel arguments.
+bool describe_matvec_rows_shared(uint32_t type, int rows, int in_w, int out_w, int compute_units, nnhip_matvec_plan_info* info);
 hipError_t launch_matvec_rows_shared(Lane* lane, uint32_t type, const float* x, const void* w, const float* bias, float* y,
                                      int rows, int in_w, int out_w);
 hipError_t launch_matvec_mfma_wide_table(Lane* lane, uint32_t type, int in_w, int inputs, const MfmaTableEntry* device_entries,

@@ -135,6 +135,14 @@ def test_matvec_plan_keeps_a_ring_turn_inside_the_result_buffer():
             for out_w in (1, 2, 63, 300, 1000, 5000, 200_000, 1_000_000):
                 for rows in (1, 2, 3, 4, 7, 16):
                     assert lib.nnhip_matvec_plan(typ, rows, in_w, out_w, 256, byref(info)) == 0, (typ, in_w, out_w, rows)
+                    if info.kernel == 2:
+                        # several input rows of a K-quant / IQ2_S matrix on the matrix cores: 16-row tiles, four rows a pass
+                        assert 2 <= rows <= 16 and typ in (12, 13, 14, 22) and rows * -(-out_w // 16) >= 2048
+                        assert info.rows_per_step == 16 and info.row_tile == min(rows, 4) and info.threads % 128 == 0
+                        assert info.steps == -(-out_w // 16) * -(-rows // 4) and info.groups == min(info.steps, 256)
+                        assert info.dynamic_lds_bytes + 8192 <= 160 * 1024
+                        seen_tiles.add((typ, "matrix core"))
+                        continue
                     if info.kernel != 0:
                         continue
                     assert info.ring_depth * info.rows_per_step * info.row_tile <= info.result_buffer_floats, \
@@ -144,7 +152,7 @@ def test_matvec_plan_keeps_a_ring_turn_inside_the_result_buffer():
                     assert info.steps == -(-out_w // info.rows_per_step) and info.groups == min(info.steps, 256)
                     assert info.dynamic_lds_bytes <= 140 * 1024
                     seen_tiles.add((typ, info.row_tile))
-    assert {(8, 1), (8, 2), (8, 4), (30, 4), (12, 1)} <= seen_tiles
+    assert {(8, 1), (8, 2), (8, 4), (30, 4), (12, 1), (12, "matrix core"), (14, "matrix core")} <= seen_tiles
     assert lib.nnhip_matvec_plan(8, 1, 32 * 5, 19, 256, byref(info)) == 0 and info.kernel == 1   # odd block count
     assert lib.nnhip_matvec_plan(12, 1, 255, 19, 256, byref(info)) == 3
     assert lib.nnhip_matvec_plan(12, 1, 256 * 300, 19, 256, byref(info)) == 8
