@@ -1,6 +1,10 @@
 // Decode mat-vec on the matrix cores for the super-block formats whose unpacking is too much vector-ALU work for the
-// lane-per-unit kernels (gemv_kernels.hip): Q4_K, Q5_K and Q6_K here.  Used for the large groups of a batched launch, where
-// it streams faster than the row-step kernels; it takes longer to start, so single launches stay with those.
+// lane-per-unit kernels (gemv_kernels.hip): Q4_K, Q5_K, Q6_K and IQ2_S here.  Used for the large groups of a batched
+// launch and for calls with 2 - 16 input rows, where it streams faster than the row-step kernels; it takes longer to
+// start, so single-row launches stay with those.  Two kernels share the tasks of the formats: matvec_mfma_kernel keeps
+// operand A in registers (rows of one or two whole stages), matvec_mfma_wide_kernel keeps the digit planes in LDS (any
+// row length, up to four input rows per pass over the weights); the text below describes the first, the second has its
+// own paragraph further down.
 //
 // y[r, o] = bias[o] + sum_k x[r, k] * w[o, k]     (NNtrain.Arc/Kernels/qwen.cl:374-406 defines the operator)
 //
@@ -859,9 +863,10 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
         return e;
     };
 
-    // this lane's pieces of a stage, as in the kernel above; rel_tail: the same for a tile's last stage, where the block
-    // columns past the row's end fetch nothing
-    uint32_t rel[LPW], rel_tail[LPW];
+    // this lane's pieces of a stage, as in the kernel above; in a tile's last stage the block columns past the row's
+    // end fetch nothing
+    uint32_t rel[LPW];
+    uint32_t in_tail = 0;                  // bit i: this lane's piece i exists in a tile's last stage
     uint32_t in_stage = 0;                 // bit i: this lane's piece i lies inside the stage buffer
 #pragma unroll
     for (int i = 0; i < LPW; ++i) {
@@ -871,7 +876,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
         const uint32_t c = q / static_cast<uint32_t>(F::kPieces);
         const bool real = r < static_cast<uint32_t>(kTileRows) && c < static_cast<uint32_t>(g.cols);
         rel[i] = real ? r * a.row_bytes + c * F::kBlockBytes + F::piece_src(q - c * F::kPieces, c & 1u) : kNoPiece;
-        rel_tail[i] = c < static_cast<uint32_t>(g.tail_cols) ? rel[i] : kNoPiece;
+        in_tail |= (real && c < static_cast<uint32_t>(g.tail_cols) ? 1u : 0u) << i;
         in_stage |= (r < static_cast<uint32_t>(kTileRows) ? 1u : 0u) << i;
     }
 
@@ -895,7 +900,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
             : kNoPiece;
         const bool tail = f_k == KC - 1;
 #pragma unroll
-        for (int i = 0; i < LPW; ++i) set[i] = stream16(f_matrix, base + (tail ? rel_tail[i] : rel[i]));
+        for (int i = 0; i < LPW; ++i) set[i] = stream16(f_matrix, tail && !((in_tail >> i) & 1u) ? kNoPiece : base + rel[i]);
         if (++f_k == KC) {
             f_k = 0;
             f_t += G;
