@@ -107,7 +107,14 @@ struct DecodeCtx {
     int dc, dh;
     int iters;               // K / 64
     int nblocks;             // K / 256
+    bool live;               // this thread has a column
 };
+
+// Decoder threads beyond the strip's columns run the same code (no branch around the loads) and store nothing.
+__device__ __forceinline__ void st128(const DecodeCtx& c, uint8_t* dst, const u32x4 v)
+{
+    if (c.live) *reinterpret_cast<u32x4*>(dst) = v;
+}
 
 __device__ __forceinline__ u32x4 gld128(const DecodeCtx& c, uint32_t uniform_off, uint32_t lane_off)
 {
@@ -164,9 +171,8 @@ struct Q4KDecode {
         for (int g = 0; g < 2; ++g) {
             const uint32_t a0 = q[2 * g], a1 = q[2 * g + 1];
             const int slot = lds_slot(c.dc, 2 * c.dh + g) * 16;
-            *reinterpret_cast<u32x4*>(lo + slot) = q4k_decode8(a0 & 0x0f0f0f0fu, a1 & 0x0f0f0f0fu, sm[4 * J], sm[4 * J + 1]);
-            *reinterpret_cast<u32x4*>(hi + slot) =
-                q4k_decode8((a0 >> 4) & 0x0f0f0f0fu, (a1 >> 4) & 0x0f0f0f0fu, sm[4 * J + 2], sm[4 * J + 3]);
+            st128(c, lo + slot, q4k_decode8(a0 & 0x0f0f0f0fu, a1 & 0x0f0f0f0fu, sm[4 * J], sm[4 * J + 1]));
+            st128(c, hi + slot, q4k_decode8((a0 >> 4) & 0x0f0f0f0fu, (a1 >> 4) & 0x0f0f0f0fu, sm[4 * J + 2], sm[4 * J + 3]));
         }
         nq[J & 1] = load_q(c, t + 2);
         if (J == 0) load_hdr(c, (t >> 2) + 1);
@@ -211,12 +217,10 @@ struct Q5KDecode {
         for (int g = 0; g < 2; ++g) {
             const uint32_t a0 = q[2 * g], a1 = q[2 * g + 1], h0 = qh[2 * g], h1 = qh[2 * g + 1];
             const int slot = lds_slot(c.dc, 2 * c.dh + g) * 16;
-            *reinterpret_cast<u32x4*>(lo + slot) =
-                q4k_decode8((a0 & 0x0f0f0f0fu) | (((h0 >> (2 * J)) & 0x01010101u) << 4),
-                            (a1 & 0x0f0f0f0fu) | (((h1 >> (2 * J)) & 0x01010101u) << 4), sm[4 * J], sm[4 * J + 1]);
-            *reinterpret_cast<u32x4*>(hi + slot) =
-                q4k_decode8(((a0 >> 4) & 0x0f0f0f0fu) | (((h0 >> (2 * J + 1)) & 0x01010101u) << 4),
-                            ((a1 >> 4) & 0x0f0f0f0fu) | (((h1 >> (2 * J + 1)) & 0x01010101u) << 4), sm[4 * J + 2], sm[4 * J + 3]);
+            st128(c, lo + slot, q4k_decode8((a0 & 0x0f0f0f0fu) | (((h0 >> (2 * J)) & 0x01010101u) << 4),
+                            (a1 & 0x0f0f0f0fu) | (((h1 >> (2 * J)) & 0x01010101u) << 4), sm[4 * J], sm[4 * J + 1]));
+            st128(c, hi + slot, q4k_decode8(((a0 >> 4) & 0x0f0f0f0fu) | (((h0 >> (2 * J + 1)) & 0x01010101u) << 4),
+                            ((a1 >> 4) & 0x0f0f0f0fu) | (((h1 >> (2 * J + 1)) & 0x01010101u) << 4), sm[4 * J + 2], sm[4 * J + 3]));
         }
         nq[J & 1] = load_q(c, t + 2);
         if (J == 0) load_hdr(c, (t >> 2) + 1);
@@ -275,12 +279,12 @@ struct Q6KDecode {
     }
     // 16 weights: bytes q (6-bit values) -> d * scale * (q - 32), as one fused multiply-add each (exact: 32 * ds is a
     // power-of-two multiple of ds, so the result is ds * (q - 32) rounded once, the reference's value)
-    static __device__ __forceinline__ void put16(uint8_t* row, int dc, int group0, const u32x4 bytes, float dsv)
+    static __device__ __forceinline__ void put16(const DecodeCtx& c, uint8_t* row, int group0, const u32x4 bytes, float dsv)
     {
         const float off = 32.0f * dsv;
 #pragma unroll
         for (int g = 0; g < 2; ++g)
-            *reinterpret_cast<u32x4*>(row + lds_slot(dc, group0 + g) * 16) = q4k_decode8(bytes[2 * g], bytes[2 * g + 1], dsv, off);
+            st128(c, row + lds_slot(c.dc, group0 + g) * 16, q4k_decode8(bytes[2 * g], bytes[2 * g + 1], dsv, off));
     }
     template <int J>
     __device__ __forceinline__ void make(const DecodeCtx& c, int t, uint8_t* lo, uint8_t* hi)
@@ -293,8 +297,8 @@ struct Q6KDecode {
             lo_b[i] = ((a[i] >> (4 * P)) & 0x0f0f0f0fu) | (((h[i] >> (4 * P)) & 0x03030303u) << 4);
             hi_b[i] = ((b[i] >> (4 * P)) & 0x0f0f0f0fu) | (((h[i] >> (4 * P + 2)) & 0x03030303u) << 4);
         }
-        put16(lo, c.dc, 2 * c.dh, lo_b, ds[4 * H + 2 * P]);
-        put16(hi, c.dc, 2 * c.dh, hi_b, ds[4 * H + 2 * P + 1]);
+        put16(c, lo, 2 * c.dh, lo_b, ds[4 * H + 2 * P]);
+        put16(c, hi, 2 * c.dh, hi_b, ds[4 * H + 2 * P + 1]);
         if (P == 1) load_half(c, (t >> 1) + 2, H);          // this half's registers are free: request the half after next
         if (J == 0) load_tail(c, (t >> 2) + 1);
         if (J == 3) block_scales();
@@ -333,10 +337,10 @@ struct Q8_0Decode {
         const float d = half_bits_to_float(dbits[J & 1]);
         uint8_t* row = c.dh ? hi : lo;
         const u32x4 a = q0[J & 1], b = q1[J & 1];
-        *reinterpret_cast<u32x4*>(row + lds_slot(c.dc, 0) * 16) = decode8(a[0], a[1], d);
-        *reinterpret_cast<u32x4*>(row + lds_slot(c.dc, 1) * 16) = decode8(a[2], a[3], d);
-        *reinterpret_cast<u32x4*>(row + lds_slot(c.dc, 2) * 16) = decode8(b[0], b[1], d);
-        *reinterpret_cast<u32x4*>(row + lds_slot(c.dc, 3) * 16) = decode8(b[2], b[3], d);
+        st128(c, row + lds_slot(c.dc, 0) * 16, decode8(a[0], a[1], d));
+        st128(c, row + lds_slot(c.dc, 1) * 16, decode8(a[2], a[3], d));
+        st128(c, row + lds_slot(c.dc, 2) * 16, decode8(b[0], b[1], d));
+        st128(c, row + lds_slot(c.dc, 3) * 16, decode8(b[2], b[3], d));
         load(c, t + 2, J & 1);
     }
 };
@@ -414,9 +418,8 @@ struct IQ2SDecode {
         for (int o = 0; o < 4; ++o) {
             const uint32_t m0 = grid[J & 1][o][0], m1 = grid[J & 1][o][1], sb = signs >> (8 * o);
             const float db = o < 2 ? db_lo : db_hi;
-            *reinterpret_cast<u32x4*>(row + lds_slot(c.dc, o) * 16) =
-                u32x4{iq_pair(db, ubyte0(m0), ubyte1(m0), sb), iq_pair(db, ubyte2(m0), ubyte3(m0), sb >> 2),
-                      iq_pair(db, ubyte0(m1), ubyte1(m1), sb >> 4), iq_pair(db, ubyte2(m1), ubyte3(m1), sb >> 6)};
+            st128(c, row + lds_slot(c.dc, o) * 16, u32x4{iq_pair(db, ubyte0(m0), ubyte1(m0), sb), iq_pair(db, ubyte2(m0), ubyte3(m0), sb >> 2),
+                      iq_pair(db, ubyte0(m1), ubyte1(m1), sb >> 4), iq_pair(db, ubyte2(m1), ubyte3(m1), sb >> 6)});
         }
         // slice t + 1 belongs to the next block when J == 3
         load_grid<(J + 1) & 3>(c, qs[(J + 1) & 3], J == 3 ? tail_next : tail, grid[(J + 1) & 1]);
@@ -492,9 +495,8 @@ struct IQ3SDecode {
 #pragma unroll
         for (int o = 0; o < 4; ++o) {
             const uint32_t m0 = grid[J & 1][2 * o], m1 = grid[J & 1][2 * o + 1], sb = signs >> (8 * o);
-            *reinterpret_cast<u32x4*>(row + lds_slot(c.dc, o) * 16) =
-                u32x4{iq_pair(db, ubyte0(m0), ubyte1(m0), sb), iq_pair(db, ubyte2(m0), ubyte3(m0), sb >> 2),
-                      iq_pair(db, ubyte0(m1), ubyte1(m1), sb >> 4), iq_pair(db, ubyte2(m1), ubyte3(m1), sb >> 6)};
+            st128(c, row + lds_slot(c.dc, o) * 16, u32x4{iq_pair(db, ubyte0(m0), ubyte1(m0), sb), iq_pair(db, ubyte2(m0), ubyte3(m0), sb >> 2),
+                      iq_pair(db, ubyte0(m1), ubyte1(m1), sb >> 4), iq_pair(db, ubyte2(m1), ubyte3(m1), sb >> 6)});
         }
         load_grid<(J + 1) & 3>(c, qs[(J + 1) & 3], J == 3 ? qh_next : qh, grid[(J + 1) & 1]);
         load_raw(c, t + 3, (J + 3) & 3);
@@ -530,7 +532,7 @@ struct BF16Decode {
     {
         uint8_t* row = c.dh ? hi : lo;
 #pragma unroll
-        for (int g = 0; g < 4; ++g) *reinterpret_cast<u32x4*>(row + lds_slot(c.dc, g) * 16) = q[J & 1][g];
+        for (int g = 0; g < 4; ++g) st128(c, row + lds_slot(c.dc, g) * 16, q[J & 1][g]);
         load(c, t + 2, J & 1);
     }
 };
@@ -581,25 +583,31 @@ __global__ __launch_bounds__(kGemmAll) void matmul_bf16_kernel(GemmArgs a)
             __syncthreads();
             int stage = 2;
             auto next_stage = [&]() { stage = stage == kStages - 1 ? 0 : stage + 1; };
+            // No test on "is there a slice i + 2": the two slices past the end are made from repeated input into stages
+            // that nobody reads any more.  With the calls unconditional the loop is one basic block per role, and the
+            // compiler's wait before a slice's registers are used counts the younger requests as still outstanding
+            // (with branches it waited for all of them, which left one iteration of cover instead of two: at 0.7 us
+            // per iteration, M <= 256, that was the memory latency).
             for (int i = 0; i < iters; i += 4) {
-                if (i + 2 < iters) make(i + 2, stage, integral_constant<int, 2>{});
+                make(i + 2, stage, integral_constant<int, 2>{});
                 next_stage();
                 __syncthreads();
-                if (i + 3 < iters) make(i + 3, stage, integral_constant<int, 3>{});
+                make(i + 3, stage, integral_constant<int, 3>{});
                 next_stage();
                 __syncthreads();
-                if (i + 4 < iters) make(i + 4, stage, integral_constant<int, 0>{});
+                make(i + 4, stage, integral_constant<int, 0>{});
                 next_stage();
                 __syncthreads();
-                if (i + 5 < iters) make(i + 5, stage, integral_constant<int, 1>{});
+                make(i + 5, stage, integral_constant<int, 1>{});
                 next_stage();
                 __syncthreads();
             }
         };
 
         if (p >= kDecoders) {
-            // ---- x movers (waves 13-15): piece q of a slice = row q / 8 of the tile, 16-byte group q % 8 of its 64
-            // values; a thread moves pieces xp, xp + 192, ...
+            // ---- x movers (waves 13-15): a piece is one 16-byte group (8 of the 64 values) of one row of the tile; a
+            // thread moves pieces xp, xp + 192, ...  Within a wave's 64 pieces (8 rows x 8 groups) a quarter-wave takes
+            // 4 rows x 4 groups of one sub-tile: 256 contiguous bytes of LDS, every bank once.
             constexpr int kXPieces = 2 * kXTile / 16;
             constexpr int kXLoads = (kXPieces + kXThreads - 1) / kXThreads;
             const int xp = p - kDecoders;
@@ -609,7 +617,8 @@ __global__ __launch_bounds__(kGemmAll) void matmul_bf16_kernel(GemmArgs a)
 #pragma unroll
             for (int i = 0; i < kXLoads; ++i) {
                 const int q = min(xp + i * kXThreads, kXPieces - 1);       // the last round is partly idle (not stored)
-                const int r = q >> 3, grp = q & 7;
+                const int l = q & 63, quarter = l >> 4, within = l & 15;
+                const int r = (q >> 6) * 8 + (quarter >> 1) * 4 + (within >> 2), grp = (quarter & 1) * 4 + (within & 3);
                 xsrc[i] = static_cast<uint32_t>((min(r, a.M - 1 - m0) * a.K + grp * 8) * 2);
                 xdst[i] = (grp >> 2) * kXTile + r * kRowBytes + lds_slot(r, grp & 3) * 16;
             }
@@ -629,7 +638,8 @@ __global__ __launch_bounds__(kGemmAll) void matmul_bf16_kernel(GemmArgs a)
                 uint8_t* xb = xs + stage * 2 * kXTile;
 #pragma unroll
                 for (int i = 0; i < kXLoads; ++i)
-                    if (xp + i * kXThreads < kXPieces) *reinterpret_cast<u32x4*>(xb + xdst[i]) = set[i];
+                    if ((i + 1) * kXThreads <= kXPieces || xp + i * kXThreads < kXPieces)
+                        *reinterpret_cast<u32x4*>(xb + xdst[i]) = set[i];
                 load_x(set, t + 2);
             });
             return;
@@ -639,7 +649,10 @@ __global__ __launch_bounds__(kGemmAll) void matmul_bf16_kernel(GemmArgs a)
         static_assert(2 * BN <= kDecoders, "two decoding threads per column");
         const int row_bytes = (a.K >> 8) * F::kBlockBytes;
         const bool d_role = p < 2 * BN;
+        if ((p & ~63) >= 2 * BN) return;        // a whole wave without columns: ended waves do not count at barriers
+
         DecodeCtx c;
+        c.live = d_role;
         c.dc = d_role ? p >> 1 : 0;
         c.dh = p & 1;
         c.wbase = a.w + static_cast<size_t>(n0) * row_bytes;                               // wave-uniform
@@ -650,7 +663,6 @@ __global__ __launch_bounds__(kGemmAll) void matmul_bf16_kernel(GemmArgs a)
         dec.start(c);
         run([&](int t, int stage, auto jt) {
             constexpr int J = decltype(jt)::value;
-            if (!d_role) return;
             uint8_t* wb = ws + stage * 2 * kWTile + c.dc * kRowBytes;
             dec.template make<J>(c, t, wb, wb + kWTile);
         });
@@ -660,7 +672,8 @@ __global__ __launch_bounds__(kGemmAll) void matmul_bf16_kernel(GemmArgs a)
     // ---------------------------------------------------------------------------------------------- consumers
     // waves w and w + 4 usually share a SIMD: giving them different column halves balances the matrix pipes
     if constexpr (BM > 128) __builtin_amdgcn_s_setprio(3);
-    const int wm = wave % WM, wn = wave / WM;
+    const int uwave = __builtin_amdgcn_readfirstlane(wave);     // wave-uniform values stay in scalar registers
+    const int wm = uwave % WM, wn = uwave / WM;
     const int ct0 = wn * CTW;                       // this wave's column tiles start here
     // operand address of this lane inside a 16-row tile: row lane % 16, k-group lane / 16
     const int frag = (lane & 15) * kRowBytes + lds_slot(lane & 15, lane >> 4) * 16;
@@ -678,43 +691,59 @@ __global__ __launch_bounds__(kGemmAll) void matmul_bf16_kernel(GemmArgs a)
         const uint8_t* xrow = xs + wm * RW * kRowBytes + frag;
         const uint8_t* wcol = ws + ct0 * 16 * kRowBytes + frag;
         __syncthreads();        // tiles 0 and 1 are ready
-        // Operand fetches run ahead of the matrix instructions that use them: a weight fragment is read one tile ahead
-        // (two registers sets alternate), the x fragments of a half-slice while the previous half is multiplied, and
-        // both continue across the barrier into the next slice, which was completed one iteration earlier.  The
-        // scheduling barriers keep the compiler from sinking the reads back down to their first use.
-        bf16x8 afrag[MT], afrag1[MT], bfrag[2];
+        // Operand fetches run ahead of the matrix instructions that use them, also across the barrier into the next
+        // slice, which was completed one iteration earlier: the x fragments of a half-slice are read while the previous
+        // half is multiplied.  The scheduling barriers keep the compiler from sinking the reads down to their first use.
+        static_assert(kStages == 3, "the slice phase below is also the LDS stage");
+        // Weight fragments in a ring of three, read two tiles ahead of their use.  The ring position of a slice's
+        // first tile and the LDS stage both repeat every three slices, so the loop is unrolled by three and both
+        // are compile-time constants; one or two more slices follow when K / 64 is not a multiple of three.
+        constexpr int kTiles = 2 * NT;
+        bf16x8 afrag[MT], afrag1[MT], bq[3];
+        auto tile_at = [&](const uint8_t* w, int u) { return w + (u / NT) * kWTile + (u % NT) * 16 * kRowBytes; };
+#pragma unroll
+        for (int u = 0; u < 2; ++u) bq[u] = *reinterpret_cast<const bf16x8*>(tile_at(wcol, u));
 #pragma unroll
         for (int i = 0; i < MT; ++i) afrag[i] = *reinterpret_cast<const bf16x8*>(xrow + i * 16 * kRowBytes);
-        bfrag[0] = *reinterpret_cast<const bf16x8*>(wcol);
-        int stage = 0;
-        for (int it = 0; it < iters; ++it) {
-            const uint8_t* xb = xrow + stage * 2 * kXTile;
-            const uint8_t* wb = wcol + stage * 2 * kWTile;
-            const int nstage = stage == kStages - 1 ? 0 : stage + 1;
-            const uint8_t* xn = xrow + nstage * 2 * kXTile;
-            const uint8_t* wn_ = wcol + nstage * 2 * kWTile;
+        auto slice = [&](auto phase) {
+            constexpr int P = decltype(phase)::value;         // iteration % 3 = LDS stage
+            constexpr int PN = (P + 1) % kStages;
+            const uint8_t* xb = xrow + P * 2 * kXTile;
+            const uint8_t* wb = wcol + P * 2 * kWTile;
+            const uint8_t* xn = xrow + PN * 2 * kXTile;
+            const uint8_t* wn_ = wcol + PN * 2 * kWTile;
 #pragma unroll
-            for (int i = 0; i < MT; ++i) afrag1[i] = *reinterpret_cast<const bf16x8*>(xb + kXTile + i * 16 * kRowBytes);
+            for (int t = 0; t < kTiles; ++t) {
+                constexpr int kShift = P * (kTiles % 3);
+                const int slot = (kShift + t) % 3;
+                bq[(slot + 2) % 3] = *reinterpret_cast<const bf16x8*>(t + 2 < kTiles ? tile_at(wb, t + 2) : tile_at(wn_, t + 2 - kTiles));
+                if (t == 0) {
 #pragma unroll
-            for (int t = 0; t < 2 * NT; ++t) {
-                // tile t: columns t % NT of half-slice t / NT; fetch tile t + 1 (or the next slice's first) meanwhile
-                const uint8_t* nb = t + 1 < NT ? wb + (t + 1) * 16 * kRowBytes
-                                    : t + 1 < 2 * NT ? wb + kWTile + (t + 1 - NT) * 16 * kRowBytes : wn_;
-                bfrag[(t + 1) & 1] = *reinterpret_cast<const bf16x8*>(nb);
+                    for (int i = 0; i < MT; ++i) afrag1[i] = *reinterpret_cast<const bf16x8*>(xb + kXTile + i * 16 * kRowBytes);
+                }
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int i = 0; i < MT; ++i)
-                    acc[i][t % NT] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(t < NT ? afrag[i] : afrag1[i], bfrag[t & 1],
-                                                                             acc[i][t % NT], 0, 0, 0);
+                    acc[i][t % NT] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(t < NT ? afrag[i] : afrag1[i], bq[slot], acc[i][t % NT], 0, 0, 0);
                 if (t == NT - 1) {
 #pragma unroll
                     for (int i = 0; i < MT; ++i) afrag[i] = *reinterpret_cast<const bf16x8*>(xn + i * 16 * kRowBytes);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
-            stage = nstage;
             __syncthreads();
+        };
+        int it = 0;
+        for (; it + 3 <= iters; it += 3) {
+            slice(std::integral_constant<int, 0>{});
+            slice(std::integral_constant<int, 1>{});
+            slice(std::integral_constant<int, 2>{});
         }
-        // accumulator element v of a tile: row 4 * (lane / 16) + v, column lane % 16
+        if (it < iters) slice(std::integral_constant<int, 0>{});
+        if (it + 1 < iters) slice(std::integral_constant<int, 1>{});
+        // accumulator element v of a tile: row 4 * (lane / 16) + v, column lane % 16.  (The lane number is taken
+        // afresh so that nothing derived from it occupies a register during the loop.)
+        const int lane = static_cast<int>(__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)));
 #pragma unroll
         for (int j = 0; j < NT; ++j) {
             const int cn = (ct0 + j) * 16 + (lane & 15);

@@ -931,9 +931,9 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
     const uint8_t* const a_zeros = diag ? nullptr : zero_area;
 
     // Turns the activations of matrix c_m (its `rows` input rows) into digit planes and sums in LDS; two barriers.
-    // Every wave has left the stage that last read the planes when this runs.  (A variant that requested all rows at once
-    // into registers, one trip to memory instead of two per row, made the compiler wait for every outstanding load
-    // before each parking write of the main loop: 12.6 instead of 8.6 us per 17408-wide Q4_K mat-vec.  Not kept.)
+    // Every wave has left the stage that last read the planes when this runs.  (Requesting the whole vector at once into
+    // registers, one trip to memory instead of two, made the compiler wait for every outstanding load before each
+    // parking write of the main loop in the one-row form: 12.6 instead of 8.6 us per 17408-wide Q4_K mat-vec.)
     auto prepare_x = [&]() {
         auto umax4 = [](uint32_t m, const float4& v) {
             m = umax_u(m, __float_as_uint(v.x) & 0x7fffffffu);
@@ -942,6 +942,81 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
             return umax_u(m, __float_as_uint(v.w) & 0x7fffffffu);
         };
         const int rows = ce.rows;
+        // With shared passes the rows are requested together when they fit kPrep float4 per lane (one trip to memory
+        // instead of two per row: 1.5 us of a 30 us call); the one-row form keeps the loops (see above).
+        // (Not with four tiles in flight per wave: the registers do not hold both.)
+        constexpr int kPrep = R > 1 && LPW <= 3 ? 8 : 0;
+        if (kPrep > 0 && rows * n4 <= kPrep * T) {
+            float4 xr[kPrep > 0 ? kPrep : 1];
+            const float4* x4 = reinterpret_cast<const float4*>(ce.x);      // the rows are consecutive: x4[r * n4 + i]
+            auto row_of = [&](int j) {                                      // wave-uniform (n4 % 64 == 0); -1 past the last row
+                const int f0 = (tid & ~63) + j * T;
+                const int r = (f0 >= n4) + (f0 >= 2 * n4) + (f0 >= 3 * n4);
+                return f0 >= rows * n4 ? -1 : __builtin_amdgcn_readfirstlane(r);
+            };
+#pragma unroll
+            for (int j = 0; j < kPrep; ++j) xr[j] = x4[row_of(j) >= 0 ? tid + j * T : 0];
+            uint32_t mx[R] = {};
+#pragma unroll
+            for (int j = 0; j < kPrep; ++j) {
+                const int rj = row_of(j);
+                const uint32_t m = umax4(0u, xr[j]);
+#pragma unroll
+                for (int r = 0; r < R; ++r) mx[r] = rj == r ? umax_u(mx[r], m) : mx[r];
+            }
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                if (r < rows) {
+                    const uint32_t m = wave_umax(mx[r]);
+                    if (lane == 0) red[r][wave] = m;
+                }
+            }
+            __syncthreads();
+            float scale[R] = {};
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                if (r < rows) {
+                    uint32_t m = 0;
+                    for (int i = 0; i < W; ++i) m = umax_u(m, red[r][i]);
+                    const int E = static_cast<int>(m >> 23);
+                    int e = 156 - E;
+                    e = e > 126 ? 126 : e;
+                    scale[r] = __uint_as_float(static_cast<uint32_t>(e + 127) << 23);
+                    inv[r] = E == 255 ? __uint_as_float(0x7fc00000u) : __uint_as_float(static_cast<uint32_t>(127 - e) << 23);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < kPrep; ++j) {
+                const int rj = row_of(j);
+                if (rj >= 0) {
+                    float sc = scale[0];
+#pragma unroll
+                    for (int r = 1; r < R; ++r) sc = rj == r ? scale[r] : sc;
+                    const int i = tid + j * T - rj * n4;
+                    const float4 v = xr[j];
+                    uint8_t* set = planes + rj * g.set_bytes;
+                    float* sumx = reinterpret_cast<float*>(set + 4 * g.plane_stride);
+                    uint32_t pl[4];
+                    digit_planes(__float2int_rn(v.x * sc), __float2int_rn(v.y * sc), __float2int_rn(v.z * sc), __float2int_rn(v.w * sc), pl);
+#pragma unroll
+                    for (int p = 0; p < 4; ++p) *reinterpret_cast<uint32_t*>(set + p * g.plane_stride + 4 * i) = pl[p];
+                    float s = (v.x + v.y) + (v.z + v.w);
+                    if (!F::kNeedsSums) {
+                    } else if (F::kSumRun == 32) {
+                        s = oct_sum(s);
+                        if ((i & 7) == 0) sumx[i >> 3] = s;
+                    } else {
+                        s += dpp_mov<0xB1>(s);
+                        s += dpp_mov<0x4E>(s);
+                        if ((i & 3) == 0) sumx[i >> 2] = s;
+                    }
+                }
+            }
+            planes_x = ce.x;
+            planes_rows = rows;
+            __syncthreads();
+            return;
+        }
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             if (r < rows) {
