@@ -1324,41 +1324,53 @@ const uint32_t kBatchTypeOrder[kBatchTypes] = {NNHIP_TYPE_Q8_0, NNHIP_TYPE_Q4_K,
 // entry: they are launched one by one.
 static_assert(sizeof(MfmaTableEntry) == sizeof(BatchEntry), "both kinds of entry fill one table slot");
 
-long build_batch(const nnhip_matvec_desc* descs, int count, BatchEntry* out, size_t cap, BatchGroup* groups, int* ngroups)
+long build_batch(const nnhip_matvec_desc* descs, int count, BatchEntry* out, size_t cap, BatchGroup* groups, int* ngroups,
+                 uint8_t* forms)
 {
     size_t n = 0;
     *ngroups = 0;
     // matrix-core groups first: per (type, in_w, form) with enough tiles.  Forms: 1 = operand A in registers (in_w splits
     // into one or two whole stages), 2 = the wide form with one input row per entry, 3 = the wide form with up to four
-    // input rows of a descriptor sharing a pass (descriptors with rows >= 2).
-    auto form_of = [&](const nnhip_matvec_desc& d) {
-        if (d.rows >= 2 && matvec_mfma_wide_geometry(d.ggml_type, d.in_w, d.out_w, d.w, 4)) return 3;
-        if (matvec_mfma_geometry(d.ggml_type, d.in_w, d.out_w, d.w, nullptr)) return 1;
-        if (matvec_mfma_wide_geometry(d.ggml_type, d.in_w, d.out_w, d.w, 1)) return 2;
-        return 0;
-    };
-    auto same_group = [&](const nnhip_matvec_desc& p, int form, const nnhip_matvec_desc& d) {
-        return d.ggml_type == p.ggml_type && d.in_w == p.in_w && form_of(d) == form;
-    };
-    auto in_mfma_group = [&](const nnhip_matvec_desc& d, int form) {
-        if (!form) return false;
-        long tiles = 0;
-        for (int j = 0; j < count; ++j)
-            if (same_group(d, form, descs[j])) tiles += static_cast<long>(descs[j].rows) * ((descs[j].out_w + 15) / 16);
-        return tiles >= kMfmaBatchMinTiles;
+    // input rows of a descriptor sharing a pass (descriptors with rows >= 2).  `forms` is `count` bytes of scratch: the
+    // form of every descriptor is worked out once (a model's batch has hundreds of descriptors).
+    for (int i = 0; i < count; ++i) {
+        const nnhip_matvec_desc& d = descs[i];
+        int form = 0;
+        if (d.rows >= 2 && matvec_mfma_wide_geometry(d.ggml_type, d.in_w, d.out_w, d.w, 4)) form = 3;
+        else if (matvec_mfma_geometry(d.ggml_type, d.in_w, d.out_w, d.w, nullptr)) form = 1;
+        else if (matvec_mfma_wide_geometry(d.ggml_type, d.in_w, d.out_w, d.w, 1)) form = 2;
+        forms[i] = static_cast<uint8_t>(form);
+    }
+    struct Key { uint32_t type; int in_w, form; long tiles; };
+    Key keys[kBatchGroupsMax - kBatchTypes];
+    int nkeys = 0;
+    auto key_of = [&](int i) {
+        for (int k = 0; k < nkeys; ++k)
+            if (keys[k].type == descs[i].ggml_type && keys[k].in_w == descs[i].in_w && keys[k].form == forms[i]) return k;
+        return -1;
     };
     for (int i = 0; i < count; ++i) {
-        const nnhip_matvec_desc& lead = descs[i];
-        const int form = form_of(lead);
-        if (!in_mfma_group(lead, form)) continue;
-        bool seen = false;
-        for (int j = 0; j < i; ++j) seen = seen || same_group(lead, form, descs[j]);
-        if (seen) continue;
-        if (*ngroups >= kBatchGroupsMax - kBatchTypes) break;      // (further groups stay with the row-step kernel)
-        BatchGroup g{lead.ggml_type, n, n, 0, lead.in_w, form};
-        for (int j = i; j < count; ++j) {
+        if (!forms[i]) continue;
+        int k = key_of(i);
+        if (k < 0) {
+            if (nkeys == kBatchGroupsMax - kBatchTypes) {      // (further kinds stay with the row-step kernel)
+                forms[i] = 0;
+                continue;
+            }
+            k = nkeys++;
+            keys[k] = Key{descs[i].ggml_type, descs[i].in_w, forms[i], 0};
+        }
+        keys[k].tiles += static_cast<long>(descs[i].rows) * ((descs[i].out_w + 15) / 16);
+    }
+    for (int i = 0; i < count; ++i)
+        if (forms[i] && keys[key_of(i)].tiles < kMfmaBatchMinTiles) forms[i] = 0;
+    for (int k = 0; k < nkeys; ++k) {
+        if (keys[k].tiles < kMfmaBatchMinTiles) continue;
+        const int form = keys[k].form;
+        BatchGroup g{keys[k].type, n, n, 0, keys[k].in_w, form};
+        for (int j = 0; j < count; ++j) {
             const nnhip_matvec_desc& d = descs[j];
-            if (!same_group(lead, form, d)) continue;
+            if (forms[j] != form || d.ggml_type != keys[k].type || d.in_w != keys[k].in_w) continue;
             const int share = form == 3 ? 4 : 1;
             for (int r = 0; r < d.rows; r += share) {
                 if (n >= cap) return -1;
@@ -1372,13 +1384,6 @@ long build_batch(const nnhip_matvec_desc* descs, int count, BatchEntry* out, siz
         g.end = n;
         groups[(*ngroups)++] = g;
     }
-    auto taken = [&](const nnhip_matvec_desc& d) {
-        const int form = form_of(d);
-        for (int k = 0; k < *ngroups; ++k)
-            if (groups[k].mfma && groups[k].mfma == form && groups[k].type == d.ggml_type && groups[k].max_in_w == d.in_w) return true;
-        return false;
-    };
-    const int mfma_groups = *ngroups;
     for (uint32_t type : kBatchTypeOrder) {
         BatchGroup g{type, n, n, 0, 0, 0};
         int max_t = 0, depth = 0;
@@ -1389,7 +1394,7 @@ long build_batch(const nnhip_matvec_desc* descs, int count, BatchEntry* out, siz
             const nnhip_matvec_desc& d = descs[i];
             if (d.ggml_type != type) continue;
             if (type == NNHIP_TYPE_Q8_0 && ((d.in_w / 32) & 1)) continue;
-            if (mfma_groups && taken(d)) continue;
+            if (forms[i]) continue;                       // in a matrix-core group
             const int upr = d.in_w / kUnitW;
             int rs = max_t / upr;
             if (rs > d.out_w) rs = d.out_w;
@@ -1469,9 +1474,10 @@ hipError_t launch_matvec_batch(Lane* lane, const nnhip_matvec_desc* descs, int c
     size_t cap = 0;
     for (int i = 0; i < count; ++i) cap += static_cast<size_t>(descs[i].rows);
     std::vector<BatchEntry> all(cap);
+    std::vector<uint8_t> forms(static_cast<size_t>(count > 0 ? count : 1));
     BatchGroup groups[kBatchGroupsMax];
     int ngroups = 0;
-    const long n = build_batch(descs, count, all.data(), cap, groups, &ngroups);
+    const long n = build_batch(descs, count, all.data(), cap, groups, &ngroups, forms.data());
     if (n < 0) return hipErrorInvalidValue;
     const size_t bytes = static_cast<size_t>(n) * sizeof(BatchEntry);
     if (bytes) {
@@ -1518,10 +1524,12 @@ hipError_t static_table_address(void** address)
 hipError_t launch_matvec_batch_static(Lane* lane, const nnhip_matvec_desc* descs, int count)
 {
     if (!lane->static_table) return hipErrorNotInitialized;
+    if (count > kStaticTableEntries) return hipErrorInvalidValue;       // (every descriptor takes at least one entry)
     BatchEntry entries[kStaticTableEntries];
+    uint8_t forms[kStaticTableEntries];
     BatchGroup groups[kBatchGroupsMax];
     int ngroups = 0;
-    const long n = build_batch(descs, count, entries, kStaticTableEntries, groups, &ngroups);
+    const long n = build_batch(descs, count, entries, kStaticTableEntries, groups, &ngroups, forms);
     if (n < 0) return hipErrorInvalidValue;
     if (n > 0) {
         const hipError_t e = write_table(lane, lane->static_table, entries, static_cast<size_t>(n));

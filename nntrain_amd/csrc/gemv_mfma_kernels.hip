@@ -407,6 +407,64 @@ struct Q6KTask {
     }
 };
 
+// Q8_0: w = d * q with 32 signed bytes q after a half-precision d, 34 bytes per 32 weights.  Eight such blocks are the
+// 256 weights of one block column here: 272 bytes = 17 pieces exactly, and rows are whole columns (in_w % 256 == 0), so
+// columns, rows and stages start on piece boundaries.  Quarter P = blocks 2P and 2P + 1 = the 68 bytes at 68 P of the
+// column: 17 dwords, of which a lane's 16 rows x 4 quarters fall into 64 different LDS banks (row stride 205 or 103
+// pieces).  The quants are the bytes of operand B as they are; those of the first block sit two bytes into their dwords
+// (v_alignbyte_b32), those of the second on dword boundaries.  No minima, no offset: no sums of x.
+struct Q8_0Task {
+    static constexpr int kBlockBytes = 8 * kQ8_0Bytes;
+    static constexpr int kPieces = 17;
+    static constexpr int kSumRun = 32;
+    static constexpr int kWideM = 1;
+    static constexpr int kWideLpw = 5;
+    static constexpr bool kNeedsSums = false;
+    static constexpr bool kTightStage = true;
+    static constexpr int kSharedM = 0, kSharedLpw = 0;     // (no shared passes: rows of a call are entries of their own)
+    static __device__ __forceinline__ void init_tables(uint8_t*, int, int) {}
+    using X = XSet<1>;
+    struct Raw { uint32_t w[17]; };
+
+    static __device__ __forceinline__ uint32_t piece_src(uint32_t q, bool) { return 16u * q; }
+
+    static __device__ __forceinline__ void load_x(X& xs, const uint8_t* plane, const float*, int b, int quarter, const uint8_t* zeros)
+    {
+        const uint8_t* src = zeros ? zeros : plane + 256 * b + 64 * quarter;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) xs.a[u] = lds128(src + 16 * u);
+    }
+
+    static __device__ __forceinline__ Raw load(const uint8_t* blk, int quarter, bool)
+    {
+        Raw r;
+        const uint32_t* src = reinterpret_cast<const uint32_t*>(blk + 68 * quarter);
+#pragma unroll
+        for (int i = 0; i < 17; ++i) r.w[i] = src[i];
+        return r;
+    }
+
+    static __device__ __forceinline__ void run(const Raw& r, const X& xs, int, const uint8_t*, float& accq, float&)
+    {
+        const u32x4 a0 = xs.a[0], a1 = xs.a[1], a2 = xs.a[2], a3 = xs.a[3];
+        uint32_t q0[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) q0[i] = __builtin_amdgcn_alignbyte(r.w[i + 1], r.w[i], 2);
+        i32x4 s0 = {0, 0, 0, 0}, s1 = {0, 0, 0, 0};
+        s0 = mfma_i8(a0[0], a0[1], q0[0], q0[1], s0);
+        s1 = mfma_i8(a2[0], a2[1], r.w[9], r.w[10], s1);
+        s0 = mfma_i8(a0[2], a0[3], q0[2], q0[3], s0);
+        s1 = mfma_i8(a2[2], a2[3], r.w[11], r.w[12], s1);
+        s0 = mfma_i8(a1[0], a1[1], q0[4], q0[5], s0);
+        s1 = mfma_i8(a3[0], a3[1], r.w[13], r.w[14], s1);
+        s0 = mfma_i8(a1[2], a1[3], q0[6], q0[7], s0);
+        s1 = mfma_i8(a3[2], a3[3], r.w[15], r.w[16], s1);
+        // |plane sum| <= 32 * 128 * 128 = 2^19: the pair sums of recombine() stay inside int32, each rounds once in FP32
+        accq = fmaf(half_bits_to_float(r.w[0]), recombine(s0), accq);
+        accq = fmaf(half_bits_to_float(r.w[8] >> 16), recombine(s1), accq);
+    }
+};
+
 // IQ2_S (NNtrain.Arc/Kernels/qwen35_iq.cl:411-419): 82 bytes = d (fp16), 32 index bytes, 32 sign bytes, 8 bytes of index
 // tops (two bits per eight weights), 8 bytes of 4-bit scales (one per 16 weights).  Eight weights are one entry of a
 // 1024-entry codebook of magnitude bytes (8, 25 or 43) with a sign bit each; w = d * (0.5 + scale) * 0.25 * magnitude *
@@ -825,6 +883,7 @@ struct WideArgs {
     int nblocks;
     uint32_t row_bytes;
     uint32_t row_pieces_magic;
+    int chunked;                   // 1: a workgroup takes consecutive tiles (few changes of activations), 0: every G-th
     WideGeom g;
     MfmaEntry inline_entries[4];   // a call with up to 16 input rows needs no table in device memory
 };
@@ -880,22 +939,48 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
         in_stage |= (r < static_cast<uint32_t>(kTileRows) ? 1u : 0u) << i;
     }
 
-    const int G = gridDim.x;
-    const int my_tiles = (a.total_tiles - static_cast<int>(blockIdx.x) + G - 1) / G;
+    // ---- this workgroup's tiles of the launch's tile sequence: every G-th, or a run of consecutive ones.  Runs are for
+    // launches whose matrices all have activations of their own (a workgroup then meets two or three vectors instead
+    // of all of them); the bits of a row are the same either way.
+    const int G = gridDim.x, bid = blockIdx.x;
+    int my_tiles, t_first, t_step;
+    if (a.chunked) {
+        const int per = a.total_tiles / G, rem = a.total_tiles - per * G;
+        my_tiles = per + (bid < rem ? 1 : 0);
+        t_first = bid * per + (bid < rem ? bid : rem);
+        t_step = 1;
+    } else {
+        my_tiles = (a.total_tiles - bid + G - 1) / G;
+        t_first = bid;
+        t_step = G;
+    }
+    const int t_end = a.chunked ? t_first + my_tiles : a.total_tiles;       // no requests from here on
     const int total = my_tiles * KC;
     const uint32_t chunk_bytes = static_cast<uint32_t>(g.cols) * F::kBlockBytes;
     const int n4 = a.in_w >> 2;
 
     // ---- prefetch side
-    int f_t = blockIdx.x, f_k = 0, f_m = 0;
-    MfmaEntry fe = entry_at(0);
+    int f_t = t_first, f_k = 0, f_m = 0;
+    if (a.chunked && my_tiles > 0) {
+        // the entry that holds this workgroup's first tile: the last one whose first_tile is not beyond it (a run may
+        // start hundreds of entries into the table, and walking there costs a trip to memory per entry)
+        int lo = 0, hi = a.entries - 1;
+        while (lo < hi) {
+            const int mid = (lo + hi + 1) >> 1;
+            if (table[mid].first_tile <= t_first) lo = mid;
+            else hi = mid - 1;
+        }
+        f_m = lo;
+    }
+    const int m_first = f_m;
+    MfmaEntry fe = entry_at(f_m);
     __amdgpu_buffer_rsrc_t f_matrix;
     auto fetch_enter = [&]() {
         while (f_t >= fe.first_tile + fe.tiles && f_m + 1 < a.entries) fe = entry_at(++f_m);
         f_matrix = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(fe.w), 0, static_cast<int>(fe.w_bytes), 0x00020000);
     };
     auto fetch = [&](u32x4 (&set)[LPW]) {
-        const uint32_t base = f_t < a.total_tiles
+        const uint32_t base = f_t < t_end
             ? static_cast<uint32_t>(f_t - fe.first_tile) * kTileRows * a.row_bytes + static_cast<uint32_t>(f_k) * chunk_bytes
             : kNoPiece;
         const bool tail = f_k == KC - 1;
@@ -903,8 +988,8 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
         for (int i = 0; i < LPW; ++i) set[i] = stream16(f_matrix, tail && !((in_tail >> i) & 1u) ? kNoPiece : base + rel[i]);
         if (++f_k == KC) {
             f_k = 0;
-            f_t += G;
-            if (f_t < a.total_tiles && f_t >= fe.first_tile + fe.tiles) fetch_enter();
+            f_t += t_step;
+            if (f_t < t_end && f_t >= fe.first_tile + fe.tiles) fetch_enter();
         }
     };
     auto park = [&](uint8_t* buf, const u32x4 (&set)[LPW]) {
@@ -921,7 +1006,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
     uint8_t* const planes = smem + 2 * g.stage_bytes;
     uint8_t* const tables = planes + R * g.set_bytes;      // the format's lookup tables (published by the first barrier)
     F::init_tables(tables, tid, T);
-    int c_t = blockIdx.x, c_k = 0, c_m = -1;
+    int c_t = t_first, c_k = 0, c_m = m_first - 1;      // (ce.tiles == 0: the first stage enters entry m_first)
     MfmaEntry ce{};
     float inv[R] = {};
     const float* planes_x = nullptr;       // the vector(s) the planes in LDS were made from
@@ -1161,7 +1246,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
             done_row0 = (c_t - ce.first_tile) * kTileRows;
             done_rows = ce.out_w - done_row0 < kTileRows ? ce.out_w - done_row0 : kTileRows;
             pbuf ^= 1;
-            c_t += G;
+            c_t += t_step;
         }
         park(nxt, landing);
         __syncthreads();
@@ -1255,6 +1340,7 @@ int block_bytes_of(uint32_t type)
     case NNHIP_TYPE_Q5_K: return Q5KTask::kBlockBytes;
     case NNHIP_TYPE_Q6_K: return Q6KTask::kBlockBytes;
     case NNHIP_TYPE_IQ2_S: return IQ2STask::kBlockBytes;
+    case NNHIP_TYPE_Q8_0: return Q8_0Task::kBlockBytes;
     default: return 0;
     }
 }
@@ -1266,6 +1352,7 @@ int block_pieces_of(uint32_t type)
     case NNHIP_TYPE_Q5_K: return Q5KTask::kPieces;
     case NNHIP_TYPE_Q6_K: return Q6KTask::kPieces;
     case NNHIP_TYPE_IQ2_S: return IQ2STask::kPieces;
+    case NNHIP_TYPE_Q8_0: return Q8_0Task::kPieces;
     default: return 0;
     }
 }
@@ -1290,6 +1377,7 @@ WideTraits wide_traits(uint32_t type, bool shared)
         t.table_bytes = IQ2STask::kTableBytes;
         return t;
     }
+    case NNHIP_TYPE_Q8_0: return shared ? WideTraits{0, 0, 0, 0, false, false} : wide_traits_of<Q8_0Task>(false);
     default: return {0, 0, 0, 0, false, false};
     }
 }
@@ -1323,7 +1411,8 @@ bool plan_wide(uint32_t type, int in_w, int inputs, WideGeom* out)
         if (g.lds_bytes + kWideStaticLds > static_cast<size_t>(160 * 1024)) continue;
         const double fill = static_cast<double>(nblocks) / (g.kchunks * g.cols);
         // (throughput grows with the waves: a stage holds W * M blocks per row and W tasks run side by side)
-        const double score = fill * W / 12.0 * (W % 4 == 0 ? 1.0 : 0.95);
+        // (and of two equal products the fuller stages win: 16 blocks go as 2 x 8 rather than 12 + 4)
+        const double score = fill * W / 12.0 * (W % 4 == 0 ? 1.0 : 0.95) * (0.9 + 0.1 * fill);
         if (score > best_score) {
             best_score = score;
             best = g;
@@ -1391,7 +1480,7 @@ MfmaTableEntry matvec_mfma_entry(uint32_t type, const float* x, const void* w, c
 
 bool matvec_mfma_geometry(uint32_t type, int in_w, int out_w, const void* w, MfmaPlan* plan)
 {
-    if (type == NNHIP_TYPE_IQ2_S) return false;            // (the codebook format has the wide form only)
+    if (type == NNHIP_TYPE_IQ2_S || type == NNHIP_TYPE_Q8_0) return false;       // (these have the wide form only)
     if (!entry_ok(type, in_w, out_w, w)) return false;
     MfmaGeom g;
     if (!plan_mfma(block_pieces_of(type), in_w, block_bytes_of(type) % 16 != 0, &g)) return false;
@@ -1445,6 +1534,10 @@ hipError_t launch_wide_args(Lane* lane, uint32_t type, int in_w, int inputs, Wid
     case NNHIP_TYPE_Q5_K: return launch_wide<Q5KTask>(lane, a, inputs);
     case NNHIP_TYPE_Q6_K: return launch_wide<Q6KTask>(lane, a, inputs);
     case NNHIP_TYPE_IQ2_S: return launch_wide<IQ2STask>(lane, a, inputs);
+    case NNHIP_TYPE_Q8_0:
+        if (inputs != 1) return hipErrorInvalidValue;
+        a.chunked = 1;          // (Q8_0 launches are whole models: hundreds of matrices, most with a vector of their own)
+        return launch_wide_of<Q8_0Task, 1>(lane, a);
     default: return hipErrorInvalidValue;
     }
 }
