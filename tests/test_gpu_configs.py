@@ -353,9 +353,9 @@ def _batch_run(lane, items):
     return out
 
 
-@pytest.mark.parametrize("typ", [GGML_Q4_K, GGML_Q5_K, GGML_Q6_K])
+@pytest.mark.parametrize("typ", [GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_Q8_0])
 def test_large_batched_groups_on_the_matrix_cores(lane, typ):
-    """Groups of Q4_K / Q5_K / Q6_K matrices with at least 2048 sixteen-row tiles go to the matrix-core mat-vec: against the
+    """Groups of Q4_K / Q5_K / Q6_K / Q8_0 matrices with at least 2048 sixteen-row tiles go to the matrix-core mat-vec: against the
     float64 oracle at both bars, with bias, ragged row counts, several input rows, activations that change and repeat
     from matrix to matrix, and two widths in one call (two launches).  A row's bits must not depend on the other
     matrices of the call or on its place in it."""
@@ -406,10 +406,11 @@ def test_large_batched_groups_on_the_matrix_cores(lane, typ):
     lane.trim()
 
 
-def test_large_batched_group_special_activations(lane):
+@pytest.mark.parametrize("typ", [GGML_Q4_K, GGML_Q8_0])
+def test_large_batched_group_special_activations(lane, typ):
     """All-zero activations give the bias; one NaN or infinity makes every output of that matrix NaN, as a floating-point
     dot product would; a huge outlier among the activations must not cost the small ones their accuracy."""
-    typ, in_w, out_w = GGML_Q4_K, 5120, 17408
+    in_w, out_w = 5120, 17408
     payload = synth.matrix(typ, out_w, in_w, seed=77)
     wd = lane.upload_raw(payload)
     bias = np.random.default_rng(3).standard_normal(out_w).astype(np.float32)
@@ -432,6 +433,54 @@ def test_large_batched_group_special_activations(lane):
         it["yd"].dispose()
     wd.dispose()
     bd.dispose()
+    lane.trim()
+
+
+def test_q8_0_model_sized_groups_on_the_matrix_cores(lane):
+    """Q8_0 groups of every row length class the matrix-core form plans differently (21504: six waves beside 86 KB of
+    activation planes, 17408: eight, 5376: twelve with a shorter last stage, 4096: two full stages of eight, 1024: four
+    waves), each with more than 2048 tiles so that workgroups take runs of consecutive tiles that start inside and cross
+    matrices.  Weights are drawn on the device; first, middle and last rows against the float64 oracle on the bytes
+    read back, at both bars, with bias, ragged row counts, two input rows and the guard elements."""
+    from nntrain_amd.synth import DeviceSynth
+    dsynth = DeviceSynth()
+    rng = np.random.default_rng(808)
+    items = []
+    for g, in_w in enumerate((21504, 17408, 5376, 4096, 1024)):
+        for j, (out_w, rows, bias) in enumerate(((33000 + g, 1, False), (37, 2, True), (4099, 1, True))):
+            row_bytes = (in_w // 32) * 34
+            wd = lane.allocate_bytes(out_w * row_bytes)
+            dsynth.q8_0(lane, wd, out_w * (in_w // 32), 4000 + 10 * g + j)
+            xh = rng.standard_normal((rows, in_w)).astype(np.float32)
+            xh[:, ::5] *= 0.003
+            bh = rng.standard_normal(out_w).astype(np.float32) if bias else None
+            items.append(dict(typ=GGML_Q8_0, in_w=in_w, out_w=out_w, rows=rows, x=xh, xd=lane.upload_raw(xh), bias=bh, wd=wd,
+                              bd=lane.upload_raw(bh) if bias else None, yd=lane.allocate(rows * out_w + 2), row_bytes=row_bytes))
+    lane.synchronize()
+    got = _batch_run(lane, items)
+
+    def check_rows(it, y):
+        assert np.all(np.isfinite(y)), (it["in_w"], it["out_w"])
+        n = min(96, it["out_w"])
+        for r0 in sorted({0, (it["out_w"] - n) // 2 // 16 * 16 + 5 if it["out_w"] > n + 5 else 0, it["out_w"] - n}):
+            raw = lane.read(it["wd"], np.uint8, n * it["row_bytes"], r0 * it["row_bytes"])
+            b = it["bias"][r0:r0 + n] if it["bias"] is not None else None
+            ref, asum = oracle.linear_f64(GGML_Q8_0, raw, it["x"], b, it["rows"], it["in_w"], n)
+            part = y[:, r0:r0 + n]
+            assert oracle.rel_l2(part, ref) <= MATVEC_BAR, (it["in_w"], it["out_w"], r0)
+            assert np.all(np.abs(part.astype(np.float64) - ref) <= 2e-6 + 3e-6 * asum), (it["in_w"], it["out_w"], r0)
+
+    for it, y in zip(items, got):
+        check_rows(it, y)
+    # the same matrices in another order and composition (every group still above the threshold): identical bits per row
+    order = [2, 0, 1, 5, 3, 8, 6, 11, 9, 14, 12]
+    again = _batch_run(lane, [items[i] for i in order])
+    for i, y in zip(order, again):
+        assert np.array_equal(_bits(y), _bits(got[i])), (items[i]["in_w"], items[i]["out_w"])
+    for it in items:
+        for key in ("xd", "wd", "bd", "yd"):
+            if it[key] is not None:
+                it[key].dispose()
     lane.trim()
 
 
