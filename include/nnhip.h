@@ -217,10 +217,11 @@ NNHIP_API int nnhip_matvec_plan(uint32_t ggml_type, int rows, int in_w, int out_
 /* `count` independent mat-vecs enqueued as one unit of work (a single launch per group of equal type), for the
  * per-token projection sets that ForwardTokenDevice issues back to back (Qwen35QuantizedModel.cs:451-513).
  * `descs` is a host array, read before the call returns.  Results are identical to `count` nnhip_quant_matvec calls,
- * with one exception: Q4_K, Q5_K, Q6_K and IQ2_S matrices of one in_w (at least 1024, a multiple of 256; an even
+ * with one exception: Q8_0, Q4_K, Q5_K, Q6_K and IQ2_S matrices of one in_w (at least 1024, a multiple of 256; an even
  * number of 256-blocks for Q6_K and IQ2_S) whose 16-row tiles, counted once per input row, add up to 2048 or more
  * within a call are multiplied on the matrix cores with the activations in 32-bit fixed point; descriptors with two or
- * more input rows share one pass over the weights between up to four rows there.  Those results are deterministic,
+ * more input rows share one pass over the weights between up to four rows there (not Q8_0: its rows go one by one).
+ * Those results are deterministic,
  * depend on the weights, in_w and the activations of the row only (not on out_w, the other matrices or input rows of
  * the call, or the order), agree with the single launch to FP32 summation accuracy (relative L2 difference below 1e-6)
  * and are closer to the exact product than it.

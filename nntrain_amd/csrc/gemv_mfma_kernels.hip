@@ -1,7 +1,8 @@
-// Decode mat-vec on the matrix cores for the super-block formats whose unpacking is too much vector-ALU work for the
-// lane-per-unit kernels (gemv_kernels.hip): Q4_K, Q5_K, Q6_K and IQ2_S here.  Used for the large groups of a batched
-// launch and for calls with 2 - 16 input rows, where it streams faster than the row-step kernels; it takes longer to
-// start, so single-row launches stay with those.  Two kernels share the tasks of the formats: matvec_mfma_kernel keeps
+// Decode mat-vec on the matrix cores: for the super-block formats whose unpacking is too much vector-ALU work for the
+// lane-per-unit kernels (gemv_kernels.hip), Q4_K, Q5_K, Q6_K and IQ2_S, and for Q8_0, whose signed bytes are operand B
+// as they lie in memory and whose lane-per-unit kernel is held back by its cached, strided loads.  Used for the large
+// groups of a batched launch and for calls with 2 - 16 input rows, where it streams faster than the row-step kernels;
+// it takes longer to start, so single-row launches stay with those.  Two kernels share the tasks of the formats: matvec_mfma_kernel keeps
 // operand A in registers (rows of one or two whole stages), matvec_mfma_wide_kernel keeps the digit planes in LDS (any
 // row length, up to four input rows per pass over the weights); the text below describes the first, the second has its
 // own paragraph further down.
@@ -422,6 +423,7 @@ struct Q8_0Task {
     static constexpr bool kNeedsSums = false;
     static constexpr bool kTightStage = true;
     static constexpr int kSharedM = 0, kSharedLpw = 0;     // (no shared passes: rows of a call are entries of their own)
+    static constexpr int kOneM = 2, kOneLpw = 8;           // one stage = a whole tile: two block columns per wave
     static __device__ __forceinline__ void init_tables(uint8_t*, int, int) {}
     using X = XSet<1>;
     struct Raw { uint32_t w[17]; };
@@ -872,7 +874,8 @@ struct WideGeom {
     int stage_bytes;
     int plane_stride;     // bytes of one digit plane (in_w + 16)
     int set_bytes;        // four planes and the sums of one input row
-    size_t lds_bytes;     // two stage buffers and R plane sets
+    int single;           // 1: one stage buffer that holds whole tiles (kchunks == 1, cols == nblocks)
+    size_t lds_bytes;     // the stage buffers and R plane sets
 };
 
 struct WideArgs {
@@ -888,7 +891,7 @@ struct WideArgs {
     MfmaEntry inline_entries[4];   // a call with up to 16 input rows needs no table in device memory
 };
 
-template <class F, int M, int LPW, int R>
+template <class F, int M, int LPW, int R, bool ONE = false>
 __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideArgs a)
 {
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
@@ -1002,8 +1005,8 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
 
     // ---- consume side
     uint8_t* const buf0 = smem;
-    uint8_t* const buf1 = smem + g.stage_bytes;
-    uint8_t* const planes = smem + 2 * g.stage_bytes;
+    uint8_t* const buf1 = smem + g.stage_bytes;             // (not with ONE: a single stage buffer)
+    uint8_t* const planes = smem + (ONE ? 1 : 2) * g.stage_bytes;
     uint8_t* const tables = planes + R * g.set_bytes;      // the format's lookup tables (published by the first barrier)
     F::init_tables(tables, tid, T);
     int c_t = t_first, c_k = 0, c_m = m_first - 1;      // (ce.tiles == 0: the first stage enters entry m_first)
@@ -1191,15 +1194,16 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
     float accq[R], accm[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) accq[r] = accm[r] = 0.0f;
-    auto stage_step = [&](uint8_t* cur, uint8_t* nxt, u32x4 (&refill)[LPW], const u32x4 (&landing)[LPW]) {
+    // The matrix of the stage about to be multiplied; true when its activations are not the ones in LDS.
+    auto enter = [&]() {
         bool new_x = false;
         if (c_k == 0 && c_t >= ce.first_tile + ce.tiles) {
             while (c_t >= ce.first_tile + ce.tiles) ce = entry_at(++c_m);
             new_x = ce.x != planes_x || ce.rows != planes_rows;
         }
-        fetch(refill);
-        if (new_x) prepare_x();
-        if (done) finalize();
+        return new_x;
+    };
+    auto compute = [&](const uint8_t* cur) {
         // task t of this wave: block column c_k * cols + t * W + wave of the row (W is even: the block's parity is the
         // wave's).  Stages whose tasks all exist run them as one straight piece of code, so that the lookups and products
         // of one task overlap the other's; a tile's last stage may hold fewer.
@@ -1248,15 +1252,44 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
             pbuf ^= 1;
             c_t += t_step;
         }
-        park(nxt, landing);
-        __syncthreads();
     };
-
-    park(buf0, regs[0]);
-    __syncthreads();
-    for (int n = 0; n < total; n += 2) {
-        stage_step(buf0, buf1, regs[0], regs[1]);
-        if (n + 1 < total) stage_step(buf1, buf0, regs[1], regs[0]);
+    if constexpr (ONE) {
+        // One stage buffer that holds a whole 16-row tile (a contiguous piece of the matrix: no line of memory is
+        // requested by two stages) and two register sets, i.e. up to two tiles on their way: a set is parked when
+        // every wave has left the tile before it, and refilled with the tile after the next right away.
+        auto one_step = [&](u32x4 (&mine)[LPW]) {
+            park(buf0, mine);
+            __syncthreads();            // the tile is in LDS
+            const bool new_x = enter();
+            fetch(mine);
+            if (new_x) prepare_x();
+            if (done) finalize();
+            compute(buf0);
+            __syncthreads();            // every wave has read its blocks
+        };
+        // (an odd last tile is taken after the loop: a conditional second step inside it would make the compiler wait
+        // for both register sets before every parking write)
+        for (int n = 0; n + 2 <= total; n += 2) {
+            one_step(regs[0]);
+            one_step(regs[1]);
+        }
+        if (total & 1) one_step(regs[0]);
+    } else {
+        auto stage_step = [&](uint8_t* cur, uint8_t* nxt, u32x4 (&refill)[LPW], const u32x4 (&landing)[LPW]) {
+            const bool new_x = enter();
+            fetch(refill);
+            if (new_x) prepare_x();
+            if (done) finalize();
+            compute(cur);
+            park(nxt, landing);
+            __syncthreads();
+        };
+        park(buf0, regs[0]);
+        __syncthreads();
+        for (int n = 0; n < total; n += 2) {
+            stage_step(buf0, buf1, regs[0], regs[1]);
+            if (n + 1 < total) stage_step(buf1, buf0, regs[1], regs[0]);
+        }
     }
     if (done) finalize();
 }
@@ -1358,12 +1391,12 @@ int block_pieces_of(uint32_t type)
 }
 
 
-struct WideTraits { int pieces, m, lpw, table_bytes; bool sums, tight; };
+struct WideTraits { int pieces, m, lpw, table_bytes; bool sums, tight; int one_m, one_lpw; };
 
 template <class F>
 constexpr WideTraits wide_traits_of(bool shared)
 {
-    return {F::kPieces, shared ? F::kSharedM : F::kWideM, shared ? F::kSharedLpw : F::kWideLpw, 0, F::kNeedsSums, F::kTightStage};
+    return {F::kPieces, shared ? F::kSharedM : F::kWideM, shared ? F::kSharedLpw : F::kWideLpw, 0, F::kNeedsSums, F::kTightStage, 0, 0};
 }
 
 WideTraits wide_traits(uint32_t type, bool shared)
@@ -1377,12 +1410,20 @@ WideTraits wide_traits(uint32_t type, bool shared)
         t.table_bytes = IQ2STask::kTableBytes;
         return t;
     }
-    case NNHIP_TYPE_Q8_0: return shared ? WideTraits{0, 0, 0, 0, false, false} : wide_traits_of<Q8_0Task>(false);
-    default: return {0, 0, 0, 0, false, false};
+    case NNHIP_TYPE_Q8_0: {
+        if (shared) return {0, 0, 0, 0, false, false, 0, 0};
+        WideTraits t = wide_traits_of<Q8_0Task>(false);
+        t.one_m = Q8_0Task::kOneM;
+        t.one_lpw = Q8_0Task::kOneLpw;
+        return t;
+    }
+    default: return {0, 0, 0, 0, false, false, 0, 0};
     }
 }
 
-constexpr int kWideStaticLds = 8 * 1024;      // room left for the kernel's static arrays (partial sums, maxima)
+// room left for the kernel's static arrays (partial sums, maxima, the zero area): 2 KB with one input row per pass,
+// 7 KB with four
+constexpr int wide_static_lds(int inputs) { return inputs > 1 ? 8 * 1024 : 2 * 1024; }
 
 // W for the wide form: even, as many of the row's blocks per stage as two stage buffers beside the plane sets of
 // `inputs` rows leave room for: the most waves, weighted by the share of block slots a tile fills and by an even
@@ -1408,7 +1449,7 @@ bool plan_wide(uint32_t type, int in_w, int inputs, WideGeom* out)
         g.plane_stride = in_w + 16;
         g.set_bytes = (4 * g.plane_stride + (tr.sums ? (in_w / 16) * 4 : 0) + 15) / 16 * 16;
         g.lds_bytes = 2 * static_cast<size_t>(g.stage_bytes) + static_cast<size_t>(inputs) * g.set_bytes + tr.table_bytes;
-        if (g.lds_bytes + kWideStaticLds > static_cast<size_t>(160 * 1024)) continue;
+        if (g.lds_bytes + wide_static_lds(inputs) > static_cast<size_t>(160 * 1024)) continue;
         const double fill = static_cast<double>(nblocks) / (g.kchunks * g.cols);
         // (throughput grows with the waves: a stage holds W * M blocks per row and W tasks run side by side)
         // (and of two equal products the fuller stages win: 16 blocks go as 2 x 8 rather than 12 + 4)
@@ -1416,6 +1457,32 @@ bool plan_wide(uint32_t type, int in_w, int inputs, WideGeom* out)
         if (score > best_score) {
             best_score = score;
             best = g;
+        }
+    }
+    const int row_bytes = nblocks * tr.pieces * 16;
+    const bool split_lines = row_bytes % 64 != 0 || (best_score >= 0 && best.kchunks > 1 && (best.cols * tr.pieces * 16) % 64 != 0);
+    if (tr.one_m && inputs == 1 && split_lines) {
+        // Whole tiles in one stage buffer, for rows whose stages would begin or end inside 64-byte lines of memory (5376 =
+        // 21 blocks: 5712-byte rows): a line shared by two stages is fetched twice by the non-temporal loads (3 % more
+        // traffic measured), while a tile of 16 rows is one contiguous, line-aligned piece of the matrix.
+        for (int W = 12; W >= 8; W -= 2) {
+            WideGeom g{};
+            g.waves = W;
+            g.cols = nblocks;
+            if (nblocks <= W * (tr.one_m - 1) || nblocks > W * tr.one_m) continue;        // (every wave's first task exists)
+            g.kchunks = 1;
+            g.tail_cols = nblocks;
+            g.row_pieces = (g.cols * tr.pieces) | 1;
+            const int loads = (kTileRows * g.row_pieces + 63) / 64;
+            if ((loads + W - 1) / W > tr.one_lpw) continue;
+            g.stage_bytes = loads * 1024;
+            g.plane_stride = in_w + 16;
+            g.set_bytes = (4 * g.plane_stride + 15) / 16 * 16;
+            g.single = 1;
+            g.lds_bytes = static_cast<size_t>(g.stage_bytes) + g.set_bytes + tr.table_bytes;
+            if (g.lds_bytes + wide_static_lds(1) > static_cast<size_t>(160 * 1024)) continue;
+            *out = g;
+            return true;
         }
     }
     if (best_score < 0) return false;
@@ -1429,7 +1496,7 @@ hipError_t launch_wide_of(Lane* lane, const WideArgs& a)
     constexpr int M = R == 1 ? F::kWideM : F::kSharedM, LPW = R == 1 ? F::kWideLpw : F::kSharedLpw;
     static LdsLimit big_lds;
     const void* fn = reinterpret_cast<const void*>(&matvec_mfma_wide_kernel<F, M, LPW, R>);
-    const hipError_t e = big_lds.ensure(lane->device, fn, 160 * 1024 - kWideStaticLds);
+    const hipError_t e = big_lds.ensure(lane->device, fn, 160 * 1024 - wide_static_lds(R));
     if (e != hipSuccess) return e;
     const int groups = a.total_tiles < lane->compute_units ? a.total_tiles : lane->compute_units;
     hipLaunchKernelGGL((matvec_mfma_wide_kernel<F, M, LPW, R>), dim3(groups), dim3(64 * a.g.waves), a.g.lds_bytes, lane->stream, a);
@@ -1537,6 +1604,16 @@ hipError_t launch_wide_args(Lane* lane, uint32_t type, int in_w, int inputs, Wid
     case NNHIP_TYPE_Q8_0:
         if (inputs != 1) return hipErrorInvalidValue;
         a.chunked = 1;          // (Q8_0 launches are whole models: hundreds of matrices, most with a vector of their own)
+        if (a.g.single) {
+            static LdsLimit big_lds;
+            const void* fn = reinterpret_cast<const void*>(&matvec_mfma_wide_kernel<Q8_0Task, Q8_0Task::kOneM, Q8_0Task::kOneLpw, 1, true>);
+            const hipError_t e = big_lds.ensure(lane->device, fn, 160 * 1024 - wide_static_lds(1));
+            if (e != hipSuccess) return e;
+            const int groups = a.total_tiles < lane->compute_units ? a.total_tiles : lane->compute_units;
+            hipLaunchKernelGGL((matvec_mfma_wide_kernel<Q8_0Task, Q8_0Task::kOneM, Q8_0Task::kOneLpw, 1, true>), dim3(groups),
+                               dim3(64 * a.g.waves), a.g.lds_bytes, lane->stream, a);
+            return hipGetLastError();
+        }
         return launch_wide_of<Q8_0Task, 1>(lane, a);
     default: return hipErrorInvalidValue;
     }

@@ -437,10 +437,10 @@ def test_large_batched_group_special_activations(lane, typ):
 
 
 def test_q8_0_model_sized_groups_on_the_matrix_cores(lane):
-    """Q8_0 groups of every row length class the matrix-core form plans differently (21504: six waves beside 86 KB of
-    activation planes, 17408: eight, 5376: twelve with a shorter last stage, 4096: two full stages of eight, 1024: four
-    waves), each with more than 2048 tiles so that workgroups take runs of consecutive tiles that start inside and cross
-    matrices.  Weights are drawn on the device; first, middle and last rows against the float64 oracle on the bytes
+    """Q8_0 groups of every row length class the matrix-core form plans differently (21504 and 17408: eight waves beside
+    70 - 86 KB of activation planes, 5376: whole tiles in a single stage buffer, two block columns per wave, 4096: two
+    full stages of eight columns, 1024: four waves), each with more than 2048 tiles so that workgroups take runs of
+    consecutive tiles that start inside and cross matrices.  Weights are drawn on the device; first, middle and last rows against the float64 oracle on the bytes
     read back, at both bars, with bias, ragged row counts, two input rows and the guard elements."""
     from nntrain_amd.synth import DeviceSynth
     dsynth = DeviceSynth()

@@ -53,14 +53,15 @@ def _short(name):
 
 
 # (task, stages per tile or tasks per wave, ...) of the variants the planners pick for the shapes of the benchmark and
-# the tests: register form <Task, KC, M, LPW>, wide form <Task, M, LPW, R>
+# the tests: register form <Task, KC, M, LPW>, wide form <Task, M, LPW, R, one stage buffer>
 USED = ["matvec_mfma_kernelINS0_7Q4KTaskELi2ELi1ELi3", "matvec_mfma_kernelINS0_7Q5KTaskELi2ELi1ELi3",
         "matvec_mfma_kernelINS0_7Q6KTaskELi2ELi1ELi4", "matvec_mfma_kernelINS0_7Q4KTaskELi1ELi1ELi3",
-        "matvec_mfma_wide_kernelINS0_7Q4KTaskELi1ELi3ELi1", "matvec_mfma_wide_kernelINS0_7Q4KTaskELi1ELi3ELi4",
-        "matvec_mfma_wide_kernelINS0_7Q5KTaskELi1ELi3ELi1", "matvec_mfma_wide_kernelINS0_7Q5KTaskELi1ELi3ELi4",
-        "matvec_mfma_wide_kernelINS0_7Q6KTaskELi1ELi4ELi1", "matvec_mfma_wide_kernelINS0_7Q6KTaskELi1ELi4ELi4",
-        "matvec_mfma_wide_kernelINS0_8IQ2STaskELi2ELi4ELi1",
-        "matvec_mfma_wide_kernelINS0_8Q8_0TaskELi1ELi5ELi1"]
+        "matvec_mfma_wide_kernelINS0_7Q4KTaskELi1ELi3ELi1ELb0", "matvec_mfma_wide_kernelINS0_7Q4KTaskELi1ELi3ELi4ELb0",
+        "matvec_mfma_wide_kernelINS0_7Q5KTaskELi1ELi3ELi1ELb0", "matvec_mfma_wide_kernelINS0_7Q5KTaskELi1ELi3ELi4ELb0",
+        "matvec_mfma_wide_kernelINS0_7Q6KTaskELi1ELi4ELi1ELb0", "matvec_mfma_wide_kernelINS0_7Q6KTaskELi1ELi4ELi4ELb0",
+        "matvec_mfma_wide_kernelINS0_8IQ2STaskELi2ELi4ELi1ELb0",
+        "matvec_mfma_wide_kernelINS0_8Q8_0TaskELi1ELi5ELi1ELb0",
+        "matvec_mfma_wide_kernelINS0_8Q8_0TaskELi2ELi8ELi1ELb1"]
 
 
 def test_parking_writes_wait_only_for_their_own_register_set(isa):
