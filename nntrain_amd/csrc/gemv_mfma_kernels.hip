@@ -1460,10 +1460,10 @@ bool plan_wide(uint32_t type, int in_w, int inputs, WideGeom* out)
         }
     }
     const int row_bytes = nblocks * tr.pieces * 16;
-    const bool split_lines = row_bytes % 64 != 0 || (best_score >= 0 && best.kchunks > 1 && (best.cols * tr.pieces * 16) % 64 != 0);
+    const bool split_lines = row_bytes % 128 != 0 || (best_score >= 0 && best.kchunks > 1 && (best.cols * tr.pieces * 16) % 128 != 0);
     if (tr.one_m && inputs == 1 && split_lines) {
-        // Whole tiles in one stage buffer, for rows whose stages would begin or end inside 64-byte lines of memory (5376 =
-        // 21 blocks: 5712-byte rows): a line shared by two stages is fetched twice by the non-temporal loads (3 % more
+        // Whole tiles in one stage buffer, for rows whose stages would begin or end inside 128-byte lines of memory (5376
+        // = 21 blocks: 5712-byte rows): a line shared by two stages is fetched twice by the non-temporal loads (3 % more
         // traffic measured), while a tile of 16 rows is one contiguous, line-aligned piece of the matrix.
         for (int W = 12; W >= 8; W -= 2) {
             WideGeom g{};
@@ -1477,7 +1477,7 @@ bool plan_wide(uint32_t type, int in_w, int inputs, WideGeom* out)
             if ((loads + W - 1) / W > tr.one_lpw) continue;
             g.stage_bytes = loads * 1024;
             g.plane_stride = in_w + 16;
-            g.set_bytes = (4 * g.plane_stride + 15) / 16 * 16;
+            g.set_bytes = (4 * g.plane_stride + (tr.sums ? (in_w / 16) * 4 : 0) + 15) / 16 * 16;
             g.single = 1;
             g.lds_bytes = static_cast<size_t>(g.stage_bytes) + g.set_bytes + tr.table_bytes;
             if (g.lds_bytes + wide_static_lds(1) > static_cast<size_t>(160 * 1024)) continue;
@@ -1548,6 +1548,7 @@ MfmaTableEntry matvec_mfma_entry(uint32_t type, const float* x, const void* w, c
 bool matvec_mfma_geometry(uint32_t type, int in_w, int out_w, const void* w, MfmaPlan* plan)
 {
     if (type == NNHIP_TYPE_IQ2_S || type == NNHIP_TYPE_Q8_0) return false;       // (these have the wide form only)
+
     if (!entry_ok(type, in_w, out_w, w)) return false;
     MfmaGeom g;
     if (!plan_mfma(block_pieces_of(type), in_w, block_bytes_of(type) % 16 != 0, &g)) return false;
