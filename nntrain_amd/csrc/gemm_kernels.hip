@@ -142,7 +142,8 @@ __device__ __forceinline__ void k4_block_scales(const u32x4 hdr, float sm[16])
 // and 16 high-nibble weights of sub-block 2J + 1.
 struct Q4KDecode {
     static constexpr int kBlockBytes = 144;
-    u32x4 nq[2];                // nibble bytes of K slices t and t + 1
+    static constexpr int kAhead = 2;       // (four slices ahead measured the same)
+    u32x4 nq[kAhead];           // nibble bytes of K slices t .. t + kAhead - 1
     u32x4 hdr;                  // header (d, dmin, packed scales) of the next 256-block
     float sm[16];               // (d * scale, dmin * min) of the eight sub-blocks of the current block
 
@@ -159,14 +160,14 @@ struct Q4KDecode {
     __device__ __forceinline__ void start(const DecodeCtx& c)
     {
         load_hdr(c, 0);
-        nq[0] = load_q(c, 0);
-        nq[1] = load_q(c, 1);
+#pragma unroll
+        for (int i = 0; i < kAhead; ++i) nq[i] = load_q(c, i);
         k4_block_scales(hdr, sm);
     }
     template <int J>
     __device__ __forceinline__ void make(const DecodeCtx& c, int t, uint8_t* lo, uint8_t* hi)
     {
-        const u32x4 q = nq[J & 1];
+        const u32x4 q = nq[J % kAhead];
 #pragma unroll
         for (int g = 0; g < 2; ++g) {
             const uint32_t a0 = q[2 * g], a1 = q[2 * g + 1];
@@ -174,7 +175,7 @@ struct Q4KDecode {
             st128(c, lo + slot, q4k_decode8(a0 & 0x0f0f0f0fu, a1 & 0x0f0f0f0fu, sm[4 * J], sm[4 * J + 1]));
             st128(c, hi + slot, q4k_decode8((a0 >> 4) & 0x0f0f0f0fu, (a1 >> 4) & 0x0f0f0f0fu, sm[4 * J + 2], sm[4 * J + 3]));
         }
-        nq[J & 1] = load_q(c, t + 2);
+        nq[J % kAhead] = load_q(c, t + kAhead);
         if (J == 0) load_hdr(c, (t >> 2) + 1);
         if (J == 3) k4_block_scales(hdr, sm);
     }
