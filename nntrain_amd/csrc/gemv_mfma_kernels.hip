@@ -89,6 +89,7 @@ struct MfmaArgs {
     int nblocks;                   // super-blocks per row
     uint32_t row_bytes;
     uint32_t row_pieces_magic;     // ceil(2^32 / row_pieces)
+    int chunked;                   // 1: a workgroup takes a run of consecutive tiles, 0: every G-th tile
     MfmaGeom g;
 };
 
@@ -636,8 +637,19 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_kernel(MfmaArgs a)
 
     // ---- the stage sequence of this workgroup: tiles blockIdx.x, blockIdx.x + G, ... of the launch's tile sequence,
     // KC stages per tile
-    const int G = gridDim.x;
-    const int my_tiles = (a.total_tiles - static_cast<int>(blockIdx.x) + G - 1) / G;
+    const int G = gridDim.x, bid = blockIdx.x;
+    int my_tiles, t_first, t_step;
+    if (a.chunked) {
+        const int per = a.total_tiles / G, rem = a.total_tiles - per * G;
+        my_tiles = per + (bid < rem ? 1 : 0);
+        t_first = bid * per + (bid < rem ? bid : rem);
+        t_step = 1;
+    } else {
+        my_tiles = (a.total_tiles - bid + G - 1) / G;
+        t_first = bid;
+        t_step = G;
+    }
+    const int t_end = a.chunked ? t_first + my_tiles : a.total_tiles;       // no requests from here on
     const int total = my_tiles * KC;
     const uint32_t chunk_bytes = static_cast<uint32_t>(g.cols) * F::kBlockBytes;
     const int n4 = a.in_w >> 2;
@@ -647,8 +659,18 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_kernel(MfmaArgs a)
     constexpr int kXRegs = KC * M;
     float4 xv[kXRegs];
     int xv_m = -1;                         // the table entry whose activations are in xv (or on their way)
-    int f_t = blockIdx.x, f_k = 0, f_m = 0;
-    MfmaEntry fe = entry_at(0);
+    int f_t = t_first, f_k = 0, f_m = 0;
+    if (a.chunked && my_tiles > 0) {       // the entry that holds the run's first tile
+        int lo = 0, hi = a.entries - 1;
+        while (lo < hi) {
+            const int mid = (lo + hi + 1) >> 1;
+            if (table[mid].first_tile <= t_first) lo = mid;
+            else hi = mid - 1;
+        }
+        f_m = lo;
+    }
+    const int m_first = f_m;
+    MfmaEntry fe = entry_at(f_m);
     const float* f_x = nullptr;            // vector of the matrix the prefetch side was in last
     __amdgpu_buffer_rsrc_t f_matrix;
     auto request_x = [&](const float* x, int m) {
@@ -672,15 +694,15 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_kernel(MfmaArgs a)
     // Requests this wave's pieces of the next stage into a register set.  Pieces that are padding, rows past the matrix
     // and stages past the end lie beyond the buffer: zeros, no memory traffic.
     auto fetch = [&](u32x4 (&set)[LPW]) {
-        const uint32_t base = f_t < a.total_tiles
+        const uint32_t base = f_t < t_end
             ? static_cast<uint32_t>(f_t - fe.first_tile) * kTileRows * a.row_bytes + static_cast<uint32_t>(f_k) * chunk_bytes
             : kNoPiece;
 #pragma unroll
         for (int i = 0; i < LPW; ++i) set[i] = stream16(f_matrix, base + rel[i]);
         if (++f_k == KC) {
             f_k = 0;
-            f_t += G;
-            if (f_t < a.total_tiles && f_t >= fe.first_tile + fe.tiles) fetch_enter();
+            f_t += t_step;
+            if (f_t < t_end && f_t >= fe.first_tile + fe.tiles) fetch_enter();
         }
     };
     // Copies a register set to its place in an LDS stage buffer.
@@ -692,7 +714,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_kernel(MfmaArgs a)
     };
 
     // ---- consume side
-    int c_t = blockIdx.x, c_m = -1;
+    int c_t = t_first, c_m = m_first - 1;
     MfmaEntry ce{};
     float inv = 0.0f;
     const float* regs_x = nullptr;         // the vector operand A in the registers below was made from
@@ -841,7 +863,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_kernel(MfmaArgs a)
             done_row0 = (c_t - ce.first_tile) * kTileRows;
             done_rows = ce.out_w - done_row0 < kTileRows ? ce.out_w - done_row0 : kTileRows;
             pbuf ^= 1;
-            c_t += G;
+            c_t += t_step;
         }
         park(nxt, landing);
         __syncthreads();                // publishes `nxt`, frees `cur`
@@ -1565,7 +1587,7 @@ bool matvec_mfma_geometry(uint32_t type, int in_w, int out_w, const void* w, Mfm
 }
 
 hipError_t launch_matvec_mfma_table(Lane* lane, uint32_t type, int in_w, const MfmaTableEntry* device_entries, int entries,
-                                    int total_tiles)
+                                    int total_tiles, bool runs)
 {
     MfmaArgs a{};
     MfmaGeom g;
@@ -1574,6 +1596,7 @@ hipError_t launch_matvec_mfma_table(Lane* lane, uint32_t type, int in_w, const M
     a.table = device_entries;
     a.entries = entries;
     a.total_tiles = total_tiles;
+    a.chunked = runs ? 1 : 0;
     switch (type) {
     case NNHIP_TYPE_Q4_K: return launch_mfma<Q4KTask>(lane, a);
     case NNHIP_TYPE_Q5_K: return launch_mfma<Q5KTask>(lane, a);
@@ -1604,7 +1627,7 @@ hipError_t launch_wide_args(Lane* lane, uint32_t type, int in_w, int inputs, Wid
     case NNHIP_TYPE_IQ2_S: return launch_wide<IQ2STask>(lane, a, inputs);
     case NNHIP_TYPE_Q8_0:
         if (inputs != 1) return hipErrorInvalidValue;
-        a.chunked = 1;          // (Q8_0 launches are whole models: hundreds of matrices, most with a vector of their own)
+        a.chunked = 1;          // (always for Q8_0, whose batches are whole models; measured level with every-G-th at one vector)
         if (a.g.single) {
             static LdsLimit big_lds;
             const void* fn = reinterpret_cast<const void*>(&matvec_mfma_wide_kernel<Q8_0Task, Q8_0Task::kOneM, Q8_0Task::kOneLpw, 1, true>);
@@ -1640,12 +1663,13 @@ bool describe_matvec_rows_shared(uint32_t type, int rows, int in_w, int out_w, i
 }
 
 hipError_t launch_matvec_mfma_wide_table(Lane* lane, uint32_t type, int in_w, int inputs, const MfmaTableEntry* device_entries,
-                                         int entries, int total_tiles)
+                                         int entries, int total_tiles, bool runs)
 {
     WideArgs a{};
     a.table = device_entries;
     a.entries = entries;
     a.total_tiles = total_tiles;
+    a.chunked = runs ? 1 : 0;
     return launch_wide_args(lane, type, in_w, inputs, a);
 }
 
@@ -1662,6 +1686,7 @@ hipError_t launch_matvec_rows_shared(Lane* lane, uint32_t type, const float* x, 
         a.inline_entries[a.entries++] = e;
         a.total_tiles += e.tiles;
     }
+    a.chunked = a.entries >= 3 ? 1 : 0;         // (9 - 16 input rows: three or four groups of rows, each with planes of its own)
     return launch_wide_args(lane, type, in_w, 4, a);
 }
 

@@ -102,8 +102,10 @@ struct MfmaTableEntry {
 static_assert(sizeof(MfmaTableEntry) == 80, "table slots are 80 bytes");
 MfmaTableEntry matvec_mfma_entry(uint32_t type, const float* x, const void* w, const float* bias, float* y, int in_w,
                                  int out_w, int first_tile);
+// `runs`: workgroups take runs of consecutive tiles instead of every G-th tile (for tables whose activations change from
+// entry to entry: a workgroup then converts two or three vectors instead of all of them; same bits per row).
 hipError_t launch_matvec_mfma_table(Lane* lane, uint32_t type, int in_w, const MfmaTableEntry* device_entries, int entries,
-                                    int total_tiles);
+                                    int total_tiles, bool runs);
 // The wide form of the matrix-core mat-vec (activation planes in LDS): any in_w of at least four super-blocks, and
 // entries of up to four input rows that share a pass over the weights (`inputs` = 1: every entry has one row).
 bool matvec_mfma_wide_geometry(uint32_t type, int in_w, int out_w, const void* w, int inputs);
@@ -115,7 +117,7 @@ bool describe_matvec_rows_shared(uint32_t type, int rows, int in_w, int out_w, i
 hipError_t launch_matvec_rows_shared(Lane* lane, uint32_t type, const float* x, const void* w, const float* bias, float* y,
                                      int rows, int in_w, int out_w);
 hipError_t launch_matvec_mfma_wide_table(Lane* lane, uint32_t type, int in_w, int inputs, const MfmaTableEntry* device_entries,
-                                         int entries, int total_tiles);
+                                         int entries, int total_tiles, bool runs);
 // The fixed device workspace: its address on the current device, and the batched launch that uses it.
 hipError_t static_table_address(void** address);
 hipError_t launch_matvec_batch_static(Lane* lane, const nnhip_matvec_desc* descs, int count);

@@ -390,6 +390,10 @@ def test_large_batched_groups_on_the_matrix_cores(lane, typ):
     again = _batch_run(lane, [items[i] for i in order])
     for i, y in zip(order, again):
         assert np.array_equal(_bits(y), _bits(got[i])), shapes[i]
+    # matrices 0 and 1 share their activations: a call of those alone deals every 256th tile to a workgroup, the calls
+    # above (activations that change along the table) gave workgroups runs of consecutive tiles: the same bits
+    shared = _batch_run(lane, [items[0], items[1], items[0]])
+    assert np.array_equal(_bits(shared[0]), _bits(got[0])) and np.array_equal(_bits(shared[1]), _bits(got[1]))
     # and the single launch agrees to FP32 summation accuracy (another kernel, another summation order)
     it = items[0]
     single = lane.allocate(it["out_w"])
