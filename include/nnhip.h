@@ -185,7 +185,7 @@ NNHIP_API int nnhip_dequantize(void* lane, uint32_t ggml_type, const void* w, fl
  * (NNtrain.Core/Tensors/Tensor.QwenQuantized.cs:29-96) for decode (rows == 1) and small row counts.  Each
  * output row of y is computed with the same operation order whatever `rows` is, so rows > 1 equals stacked
  * rows == 1 calls bit for bit (Qwen35InferencePrefillLinearTests.cs:64-77), except for calls with 2 - 16 input rows
- * on Q4_K / Q5_K / Q6_K / IQ2_S matrices with rows x ceil(out_w / 16) >= 2048: those take the matrix-core path described
+ * on Q4_K / Q5_K / Q6_K / IQ2_S matrices (3 - 16 on Q8_0) with rows x ceil(out_w / 16) >= 2048: those take the matrix-core path described
  * at nnhip_quant_matvec_batch (up to four input rows per pass over the weights; a row's bits do not depend on the
  * rows it travels with; 1e-6 from the rows == 1 result).  bias may be null (zero).  Asynchronous. */
 NNHIP_API int nnhip_quant_matvec(void* lane, uint32_t ggml_type, const float* x, const void* w, const float* bias,
@@ -220,7 +220,7 @@ NNHIP_API int nnhip_matvec_plan(uint32_t ggml_type, int rows, int in_w, int out_
  * with one exception: Q8_0, Q4_K, Q5_K, Q6_K and IQ2_S matrices of one in_w (at least 1024, a multiple of 256; an even
  * number of 256-blocks for Q6_K and IQ2_S) whose 16-row tiles, counted once per input row, add up to 2048 or more
  * within a call are multiplied on the matrix cores with the activations in 32-bit fixed point; descriptors with two or
- * more input rows share one pass over the weights between up to four rows there (not Q8_0: its rows go one by one).
+ * more input rows (Q8_0: three or more) share one pass over the weights between up to four rows there.
  * Those results are deterministic,
  * depend on the weights, in_w and the activations of the row only (not on out_w, the other matrices or input rows of
  * the call, or the order), agree with the single launch to FP32 summation accuracy (relative L2 difference below 1e-6)

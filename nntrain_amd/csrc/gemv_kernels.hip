@@ -1325,6 +1325,11 @@ const uint32_t kBatchTypeOrder[kBatchTypes] = {NNHIP_TYPE_Q8_0, NNHIP_TYPE_Q4_K,
 // entry: they are launched one by one.
 static_assert(sizeof(MfmaTableEntry) == sizeof(BatchEntry), "both kinds of entry fill one table slot");
 
+// Fewest input rows of a descriptor for which a shared pass on the matrix cores beats the row-step kernels: Q8_0's
+// row-step kernel already reads the matrix once for up to four rows and wins at two (31.8 against 35.7 us on
+// 21504 x 5376), loses from three on (four rows: 52.8 against 39.6 us).
+int shared_pass_min_rows(uint32_t type) { return type == NNHIP_TYPE_Q8_0 ? 3 : 2; }
+
 long build_batch(const nnhip_matvec_desc* descs, int count, BatchEntry* out, size_t cap, BatchGroup* groups, int* ngroups,
                  uint8_t* forms)
 {
@@ -1337,7 +1342,7 @@ long build_batch(const nnhip_matvec_desc* descs, int count, BatchEntry* out, siz
     for (int i = 0; i < count; ++i) {
         const nnhip_matvec_desc& d = descs[i];
         int form = 0;
-        if (d.rows >= 2 && matvec_mfma_wide_geometry(d.ggml_type, d.in_w, d.out_w, d.w, 4)) form = 3;
+        if (d.rows >= shared_pass_min_rows(d.ggml_type) && matvec_mfma_wide_geometry(d.ggml_type, d.in_w, d.out_w, d.w, 4)) form = 3;
         else if (matvec_mfma_geometry(d.ggml_type, d.in_w, d.out_w, d.w, nullptr)) form = 1;
         else if (matvec_mfma_wide_geometry(d.ggml_type, d.in_w, d.out_w, d.w, 1)) form = 2;
         forms[i] = static_cast<uint8_t>(form);
@@ -1518,8 +1523,8 @@ hipError_t launch_matvec_batch(Lane* lane, const nnhip_matvec_desc* descs, int c
 
 bool matvec_rows_share_pass(uint32_t type, int rows, int in_w, int out_w, const void* w)
 {
-    return rows >= 2 && rows <= 16 && static_cast<long>(rows) * ((out_w + 15) / 16) >= kMfmaBatchMinTiles &&
-           matvec_mfma_wide_geometry(type, in_w, out_w, w, 4);
+    return rows >= shared_pass_min_rows(type) && rows <= 16 &&
+           static_cast<long>(rows) * ((out_w + 15) / 16) >= kMfmaBatchMinTiles && matvec_mfma_wide_geometry(type, in_w, out_w, w, 4);
 }
 
 hipError_t static_table_address(void** address)

@@ -169,6 +169,7 @@ __device__ __forceinline__ i32x4 mfma_i8(uint32_t a0, uint32_t a1, uint32_t b0, 
 }
 
 __device__ __forceinline__ u32x4 lds128(const uint8_t* p) { return *reinterpret_cast<const u32x4*>(p); }
+__device__ __forceinline__ u32x2 lds64(const uint8_t* p) { return *reinterpret_cast<const u32x2*>(p); }
 
 // This lane's part of operand A for one super-block column: 64 bytes (its digit plane of its quarter's 64 activations;
 // zeros in the lanes outside the block diagonal) and the FP32 sums of x over the quarter's NS scale groups.
@@ -216,6 +217,48 @@ struct Q4KTask {
         r.q2 = lds128(blk + 32 + 32 * quarter);
         r.h = lds128(blk);
         return r;
+    }
+
+    // The form for passes that several input rows share (see the kernel): one MFMA per 32-weight sub-block, operand A = the
+    // four digit planes of up to four input rows, K group g = weights 8 g .. 8 g + 7 of the sub-block.  This lane supplies
+    // those eight weights of its matrix row (`g` = lane / 16) and receives the plane sums of input row lane / 16.
+    static constexpr bool kStacked = true;
+    struct RawS { u32x4 h; u32x2 q[4]; };
+
+    static __device__ __forceinline__ RawS load_stacked(const uint8_t* blk, int g, bool)
+    {
+        RawS r;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) r.q[j] = lds64(blk + 16 + 32 * j + 8 * g);
+        r.h = lds128(blk);
+        return r;
+    }
+
+    // a_plane = this lane's digit plane (as a supplier of operand A) at the block's first activation + 8 g; sums = the
+    // eight sub-block sums of x of the input row this lane receives
+    static __device__ __forceinline__ void run_stacked(const RawS& r, const uint8_t* a_plane, const float* sums, const uint8_t*,
+                                                       float& accq, float& accm)
+    {
+        constexpr uint32_t kLow = 0x0f0f0f0fu;
+        u32x2 a[8];
+#pragma unroll
+        for (int sb = 0; sb < 8; ++sb) a[sb] = lds64(a_plane + 32 * sb);
+        float2 sx[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) sx[j] = *reinterpret_cast<const float2*>(sums + 2 * j);
+        const float d = half_bits_to_float(r.h[0]), dmin = half_bits_to_float(r.h[0] >> 16);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const i32x4 zero = {0, 0, 0, 0};
+            const i32x4 s_lo = mfma_i8(a[2 * j][0], a[2 * j][1], r.q[j][0] & kLow, r.q[j][1] & kLow, zero);
+            const i32x4 s_hi = mfma_i8(a[2 * j + 1][0], a[2 * j + 1][1], (r.q[j][0] >> 4) & kLow, (r.q[j][1] >> 4) & kLow, zero);
+            uint32_t sc, mn;
+            k4_scale_pair(r.h[1], r.h[2], r.h[3], j, sc, mn);
+            accq = fmaf(d * ubyte0(sc), recombine(s_lo), accq);
+            accq = fmaf(d * ubyte1(sc), recombine(s_hi), accq);
+            accm = fmaf(dmin * ubyte0(mn), sx[j].x, accm);
+            accm = fmaf(dmin * ubyte1(mn), sx[j].y, accm);
+        }
     }
 
     static __device__ __forceinline__ void run(const Raw& r, const X& xs, int quarter, const uint8_t*, float& accq, float& accm)
@@ -276,6 +319,47 @@ struct Q5KTask {
         return r;
     }
 
+    // shared passes: as Q4KTask::run_stacked, the fifth bits of sub-block s being bit s of the qh bytes 8 g .. 8 g + 7
+    static constexpr bool kStacked = true;
+    struct RawS { u32x4 h; u32x2 hq; u32x2 q[4]; };
+
+    static __device__ __forceinline__ RawS load_stacked(const uint8_t* blk, int g, bool)
+    {
+        RawS r;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) r.q[j] = lds64(blk + 48 + 32 * j + 8 * g);
+        r.hq = lds64(blk + 16 + 8 * g);
+        r.h = lds128(blk);
+        return r;
+    }
+
+    static __device__ __forceinline__ void run_stacked(const RawS& r, const uint8_t* a_plane, const float* sums, const uint8_t*,
+                                                       float& accq, float& accm)
+    {
+        constexpr uint32_t kLow = 0x0f0f0f0fu, kBit4 = 0x10101010u;
+        u32x2 a[8];
+#pragma unroll
+        for (int sb = 0; sb < 8; ++sb) a[sb] = lds64(a_plane + 32 * sb);
+        float2 sx[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) sx[j] = *reinterpret_cast<const float2*>(sums + 2 * j);
+        const float d = half_bits_to_float(r.h[0]), dmin = half_bits_to_float(r.h[0] >> 16);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const i32x4 zero = {0, 0, 0, 0};
+            auto lo5 = [&](uint32_t q, uint32_t hq) { return (q & kLow) | (((hq >> (2 * j)) << 4) & kBit4); };
+            auto hi5 = [&](uint32_t q, uint32_t hq) { return ((q >> 4) & kLow) | (((hq >> (2 * j)) << 3) & kBit4); };
+            const i32x4 s_lo = mfma_i8(a[2 * j][0], a[2 * j][1], lo5(r.q[j][0], r.hq[0]), lo5(r.q[j][1], r.hq[1]), zero);
+            const i32x4 s_hi = mfma_i8(a[2 * j + 1][0], a[2 * j + 1][1], hi5(r.q[j][0], r.hq[0]), hi5(r.q[j][1], r.hq[1]), zero);
+            uint32_t sc, mn;
+            k4_scale_pair(r.h[1], r.h[2], r.h[3], j, sc, mn);
+            accq = fmaf(d * ubyte0(sc), recombine(s_lo), accq);
+            accq = fmaf(d * ubyte1(sc), recombine(s_hi), accq);
+            accm = fmaf(dmin * ubyte0(mn), sx[j].x, accm);
+            accm = fmaf(dmin * ubyte1(mn), sx[j].y, accm);
+        }
+    }
+
     static __device__ __forceinline__ void run(const Raw& r, const X& xs, int quarter, const uint8_t*, float& accq, float& accm)
     {
         constexpr uint32_t kLow = 0x0f0f0f0fu, kBit4 = 0x10101010u;
@@ -311,6 +395,7 @@ struct Q5KTask {
 // A block is 2-byte aligned in memory; a stage gives it 14 pieces (224 bytes) so that it starts 16-byte aligned in LDS.
 struct Q6KTask {
     static constexpr int kBlockBytes = kQ6KBytes;
+    static constexpr bool kStacked = false;
     static constexpr int kPieces = 14;
     static constexpr int kSumRun = 16;
     static constexpr int kWideM = 1;
@@ -423,7 +508,7 @@ struct Q8_0Task {
     static constexpr int kWideLpw = 5;
     static constexpr bool kNeedsSums = false;
     static constexpr bool kTightStage = true;
-    static constexpr int kSharedM = 0, kSharedLpw = 0;     // (no shared passes: rows of a call are entries of their own)
+    static constexpr int kSharedM = 1, kSharedLpw = 5;     // the same with four input rows per pass
     static constexpr int kOneM = 2, kOneLpw = 8;           // one stage = a whole tile: two block columns per wave
     static __device__ __forceinline__ void init_tables(uint8_t*, int, int) {}
     using X = XSet<1>;
@@ -445,6 +530,41 @@ struct Q8_0Task {
 #pragma unroll
         for (int i = 0; i < 17; ++i) r.w[i] = src[i];
         return r;
+    }
+
+    // Shared passes (see Q4KTask::run_stacked): one MFMA per 34-byte block, K group g = its quants 8 g .. 8 g + 7, which
+    // start two bytes into a dword in the even blocks of a column and on a dword boundary in the odd ones.
+    static constexpr bool kStacked = true;
+    struct RawS { uint32_t w[8][3]; uint32_t d[8]; };
+
+    static __device__ __forceinline__ RawS load_stacked(const uint8_t* blk, int g, bool)
+    {
+        RawS r;
+#pragma unroll
+        for (int bi = 0; bi < 8; ++bi) {
+            const uint32_t* src = reinterpret_cast<const uint32_t*>(blk + 34 * bi + ((bi & 1) ? 2 : 0) + 8 * g);
+            r.w[bi][0] = src[0];
+            r.w[bi][1] = src[1];
+            r.w[bi][2] = (bi & 1) ? 0u : src[2];
+            r.d[bi] = *reinterpret_cast<const uint16_t*>(blk + 34 * bi);
+        }
+        return r;
+    }
+
+    static __device__ __forceinline__ void run_stacked(const RawS& r, const uint8_t* a_plane, const float*, const uint8_t*,
+                                                       float& accq, float&)
+    {
+        u32x2 a[8];
+#pragma unroll
+        for (int bi = 0; bi < 8; ++bi) a[bi] = lds64(a_plane + 32 * bi);
+#pragma unroll
+        for (int bi = 0; bi < 8; ++bi) {
+            const uint32_t q_lo = (bi & 1) ? r.w[bi][0] : __builtin_amdgcn_alignbyte(r.w[bi][1], r.w[bi][0], 2);
+            const uint32_t q_hi = (bi & 1) ? r.w[bi][1] : __builtin_amdgcn_alignbyte(r.w[bi][2], r.w[bi][1], 2);
+            const i32x4 zero = {0, 0, 0, 0};
+            const i32x4 sum = mfma_i8(a[bi][0], a[bi][1], q_lo, q_hi, zero);
+            accq = fmaf(half_bits_to_float(r.d[bi]), recombine(sum), accq);
+        }
     }
 
     static __device__ __forceinline__ void run(const Raw& r, const X& xs, int, const uint8_t*, float& accq, float&)
@@ -481,6 +601,7 @@ __device__ const uint64_t g_iq2s_grid_mv[1024] = { NNHIP_IQ2S_GRID_VALUES };
 
 struct IQ2STask {
     static constexpr int kBlockBytes = kIQ2SBytes;
+    static constexpr bool kStacked = false;
     static constexpr int kPieces = 6;
     static constexpr int kSumRun = 32;
     static constexpr int kWideM = 2;                  // (the blocks are small: two per wave make a stage worth its barrier;
@@ -919,6 +1040,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
     __shared__ float part[2][R][kMaxWaves][kTileRows];
     __shared__ uint32_t red[R][kMaxWaves];
+    __shared__ float inv_of_row[R];                                       // 2^-e of each input row's fixed-point scale
     __shared__ __attribute__((aligned(16))) uint8_t zero_area[256];       // operand A outside the block diagonal
 
     const WideGeom& g = a.g;
@@ -1093,6 +1215,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
                     e = e > 126 ? 126 : e;
                     scale[r] = __uint_as_float(static_cast<uint32_t>(e + 127) << 23);
                     inv[r] = E == 255 ? __uint_as_float(0x7fc00000u) : __uint_as_float(static_cast<uint32_t>(127 - e) << 23);
+                    if (tid == 0) inv_of_row[r] = inv[r];
                 }
             }
 #pragma unroll
@@ -1150,6 +1273,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
                 const float scale = __uint_as_float(static_cast<uint32_t>(e + 127) << 23);
                 // a NaN or an infinity among the activations makes every output of the row NaN
                 inv[r] = E == 255 ? __uint_as_float(0x7fc00000u) : __uint_as_float(static_cast<uint32_t>(127 - e) << 23);
+                if (tid == 0) inv_of_row[r] = inv[r];
                 uint8_t* set = planes + r * g.set_bytes;
                 float* sumx = reinterpret_cast<float*>(set + 4 * g.plane_stride);
                 const float4* x4 = reinterpret_cast<const float4*>(ce.x + static_cast<size_t>(r) * a.in_w);
@@ -1225,7 +1349,41 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
         }
         return new_x;
     };
+    // Shared passes of the formats with one scale per 32 weights: one MFMA serves up to four input rows (operand A = their
+    // digit planes stacked, lane quarter q' receives input row q'), see run_stacked of the task.
+    constexpr bool kStack = R > 1 && F::kStacked;
+    float acc_sq = 0.0f, acc_sm = 0.0f;
     auto compute = [&](const uint8_t* cur) {
+        if constexpr (kStack) {
+            const uint8_t* a_plane = planes + (row_l >> 2) * g.set_bytes + (row_l & 3) * g.plane_stride + 8 * quarter;
+            const float* d_sums = reinterpret_cast<const float*>(planes + quarter * g.set_bytes + 4 * g.plane_stride);
+            const int b0 = c_k * g.cols + wave;
+            const uint8_t* stage = cur + row_off;
+            constexpr int kSumsPerBlock = 256 / F::kSumRun;
+#pragma unroll
+            for (int t = 0; t < M; ++t) {
+                const int b = b0 + t * W;
+                if (b < a.nblocks)
+                    F::run_stacked(F::load_stacked(stage + t * W * (16 * F::kPieces), quarter, (wave & 1) != 0), a_plane + 256 * b,
+                                   d_sums + kSumsPerBlock * b, tables, acc_sq, acc_sm);
+            }
+            if (++c_k == KC) {
+                c_k = 0;
+                const float p = fmaf(acc_sq, inv_of_row[quarter], -acc_sm);     // (from LDS: a register array indexed by the lane would go to scratch memory)
+                if (quarter < ce.rows) part[pbuf][quarter][wave][row_l] = p;
+                acc_sq = 0.0f;
+                acc_sm = 0.0f;
+                done = true;
+                done_y = ce.y;
+                done_bias = ce.bias;
+                done_out_w = ce.out_w;
+                done_inputs = ce.rows;
+                done_row0 = (c_t - ce.first_tile) * kTileRows;
+                done_rows = ce.out_w - done_row0 < kTileRows ? ce.out_w - done_row0 : kTileRows;
+                pbuf ^= 1;
+                c_t += t_step;
+            }
+        } else {
         // task t of this wave: block column c_k * cols + t * W + wave of the row (W is even: the block's parity is the
         // wave's).  Stages whose tasks all exist run them as one straight piece of code, so that the lookups and products
         // of one task overlap the other's; a tile's last stage may hold fewer.
@@ -1273,6 +1431,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
             done_rows = ce.out_w - done_row0 < kTileRows ? ce.out_w - done_row0 : kTileRows;
             pbuf ^= 1;
             c_t += t_step;
+        }
         }
     };
     if constexpr (ONE) {
@@ -1433,8 +1592,8 @@ WideTraits wide_traits(uint32_t type, bool shared)
         return t;
     }
     case NNHIP_TYPE_Q8_0: {
-        if (shared) return {0, 0, 0, 0, false, false, 0, 0};
-        WideTraits t = wide_traits_of<Q8_0Task>(false);
+        WideTraits t = wide_traits_of<Q8_0Task>(shared);
+        if (shared) return t;
         t.one_m = Q8_0Task::kOneM;
         t.one_lpw = Q8_0Task::kOneLpw;
         return t;
@@ -1626,7 +1785,7 @@ hipError_t launch_wide_args(Lane* lane, uint32_t type, int in_w, int inputs, Wid
     case NNHIP_TYPE_Q6_K: return launch_wide<Q6KTask>(lane, a, inputs);
     case NNHIP_TYPE_IQ2_S: return launch_wide<IQ2STask>(lane, a, inputs);
     case NNHIP_TYPE_Q8_0:
-        if (inputs != 1) return hipErrorInvalidValue;
+        if (inputs != 1) return launch_wide_of<Q8_0Task, 4>(lane, a);
         a.chunked = 1;          // (always for Q8_0, whose batches are whole models; measured level with every-G-th at one vector)
         if (a.g.single) {
             static LdsLimit big_lds;

@@ -537,10 +537,11 @@ def test_matrix_core_groups_with_long_rows_and_shared_passes(lane, typ):
     lane.trim()
 
 
-@pytest.mark.parametrize("typ", [GGML_Q4_K, GGML_Q6_K])
+@pytest.mark.parametrize("typ", [GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_Q8_0])
 def test_several_input_rows_share_a_pass_in_a_single_call(lane, typ):
-    """nnhip_quant_matvec with 2 - 9 input rows on a K-quant matrix large enough for the matrix cores (rows x 16-row
-    tiles >= 2048): up to four rows share a pass over the weights.  Both bars against the oracle, the guard elements,
+    """nnhip_quant_matvec with 2 - 9 input rows (Q8_0: 3 - 9, two rows stay with its row-tiled kernel) on a matrix large
+    enough for the matrix cores (rows x 16-row tiles >= 2048): up to four rows share a pass over the weights (Q4_K, Q5_K
+    and Q8_0 with the rows stacked in operand A, Q6_K one row after the other on the unpacked quants).  Both bars against the oracle, the guard elements,
     no transfers, and a row's bits do not depend on the rows it travels with; the same call inside a captured graph
     gives the same bits on every replay."""
     in_w, out_w = 5120, 17408
@@ -554,7 +555,8 @@ def test_several_input_rows_share_a_pass_in_a_single_call(lane, typ):
     x[5] *= 4e3
     xd = lane.upload_raw(x)
     results = {}
-    for rows in (2, 4, 9):
+    fewest = 3 if typ == GGML_Q8_0 else 2
+    for rows in (fewest, 4, 9):
         yd = lane.allocate(rows * out_w + 2)
         lane.fill_u32(yd, NAN_BITS, rows * out_w + 2)
         before = lane.counters()
@@ -571,7 +573,7 @@ def test_several_input_rows_share_a_pass_in_a_single_call(lane, typ):
         results[rows] = y
         yd.dispose()
     assert np.array_equal(_bits(results[9][:4]), _bits(results[4]))
-    assert np.array_equal(_bits(results[4][:2]), _bits(results[2]))
+    assert np.array_equal(_bits(results[4][:fewest]), _bits(results[fewest]))
     # captured: the descriptor table write is recorded with the launch
     yd = lane.allocate(4 * out_w)
     lane.graph_begin()
@@ -579,7 +581,7 @@ def test_several_input_rows_share_a_pass_in_a_single_call(lane, typ):
     graph = lane.graph_end()
     for _ in range(3):
         lane.fill_u32(yd, NAN_BITS, 4 * out_w)
-        mat.forward(lane, xd, None, 2)              # eager work between the replays uses the same table
+        mat.forward(lane, xd, None, fewest)         # eager work between the replays uses the same table
         lane.synchronize()
         lane.graph_launch(graph)
         lane.synchronize()
