@@ -162,6 +162,9 @@ __device__ __forceinline__ float recombine_wide(i32x4 s)
     return fmaf(hi, 65536.0f, lo);
 }
 
+// a * b for operands inside 24 signed bits (v_mul_i32_i24 / v_mad_i32_i24: full rate; the 32-bit multiply is quarter rate)
+__device__ __forceinline__ int mul24(int a, int b) { return __mul24(a, b); }
+
 __device__ __forceinline__ i32x4 mfma_i8(uint32_t a0, uint32_t a1, uint32_t b0, uint32_t b1, i32x4 c)
 {
     return __builtin_amdgcn_mfma_i32_16x16x32_i8(__builtin_bit_cast(long, u32x2{a0, a1}), __builtin_bit_cast(long, u32x2{b0, b1}),
@@ -247,18 +250,30 @@ struct Q4KTask {
 #pragma unroll
         for (int j = 0; j < 4; ++j) sx[j] = *reinterpret_cast<const float2*>(sums + 2 * j);
         const float d = half_bits_to_float(r.h[0]), dmin = half_bits_to_float(r.h[0] >> 16);
+        // the 6-bit scales are multiplied into the integer plane sums (|sum| <= 32 * 15 * 128 < 2^16, eight of them times
+        // 63 stay below 2^25) and the block is recombined once; the minima are summed before dmin multiplies them
+        i32x4 total = {0, 0, 0, 0};
+        float mins = 0.0f;
+        i32x4 s_lo[4], s_hi[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {           // (all eight products first: their results are not needed one by one)
+            const i32x4 zero = {0, 0, 0, 0};
+            s_lo[j] = mfma_i8(a[2 * j][0], a[2 * j][1], r.q[j][0] & kLow, r.q[j][1] & kLow, zero);
+            s_hi[j] = mfma_i8(a[2 * j + 1][0], a[2 * j + 1][1], (r.q[j][0] >> 4) & kLow, (r.q[j][1] >> 4) & kLow, zero);
+        }
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const i32x4 zero = {0, 0, 0, 0};
-            const i32x4 s_lo = mfma_i8(a[2 * j][0], a[2 * j][1], r.q[j][0] & kLow, r.q[j][1] & kLow, zero);
-            const i32x4 s_hi = mfma_i8(a[2 * j + 1][0], a[2 * j + 1][1], (r.q[j][0] >> 4) & kLow, (r.q[j][1] >> 4) & kLow, zero);
             uint32_t sc, mn;
             k4_scale_pair(r.h[1], r.h[2], r.h[3], j, sc, mn);
-            accq = fmaf(d * ubyte0(sc), recombine(s_lo), accq);
-            accq = fmaf(d * ubyte1(sc), recombine(s_hi), accq);
-            accm = fmaf(dmin * ubyte0(mn), sx[j].x, accm);
-            accm = fmaf(dmin * ubyte1(mn), sx[j].y, accm);
+            const int f_lo = static_cast<int>(sc & 0xffu), f_hi = static_cast<int>((sc >> 8) & 0xffu);
+#pragma unroll
+            for (int p = 0; p < 4; ++p) total[p] += mul24(f_lo, s_lo[j][p]) + mul24(f_hi, s_hi[j][p]);      // (24-bit operands: one full-rate instruction each)
+            mins = fmaf(ubyte0(mn), sx[j].x, mins);
+            mins = fmaf(ubyte1(mn), sx[j].y, mins);
         }
+        accq = fmaf(d, recombine_wide(total), accq);
+        accm = fmaf(dmin, mins, accm);
     }
 
     static __device__ __forceinline__ void run(const Raw& r, const X& xs, int quarter, const uint8_t*, float& accq, float& accm)
@@ -344,6 +359,8 @@ struct Q5KTask {
 #pragma unroll
         for (int j = 0; j < 4; ++j) sx[j] = *reinterpret_cast<const float2*>(sums + 2 * j);
         const float d = half_bits_to_float(r.h[0]), dmin = half_bits_to_float(r.h[0] >> 16);
+        i32x4 total = {0, 0, 0, 0};
+        float mins = 0.0f;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const i32x4 zero = {0, 0, 0, 0};
@@ -353,11 +370,14 @@ struct Q5KTask {
             const i32x4 s_hi = mfma_i8(a[2 * j + 1][0], a[2 * j + 1][1], hi5(r.q[j][0], r.hq[0]), hi5(r.q[j][1], r.hq[1]), zero);
             uint32_t sc, mn;
             k4_scale_pair(r.h[1], r.h[2], r.h[3], j, sc, mn);
-            accq = fmaf(d * ubyte0(sc), recombine(s_lo), accq);
-            accq = fmaf(d * ubyte1(sc), recombine(s_hi), accq);
-            accm = fmaf(dmin * ubyte0(mn), sx[j].x, accm);
-            accm = fmaf(dmin * ubyte1(mn), sx[j].y, accm);
+            const int f_lo = static_cast<int>(sc & 0xffu), f_hi = static_cast<int>((sc >> 8) & 0xffu);
+#pragma unroll
+            for (int p = 0; p < 4; ++p) total[p] += mul24(f_lo, s_lo[p]) + mul24(f_hi, s_hi[p]);      // (|sum| <= 32 * 31 * 128 < 2^17, 24-bit multiplies: below 2^26)
+            mins = fmaf(ubyte0(mn), sx[j].x, mins);
+            mins = fmaf(ubyte1(mn), sx[j].y, mins);
         }
+        accq = fmaf(d, recombine_wide(total), accq);
+        accm = fmaf(dmin, mins, accm);
     }
 
     static __device__ __forceinline__ void run(const Raw& r, const X& xs, int quarter, const uint8_t*, float& accq, float& accm)
@@ -692,7 +712,7 @@ struct IQ2STask {
         for (int k = 0; k < 4; ++k) {
             const int factor = static_cast<int>(2u * ((r.scales >> (4 * k)) & 15u) + 1u);    // nibble k & 1 of scale byte k >> 1
 #pragma unroll
-            for (int p = 0; p < 4; ++p) total[p] += factor * acc[k][p];
+            for (int p = 0; p < 4; ++p) total[p] += mul24(factor, acc[k][p]);     // (24-bit operands: v_mad_i32_i24, not the quarter-rate 32-bit multiply)
         }
         accq = fmaf(half_bits_to_float(r.d) * 0.125f, recombine_wide(total), accq);
     }
