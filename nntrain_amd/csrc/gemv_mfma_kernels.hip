@@ -1332,10 +1332,14 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
                              static_cast<uint32_t>(wave) * (16u * F::kPieces);
     int pbuf = 0;
     bool done = false;
-    float* done_y = nullptr;
-    const float* done_bias = nullptr;
-    int done_row0 = 0, done_rows = 0, done_out_w = 0, done_inputs = 0;
+    int done_row0 = 0;
+    // Adds up and stores the tile whose wave partials sit in part[pbuf ^ 1].  It runs before the next stage enters its
+    // matrix, so the tile's matrix is still `ce` (no copies of its fields: the kernel is short of scalar registers).
     auto finalize = [&]() {
+        const int done_rows = ce.out_w - done_row0 < kTileRows ? ce.out_w - done_row0 : kTileRows;
+        const int done_out_w = ce.out_w, done_inputs = ce.rows;
+        float* const done_y = ce.y;
+        const float* const done_bias = ce.bias;
         if (tid < kTileRows * R) {
             const int r = tid >> 4, j0 = tid & 15;
             if (r < done_inputs) {
@@ -1394,12 +1398,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
                 acc_sq = 0.0f;
                 acc_sm = 0.0f;
                 done = true;
-                done_y = ce.y;
-                done_bias = ce.bias;
-                done_out_w = ce.out_w;
-                done_inputs = ce.rows;
                 done_row0 = (c_t - ce.first_tile) * kTileRows;
-                done_rows = ce.out_w - done_row0 < kTileRows ? ce.out_w - done_row0 : kTileRows;
                 pbuf ^= 1;
                 c_t += t_step;
             }
@@ -1443,12 +1442,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
                 accm[r] = 0.0f;
             }
             done = true;
-            done_y = ce.y;
-            done_bias = ce.bias;
-            done_out_w = ce.out_w;
-            done_inputs = ce.rows;
             done_row0 = (c_t - ce.first_tile) * kTileRows;
-            done_rows = ce.out_w - done_row0 < kTileRows ? ce.out_w - done_row0 : kTileRows;
             pbuf ^= 1;
             c_t += t_step;
         }
@@ -1461,10 +1455,9 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
         auto one_step = [&](u32x4 (&mine)[LPW]) {
             park(buf0, mine);
             __syncthreads();            // the tile is in LDS
-            const bool new_x = enter();
             fetch(mine);
-            if (new_x) prepare_x();
             if (done) finalize();
+            if (enter()) prepare_x();
             compute(buf0);
             __syncthreads();            // every wave has read its blocks
         };
@@ -1477,10 +1470,9 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
         if (total & 1) one_step(regs[0]);
     } else {
         auto stage_step = [&](uint8_t* cur, uint8_t* nxt, u32x4 (&refill)[LPW], const u32x4 (&landing)[LPW]) {
-            const bool new_x = enter();
             fetch(refill);
-            if (new_x) prepare_x();
             if (done) finalize();
+            if (enter()) prepare_x();
             compute(cur);
             park(nxt, landing);
             __syncthreads();
