@@ -187,6 +187,7 @@ struct XSet {
 // fixed-point units) and accm (the minimum part).
 struct Q4KTask {
     static constexpr int kBlockBytes = kQ4KBytes;     // 144 = 9 pieces; blocks and rows are 16-byte aligned
+    static constexpr int kLdsTableBytes = 0;          // no lookup tables in LDS
     static constexpr int kPieces = 9;                 // 16-byte pieces a block takes in a stage
     static constexpr int kSumRun = 32;                // activations per FP32 sum (one sub-block)
     static constexpr int kWideM = 1;                  // wide form: block columns per wave and stage,
@@ -305,6 +306,7 @@ struct Q4KTask {
 // qh, 128 nibble bytes: 176 = 11 pieces).
 struct Q5KTask {
     static constexpr int kBlockBytes = kQ5KBytes;
+    static constexpr int kLdsTableBytes = 0;          // no lookup tables in LDS
     static constexpr int kPieces = 11;
     static constexpr int kSumRun = 32;
     static constexpr int kWideM = 1;
@@ -416,6 +418,7 @@ struct Q5KTask {
 struct Q6KTask {
     static constexpr int kBlockBytes = kQ6KBytes;
     static constexpr bool kStacked = false;
+    static constexpr int kLdsTableBytes = 0;          // no lookup tables in LDS
     static constexpr int kPieces = 14;
     static constexpr int kSumRun = 16;
     static constexpr int kWideM = 1;
@@ -522,6 +525,7 @@ struct Q6KTask {
 // (v_alignbyte_b32), those of the second on dword boundaries.  No minima, no offset: no sums of x.
 struct Q8_0Task {
     static constexpr int kBlockBytes = 8 * kQ8_0Bytes;
+    static constexpr int kLdsTableBytes = 0;          // no lookup tables in LDS
     static constexpr int kPieces = 17;
     static constexpr int kSumRun = 32;
     static constexpr int kWideM = 1;
@@ -632,6 +636,7 @@ struct IQ2STask {
     static constexpr bool kTightStage = true;         // 17408-wide planes leave no room for whole 1 KB slots per wave
     static constexpr int kGridBytes = 8192;
     static constexpr int kTableBytes = kGridBytes + 2048;     // the codebook and 256 selector pairs
+    static constexpr int kLdsTableBytes = kTableBytes;        // (a static LDS array of the kernel)
     using X = XSet<1>;
     struct Raw { uint32_t q[2], s[2], tops, scales, d; };
 
@@ -1168,10 +1173,13 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
     };
 
     // ---- consume side
+    // The format's lookup tables are a static array: its address is a constant of the program, so a table read takes its
+    // base from the instruction's offset field instead of an addition per lookup (sixteen per IQ2_S task).
+    __shared__ __attribute__((aligned(16))) uint8_t table_area[F::kLdsTableBytes > 0 ? F::kLdsTableBytes : 16];
+    uint8_t* const tables = table_area;                    // (published by the first barrier)
     uint8_t* const buf0 = smem;
-    uint8_t* const buf1 = smem + g.stage_bytes;             // (not with ONE: a single stage buffer)
+    uint8_t* const buf1 = smem + g.stage_bytes;            // (not with ONE: a single stage buffer)
     uint8_t* const planes = smem + (ONE ? 1 : 2) * g.stage_bytes;
-    uint8_t* const tables = planes + R * g.set_bytes;      // the format's lookup tables (published by the first barrier)
     F::init_tables(tables, tid, T);
     int c_t = t_first, c_k = 0, c_m = m_first - 1;      // (ce.tiles == 0: the first stage enters entry m_first)
     MfmaEntry ce{};
@@ -1641,8 +1649,8 @@ bool plan_wide(uint32_t type, int in_w, int inputs, WideGeom* out)
         g.stage_bytes = (tr.tight ? loads : tr.lpw * W) * 1024;      // to the last row's end, or every wave's slots
         g.plane_stride = in_w + 16;
         g.set_bytes = (4 * g.plane_stride + (tr.sums ? (in_w / 16) * 4 : 0) + 15) / 16 * 16;
-        g.lds_bytes = 2 * static_cast<size_t>(g.stage_bytes) + static_cast<size_t>(inputs) * g.set_bytes + tr.table_bytes;
-        if (g.lds_bytes + wide_static_lds(inputs) > static_cast<size_t>(160 * 1024)) continue;
+        g.lds_bytes = 2 * static_cast<size_t>(g.stage_bytes) + static_cast<size_t>(inputs) * g.set_bytes;
+        if (g.lds_bytes + wide_static_lds(inputs) + tr.table_bytes > static_cast<size_t>(160 * 1024)) continue;
         const double fill = static_cast<double>(nblocks) / (g.kchunks * g.cols);
         // (throughput grows with the waves: a stage holds W * M blocks per row and W tasks run side by side)
         // (and of two equal products the fuller stages win: 16 blocks go as 2 x 8 rather than 12 + 4)
@@ -1672,8 +1680,8 @@ bool plan_wide(uint32_t type, int in_w, int inputs, WideGeom* out)
             g.plane_stride = in_w + 16;
             g.set_bytes = (4 * g.plane_stride + (tr.sums ? (in_w / 16) * 4 : 0) + 15) / 16 * 16;
             g.single = 1;
-            g.lds_bytes = static_cast<size_t>(g.stage_bytes) + g.set_bytes + tr.table_bytes;
-            if (g.lds_bytes + wide_static_lds(1) > static_cast<size_t>(160 * 1024)) continue;
+            g.lds_bytes = static_cast<size_t>(g.stage_bytes) + g.set_bytes;
+            if (g.lds_bytes + wide_static_lds(1) + tr.table_bytes > static_cast<size_t>(160 * 1024)) continue;
             *out = g;
             return true;
         }
@@ -1689,7 +1697,7 @@ hipError_t launch_wide_of(Lane* lane, const WideArgs& a)
     constexpr int M = R == 1 ? F::kWideM : F::kSharedM, LPW = R == 1 ? F::kWideLpw : F::kSharedLpw;
     static LdsLimit big_lds;
     const void* fn = reinterpret_cast<const void*>(&matvec_mfma_wide_kernel<F, M, LPW, R>);
-    const hipError_t e = big_lds.ensure(lane->device, fn, 160 * 1024 - wide_static_lds(R));
+    const hipError_t e = big_lds.ensure(lane->device, fn, 160 * 1024 - wide_static_lds(R) - F::kLdsTableBytes);
     if (e != hipSuccess) return e;
     const int groups = a.total_tiles < lane->compute_units ? a.total_tiles : lane->compute_units;
     hipLaunchKernelGGL((matvec_mfma_wide_kernel<F, M, LPW, R>), dim3(groups), dim3(64 * a.g.waves), a.g.lds_bytes, lane->stream, a);
