@@ -43,6 +43,14 @@ internal static unsafe partial class NnHipNative
         internal int DynamicLdsBytes;
     }
 
+    [StructLayout(LayoutKind.Sequential)]
+    internal struct BatchLaunchInfo
+    {
+        internal uint StructSize; internal uint GgmlType; internal int Kernel; internal int InW; internal int Entries;
+        internal int Units; internal int Groups; internal int Threads; internal int RowsPerPass; internal int ConsecutiveRuns;
+        internal int StageBuffers; internal int ActivationsInLds; internal int DynamicLdsBytes;
+    }
+
     internal const uint PreNone = 0, PreRmsNorm = 1, PreSiluMultiply = 2;
 
     [StructLayout(LayoutKind.Sequential)]
@@ -78,6 +86,7 @@ internal static unsafe partial class NnHipNative
     [LibraryImport(Library)] internal static partial int nnhip_dequantize(nint lane, uint ggmlType, nint w, nint output, long elements);
     [LibraryImport(Library)] internal static partial int nnhip_quant_matvec(nint lane, uint ggmlType, nint x, nint w, nint bias, nint y, int rows, int inW, int outW);
     [LibraryImport(Library)] internal static partial int nnhip_matvec_plan(uint ggmlType, int rows, int inW, int outW, int computeUnits, MatvecPlanInfo* info);
+    [LibraryImport(Library)] internal static partial int nnhip_matvec_batch_plan(MatvecDesc* descs, int count, int computeUnits, BatchLaunchInfo* launches, int capacity, out int launchCount);
     [LibraryImport(Library)] internal static partial int nnhip_quant_matvec_batch(nint lane, MatvecDesc* descs, int count);
     [LibraryImport(Library)] internal static partial int nnhip_quant_matvec_batch_static(nint lane, MatvecDesc* descs, int count);
     [LibraryImport(Library)] internal static partial int nnhip_quant_matvec_fused(nint lane, FusedMatvecDesc* desc);

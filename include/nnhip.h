@@ -232,6 +232,32 @@ NNHIP_API int nnhip_matvec_plan(uint32_t ggml_type, int rows, int in_w, int out_
  * kept until the lane is destroyed.  Asynchronous. */
 NNHIP_API int nnhip_quant_matvec_batch(void* lane, const nnhip_matvec_desc* descs, int count);
 
+/* The launches nnhip_quant_matvec_batch would split `count` descriptors into, without a device: one structure per launch,
+ * in launch order.  No counterpart in the reference, which issues one kernel per matrix; it exists for reporting and so
+ * that the grouping rules above (which matrices reach the matrix cores, which input rows share passes, how tiles are
+ * dealt to the workgroups) can be checked in tests on a machine without a GPU.  The descriptors are checked as for the
+ * batch itself; their pointers are inspected for alignment and equality only, never followed.  `launches` has room for
+ * `capacity` structures, each with struct_size set; *n_launches receives the number of launches, which may exceed
+ * `capacity` (then only the first `capacity` are described). */
+typedef struct nnhip_batch_launch_info {
+    uint32_t struct_size;
+    uint32_t ggml_type;
+    int32_t kernel;                 /* NNHIP_MATVEC_KERNEL_*                                                          */
+    int32_t in_w;                   /* matrix core: the row length all entries share; row-step: the longest           */
+    int32_t entries;                /* table entries: one per matrix and input row (or group of up to four rows)      */
+    int32_t units;                  /* work items dealt to the workgroups: 16-row tiles, or chunks of row steps       */
+    int32_t groups;                 /* workgroups: min(units, compute_units)                                          */
+    int32_t threads;                /* lanes per workgroup                                                            */
+    int32_t rows_per_pass;          /* most input rows of an entry that share a pass over the weights (1 - 4)         */
+    int32_t consecutive_runs;       /* 1: a workgroup takes a run of consecutive tiles; 0: every groups-th tile       */
+    int32_t stage_buffers;          /* matrix core: weight stages in LDS (1 = one buffer holding a whole tile)        */
+    int32_t activations_in_lds;     /* matrix core: 1 = digit planes in LDS (the wide form), 0 = in registers         */
+    int32_t dynamic_lds_bytes;
+} nnhip_batch_launch_info;
+
+NNHIP_API int nnhip_matvec_batch_plan(const nnhip_matvec_desc* descs, int count, int compute_units,
+                                      nnhip_batch_launch_info* launches, int capacity, int* n_launches);
+
 /* nnhip_quant_matvec_batch for callers that cannot allocate device memory: code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same arguments and bit-identical
  * results to nnhip_quant_matvec_batch; the descriptor table lives in a fixed array inside the library's device image (80 bytes per mat-vec row,

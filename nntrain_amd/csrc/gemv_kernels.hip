@@ -1521,6 +1521,74 @@ hipError_t launch_matvec_batch(Lane* lane, const nnhip_matvec_desc* descs, int c
     return launch_batch_groups(lane, lane->batch_table, groups, ngroups, descs, count);
 }
 
+int plan_matvec_batch(const nnhip_matvec_desc* descs, int count, int compute_units, nnhip_batch_launch_info* launches,
+                      int capacity)
+{
+    size_t cap = 0;
+    for (int i = 0; i < count; ++i) cap += static_cast<size_t>(descs[i].rows);
+    std::vector<BatchEntry> all(cap ? cap : 1);
+    std::vector<uint8_t> forms(static_cast<size_t>(count > 0 ? count : 1));
+    BatchGroup groups[kBatchGroupsMax];
+    int ngroups = 0;
+    if (build_batch(descs, count, all.data(), cap, groups, &ngroups, forms.data()) < 0) return -1;
+    int n = 0;
+    auto next = [&]() -> nnhip_batch_launch_info* {
+        nnhip_batch_launch_info* slot = n < capacity ? &launches[n] : nullptr;
+        n += 1;
+        if (slot) {
+            const uint32_t size = slot->struct_size;
+            *slot = nnhip_batch_launch_info{};
+            slot->struct_size = size;
+        }
+        return slot;
+    };
+    for (int i = 0; i < ngroups; ++i) {
+        const BatchGroup& g = groups[i];
+        nnhip_batch_launch_info* info = next();
+        if (!info) continue;
+        info->ggml_type = g.type;
+        info->in_w = g.max_in_w;
+        info->entries = static_cast<int32_t>(g.end - g.begin);
+        info->units = g.total_chunks;
+        info->groups = g.total_chunks < compute_units ? g.total_chunks : compute_units;
+        info->rows_per_pass = 1;
+        if (g.mfma) {
+            info->kernel = NNHIP_MATVEC_KERNEL_MATRIX_CORE;
+            if (!describe_matvec_mfma_launch(g.type, g.max_in_w, g.mfma, g.x_changes >= 2, info)) return -1;
+            if (g.mfma == 3) {
+                const MfmaTableEntry* e = reinterpret_cast<const MfmaTableEntry*>(all.data()) + g.begin;
+                for (size_t k = 0; k < g.end - g.begin; ++k)
+                    if (e[k].rows > info->rows_per_pass) info->rows_per_pass = e[k].rows;
+            }
+        } else {
+            int max_t = 0, depth = 0;
+            shape_of(g.type, &max_t, &depth);
+            info->kernel = NNHIP_MATVEC_KERNEL_ROWSTEP;
+            info->threads = max_t;
+            info->dynamic_lds_bytes = static_cast<int32_t>(static_cast<size_t>(kChunkPieces) * (g.max_in_w / kUnitW) * sizeof(float4));
+        }
+    }
+    for (int i = 0; i < count; ++i) {           // (Q8_0 rows with an odd number of blocks: one launch each)
+        const nnhip_matvec_desc& d = descs[i];
+        if (d.ggml_type != NNHIP_TYPE_Q8_0 || !((d.in_w / 32) & 1)) continue;
+        nnhip_batch_launch_info* info = next();
+        if (!info) continue;
+        nnhip_matvec_plan_info single{};
+        single.struct_size = sizeof(single);
+        if (!describe_matvec(d.ggml_type, d.rows, d.in_w, d.out_w, compute_units, &single)) return -1;
+        info->ggml_type = d.ggml_type;
+        info->kernel = single.kernel;
+        info->in_w = d.in_w;
+        info->entries = 1;
+        info->units = single.steps;
+        info->groups = single.groups;
+        info->threads = single.threads;
+        info->rows_per_pass = single.row_tile;
+        info->dynamic_lds_bytes = single.dynamic_lds_bytes;
+    }
+    return n;
+}
+
 bool matvec_rows_share_pass(uint32_t type, int rows, int in_w, int out_w, const void* w)
 {
     return rows >= shared_pass_min_rows(type) && rows <= 16 &&

@@ -1841,6 +1841,28 @@ bool describe_matvec_rows_shared(uint32_t type, int rows, int in_w, int out_w, i
     return true;
 }
 
+bool describe_matvec_mfma_launch(uint32_t type, int in_w, int form, bool runs, nnhip_batch_launch_info* info)
+{
+    if (form == 1) {
+        MfmaGeom g;
+        if (!plan_mfma(block_pieces_of(type), in_w, block_bytes_of(type) % 16 != 0, &g)) return false;
+        info->threads = 64 * g.waves;
+        info->stage_buffers = g.stages;
+        info->dynamic_lds_bytes = static_cast<int32_t>(g.lds_bytes);
+        info->activations_in_lds = 0;
+        info->consecutive_runs = runs ? 1 : 0;
+        return true;
+    }
+    WideGeom g;
+    if (!plan_wide(type, in_w, form == 3 ? 4 : 1, &g)) return false;
+    info->threads = 64 * g.waves;
+    info->stage_buffers = g.single ? 1 : 2;
+    info->dynamic_lds_bytes = static_cast<int32_t>(g.lds_bytes);
+    info->activations_in_lds = 1;
+    info->consecutive_runs = (runs || (type == NNHIP_TYPE_Q8_0 && form == 2)) ? 1 : 0;      // (as launch_wide_args)
+    return true;
+}
+
 hipError_t launch_matvec_mfma_wide_table(Lane* lane, uint32_t type, int in_w, int inputs, const MfmaTableEntry* device_entries,
                                          int entries, int total_tiles, bool runs)
 {

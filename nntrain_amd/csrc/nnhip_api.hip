@@ -646,6 +646,29 @@ int nnhip_quant_matvec_batch(void* handle, const nnhip_matvec_desc* descs, int c
     return NNHIP_OK;
 }
 
+int nnhip_matvec_batch_plan(const nnhip_matvec_desc* descs, int count, int compute_units, nnhip_batch_launch_info* launches,
+                            int capacity, int* n_launches)
+{
+    if (count < 0 || (count > 0 && !descs) || capacity < 0 || (capacity > 0 && !launches) || !n_launches || compute_units < 1)
+        return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_MATVEC_BATCH, -1, 0, "null array, negative count or capacity, or compute_units < 1");
+    for (int i = 0; i < capacity; ++i)
+        if (launches[i].struct_size != sizeof(nnhip_batch_launch_info))
+            return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_MATVEC_BATCH, -1, 0, "launches[%d] has the wrong struct_size", i);
+    Lane nowhere;
+    nowhere.device = -1;
+    for (int i = 0; i < count; ++i) {
+        const nnhip_matvec_desc& d = descs[i];
+        int rc = check_linear(NNHIP_OP_MATVEC_BATCH, &nowhere, d.ggml_type, d.x, d.w, d.y, d.rows, d.in_w, d.out_w);
+        if (rc != NNHIP_OK) return rc;
+        if (d.in_w > matvec_max_in_w(d.ggml_type))
+            return fail(NNHIP_ERR_TOO_LARGE, NNHIP_OP_MATVEC_BATCH, -1, 0, "descriptor %d: in_w %d exceeds the %d values one workgroup can stage", i, d.in_w, matvec_max_in_w(d.ggml_type));
+    }
+    const int n = plan_matvec_batch(descs, count, compute_units, launches, capacity);
+    if (n < 0) return fail(NNHIP_ERR_TOO_LARGE, NNHIP_OP_MATVEC_BATCH, -1, 0, "no kernel takes one of the shapes");
+    *n_launches = n;
+    return NNHIP_OK;
+}
+
 int nnhip_quant_matvec_batch_static(void* handle, const nnhip_matvec_desc* descs, int count)
 {
     NNHIP_LANE(handle, NNHIP_OP_MATVEC_BATCH)

@@ -118,6 +118,12 @@ hipError_t launch_matvec_rows_shared(Lane* lane, uint32_t type, const float* x, 
                                      int rows, int in_w, int out_w);
 hipError_t launch_matvec_mfma_wide_table(Lane* lane, uint32_t type, int in_w, int inputs, const MfmaTableEntry* device_entries,
                                          int entries, int total_tiles, bool runs);
+// Geometry of one matrix-core launch of a batch (`form` 1: operand A in registers, 2: the wide form, 3: the wide form
+// with shared passes), and the launches a whole batch splits into; no device needed.  plan_matvec_batch returns the
+// number of launches, of which it describes the first `capacity`.
+bool describe_matvec_mfma_launch(uint32_t type, int in_w, int form, bool runs, nnhip_batch_launch_info* info);
+int plan_matvec_batch(const nnhip_matvec_desc* descs, int count, int compute_units, nnhip_batch_launch_info* launches,
+                      int capacity);
 // The fixed device workspace: its address on the current device, and the batched launch that uses it.
 hipError_t static_table_address(void** address);
 hipError_t launch_matvec_batch_static(Lane* lane, const nnhip_matvec_desc* descs, int count);

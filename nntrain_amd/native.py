@@ -57,6 +57,13 @@ class MatvecPlanInfo(Structure):
                 ("result_buffer_floats", c_int32), ("dynamic_lds_bytes", c_int32)]
 
 
+class BatchLaunchInfo(Structure):
+    _fields_ = [("struct_size", c_uint32), ("ggml_type", c_uint32), ("kernel", c_int32), ("in_w", c_int32),
+                ("entries", c_int32), ("units", c_int32), ("groups", c_int32), ("threads", c_int32),
+                ("rows_per_pass", c_int32), ("consecutive_runs", c_int32), ("stage_buffers", c_int32),
+                ("activations_in_lds", c_int32), ("dynamic_lds_bytes", c_int32)]
+
+
 PRE_NONE, PRE_RMS_NORM, PRE_SILU_MULTIPLY = 0, 1, 2
 
 # name -> (restype, argtypes); exactly the prototypes of include/nnhip.h
@@ -84,6 +91,7 @@ PROTOTYPES = {
     "nnhip_dequantize": (c_int, [c_void_p, c_uint32, c_void_p, c_void_p, c_int64]),
     "nnhip_quant_matvec": (c_int, [c_void_p, c_uint32, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int]),
     "nnhip_matvec_plan": (c_int, [c_uint32, c_int, c_int, c_int, c_int, POINTER(MatvecPlanInfo)]),
+    "nnhip_matvec_batch_plan": (c_int, [POINTER(MatvecDesc), c_int, c_int, POINTER(BatchLaunchInfo), c_int, POINTER(c_int)]),
     "nnhip_quant_matvec_batch": (c_int, [c_void_p, POINTER(MatvecDesc), c_int]),
     "nnhip_quant_matvec_batch_static": (c_int, [c_void_p, POINTER(MatvecDesc), c_int]),
     "nnhip_quant_matvec_fused": (c_int, [c_void_p, POINTER(FusedMatvecDesc)]),

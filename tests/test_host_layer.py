@@ -83,13 +83,15 @@ def test_csharp_declarations_match_the_header():
     # structure sizes: C# field lists (4-byte scalars, 8-byte nint / ulong) against the ctypes structures
     sizes = {"uint": 4, "int": 4, "float": 4, "nint": 8, "ulong": 8}
     for cs_name, ct in (("ErrorInfo", native.ErrorInfo), ("LaneCounters", native.LaneCounters), ("MatvecDesc", native.MatvecDesc),
-                        ("FusedMatvecDesc", native.FusedMatvecDesc), ("MatvecPlanInfo", native.MatvecPlanInfo)):
+                        ("FusedMatvecDesc", native.FusedMatvecDesc), ("MatvecPlanInfo", native.MatvecPlanInfo),
+                        ("BatchLaunchInfo", native.BatchLaunchInfo)):
         body = re.search(r"internal struct %s\s*\{(.*?)\n    \}" % cs_name, cs, re.S).group(1)
         fields = re.findall(r"internal (\w+) \w+;", body)
         offset = 0
         for f in fields:
             offset = (offset + sizes[f] - 1) // sizes[f] * sizes[f] + sizes[f]
-        assert (offset + 7) // 8 * 8 == ctypes.sizeof(ct), (cs_name, offset, ctypes.sizeof(ct))
+        align = max(sizes[f] for f in fields)
+        assert (offset + align - 1) // align * align == ctypes.sizeof(ct), (cs_name, offset, ctypes.sizeof(ct))
         assert len(fields) == len(ct._fields_), cs_name
     assert ctypes.sizeof(native.FusedMatvecDesc) == 120
 
@@ -161,6 +163,138 @@ def test_matvec_plan_keeps_a_ring_turn_inside_the_result_buffer():
     assert lib.nnhip_matvec_plan(99, 1, 256, 19, 256, byref(info)) == 2
     info.struct_size = 8
     assert lib.nnhip_matvec_plan(12, 1, 256, 19, 256, byref(info)) == 1
+
+
+def _batch_plan(lib, descs, compute_units=256, capacity=16):
+    arr = (native.MatvecDesc * max(len(descs), 1))(*descs)
+    out = (native.BatchLaunchInfo * max(capacity, 1))()
+    for o in out:
+        o.struct_size = ctypes.sizeof(native.BatchLaunchInfo)
+    n = c_int(-1)
+    rc = lib.nnhip_matvec_batch_plan(arr, len(descs), compute_units, out if capacity else None, capacity, byref(n))
+    assert rc == 0, native.last_error()[1]
+    return [out[i] for i in range(min(n.value, capacity))], n.value
+
+
+def _desc(typ, rows, in_w, out_w, x=0x1000, w=0x100000, y=0x2000):
+    # (addresses are compared and checked for alignment, never followed: no device is needed)
+    return native.MatvecDesc(x=x, w=w, bias=None, y=y, ggml_type=typ, rows=rows, in_w=in_w, out_w=out_w)
+
+
+def test_batch_plan_groups_a_models_projections_by_type_and_row_length():
+    """The decode batch of a Q8_0 model: one matrix-core launch per row length, every 16-row tile counted once, runs of
+    consecutive tiles per workgroup, and whole tiles in one stage buffer where rows are not a multiple of 128 bytes
+    (5376 weights = 5712 bytes)."""
+    lib = native.load_library()
+    descs = []
+    for layer in range(48):
+        descs += [_desc(8, 1, 5376, 21504, x=0x1000 + layer * 0x10000), _desc(8, 1, 5376, 21504, x=0x1000 + layer * 0x10000),
+                  _desc(8, 1, 21504, 5376, x=0x8000 + layer * 0x10000), _desc(8, 1, 4096, 5376, x=0xc000 + layer * 0x10000)]
+    launches, n = _batch_plan(lib, descs)
+    assert n == 3 and [(l.ggml_type, l.kernel, l.in_w) for l in launches] == [(8, 2, 5376), (8, 2, 21504), (8, 2, 4096)]
+    assert [l.entries for l in launches] == [96, 48, 48]
+    assert [l.units for l in launches] == [96 * 1344, 48 * 336, 48 * 336]
+    for l in launches:
+        assert l.groups == 256 and l.rows_per_pass == 1 and l.consecutive_runs == 1 and l.activations_in_lds == 1
+        assert l.threads % 128 == 0 and 512 <= l.threads <= 768
+        assert l.dynamic_lds_bytes + 2048 <= 160 * 1024
+    assert [l.stage_buffers for l in launches] == [1, 2, 2]
+    # a stage buffer of the 5376-wide launch holds a whole tile (16 rows of 5712 bytes) beside the four digit planes
+    assert launches[0].dynamic_lds_bytes >= 16 * 5712 + 4 * 5376
+    # fewer compute units than tiles or more: one workgroup per unit at most
+    launches, _ = _batch_plan(lib, [_desc(8, 1, 4096, 16 * 2100)], compute_units=4096)
+    assert launches[0].kernel == 2 and launches[0].groups == 2100
+
+
+def test_batch_plan_threshold_counts_tiles_once_per_input_row():
+    lib = native.load_library()
+    # 2047 tiles: the row-step kernel; one more tile from a second matrix of the same type and row length: the matrix cores
+    launches, n = _batch_plan(lib, [_desc(12, 1, 4096, 16 * 2047)])
+    assert n == 1 and launches[0].kernel == 0 and launches[0].stage_buffers == 0
+    launches, n = _batch_plan(lib, [_desc(12, 1, 4096, 16 * 2047), _desc(12, 1, 4096, 9)])
+    assert n == 1 and launches[0].kernel == 2 and launches[0].units == 2048 and launches[0].entries == 2
+    # a different row length or type does not count towards the group
+    launches, n = _batch_plan(lib, [_desc(12, 1, 4096, 16 * 2047), _desc(12, 1, 5120, 16), _desc(13, 1, 4096, 16)])
+    assert n == 2 and all(l.kernel == 0 for l in launches) and [l.ggml_type for l in launches] == [12, 13]
+    assert launches[0].entries == 2 and launches[0].in_w == 5120
+    # input rows count: 4 rows x 512 tiles
+    launches, n = _batch_plan(lib, [_desc(12, 4, 4096, 16 * 512)])
+    assert n == 1 and launches[0].kernel == 2 and launches[0].rows_per_pass == 4 and launches[0].units == 512
+    launches, n = _batch_plan(lib, [_desc(12, 4, 4096, 16 * 511)])
+    assert n == 1 and launches[0].kernel == 0 and launches[0].entries == 4
+    # a weight pointer the 16-byte loads cannot take keeps a Q6_K matrix with the row-step kernel (4-byte alignment is its rule)
+    launches, n = _batch_plan(lib, [_desc(14, 1, 4096, 16 * 3000, w=0x100004)])
+    assert n == 1 and launches[0].kernel == 0
+    # Q6_K and IQ2_S rows must hold an even number of 256-blocks for the matrix cores
+    for typ in (14, 22):
+        assert _batch_plan(lib, [_desc(typ, 1, 256 * 17, 16 * 3000)])[0][0].kernel == 0
+        assert _batch_plan(lib, [_desc(typ, 1, 256 * 18, 16 * 3000)])[0][0].kernel == 2
+    # below 1024 weights a row: never
+    assert _batch_plan(lib, [_desc(12, 1, 768, 16 * 5000)])[0][0].kernel == 0
+
+
+def test_batch_plan_shared_passes_and_tile_order():
+    lib = native.load_library()
+    # twenty matrices on one activation vector: every groups-th tile; a vector per matrix: runs of consecutive tiles
+    shared, _ = _batch_plan(lib, [_desc(12, 1, 5120, 17408)] * 20)
+    own, _ = _batch_plan(lib, [_desc(12, 1, 5120, 17408, x=0x1000 + i * 0x10000) for i in range(20)])
+    assert shared[0].kernel == own[0].kernel == 2 and shared[0].units == own[0].units == 20 * 1088
+    assert (shared[0].consecutive_runs, own[0].consecutive_runs) == (0, 1)
+    assert shared[0].activations_in_lds == 0                  # (5120 = 20 blocks fit the register form)
+    # two vectors (one change along the table) still deal every groups-th tile
+    two, _ = _batch_plan(lib, [_desc(12, 1, 5120, 17408)] * 10 + [_desc(12, 1, 5120, 17408, x=0x9000)] * 10)
+    assert two[0].consecutive_runs == 0
+    # input rows of a descriptor share passes four at a time; K-quants from two rows on, Q8_0 from three
+    for typ, rows, entries, per_pass in ((12, 2, 1, 2), (12, 4, 1, 4), (12, 6, 2, 4), (13, 9, 3, 4), (14, 16, 4, 4), (22, 5, 2, 4),
+                                         (8, 2, 2, 1), (8, 3, 1, 3), (8, 7, 2, 4)):
+        in_w = 5376 if typ == 8 else 5120 if typ != 22 else 4096
+        launches, n = _batch_plan(lib, [_desc(typ, rows, in_w, 17408)])
+        l = launches[0]
+        assert n == 1 and l.kernel == 2 and (l.entries, l.rows_per_pass) == (entries, per_pass), (typ, rows, l.entries, l.rows_per_pass)
+        assert l.units == entries * 1088 and l.activations_in_lds == 1
+        assert l.dynamic_lds_bytes + (8192 if per_pass > 1 else 2048) + (2048 if typ == 22 else 0) <= 160 * 1024
+    # 21504-wide planes of four rows do not fit LDS: those rows get an entry each
+    launches, _ = _batch_plan(lib, [_desc(8, 4, 21504, 16384)])
+    assert launches[0].kernel == 2 and (launches[0].entries, launches[0].rows_per_pass) == (4, 1)
+    # descriptors with and without shared passes of one type and row length make two launches
+    launches, n = _batch_plan(lib, [_desc(12, 1, 4096, 16 * 2048), _desc(12, 3, 4096, 16 * 2048)])
+    assert n == 2 and sorted(l.rows_per_pass for l in launches) == [1, 3]
+
+
+def test_batch_plan_mixed_types_and_errors():
+    lib = native.load_library()
+    descs = [_desc(12, 1, 4096, 16 * 3000), _desc(14, 1, 4096, 16 * 3000), _desc(21, 1, 4096, 100), _desc(8, 1, 160, 19),
+             _desc(22, 1, 4096, 16 * 3000), _desc(30, 2, 4096, 77), _desc(8, 1, 64, 5)]
+    launches, n = _batch_plan(lib, descs)
+    kinds = [(l.ggml_type, l.kernel) for l in launches]
+    # matrix-core groups first, then the row-step launches in type order, then Q8_0 rows with an odd number of blocks
+    assert n == 7 and kinds == [(12, 2), (14, 2), (22, 2), (8, 0), (21, 0), (30, 0), (8, 1)]
+    assert launches[5].entries == 2 and launches[6].in_w == 160 and launches[6].entries == 1
+    # a small capacity still reports the count and fills what fits
+    few, n = _batch_plan(lib, descs, capacity=2)
+    assert n == 7 and [(l.ggml_type, l.kernel) for l in few] == kinds[:2]
+    none, n = _batch_plan(lib, descs, capacity=0)
+    assert n == 7 and none == []
+    assert _batch_plan(lib, [])[1] == 0
+    # the descriptor checks of the batch itself
+    n = c_int()
+    out = (native.BatchLaunchInfo * 1)()
+    out[0].struct_size = ctypes.sizeof(native.BatchLaunchInfo)
+    one = (native.MatvecDesc * 1)
+
+    def status(d, cus=256):
+        return lib.nnhip_matvec_batch_plan(one(d), 1, cus, out, 1, byref(n))
+
+    assert status(_desc(12, 1, 4096, 16, w=0x100004)) == 1 and "16-byte" in native.last_error()[1]
+    assert status(_desc(12, 1, 4000, 16)) == 3
+    assert status(_desc(99, 1, 4096, 16)) == 2
+    assert status(_desc(12, 0, 4096, 16)) == 1
+    assert status(_desc(12, 1, 256 * 300, 16)) == 8
+    assert status(_desc(12, 1, 4096, 16, x=0)) == 1
+    assert status(_desc(12, 1, 4096, 16), cus=0) == 1
+    assert lib.nnhip_matvec_batch_plan(one(_desc(12, 1, 4096, 16)), 1, 256, out, 1, None) == 1
+    out[0].struct_size = 8
+    assert status(_desc(12, 1, 4096, 16)) == 1 and "struct_size" in native.last_error()[1]
 
 
 def test_bad_handles_are_reported_not_dereferenced():
