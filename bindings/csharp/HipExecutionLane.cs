@@ -49,6 +49,33 @@ public sealed unsafe class HipExecutionLane : IDisposable
         return buffer;
     }
 
+    /// <summary>Uploads <paramref name="bytes"/> bytes that sit at <paramref name="fileOffset"/> of an open file: the
+    /// library reads the range through two pinned buffers of its own, one travelling while the other is filled, so no
+    /// managed array of the tensor's size exists (the pair ReadTensorBytes + UploadRaw of
+    /// Qwen35QuantizedModel.LoadTensor in one call).  On Linux a SafeFileHandle's handle is the descriptor.</summary>
+    public HipBuffer UploadFromFile(Microsoft.Win32.SafeHandles.SafeFileHandle file, long fileOffset, long bytes)
+    {
+        HipBuffer buffer = AllocateBytes(Math.Max(bytes, 4));
+        bool held = false;
+        try
+        {
+            file.DangerousAddRef(ref held);
+            lock (_sync)
+                NnHipNative.Check(NnHipNative.nnhip_upload_from_file(Handle, buffer.Pointer, 0, (int)file.DangerousGetHandle(),
+                                                                     (ulong)fileOffset, (nuint)bytes), "upload");
+        }
+        catch
+        {
+            buffer.Dispose();
+            throw;
+        }
+        finally
+        {
+            if (held) file.DangerousRelease();
+        }
+        return buffer;
+    }
+
     public void Read(HipBuffer buffer, Span<float> values)
     {
         lock (_sync)

@@ -77,6 +77,7 @@ internal static unsafe partial class NnHipNative
     [LibraryImport(Library)] internal static partial int nnhip_free(nint lane, nint dptr);
     [LibraryImport(Library)] internal static partial int nnhip_lane_trim(nint lane);
     [LibraryImport(Library)] internal static partial int nnhip_upload(nint lane, nint dptr, nuint offset, void* host, nuint bytes);
+    [LibraryImport(Library)] internal static partial int nnhip_upload_from_file(nint lane, nint dptr, nuint offset, int fd, ulong fileOffset, nuint bytes);
     [LibraryImport(Library)] internal static partial int nnhip_download(nint lane, nint dptr, nuint offset, void* host, nuint bytes);
     [LibraryImport(Library)] internal static partial int nnhip_copy(nint lane, nint dst, nuint dstOffset, nint src, nuint srcOffset, nuint bytes);
     [LibraryImport(Library)] internal static partial int nnhip_fill_u32(nint lane, nint dptr, nuint offset, uint value, nuint count);

@@ -154,6 +154,14 @@ NNHIP_API int nnhip_lane_trim(void* lane);
  * interpreted: GGUF blocks go up exactly as they sit in the file. */
 NNHIP_API int nnhip_upload(void* lane, void* dptr, size_t offset, const void* host, size_t bytes);
 NNHIP_API int nnhip_download(void* lane, const void* dptr, size_t offset, void* host, size_t bytes);
+/* nnhip_upload of `bytes` bytes that sit at `file_offset` of the open file `fd` (a POSIX descriptor; the file position
+ * is not used or moved): the library reads the range piece by piece into two pinned buffers of its own and copies one
+ * piece while it reads the next, so the caller holds no copy of the tensor and the copy does not wait for the read.
+ * Replaces the pair GgufReader.ReadTensorBytes (GgufReader.cs:107-123) + UploadRaw that
+ * Qwen35QuantizedModel.LoadTensor issues per tensor (Qwen35QuantizedModel.cs:234-243).  Blocking; a range that
+ * reaches past the end of the file is NNHIP_ERR_INVALID_ARGUMENT (what arrived before it is counted in h2d_bytes).
+ * One lane = one thread at a time, as for every call; lanes of several threads may read one descriptor. */
+NNHIP_API int nnhip_upload_from_file(void* lane, void* dptr, size_t offset, int fd, uint64_t file_offset, size_t bytes);
 /* Device-to-device copy on the lane's stream (asynchronous).  Replaces the lane's CopyBuffer used for KV
  * growth and staging (Qwen35QuantizedModel.cs:1037-1061). */
 NNHIP_API int nnhip_copy(void* lane, void* dst, size_t dst_offset, const void* src, size_t src_offset, size_t bytes);

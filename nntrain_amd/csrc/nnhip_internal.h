@@ -19,6 +19,7 @@ constexpr uint32_t kGraphMagic = 0x4e475248u;  // "NGRH"
 
 constexpr size_t kCacheBlockMax = 64u << 20;   // larger blocks (weights) are returned to the driver when freed
 constexpr size_t kCacheTotalMax = 1u << 30;    // most bytes a lane keeps for reuse
+constexpr size_t kStagingBytes = 16u << 20;    // one pinned staging buffer of a file upload
 
 struct Lane {
     uint32_t magic = kLaneMagic;
@@ -39,6 +40,10 @@ struct Lane {
     std::vector<void*> retired_tables;          // outgrown tables: freed with the lane, a captured graph may name them
     std::vector<char> batch_shadow;             // the entries the device table holds now (empty: unknown)
     void* static_table = nullptr;               // this device's address of the library's fixed batch workspace
+    // Two pinned host buffers (and an event each) through which nnhip_upload_from_file moves a file range: the next piece
+    // is read while the last one travels.  Allocated by the first such upload, freed with the lane.
+    void* staging[2] = {nullptr, nullptr};
+    hipEvent_t staging_done[2] = {nullptr, nullptr};
 };
 
 struct Event {

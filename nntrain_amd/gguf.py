@@ -240,6 +240,18 @@ class GgufReader:
             done += len(piece)
         return chunks[0] if len(chunks) == 1 else b"".join(chunks)
 
+    def tensor_file_range(self, tensor: GgufTensorInfo, start: int, byte_count: int) -> tuple[int, int]:
+        """(file descriptor, absolute file offset) of bytes [start, start + byte_count) of a tensor's payload, after the
+        same checks as read_tensor_range: for uploads that read the file themselves (positional reads: the descriptor's
+        own position is neither used nor moved)."""
+        total = tensor.byte_count()
+        if start < 0 or byte_count < 0 or start + byte_count > total:
+            raise ValueError("range is outside the tensor payload")
+        offset = self._data_offset + tensor.offset + start
+        if offset > self._size or byte_count > self._size - offset:
+            raise EOFError("tensor payload exceeds the file")
+        return self._fd, offset
+
     def matrix_dims(self, tensor: GgufTensorInfo) -> tuple[int, int]:
         """(input_width, output_width) of a 2-D weight: GGUF stores ne0 = K first (Qwen35Gguf.cs:170-182)."""
         if len(tensor.shape) != 2:

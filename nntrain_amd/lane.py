@@ -156,6 +156,13 @@ class HipExecutionLane:
         check(self._lib.nnhip_upload(self._handle, c_void_p(buf._require()), offset, a.ctypes.data_as(c_void_p), a.nbytes),
               "upload")
 
+    def write_from_file(self, buf: HipBuffer, fd: int, file_offset: int, nbytes: int, offset: int = 0) -> None:
+        """`nbytes` bytes at `file_offset` of the open file `fd` into the buffer at `offset`: read and copied by the
+        library through its pinned staging buffers, a piece travelling while the next is read."""
+        if nbytes < 0 or offset < 0 or offset + nbytes > buf.nbytes:
+            raise ValueError("write exceeds the buffer")
+        check(self._lib.nnhip_upload_from_file(self._handle, c_void_p(buf._require()), offset, fd, file_offset, nbytes), "upload")
+
     def read(self, buf: HipBuffer, dtype=np.float32, count: int | None = None, offset: int = 0) -> np.ndarray:
         itemsize = np.dtype(dtype).itemsize
         if count is None:

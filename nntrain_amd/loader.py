@@ -120,16 +120,19 @@ def widen_dense(tensor_type: int, payload: bytes) -> np.ndarray:
 class HipGgufLoader:
     """Uploads tensors of one GGUF file to one lane.
 
-    A quantized matrix is read and uploaded in pieces of `chunk_bytes`, so the host never holds more than one piece of
-    it; the reads are positional, so several loaders (one per lane, one thread each) may share a reader.
+    A quantized matrix goes from the file to the device inside the library (`staged`, the default: positional reads
+    into two pinned buffers, one travelling while the other is filled), or is read here and uploaded in pieces of
+    `chunk_bytes`; either way the host never holds more than a piece of it, and the reads are positional, so several
+    loaders (one per lane, one thread each) may share a reader.
     """
 
-    def __init__(self, lane: HipExecutionLane, reader: GgufReader, chunk_bytes: int = 64 << 20):
+    def __init__(self, lane: HipExecutionLane, reader: GgufReader, chunk_bytes: int = 64 << 20, staged: bool = True):
         if chunk_bytes <= 0:
             raise ValueError("chunk_bytes must be positive")
         self.lane = lane
         self.reader = reader
         self.chunk_bytes = chunk_bytes
+        self.staged = staged
         self.quantized_bytes = 0
         self.dense_bytes = 0
 
@@ -143,11 +146,15 @@ class HipGgufLoader:
             raise InvalidDataError(f"Matrix '{info.name}' has an inconsistent block geometry.")
         buffer = self.lane.allocate_bytes(nbytes)
         try:
-            done = 0
-            while done < nbytes:
-                piece = self.reader.read_tensor_range(info, done, min(self.chunk_bytes, nbytes - done))
-                self.lane.write(buffer, np.frombuffer(piece, dtype=np.uint8), offset=done)
-                done += len(piece)
+            if self.staged:
+                fd, file_offset = self.reader.tensor_file_range(info, 0, nbytes)
+                self.lane.write_from_file(buffer, fd, file_offset, nbytes)
+            else:
+                done = 0
+                while done < nbytes:
+                    piece = self.reader.read_tensor_range(info, done, min(self.chunk_bytes, nbytes - done))
+                    self.lane.write(buffer, np.frombuffer(piece, dtype=np.uint8), offset=done)
+                    done += len(piece)
         except BaseException:
             buffer.dispose()
             raise

@@ -82,6 +82,7 @@ PROTOTYPES = {
     "nnhip_free": (c_int, [c_void_p, c_void_p]),
     "nnhip_lane_trim": (c_int, [c_void_p]),
     "nnhip_upload": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p, c_size_t]),
+    "nnhip_upload_from_file": (c_int, [c_void_p, c_void_p, c_size_t, c_int, c_uint64, c_size_t]),
     "nnhip_download": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p, c_size_t]),
     "nnhip_copy": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p, c_size_t, c_size_t]),
     "nnhip_fill_u32": (c_int, [c_void_p, c_void_p, c_size_t, c_uint32, c_size_t]),

@@ -75,7 +75,7 @@ def _model(tmp_path, name, qkv_types=(GGML_Q4_K,) * 3, tied=False, extra=None, d
     return write_gguf(tmp_path / name, tensors, kvs), host
 
 
-def _cpu_logits(host, token, tied=False):
+def _cpu_logits(host, token, tied=False, trace=None):
     def w(name):
         typ, raw, out_w, in_w = host[name]
         return oracle.dequantize(typ, raw).reshape(out_w, in_w).astype(np.float64)
@@ -88,6 +88,8 @@ def _cpu_logits(host, token, tied=False):
         p = f"blk.{i}."
         n = oracle.rms_norm(hidden, host[p + "attn_norm.weight"], 1, EMB, EPS).ravel()
         v = mv(p + "attn_v.weight", n).reshape(KV, HW)
+        if trace is not None:           # (the last layer's projections stay: the loop's q|k|v buffer holds them afterwards)
+            trace["qkv"] = np.concatenate([mv(p + "attn_q.weight", n), mv(p + "attn_k.weight", n), v.ravel()])
         ctx = np.repeat(v, HEADS // KV, axis=0).ravel()
         attn = mv(p + "attn_output.weight", ctx)
         hidden, m = oracle.add_rms_norm(hidden, attn, host[p + "ffn_norm.weight"], 1, EMB, EPS)
@@ -115,9 +117,16 @@ def test_logits_match_the_cpu_restatement_and_all_three_loops_agree_bitwise(lane
                 assert after["kernel_launches"] - mid["kernel_launches"] == 1 + 12 * LAYERS + 2
                 assert mid["h2d_bytes"] == before["h2d_bytes"] and mid["allocated_bytes"] == before["allocated_bytes"]
                 assert np.array_equal(got.view(np.uint32), ref.view(np.uint32))
-                want = _cpu_logits(host, token)
+                trace = {}
+                want = _cpu_logits(host, token, trace=trace)
                 assert oracle.rel_l2(got, want) <= 1e-5
                 assert int(np.argmax(got)) == int(np.argmax(want))
+                # the query and key projections feed nothing in a first-token pass (attention over one position returns
+                # the values), so the logits do not cover them: the last layer's q | k | v against the CPU, piece by piece
+                for dec in (fused, plain):
+                    qkv = lane.read(dec._qkv, count=(HEADS + 2 * KV) * HW)
+                    for lo, hi in ((0, HEADS * HW), (HEADS * HW, (HEADS + KV) * HW), ((HEADS + KV) * HW, (HEADS + 2 * KV) * HW)):
+                        assert oracle.rel_l2(qkv[lo:hi], trace["qkv"][lo:hi]) <= 1e-5, (dec is fused, lo)
             # graph replay of the layers and the head
             eager = [lane.read(fused.forward_token(t), count=VOCAB) for t in (3, 11, 5)]
             fused.capture_graph()

@@ -300,6 +300,7 @@ def test_batch_plan_mixed_types_and_errors():
 def test_bad_handles_are_reported_not_dereferenced():
     lib = native.load_library()
     assert lib.nnhip_synchronize(None) == 7
+    assert lib.nnhip_upload_from_file(None, None, 0, 0, 0, 16) == 7
     p = c_void_p()
     assert lib.nnhip_alloc(None, 16, byref(p)) == 7
     assert lib.nnhip_quant_matvec(None, 8, None, None, None, None, 1, 32, 1) == 7
