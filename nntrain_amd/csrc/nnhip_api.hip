@@ -61,6 +61,58 @@ int check_linear(uint32_t op, Lane* lane, uint32_t type, const void* x, const vo
     return NNHIP_OK;
 }
 
+// Moves `bytes` bytes to the device through the lane's two pinned staging buffers: `fill(dst, done, want)` puts bytes
+// [done, done + want) of the source into `dst` (returning a status), and piece i is filled into buffer i % 2 while
+// piece i - 1 travels from the other one; a buffer is reused once the copy that last read it has completed.  On any
+// failure the stream is drained before returning: no copy may still read a buffer that the next call fills.
+template <class Fill>
+int staged_upload(nnhip::Lane* lane, void* dptr, size_t offset, size_t bytes, Fill&& fill)
+{
+    for (int i = 0; i < 2; ++i) {
+        if (!lane->staging[i]) {
+            const hipError_t e = hipHostMalloc(&lane->staging[i], kStagingBytes, hipHostMallocDefault);
+            if (e != hipSuccess) {
+                lane->staging[i] = nullptr;
+                return hip_fail(e, NNHIP_OP_UPLOAD, lane->device, "pinned staging buffer");
+            }
+        }
+        if (!lane->staging_done[i]) {
+            const hipError_t e = hipEventCreateWithFlags(&lane->staging_done[i], hipEventDisableTiming);
+            if (e != hipSuccess) {
+                lane->staging_done[i] = nullptr;
+                return hip_fail(e, NNHIP_OP_UPLOAD, lane->device, "staging event");
+            }
+        }
+    }
+    size_t done = 0;
+    int status = NNHIP_OK;
+    for (int piece = 0; done < bytes; ++piece) {
+        const int slot = piece & 1;
+        if (piece >= 2) {
+            const hipError_t e = hipEventSynchronize(lane->staging_done[slot]);
+            if (e != hipSuccess) {
+                status = hip_fail(e, NNHIP_OP_UPLOAD, lane->device, "waiting for a staging buffer");
+                break;
+            }
+        }
+        const size_t want = bytes - done < kStagingBytes ? bytes - done : kStagingBytes;
+        status = fill(lane->staging[slot], done, want);
+        if (status != NNHIP_OK) break;
+        hipError_t e = hipMemcpyAsync(static_cast<char*>(dptr) + offset + done, lane->staging[slot], want, hipMemcpyHostToDevice, lane->stream);
+        if (e == hipSuccess) e = hipEventRecord(lane->staging_done[slot], lane->stream);
+        if (e != hipSuccess) {
+            status = hip_fail(e, NNHIP_OP_UPLOAD, lane->device, "host-to-device copy");
+            break;
+        }
+        done += want;
+    }
+    const hipError_t e = hipStreamSynchronize(lane->stream);
+    if (status == NNHIP_OK && e != hipSuccess) status = hip_fail(e, NNHIP_OP_UPLOAD, lane->device, "host-to-device copy");
+    std::lock_guard<std::mutex> guard(lane->mutex);
+    lane->counters.h2d_bytes += done;
+    return status;
+}
+
 }  // namespace
 
 bool type_block(uint32_t type, int* elems, int* bytes)
@@ -362,66 +414,22 @@ int nnhip_upload_from_file(void* handle, void* dptr, size_t offset, int fd, uint
     if (bytes == 0) return NNHIP_OK;
     if (!dptr || fd < 0) return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_UPLOAD, lane->device, 0, "null device pointer or negative file descriptor");
     if (lane->capturing) return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_UPLOAD, lane->device, 0, "no transfer while a graph is being captured");
-    for (int i = 0; i < 2; ++i) {
-        if (!lane->staging[i]) {
-            const hipError_t e = hipHostMalloc(&lane->staging[i], kStagingBytes, hipHostMallocDefault);
-            if (e != hipSuccess) {
-                lane->staging[i] = nullptr;
-                return hip_fail(e, NNHIP_OP_UPLOAD, lane->device, "pinned staging buffer");
-            }
-        }
-        if (!lane->staging_done[i]) {
-            const hipError_t e = hipEventCreateWithFlags(&lane->staging_done[i], hipEventDisableTiming);
-            if (e != hipSuccess) {
-                lane->staging_done[i] = nullptr;
-                return hip_fail(e, NNHIP_OP_UPLOAD, lane->device, "staging event");
-            }
-        }
-    }
-    // Piece i is read into buffer i % 2 while piece i - 1 travels from the other one; a buffer is reused once the copy
-    // that last read it has completed.  On any failure the stream is drained before returning: no copy may still read
-    // a buffer that the next call fills.
-    size_t done = 0;
-    int status = NNHIP_OK;
-    for (int piece = 0; done < bytes && status == NNHIP_OK; ++piece) {
-        const int slot = piece & 1;
-        if (piece >= 2) {
-            const hipError_t e = hipEventSynchronize(lane->staging_done[slot]);
-            if (e != hipSuccess) {
-                status = hip_fail(e, NNHIP_OP_UPLOAD, lane->device, "waiting for a staging buffer");
-                break;
-            }
-        }
-        const size_t want = bytes - done < kStagingBytes ? bytes - done : kStagingBytes;
+    const int device = lane->device;
+    return staged_upload(lane, dptr, offset, bytes, [&](void* dst, size_t done, size_t want) {
         size_t got = 0;
         while (got < want) {
-            const ssize_t n = pread(fd, static_cast<char*>(lane->staging[slot]) + got, want - got,
-                                    static_cast<off_t>(file_offset + done + got));
+            const ssize_t n = pread(fd, static_cast<char*>(dst) + got, want - got, static_cast<off_t>(file_offset + done + got));
             if (n > 0) {
                 got += static_cast<size_t>(n);
             } else if (n == 0) {
-                status = fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_UPLOAD, lane->device, 0,
-                              "the file ends %zu bytes before the end of the range", bytes - done - got);
-                break;
+                return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_UPLOAD, device, 0,
+                            "the file ends %zu bytes before the end of the range", bytes - done - got);
             } else if (errno != EINTR) {
-                status = fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_UPLOAD, lane->device, 0, "reading the file failed: %s", strerror(errno));
-                break;
+                return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_UPLOAD, device, 0, "reading the file failed: %s", strerror(errno));
             }
         }
-        if (status != NNHIP_OK) break;
-        hipError_t e = hipMemcpyAsync(static_cast<char*>(dptr) + offset + done, lane->staging[slot], want, hipMemcpyHostToDevice, lane->stream);
-        if (e == hipSuccess) e = hipEventRecord(lane->staging_done[slot], lane->stream);
-        if (e != hipSuccess) {
-            status = hip_fail(e, NNHIP_OP_UPLOAD, lane->device, "host-to-device copy");
-            break;
-        }
-        done += want;
-    }
-    const hipError_t e = hipStreamSynchronize(lane->stream);
-    if (status == NNHIP_OK && e != hipSuccess) status = hip_fail(e, NNHIP_OP_UPLOAD, lane->device, "host-to-device copy");
-    std::lock_guard<std::mutex> guard(lane->mutex);
-    lane->counters.h2d_bytes += done;
-    return status;
+        return static_cast<int>(NNHIP_OK);
+    });
 }
 
 int nnhip_download(void* handle, const void* dptr, size_t offset, void* host, size_t bytes)
