@@ -8,6 +8,9 @@ per token).  A "step" is one token: every mat-vec of the set once, fresh N(0,1) 
 
 Other workloads (`--workload gemv|prefill|ffn|decode_loop|decode27b_chained|all`) time the single-matrix configurations,
 the fused layer half, the GGUF decode loop and the 27B-shape token in dependency order; they are reported under "also".
+`--workload library_gemm` (never part of "all") times the ROCm library's bfloat16 GEMM on the prefill shape through
+torch.matmul, weights already decoded, as a yardstick for the machine; it does not load this library (PyTorch carries a
+HIP runtime of its own, and two of them in one process do not both see the device).
 
 One JSON line on stdout; progress on stderr.
 """
@@ -760,12 +763,48 @@ def _prefill_of(lane, nn, oracle, typ, tname, ms_list):
     return out
 
 
+def library_gemm_yardstick(ms_list=(128, 256, 512, 2048)):
+    """What the ROCm library GEMM (torch.matmul, bfloat16 weights already decoded and resident) reaches on the prefill
+    shape on this box: a yardstick to read the prefill kernel's own figures against, nothing the product uses."""
+    try:
+        import torch
+        if not torch.cuda.is_available():
+            return {"unavailable": "torch sees no device"}
+        in_w, out_w = 5120, 17408
+        w = torch.randn(out_w, in_w, device="cuda", dtype=torch.bfloat16)
+        out = {}
+        for m in ms_list:
+            x = torch.randn(m, in_w, device="cuda", dtype=torch.bfloat16)
+            for _ in range(5):
+                y = x @ w.t()
+            torch.cuda.synchronize()
+            samples = []
+            for _ in range(5):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for _ in range(5):
+                    y = x @ w.t()
+                e1.record()
+                torch.cuda.synchronize()
+                samples.append(e0.elapsed_time(e1) / 5)
+            ms = float(np.median(samples))
+            flops = 2.0 * m * in_w * out_w
+            out[f"M={m}"] = {"ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 1),
+                             "vs_2500_TFLOPs_bf16": round(flops / ms / 1e9 / BF16_PEAK_TFLOPS, 4)}
+            log(f"[prefill] library bf16 GEMM (torch.matmul) M={m}: {ms:.3f} ms, {flops / ms / 1e9:.0f} TFLOP/s")
+            del x, y
+        return out
+    except Exception as e:          # a yardstick only: its absence must not fail the run
+        return {"unavailable": f"{type(e).__name__}: {e}"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", choices=["decode27b", "decode27b_chained", "gemv", "prefill", "ffn", "decode_loop", "all"], default="all")
+    ap.add_argument("--workload", choices=["decode27b", "decode27b_chained", "gemv", "prefill", "ffn", "decode_loop", "all", "library_gemm"],
+                    default="all")
     ap.add_argument("--mode", choices=["forward", "graph", "batch"], default="batch",
                     help="decode27b: one launch per matrix, the same captured in a HIP graph, or the batched entry point")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -778,6 +817,16 @@ def main():
     if args.gpus != 1:
         raise SystemExit("this build measures one GPU: the quantized linear path has no collectives and every box has a "
                          "single MI355X; run with --gpus 1")
+
+    if args.workload == "library_gemm":
+        res = library_gemm_yardstick()
+        at512 = res.get("M=512", {})
+        print(json.dumps({"metric": "library bf16 GEMM on the prefill shape (torch.matmul), TFLOP/s at M=512", "value": at512.get("tflops"),
+                          "unit": "TFLOP/s", "n_gpus": 1, "steps": 25, "warmup": 5, "ms_per_step": at512.get("ms"),
+                          "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+                          "config": {"workload": "library_gemm 17408x5120, M = 128 / 256 / 512 / 2048"}, "roofline": None,
+                          "cpu_baseline": None, "also": {"library_bf16_gemm": res}}), flush=True)
+        return
 
     import nntrain_amd as nn
     import oracle
