@@ -222,6 +222,9 @@ typedef struct nnhip_matvec_plan_info {
 NNHIP_API int nnhip_matvec_plan(uint32_t ggml_type, int rows, int in_w, int out_w, int compute_units,
                                 nnhip_matvec_plan_info* info);
 
+/* Most mat-vec rows (descriptors counted once per input row) one batched call takes: 80 MB of descriptor table. */
+#define NNHIP_BATCH_MAX_ENTRIES (1 << 20)
+
 /* `count` independent mat-vecs enqueued as one unit of work (a single launch per group of equal type), for the
  * per-token projection sets that ForwardTokenDevice issues back to back (Qwen35QuantizedModel.cs:451-513).
  * `descs` is a host array, read before the call returns.  Results are identical to `count` nnhip_quant_matvec calls,
@@ -237,7 +240,8 @@ NNHIP_API int nnhip_matvec_plan(uint32_t ggml_type, int rows, int in_w, int out_
  * (skipped when the table already holds them), so the call never waits for the device.  Under graph capture the write
  * is recorded with the launch and a replay restores the table it needs; the table cannot grow during a capture
  * (NNHIP_ERR_INVALID_ARGUMENT: issue a batch at least as large once before capturing), and tables a graph may name are
- * kept until the lane is destroyed.  Asynchronous. */
+ * kept until the lane is destroyed.  A descriptor takes at most 65535 input rows and a call at most
+ * NNHIP_BATCH_MAX_ENTRIES rows in all (NNHIP_ERR_TOO_LARGE).  Asynchronous. */
 NNHIP_API int nnhip_quant_matvec_batch(void* lane, const nnhip_matvec_desc* descs, int count);
 
 /* The launches nnhip_quant_matvec_batch would split `count` descriptors into, without a device: one structure per launch,

@@ -707,20 +707,43 @@ int nnhip_lora_b(void* handle, const float* z, const float* b, float* y, int row
     return NNHIP_OK;
 }
 
-int nnhip_quant_matvec_batch(void* handle, const nnhip_matvec_desc* descs, int count)
+// The checks every entry point that takes a descriptor array makes; *entries receives the mat-vec rows of the batch.
+static int check_batch(nnhip::Lane* lane, const nnhip_matvec_desc* descs, int count, long* entries)
 {
-    NNHIP_LANE(handle, NNHIP_OP_MATVEC_BATCH)
+    using namespace nnhip;
     if (count < 0 || (count > 0 && !descs))
         return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_MATVEC_BATCH, lane->device, 0, "descriptor array is null or count negative");
+    long total = 0;
     for (int i = 0; i < count; ++i) {
         const nnhip_matvec_desc& d = descs[i];
         int rc = check_linear(NNHIP_OP_MATVEC_BATCH, lane, d.ggml_type, d.x, d.w, d.y, d.rows, d.in_w, d.out_w);
         if (rc != NNHIP_OK) return rc;
         if (d.in_w > matvec_max_in_w(d.ggml_type))
             return fail(NNHIP_ERR_TOO_LARGE, NNHIP_OP_MATVEC_BATCH, lane->device, 0, "descriptor %d: in_w %d exceeds the %d values one workgroup can stage", i, d.in_w, matvec_max_in_w(d.ggml_type));
+        if (d.rows > 65535)
+            return fail(NNHIP_ERR_TOO_LARGE, NNHIP_OP_MATVEC_BATCH, lane->device, 0, "descriptor %d: rows %d exceeds 65535", i, d.rows);
+        total += d.rows;
     }
+    if (total > NNHIP_BATCH_MAX_ENTRIES)
+        return fail(NNHIP_ERR_TOO_LARGE, NNHIP_OP_MATVEC_BATCH, lane->device, 0,
+                    "the batch has %ld mat-vec rows; a call takes at most %d (split the batch)", total, NNHIP_BATCH_MAX_ENTRIES);
+    *entries = total;
+    return NNHIP_OK;
+}
+
+int nnhip_quant_matvec_batch(void* handle, const nnhip_matvec_desc* descs, int count)
+{
+    NNHIP_LANE(handle, NNHIP_OP_MATVEC_BATCH)
+    long entries = 0;
+    const int rc = check_batch(lane, descs, count, &entries);
+    if (rc != NNHIP_OK) return rc;
     if (count == 0) return NNHIP_OK;
-    hipError_t e = launch_matvec_batch(lane, descs, count);
+    hipError_t e = hipSuccess;
+    try {
+        e = launch_matvec_batch(lane, descs, count);
+    } catch (const std::bad_alloc&) {       // (the host copy of the table)
+        return fail(NNHIP_ERR_OUT_OF_MEMORY, NNHIP_OP_MATVEC_BATCH, lane->device, 0, "host memory for the descriptor table");
+    }
     if (e == hipErrorStreamCaptureUnsupported)
         return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_MATVEC_BATCH, lane->device, static_cast<uint32_t>(e),
                     "the batch needs a larger descriptor table than the lane holds, and a table cannot grow while a graph is "
@@ -739,14 +762,15 @@ int nnhip_matvec_batch_plan(const nnhip_matvec_desc* descs, int count, int compu
             return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_MATVEC_BATCH, -1, 0, "launches[%d] has the wrong struct_size", i);
     Lane nowhere;
     nowhere.device = -1;
-    for (int i = 0; i < count; ++i) {
-        const nnhip_matvec_desc& d = descs[i];
-        int rc = check_linear(NNHIP_OP_MATVEC_BATCH, &nowhere, d.ggml_type, d.x, d.w, d.y, d.rows, d.in_w, d.out_w);
-        if (rc != NNHIP_OK) return rc;
-        if (d.in_w > matvec_max_in_w(d.ggml_type))
-            return fail(NNHIP_ERR_TOO_LARGE, NNHIP_OP_MATVEC_BATCH, -1, 0, "descriptor %d: in_w %d exceeds the %d values one workgroup can stage", i, d.in_w, matvec_max_in_w(d.ggml_type));
+    long entries = 0;
+    const int rc = check_batch(&nowhere, descs, count, &entries);
+    if (rc != NNHIP_OK) return rc;
+    int n = 0;
+    try {
+        n = plan_matvec_batch(descs, count, compute_units, launches, capacity);
+    } catch (const std::bad_alloc&) {
+        return fail(NNHIP_ERR_OUT_OF_MEMORY, NNHIP_OP_MATVEC_BATCH, -1, 0, "host memory for the descriptor table");
     }
-    const int n = plan_matvec_batch(descs, count, compute_units, launches, capacity);
     if (n < 0) return fail(NNHIP_ERR_TOO_LARGE, NNHIP_OP_MATVEC_BATCH, -1, 0, "no kernel takes one of the shapes");
     *n_launches = n;
     return NNHIP_OK;
@@ -755,17 +779,9 @@ int nnhip_matvec_batch_plan(const nnhip_matvec_desc* descs, int count, int compu
 int nnhip_quant_matvec_batch_static(void* handle, const nnhip_matvec_desc* descs, int count)
 {
     NNHIP_LANE(handle, NNHIP_OP_MATVEC_BATCH)
-    if (count < 0 || (count > 0 && !descs))
-        return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_MATVEC_BATCH, lane->device, 0, "descriptor array is null or count negative");
     long entries = 0;
-    for (int i = 0; i < count; ++i) {
-        const nnhip_matvec_desc& d = descs[i];
-        int rc = check_linear(NNHIP_OP_MATVEC_BATCH, lane, d.ggml_type, d.x, d.w, d.y, d.rows, d.in_w, d.out_w);
-        if (rc != NNHIP_OK) return rc;
-        if (d.in_w > matvec_max_in_w(d.ggml_type))
-            return fail(NNHIP_ERR_TOO_LARGE, NNHIP_OP_MATVEC_BATCH, lane->device, 0, "descriptor %d: in_w %d exceeds the %d values one workgroup can stage", i, d.in_w, matvec_max_in_w(d.ggml_type));
-        entries += d.rows;
-    }
+    const int rc = check_batch(lane, descs, count, &entries);
+    if (rc != NNHIP_OK) return rc;
     if (entries > NNHIP_STATIC_BATCH_MAX_ENTRIES)
         return fail(NNHIP_ERR_TOO_LARGE, NNHIP_OP_MATVEC_BATCH, lane->device, 0,
                     "the batch has %ld mat-vec rows; the fixed workspace holds %d (use nnhip_quant_matvec_batch, or split the batch)",

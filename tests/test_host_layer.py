@@ -293,6 +293,12 @@ def test_batch_plan_mixed_types_and_errors():
     assert status(_desc(12, 1, 4096, 16, x=0)) == 1
     assert status(_desc(12, 1, 4096, 16), cus=0) == 1
     assert lib.nnhip_matvec_batch_plan(one(_desc(12, 1, 4096, 16)), 1, 256, out, 1, None) == 1
+    # size limits of a batched call: 65535 input rows a descriptor, 2^20 mat-vec rows a call
+    assert status(_desc(12, 65535, 256, 16)) == 0
+    assert status(_desc(12, 65536, 256, 16)) == 8 and "65535" in native.last_error()[1]
+    many = (native.MatvecDesc * 17)(*[_desc(12, 65535, 256, 16)] * 17)
+    assert lib.nnhip_matvec_batch_plan(many, 16, 256, out, 1, byref(n)) == 0
+    assert lib.nnhip_matvec_batch_plan(many, 17, 256, out, 1, byref(n)) == 8 and "split the batch" in native.last_error()[1]
     out[0].struct_size = 8
     assert status(_desc(12, 1, 4096, 16)) == 1 and "struct_size" in native.last_error()[1]
 
