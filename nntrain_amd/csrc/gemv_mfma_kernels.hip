@@ -681,11 +681,15 @@ struct IQ2STask {
         return r;
     }
 
-    static __device__ __forceinline__ void run(const Raw& r, const X& xs, int, const uint8_t* tables, float& accq, float&)
+    // The sixteen lookups of a task and the products that use them are separate steps: with several input rows sharing
+    // a pass the lookups are made once and every row multiplies with them.
+    static constexpr bool kSplitLookups = true;
+    struct Looked { u32x2 mag[8], sel[8]; };
+
+    static __device__ __forceinline__ void lookup(const Raw& r, const uint8_t* tables, Looked& lk)
     {
-        // every lookup of the task is requested before the first result is used (the scheduling barrier keeps the
-        // compiler from folding the reads back into a chain of eight round trips to LDS)
-        u32x2 mag[8], sel[8];
+        u32x2 (&mag)[8] = lk.mag;
+        u32x2 (&sel)[8] = lk.sel;
 #pragma unroll
         for (int g = 0; g < 2; ++g) {
             // the two top bits of entry o of the group as byte o, then index bytes and tops interleaved into 16-bit indices
@@ -700,7 +704,12 @@ struct IQ2STask {
                 sel[4 * g + o] = *reinterpret_cast<const u32x2*>(tables + kGridBytes + 8u * sign);
             }
         }
-        __builtin_amdgcn_sched_barrier(0);
+    }
+
+    static __device__ __forceinline__ void finish(const Raw& r, const Looked& lk, const X& xs, float& accq)
+    {
+        const u32x2 (&mag)[8] = lk.mag;
+        const u32x2 (&sel)[8] = lk.sel;
         i32x4 acc[4] = {{0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}};
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
@@ -720,6 +729,16 @@ struct IQ2STask {
             for (int p = 0; p < 4; ++p) total[p] += mul24(factor, acc[k][p]);     // (24-bit operands: v_mad_i32_i24, not the quarter-rate 32-bit multiply)
         }
         accq = fmaf(half_bits_to_float(r.d) * 0.125f, recombine_wide(total), accq);
+    }
+
+    static __device__ __forceinline__ void run(const Raw& r, const X& xs, int, const uint8_t* tables, float& accq, float&)
+    {
+        // every lookup of the task is requested before the first result is used (the scheduling barrier keeps the
+        // compiler from folding the reads back into a chain of eight round trips to LDS)
+        Looked lk;
+        lookup(r, tables, lk);
+        __builtin_amdgcn_sched_barrier(0);
+        finish(r, lk, xs, accq);
     }
 };
 
@@ -1033,6 +1052,9 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_kernel(MfmaArgs a)
 // registers), a tile takes ceil(nblocks / W) stages of W block columns, the last one partly empty, and a task multiplies
 // the unpacked quants with the operand A of every input row of the entry.  Rows, planes and results of input row r of
 // an entry are x + r * in_w, the r-th plane set and y + r * out_w.
+template <class F, class = void> struct SplitLookups { static constexpr bool value = false; };
+template <class F> struct SplitLookups<F, std::enable_if_t<F::kSplitLookups>> { static constexpr bool value = true; };
+
 struct WideGeom {
     int waves;            // W (even: block parity is wave parity)
     int cols;             // block columns per stage = W * M
@@ -1415,14 +1437,30 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
         // wave's).  Stages whose tasks all exist run them as one straight piece of code, so that the lookups and products
         // of one task overlap the other's; a tile's last stage may hold fewer.
         auto task = [&](const typename F::Raw& raw, int b) {
+            if constexpr (SplitLookups<F>::value && R > 1) {
+                // what the block's lookups return does not depend on the input row: made once, used by every row
+                typename F::Looked lk;
+                F::lookup(raw, tables, lk);
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int r = 0; r < R; ++r) {
-                if (r < ce.rows) {
-                    const uint8_t* set = planes + r * g.set_bytes;
-                    typename F::X xs;
-                    F::load_x(xs, set + (row_l & 3) * g.plane_stride, reinterpret_cast<const float*>(set + 4 * g.plane_stride), b,
-                              quarter, a_zeros);
-                    F::run(raw, xs, quarter, tables, accq[r], accm[r]);
+                for (int r = 0; r < R; ++r) {
+                    if (r < ce.rows) {
+                        const uint8_t* set = planes + r * g.set_bytes;
+                        typename F::X xs;
+                        F::load_x(xs, set + (row_l & 3) * g.plane_stride, nullptr, b, quarter, a_zeros);
+                        F::finish(raw, lk, xs, accq[r]);
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    if (r < ce.rows) {
+                        const uint8_t* set = planes + r * g.set_bytes;
+                        typename F::X xs;
+                        F::load_x(xs, set + (row_l & 3) * g.plane_stride, reinterpret_cast<const float*>(set + 4 * g.plane_stride), b,
+                                  quarter, a_zeros);
+                        F::run(raw, xs, quarter, tables, accq[r], accm[r]);
+                    }
                 }
             }
         };

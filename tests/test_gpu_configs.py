@@ -537,11 +537,12 @@ def test_matrix_core_groups_with_long_rows_and_shared_passes(lane, typ):
     lane.trim()
 
 
-@pytest.mark.parametrize("typ", [GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_Q8_0])
+@pytest.mark.parametrize("typ", [GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_Q8_0, GGML_IQ2_S])
 def test_several_input_rows_share_a_pass_in_a_single_call(lane, typ):
     """nnhip_quant_matvec with 2 - 9 input rows (Q8_0: 3 - 9, two rows stay with its row-tiled kernel) on a matrix large
     enough for the matrix cores (rows x 16-row tiles >= 2048): up to four rows share a pass over the weights (Q4_K, Q5_K
-    and Q8_0 with the rows stacked in operand A, Q6_K one row after the other on the unpacked quants).  Both bars against the oracle, the guard elements,
+    and Q8_0 with the rows stacked in operand A, Q6_K one row after the other on the unpacked quants, IQ2_S one row after
+    the other on one set of codebook lookups).  Both bars against the oracle, the guard elements,
     no transfers, and a row's bits do not depend on the rows it travels with; the same call inside a captured graph
     gives the same bits on every replay."""
     in_w, out_w = 5120, 17408

@@ -59,7 +59,7 @@ USED = ["matvec_mfma_kernelINS0_7Q4KTaskELi2ELi1ELi3", "matvec_mfma_kernelINS0_7
         "matvec_mfma_wide_kernelINS0_7Q4KTaskELi1ELi3ELi1ELb0", "matvec_mfma_wide_kernelINS0_7Q4KTaskELi1ELi3ELi4ELb0",
         "matvec_mfma_wide_kernelINS0_7Q5KTaskELi1ELi3ELi1ELb0", "matvec_mfma_wide_kernelINS0_7Q5KTaskELi1ELi3ELi4ELb0",
         "matvec_mfma_wide_kernelINS0_7Q6KTaskELi1ELi4ELi1ELb0", "matvec_mfma_wide_kernelINS0_7Q6KTaskELi1ELi4ELi4ELb0",
-        "matvec_mfma_wide_kernelINS0_8IQ2STaskELi2ELi4ELi1ELb0",
+        "matvec_mfma_wide_kernelINS0_8IQ2STaskELi2ELi4ELi1ELb0", "matvec_mfma_wide_kernelINS0_8IQ2STaskELi1ELi2ELi4ELb0",
         "matvec_mfma_wide_kernelINS0_8Q8_0TaskELi1ELi5ELi1ELb0",
         "matvec_mfma_wide_kernelINS0_8Q8_0TaskELi2ELi8ELi1ELb1",
         "matvec_mfma_wide_kernelINS0_8Q8_0TaskELi1ELi5ELi4ELb0"]
