@@ -488,6 +488,51 @@ struct Q6KTask {
         return r;
     }
 
+    // The 6-bit quants of the task as operand B, and the scales: the same for every input row of a shared pass.
+    static constexpr bool kSplitLookups = true;
+    struct Looked { uint32_t lo[8], hi[8]; float d, c0, c1, c2, c3; };
+
+    static __device__ __forceinline__ void lookup(const Raw& r, int quarter, const uint8_t*, Looked& lk)
+    {
+        constexpr uint32_t kLow = 0x0f0f0f0fu, kTop = 0x30303030u;
+        const int sh = 2 * (quarter & 1);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            lk.lo[i] = (r.la[i] & kLow) | (((r.ha[i] >> sh) << 4) & kTop);
+            lk.hi[i] = ((r.la[i] >> 4) & kLow) | ((r.ha[i] >> sh) & kTop);
+            lk.lo[4 + i] = (r.lb[i] & kLow) | (((r.hb[i] >> sh) << 4) & kTop);
+            lk.hi[4 + i] = ((r.lb[i] >> 4) & kLow) | ((r.hb[i] >> sh) & kTop);
+        }
+        // scales 8h + 2e + {0, 1} and 8h + 4 + 2e + {0, 1}: bytes 2e, 2e + 1 of the two dwords read for half h
+        const uint32_t w0 = r.sc[0] >> (8 * sh), w1 = r.sc[1] >> (8 * sh);
+        lk.d = half_bits_to_float(r.d);
+        lk.c0 = sbyte0(w0);
+        lk.c1 = sbyte1(w0);
+        lk.c2 = sbyte0(w1);
+        lk.c3 = sbyte1(w1);
+    }
+
+    static __device__ __forceinline__ void finish(const Raw&, const Looked& lk, const X& xs, float& accq, float& accm)
+    {
+        const u32x4 a0 = xs.a[0], a1 = xs.a[1], a2 = xs.a[2], a3 = xs.a[3];
+        i32x4 s0 = {0, 0, 0, 0}, s1 = {0, 0, 0, 0}, s2 = {0, 0, 0, 0}, s3 = {0, 0, 0, 0};
+        s0 = mfma_i8(a0[0], a0[1], lk.lo[0], lk.lo[1], s0);
+        s2 = mfma_i8(a2[0], a2[1], lk.hi[0], lk.hi[1], s2);
+        s0 = mfma_i8(a0[2], a0[3], lk.lo[2], lk.lo[3], s0);
+        s2 = mfma_i8(a2[2], a2[3], lk.hi[2], lk.hi[3], s2);
+        s1 = mfma_i8(a1[0], a1[1], lk.lo[4], lk.lo[5], s1);
+        s3 = mfma_i8(a3[0], a3[1], lk.hi[4], lk.hi[5], s3);
+        s1 = mfma_i8(a1[2], a1[3], lk.lo[6], lk.lo[7], s1);
+        s3 = mfma_i8(a3[2], a3[3], lk.hi[6], lk.hi[7], s3);
+        const float d = lk.d, c0 = lk.c0, c1 = lk.c1, c2 = lk.c2, c3 = lk.c3;
+        accq = fmaf(d * c0, recombine(s0), accq);
+        accq = fmaf(d * c1, recombine(s1), accq);
+        accq = fmaf(d * c2, recombine(s2), accq);
+        accq = fmaf(d * c3, recombine(s3), accq);
+        const float t = fmaf(c0, xs.sx[0], fmaf(c1, xs.sx[1], fmaf(c2, xs.sx[2], c3 * xs.sx[3])));
+        accm = fmaf(32.0f * d, t, accm);
+    }
+
     static __device__ __forceinline__ void run(const Raw& r, const X& xs, int quarter, const uint8_t*, float& accq, float& accm)
     {
         constexpr uint32_t kLow = 0x0f0f0f0fu, kTop = 0x30303030u;
@@ -686,7 +731,7 @@ struct IQ2STask {
     static constexpr bool kSplitLookups = true;
     struct Looked { u32x2 mag[8], sel[8]; };
 
-    static __device__ __forceinline__ void lookup(const Raw& r, const uint8_t* tables, Looked& lk)
+    static __device__ __forceinline__ void lookup(const Raw& r, int, const uint8_t* tables, Looked& lk)
     {
         u32x2 (&mag)[8] = lk.mag;
         u32x2 (&sel)[8] = lk.sel;
@@ -706,7 +751,7 @@ struct IQ2STask {
         }
     }
 
-    static __device__ __forceinline__ void finish(const Raw& r, const Looked& lk, const X& xs, float& accq)
+    static __device__ __forceinline__ void finish(const Raw& r, const Looked& lk, const X& xs, float& accq, float&)
     {
         const u32x2 (&mag)[8] = lk.mag;
         const u32x2 (&sel)[8] = lk.sel;
@@ -736,9 +781,10 @@ struct IQ2STask {
         // every lookup of the task is requested before the first result is used (the scheduling barrier keeps the
         // compiler from folding the reads back into a chain of eight round trips to LDS)
         Looked lk;
-        lookup(r, tables, lk);
+        float unused = 0.0f;
+        lookup(r, 0, tables, lk);
         __builtin_amdgcn_sched_barrier(0);
-        finish(r, lk, xs, accq);
+        finish(r, lk, xs, accq, unused);
     }
 };
 
@@ -1440,15 +1486,16 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
             if constexpr (SplitLookups<F>::value && R > 1) {
                 // what the block's lookups return does not depend on the input row: made once, used by every row
                 typename F::Looked lk;
-                F::lookup(raw, tables, lk);
+                F::lookup(raw, quarter, tables, lk);
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
                     if (r < ce.rows) {
                         const uint8_t* set = planes + r * g.set_bytes;
                         typename F::X xs;
-                        F::load_x(xs, set + (row_l & 3) * g.plane_stride, nullptr, b, quarter, a_zeros);
-                        F::finish(raw, lk, xs, accq[r]);
+                        F::load_x(xs, set + (row_l & 3) * g.plane_stride, reinterpret_cast<const float*>(set + 4 * g.plane_stride), b,
+                                  quarter, a_zeros);
+                        F::finish(raw, lk, xs, accq[r], accm[r]);
                     }
                 }
             } else {
