@@ -382,9 +382,9 @@ def run_gemv(args, lane, nn, oracle):
             out[name]["cpu_baseline"] = {"gb_per_s": round(nbytes / per_pass / 1e9, 2), "us_per_matvec": round(per_pass * 1e6, 1),
                                          "cores": threads, "one_thread_gb_per_s": round(nbytes / one / 1e9, 3), "kind": "port"}
             log(f"[gemv] {name}: CPU port {nbytes / per_pass / 1e9:.1f} GB/s on {threads} threads, {nbytes / one / 1e9:.2f} GB/s on one")
-        if tname == "GGML_Q8_0" or name.startswith("cfg2 Q4_K"):
-            # several input rows in one call (weights rotated as above): microseconds per call.  Q8_0: four rows per pass
-            # of the row-step kernel; Q4_K: four rows per pass of the matrix-core kernel
+        if tname == "GGML_Q8_0" or name.startswith("cfg2"):
+            # several input rows in one call (weights rotated as above): microseconds per call, up to four rows sharing a
+            # pass over the weights (Q8_0 with two rows: its row-tiled lane-per-unit kernel; otherwise the matrix cores)
             per_rows = {}
             for rows in (2, 4, 8):
                 xr = lane.upload_raw(synth.activations(rows, in_w, xseed + rows))
