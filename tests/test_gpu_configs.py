@@ -239,6 +239,9 @@ def test_allocate_forward_dispose_pattern_does_not_wait_for_the_device(lane):
     alloc_enqueue, alloc_total = wall(allocating)
     assert lane.counters()["kernel_launches"] - launches == rounds
     pre_enqueue, pre_total = wall(preallocated)
+    for _ in range(2):          # best of three each: one descheduled host thread must not decide the comparison
+        alloc_enqueue, alloc_total = min((alloc_enqueue, alloc_total), wall(allocating), key=lambda t: t[1])
+        pre_enqueue, pre_total = min((pre_enqueue, pre_total), wall(preallocated), key=lambda t: t[1])
     print(f"1000 projections: preallocated {pre_total * 1e3:.1f} ms (enqueue {pre_enqueue * 1e3:.1f}), "
           f"allocate+dispose {alloc_total * 1e3:.1f} ms (enqueue {alloc_enqueue * 1e3:.1f})")
     assert alloc_total <= 1.2 * pre_total + 2e-3
