@@ -52,6 +52,7 @@ internal static unsafe partial class NnHipNative
     }
 
     internal const uint PreNone = 0, PreRmsNorm = 1, PreSiluMultiply = 2;
+    internal const uint PostNone = 0, PostSiluPair = 1;
 
     [StructLayout(LayoutKind.Sequential)]
     internal struct FusedMatvecDesc
@@ -61,6 +62,7 @@ internal static unsafe partial class NnHipNative
         internal nint W; internal nint Bias; internal nint Addend; internal nint Y;
         internal int InW; internal int OutW;
         internal nint LoraZ; internal nint LoraB; internal int LoraRank; internal float LoraScale;
+        internal int XHeadWidth; internal int XHeadGroup; internal uint PostOp; internal uint Reserved;
     }
 
     [LibraryImport(Library)] internal static partial uint nnhip_abi_version();
@@ -91,6 +93,11 @@ internal static unsafe partial class NnHipNative
     [LibraryImport(Library)] internal static partial int nnhip_quant_matvec_batch(nint lane, MatvecDesc* descs, int count);
     [LibraryImport(Library)] internal static partial int nnhip_quant_matvec_batch_static(nint lane, MatvecDesc* descs, int count);
     [LibraryImport(Library)] internal static partial int nnhip_quant_matvec_fused(nint lane, FusedMatvecDesc* desc);
+    [LibraryImport(Library)] internal static partial int nnhip_chain_create(nint lane, FusedMatvecDesc* steps, int count, out nint chain);
+    [LibraryImport(Library)] internal static partial int nnhip_chain_launch(nint lane, nint chain);
+    [LibraryImport(Library)] internal static partial int nnhip_chain_status(nint lane, nint chain, out int gaveUp);
+    [LibraryImport(Library)] internal static partial int nnhip_chain_launches(nint lane, nint chain, out int launches);
+    [LibraryImport(Library)] internal static partial int nnhip_chain_destroy(nint lane, nint chain);
     [LibraryImport(Library)] internal static partial int nnhip_quant_matmul(nint lane, uint ggmlType, nint x, nint w, nint bias, nint y, int rows, int inW, int outW);
     [LibraryImport(Library)] internal static partial int nnhip_quant_matmul_bf16(nint lane, uint ggmlType, nint xBf16, nint w, nint bias, nint y, int rows, int inW, int outW);
     [LibraryImport(Library)] internal static partial int nnhip_rms_norm(nint lane, nint input, nint weight, nint output, int rows, int width, int inputStride, float epsilon);

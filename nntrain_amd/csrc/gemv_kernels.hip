@@ -66,26 +66,6 @@ struct MatvecArgs {
 
 enum : int { kPreNone = 0, kPreRmsNorm = 1, kPreSiluMultiply = 2 };
 
-__device__ __forceinline__ float4 add4(const float4 a, const float4 b) { return make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w); }
-
-// gate * sigmoid(gate) * up with the two-sided sigmoid of the reference (NNtrain.Arc/Kernels/qwen35_attention.cl:9-14,
-// 38-43): exp never sees a positive argument.
-__device__ __forceinline__ float silu_mul1(float g, float u)
-{
-    float sig;
-    if (g >= 0.0f) {
-        sig = 1.0f / (1.0f + expf(-g));
-    } else {
-        const float e = expf(g);
-        sig = e / (1.0f + e);
-    }
-    return g * sig * u;
-}
-__device__ __forceinline__ float4 silu_mul4(const float4 g, const float4 u)
-{
-    return make_float4(silu_mul1(g.x, u.x), silu_mul1(g.y, u.y), silu_mul1(g.z, u.z), silu_mul1(g.w, u.w));
-}
-
 __device__ __forceinline__ float dot4s(uint32_t v, const float4 x, float acc)  // 4 signed bytes . x
 {
     acc = fmaf(sbyte0(v), x.x, acc);
@@ -1234,6 +1214,18 @@ hipError_t launch_matvec(Lane* lane, uint32_t type, const float* x, const void* 
         hipLaunchKernelGGL(matvec_q8_0_oddrow_kernel, dim3((out_w + 3) / 4, rows), dim3(256), 0, lane->stream, a);
         return hipGetLastError();
     }
+    if (rows == 1 && matvec_stream_takes(type, NNHIP_PRE_NONE, x, w, in_w, out_w)) {
+        nnhip_fused_matvec_desc d{};
+        d.ggml_type = type;
+        d.pre_op = NNHIP_PRE_NONE;
+        d.x = x;
+        d.w = w;
+        d.bias = bias;
+        d.y = y;
+        d.in_w = in_w;
+        d.out_w = out_w;
+        return launch_matvec_stream(lane, d);
+    }
 
     a.units_per_row = in_w / kUnitW;
     a.magic = static_cast<uint32_t>((0x100000000ull + a.units_per_row - 1) / a.units_per_row);
@@ -1272,6 +1264,9 @@ bool matvec_fused_supported(uint32_t type, int in_w)
 
 hipError_t launch_matvec_fused(Lane* lane, const nnhip_fused_matvec_desc& d)
 {
+    if (matvec_stream_takes(d.ggml_type, static_cast<int>(d.pre_op), d.x, d.w, d.in_w, d.out_w) &&
+        !(reinterpret_cast<uintptr_t>(d.x2) & 15u) && !(reinterpret_cast<uintptr_t>(d.norm_weight) & 15u))
+        return launch_matvec_stream(lane, d);
     int elems = 0, bytes = 0;
     type_block(d.ggml_type, &elems, &bytes);
     MatvecArgs a{};

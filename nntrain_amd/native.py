@@ -48,7 +48,8 @@ class FusedMatvecDesc(Structure):
                 ("x", c_void_p), ("x2", c_void_p), ("norm_weight", c_void_p), ("x_out", c_void_p), ("sum_out", c_void_p),
                 ("w", c_void_p), ("bias", c_void_p), ("addend", c_void_p), ("y", c_void_p), ("in_w", c_int32),
                 ("out_w", c_int32), ("lora_z", c_void_p), ("lora_b", c_void_p), ("lora_rank", c_int32),
-                ("lora_scale", c_float)]
+                ("lora_scale", c_float), ("x_head_width", c_int32), ("x_head_group", c_int32), ("post_op", c_uint32),
+                ("reserved", c_uint32)]
 
 
 class MatvecPlanInfo(Structure):
@@ -65,6 +66,7 @@ class BatchLaunchInfo(Structure):
 
 
 PRE_NONE, PRE_RMS_NORM, PRE_SILU_MULTIPLY = 0, 1, 2
+POST_NONE, POST_SILU_PAIR = 0, 1
 
 # name -> (restype, argtypes); exactly the prototypes of include/nnhip.h
 PROTOTYPES = {
@@ -96,6 +98,11 @@ PROTOTYPES = {
     "nnhip_quant_matvec_batch": (c_int, [c_void_p, POINTER(MatvecDesc), c_int]),
     "nnhip_quant_matvec_batch_static": (c_int, [c_void_p, POINTER(MatvecDesc), c_int]),
     "nnhip_quant_matvec_fused": (c_int, [c_void_p, POINTER(FusedMatvecDesc)]),
+    "nnhip_chain_create": (c_int, [c_void_p, POINTER(FusedMatvecDesc), c_int, POINTER(c_void_p)]),
+    "nnhip_chain_launch": (c_int, [c_void_p, c_void_p]),
+    "nnhip_chain_status": (c_int, [c_void_p, c_void_p, POINTER(c_int)]),
+    "nnhip_chain_launches": (c_int, [c_void_p, c_void_p, POINTER(c_int)]),
+    "nnhip_chain_destroy": (c_int, [c_void_p, c_void_p]),
     "nnhip_quant_matmul": (c_int, [c_void_p, c_uint32, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int]),
     "nnhip_quant_matmul_bf16": (c_int, [c_void_p, c_uint32, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int]),
     "nnhip_rms_norm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float]),

@@ -157,6 +157,36 @@ class HipQuantizedMatrix:
             raise
         return y
 
+    def fused_descriptor(self, lane: HipExecutionLane, x: HipBuffer, *, pre_op: int = PRE_NONE, x2: HipBuffer | None = None,
+                         norm_weight: HipBuffer | None = None, epsilon: float = 0.0, x_out: HipBuffer | None = None,
+                         sum_out: HipBuffer | None = None, bias: HipBuffer | None = None, addend: HipBuffer | None = None,
+                         out: HipBuffer, lora_z: HipBuffer | None = None, lora_b: HipBuffer | None = None,
+                         lora_rank: int = 0, lora_scale: float = 0.0, x_head_width: int = 0,
+                         x_head_group: int = 0, post_op: int = 0) -> FusedMatvecDesc:
+        """The native descriptor of forward_fused with these arguments (also one step of a HipMatvecChain, where
+        x_head_width / x_head_group gather x by heads first: v[h * width + j] = x[(h // group) * width + j], and
+        post_op POST_SILU_PAIR stores SiLU(z[o]) * z[out / 2 + o] for the first half of the rows instead of z)."""
+        if lora_rank < 0:
+            raise ValueError("lora_rank must not be negative.")
+        if lora_rank > 0 and (lora_z is None or lora_b is None or lora_z.nbytes < 4 * lora_rank
+                              or lora_b.nbytes < 4 * lora_rank * self.output_width):
+            raise ValueError("LoRA buffers do not match lora_rank.")
+        n_in, n_out = 4 * self.input_width, 4 * self.output_width
+        n_y = n_out // 2 if post_op else n_out
+        n_x = n_in // x_head_group if x_head_group > 0 else n_in
+        for name, buf, need in (("x", x, n_x), ("x2", x2, n_in), ("norm_weight", norm_weight, n_in), ("x_out", x_out, n_in),
+                                ("sum_out", sum_out, n_in), ("bias", bias, n_out), ("addend", addend, n_out), ("out", out, n_y)):
+            if buf is not None and buf.nbytes < need:
+                raise ValueError(f"Quantized linear '{name}' width mismatch.")
+        w = self.device_payload(lane)
+        ptr = lambda b: c_void_p(b._require()) if b is not None else None   # noqa: E731
+        return FusedMatvecDesc(struct_size=ctypes.sizeof(FusedMatvecDesc), ggml_type=self.ggml_type, pre_op=pre_op,
+                               epsilon=epsilon, x=ptr(x), x2=ptr(x2), norm_weight=ptr(norm_weight), x_out=ptr(x_out),
+                               sum_out=ptr(sum_out), w=ptr(w), bias=ptr(bias), addend=ptr(addend), y=ptr(out),
+                               in_w=self.input_width, out_w=self.output_width, lora_z=ptr(lora_z), lora_b=ptr(lora_b),
+                               lora_rank=lora_rank, lora_scale=lora_scale, x_head_width=x_head_width,
+                               x_head_group=x_head_group, post_op=post_op)
+
     def forward_fused(self, lane: HipExecutionLane, x: HipBuffer, *, pre_op: int = PRE_NONE, x2: HipBuffer | None = None,
                       norm_weight: HipBuffer | None = None, epsilon: float = 0.0, x_out: HipBuffer | None = None,
                       sum_out: HipBuffer | None = None, bias: HipBuffer | None = None, addend: HipBuffer | None = None,
@@ -167,25 +197,13 @@ class HipQuantizedMatrix:
         x_out / sum_out receive v and x + x2 when given.  `out` may be `addend` (the residual stream updated in place).
         lora_z [rank] and lora_b [out, rank] add the low-rank adapter branch lora_scale * z . b^T before the addend
         (Matrix.ForwardFusedLora, Qwen35QuantizedModel.cs:1387)."""
-        if lora_rank < 0:
-            raise ValueError("lora_rank must not be negative.")
-        if lora_rank > 0 and (lora_z is None or lora_b is None or lora_z.nbytes < 4 * lora_rank
-                              or lora_b.nbytes < 4 * lora_rank * self.output_width):
-            raise ValueError("LoRA buffers do not match lora_rank.")
-        n_in, n_out = 4 * self.input_width, 4 * self.output_width
-        for name, buf, need in (("x", x, n_in), ("x2", x2, n_in), ("norm_weight", norm_weight, n_in), ("x_out", x_out, n_in),
-                                ("sum_out", sum_out, n_in), ("bias", bias, n_out), ("addend", addend, n_out), ("out", out, n_out)):
-            if buf is not None and buf.nbytes < need:
-                raise ValueError(f"Quantized linear '{name}' width mismatch.")
-        w = self.device_payload(lane)
+        if out is not None and out.nbytes < 4 * self.output_width:
+            raise ValueError("Quantized linear 'out' width mismatch.")
         y = out if out is not None else lane.allocate(self.output_width)
-        ptr = lambda b: c_void_p(b._require()) if b is not None else None   # noqa: E731
-        desc = FusedMatvecDesc(struct_size=ctypes.sizeof(FusedMatvecDesc), ggml_type=self.ggml_type, pre_op=pre_op,
-                               epsilon=epsilon, x=ptr(x), x2=ptr(x2), norm_weight=ptr(norm_weight), x_out=ptr(x_out),
-                               sum_out=ptr(sum_out), w=ptr(w), bias=ptr(bias), addend=ptr(addend), y=ptr(y),
-                               in_w=self.input_width, out_w=self.output_width, lora_z=ptr(lora_z), lora_b=ptr(lora_b),
-                               lora_rank=lora_rank, lora_scale=lora_scale)
         try:
+            desc = self.fused_descriptor(lane, x, pre_op=pre_op, x2=x2, norm_weight=norm_weight, epsilon=epsilon, x_out=x_out,
+                                         sum_out=sum_out, bias=bias, addend=addend, out=y, lora_z=lora_z, lora_b=lora_b,
+                                         lora_rank=lora_rank, lora_scale=lora_scale)
             with lane.kernel("quant_matvec_fused"):
                 check(lane._lib.nnhip_quant_matvec_fused(lane._handle, ctypes.byref(desc)), "quant_matvec_fused")
         except BaseException:

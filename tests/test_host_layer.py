@@ -93,7 +93,7 @@ def test_csharp_declarations_match_the_header():
         align = max(sizes[f] for f in fields)
         assert (offset + align - 1) // align * align == ctypes.sizeof(ct), (cs_name, offset, ctypes.sizeof(ct))
         assert len(fields) == len(ct._fields_), cs_name
-    assert ctypes.sizeof(native.FusedMatvecDesc) == 120
+    assert ctypes.sizeof(native.FusedMatvecDesc) == 136
 
 
 def test_abi_version_and_struct_layouts():
@@ -102,7 +102,7 @@ def test_abi_version_and_struct_layouts():
     assert ctypes.sizeof(native.MatvecDesc) == 48
     assert ctypes.sizeof(native.LaneCounters) == 48
     assert ctypes.sizeof(native.MatvecPlanInfo) == 40
-    assert ctypes.sizeof(native.FusedMatvecDesc) == 120
+    assert ctypes.sizeof(native.FusedMatvecDesc) == 136
 
 
 def test_geometry_queries_without_a_gpu():
