@@ -608,7 +608,7 @@ def run_decode_loop(args, lane, nn, oracle):
            "weight_bytes_streamed_per_token": weight_bytes,
            "ms_per_token": {"one_launch_per_operation": round(ms_plain, 4), "fused_launches": round(ms_fused, 4),
                             "fused_launches_hip_graph": round(ms_graph, 4)},
-           "launches_per_token": {"one_launch_per_operation": 1 + 12 * layers + 2, "fused_launches": 1 + 5 * layers + 1},
+           "launches_per_token": {"one_launch_per_operation": 1 + 12 * layers + 2, "fused_launches": 1 + 4 * layers + 1},
            "gb_per_s_fused_graph": round(weight_bytes / ms_graph / 1e6, 1),
            "frac_of_8TBs_fused_graph": round(weight_bytes / ms_graph / 1e6 / HBM_PEAK_GBS, 4),
            "greedy_generation_with_host_argmax": {"tokens": timing.generated_tokens,
@@ -692,39 +692,13 @@ def run_decode27b_chained(args, lane, nn, oracle):
         return {"ms_per_token": round(ms, 4), "tokens_per_s": round(1e3 / ms, 2), "gb_per_s": round(weight_bytes / ms / 1e6, 1),
                 "frac_of_8TBs": round(weight_bytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
 
-    # the same steps handed over as chains: per layer one chain and the attention launch, or the whole token as one chain
-    # with the first-token attention folded into the o projection's input
-    reference_logits = lane.read(plain.forward_token(tokens[1]), np.float32, count=vocab)
-    chained = {}
-    for key, fold in (("chains_per_layer", False), ("one_chain_per_token", True)):
-        fused.release_graph()
-        fused.build_chains(fold_attention=fold)
-        got = lane.read(fused.forward_token(tokens[1]), np.float32, count=vocab)
-        rel_c = oracle.rel_l2(got, reference_logits)
-        if fused.chains_gave_up() or not (np.all(np.isfinite(got)) and rel_c <= 1e-5):
-            raise SystemExit(f"decode27b_chained: {key}: logits differ from the launch-per-operation form, rel-L2 {rel_c:.3e}")
-        ms_eager = per_token(fused)
-        launches = fused.chain_launches
-        fused.capture_graph()
-        again = lane.read(fused.forward_token(tokens[1]), np.uint32, count=vocab)
-        if not np.array_equal(again, got.view(np.uint32)):
-            raise SystemExit(f"decode27b_chained: {key}: graph replay differs bitwise")
-        ms_g = per_token(fused)
-        if fused.chains_gave_up():
-            raise SystemExit(f"decode27b_chained: {key}: a workgroup gave up waiting")
-        chained[key] = {"eager": entry(ms_eager), "hip_graph": entry(ms_g), "launches_per_token": 1 + launches,
-                        "rel_l2_logits_vs_launch_per_operation": rel_c}
-        log(f"[decode27b_chained] {key}: {ms_eager:.3f} ms eager, {ms_g:.3f} ms from a graph ({1e3 / min(ms_eager, ms_g):.1f} tok/s), "
-            f"{1 + launches} launches, rel-L2 vs launch per operation {rel_c:.2e}")
-        fused.release_chains()
-
     layers = d.layer_count
     out = {"config": "62 layers, hidden 5376, feed-forward 21504, heads 32/16 x 128, vocabulary 262144 (head tied to the "
                      "embedding), Q8_0, first-token attention (no cache)",
            "weight_bytes_streamed_per_token": weight_bytes,
            "one_launch_per_operation": entry(ms_plain), "fused_launches": entry(ms_fused),
-           "fused_launches_hip_graph": entry(ms_graph), "chained": chained,
-           "launches_per_token": {"one_launch_per_operation": 1 + 12 * layers + 2, "fused_launches": 1 + 5 * layers + 1},
+           "fused_launches_hip_graph": entry(ms_graph),
+           "launches_per_token": {"one_launch_per_operation": 1 + 12 * layers + 2, "fused_launches": 1 + 4 * layers + 1},
            "rel_l2_head_vs_f64_oracle": rel, "bitwise_equal": True}
     log(f"[decode27b_chained] per token: {ms_plain:.3f} ms one launch per operation, {ms_fused:.3f} ms fused, "
         f"{ms_graph:.3f} ms fused + graph ({weight_bytes / ms_graph / 1e6:.0f} GB/s, {1e3 / ms_graph:.1f} tok/s)")

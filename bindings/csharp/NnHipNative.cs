@@ -93,11 +93,6 @@ internal static unsafe partial class NnHipNative
     [LibraryImport(Library)] internal static partial int nnhip_quant_matvec_batch(nint lane, MatvecDesc* descs, int count);
     [LibraryImport(Library)] internal static partial int nnhip_quant_matvec_batch_static(nint lane, MatvecDesc* descs, int count);
     [LibraryImport(Library)] internal static partial int nnhip_quant_matvec_fused(nint lane, FusedMatvecDesc* desc);
-    [LibraryImport(Library)] internal static partial int nnhip_chain_create(nint lane, FusedMatvecDesc* steps, int count, out nint chain);
-    [LibraryImport(Library)] internal static partial int nnhip_chain_launch(nint lane, nint chain);
-    [LibraryImport(Library)] internal static partial int nnhip_chain_status(nint lane, nint chain, out int gaveUp);
-    [LibraryImport(Library)] internal static partial int nnhip_chain_launches(nint lane, nint chain, out int launches);
-    [LibraryImport(Library)] internal static partial int nnhip_chain_destroy(nint lane, nint chain);
     [LibraryImport(Library)] internal static partial int nnhip_quant_matmul(nint lane, uint ggmlType, nint x, nint w, nint bias, nint y, int rows, int inW, int outW);
     [LibraryImport(Library)] internal static partial int nnhip_quant_matmul_bf16(nint lane, uint ggmlType, nint xBf16, nint w, nint bias, nint y, int rows, int inW, int outW);
     [LibraryImport(Library)] internal static partial int nnhip_rms_norm(nint lane, nint input, nint weight, nint output, int rows, int width, int inputStride, float epsilon);

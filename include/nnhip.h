@@ -68,7 +68,7 @@ enum {
     NNHIP_OP_UPLOAD, NNHIP_OP_DOWNLOAD, NNHIP_OP_COPY, NNHIP_OP_SYNCHRONIZE, NNHIP_OP_DEQUANTIZE,
     NNHIP_OP_MATVEC, NNHIP_OP_MATVEC_BATCH, NNHIP_OP_MATMUL_BF16, NNHIP_OP_EVENT, NNHIP_OP_GRAPH,
     NNHIP_OP_DEVICE_QUERY, NNHIP_OP_FILL, NNHIP_OP_RMS_NORM, NNHIP_OP_SILU_MULTIPLY, NNHIP_OP_ADD_IN_PLACE,
-    NNHIP_OP_MATVEC_FUSED, NNHIP_OP_LORA, NNHIP_OP_ATTENTION, NNHIP_OP_MATMUL, NNHIP_OP_CHAIN
+    NNHIP_OP_MATVEC_FUSED, NNHIP_OP_LORA, NNHIP_OP_ATTENTION, NNHIP_OP_MATMUL
 };
 
 /* Same field order as the reference's NativeErrorInfo (CudaNativeGateway.cs:1360-1371). */
@@ -340,6 +340,13 @@ NNHIP_API int nnhip_add_in_place(void* lane, float* destination, const float* so
  *   217-275; Matrix.ForwardFusedLora, Qwen35QuantizedModel.cs:1387) and is bit-identical to nnhip_lora_b applied to
  *   the plain result; addend may be null, and may be y itself (the residual stream: replaces q35a_add_in_place after
  *   the down projection).  bias may be null.
+ *   x_head_width / x_head_group > 0 (with NNHIP_PRE_NONE): x holds in_w / x_head_group floats, kv heads of x_head_width
+ *   values, and v[h * width + j] = x[(h / group) * width + j]: the launch reads the value heads as
+ *   nnhip_first_token_attention would have copied them (replaces that launch in front of the o projection).
+ *   post_op NNHIP_POST_SILU_PAIR (out_w even; no addend, no low-rank branch): w stacks two projections of out_w / 2 rows
+ *   (gate | up) and y receives out_w / 2 values, y[o] = SiLU(z[o]) * z[out_w / 2 + o] with z = bias + W v and the SiLU of
+ *   nnhip_silu_multiply: replaces the two projections and q35a_silu_multiply (Qwen35QuantizedModel.cs:489-496) with one
+ *   launch, bit-identical to them.
  * The mat-vec part is bit-identical to nnhip_quant_matvec on the same v.  x, x2, norm_weight hold in_w floats;
  * x_out and sum_out must not overlap x or x2 (every workgroup reads those while workgroup 0 writes).  Q8_0 rows with
  * an odd number of blocks are not covered (NNHIP_ERR_INVALID_ARGUMENT).  struct_size = sizeof of this structure.
@@ -367,38 +374,13 @@ typedef struct nnhip_fused_matvec_desc {
     const float* lora_b;        /* [out_w, lora_rank] FP32                                                             */
     int32_t lora_rank;
     float lora_scale;
-    int32_t x_head_width;       /* steps of a chain only (0 elsewhere): > 0 gathers x by heads before the pre-op,         */
-    int32_t x_head_group;       /* v[h * width + j] = x[(h / group) * width + j], the first-token attention result       */
-    uint32_t post_op;           /* steps of a chain only: NNHIP_POST_SILU_PAIR stores y[o] = SiLU(z[o]) * z[out_w / 2 + o]  */
-    uint32_t reserved;          /* for o < out_w / 2, z = bias + W v: a stacked gate | up projection leaves the product   */
+    int32_t x_head_width;       /* > 0: x is gathered by heads first, v[h * width + j] = x[(h / x_head_group) * width + j]   */
+    int32_t x_head_group;       /* (x then holds in_w / x_head_group floats); both 0: x is used as it is                       */
+    uint32_t post_op;           /* NNHIP_POST_SILU_PAIR: y[o] = SiLU(z[o]) * z[out_w / 2 + o] for o < out_w / 2, z = bias + W v */
+    uint32_t reserved;          /* 0                                                                                           */
 } nnhip_fused_matvec_desc;
 
 NNHIP_API int nnhip_quant_matvec_fused(void* lane, const nnhip_fused_matvec_desc* desc);
-
-/* A chain: `count` fused mat-vecs of which each may consume what the one before it produced (its x, x2 or addend is
- * the y, x_out or sum_out of an earlier step), enqueued as ONE unit of work for the per-token sequence that
- * ForwardTokenDevice issues launch by launch (Qwen35QuantizedModel.cs:451-513: projection, norm, projection ...).  It has
- * no counterpart in the reference, which has nothing between "one kernel per operation" and BatchDispatch.  Consecutive
- * steps of one storage type among Q8_0 / Q4_K / Q5_K / Q6_K / IQ2_S with in_w a multiple of 256 in 1024 .. 22528 (RMSNorm
- * steps: at most 8192) and 16-byte aligned w run as a single launch on the matrix cores: all workgroups stay resident, the
- * weight stream of the next step is requested while the last rows of a step are still being multiplied, and only the
- * preparation of the next vector waits for the previous step (device-wide counters, no host involvement).  Other steps are
- * launched in between exactly as nnhip_quant_matvec_fused would.  Results: the activations of the matrix-core steps go
- * through 32-bit fixed point with one exponent per 32 values (error per element at most 2^-31 of the largest magnitude
- * among its 32 neighbours; FP32 accumulation), so they agree with nnhip_quant_matvec_fused to FP32 summation accuracy
- * (relative L2 difference below 1e-6), not bit for bit; they are deterministic, and a row's bits depend on its weights,
- * in_w and the prepared vector only.  x_head_width / x_head_group of a step are honoured only here.
- * nnhip_chain_create validates every step like nnhip_quant_matvec_fused, allocates and uploads the step table (blocking;
- * not allowed while a graph is captured); nnhip_chain_launch enqueues the chain (asynchronous, allocates nothing, may be
- * captured) - the same chain must not be in flight twice at once, and no other work may occupy the device's compute units
- * while it runs (its workgroups wait for each other: the waits are bounded, and nnhip_chain_status, which blocks until the
- * lane's stream has drained, reports in *gave_up whether any wait ran out since it was last asked - results are then
- * undefined).  nnhip_chain_launches returns the number of kernel launches per nnhip_chain_launch. */
-NNHIP_API int nnhip_chain_create(void* lane, const nnhip_fused_matvec_desc* steps, int count, void** chain);
-NNHIP_API int nnhip_chain_launch(void* lane, void* chain);
-NNHIP_API int nnhip_chain_status(void* lane, void* chain, int* gave_up);
-NNHIP_API int nnhip_chain_launches(void* lane, void* chain, int* launches);
-NNHIP_API int nnhip_chain_destroy(void* lane, void* chain);
 
 /* out[h, :] = v[h / (heads / kv_heads), :] for h < heads: the result of causal grouped-query attention for the first
  * token of a sequence (a single key has softmax weight 1 whatever the query), which lets a decode loop exercise every

@@ -14,6 +14,5 @@ from .quantized_matrix import (BLOCK_BYTES, BLOCK_ELEMS, GGML_BF16, GGML_IQ2_S, 
                                GGML_Q5_K, GGML_Q6_K, GGML_Q8_0, HipQuantizedMatrix)
 from .gguf import GgufReader, GgufReadLimits, GgufTensorInfo, InvalidDataError  # noqa: F401
 from .loader import GgufTensorDirectory, HipGgufLoader, NotSupportedError  # noqa: F401
-from .chain import HipMatvecChain  # noqa: F401
 from . import qwen35_gpu  # noqa: F401
 from .decoder import DecoderDescriptor, GenerationTiming, QuantizedDecoder  # noqa: F401

@@ -62,9 +62,32 @@ struct MatvecArgs {
     const float* lora_b;
     int lora_rank;         // 0: no low-rank branch
     float lora_scale;
+    int head4;             // kPreHeadGather: float4 per head, and the heads that share a source head:
+    int head_group;        //   v[h * width + j] = x[(h / group) * width + j] (first-token attention)
+    int pair_rows;         // PAIR: out_w / 2; rows o and pair_rows + o leave y[o] = SiLU(z[o]) * z[pair_rows + o]
 };
 
-enum : int { kPreNone = 0, kPreRmsNorm = 1, kPreSiluMultiply = 2 };
+enum : int { kPreNone = 0, kPreRmsNorm = 1, kPreSiluMultiply = 2, kPreHeadGather = 3 };
+
+__device__ __forceinline__ float4 add4(const float4 a, const float4 b) { return make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w); }
+
+// gate * sigmoid(gate) * up with the two-sided sigmoid of the reference (NNtrain.Arc/Kernels/qwen35_attention.cl:9-14,
+// 38-43): exp never sees a positive argument.
+__device__ __forceinline__ float silu_mul1(float g, float u)
+{
+    float sig;
+    if (g >= 0.0f) {
+        sig = 1.0f / (1.0f + expf(-g));
+    } else {
+        const float e = expf(g);
+        sig = e / (1.0f + e);
+    }
+    return g * sig * u;
+}
+__device__ __forceinline__ float4 silu_mul4(const float4 g, const float4 u)
+{
+    return make_float4(silu_mul1(g.x, u.x), silu_mul1(g.y, u.y), silu_mul1(g.z, u.z), silu_mul1(g.w, u.w));
+}
 
 __device__ __forceinline__ float dot4s(uint32_t v, const float4 x, float acc)  // 4 signed bytes . x
 {
@@ -521,11 +544,16 @@ template <> struct Shape<BF16Unit> { static constexpr int kMaxT = 512, kWavesPer
 // weights are streamed once per MR rows.  A lane cannot hold MR x 64 activations in registers: the vectors stay in LDS and
 // the lane re-reads its 64 values of a row for every step; the arithmetic and the summation order per input row are
 // those of MR = 1, so results do not depend on how the rows were grouped.
-template <class Q, int PRE = kPreNone, int MR = 1>
+// PAIR (a stacked gate | up projection, NNtrain.Core/Modules/Qwen35QuantizedModel.cs:489-496 runs the two and then
+// q35a_silu_multiply): a row step is RS / 2 rows of the first half of the matrix and the matching rows of the second, and
+// what is stored is SiLU(first) * second, so the product is formed once, by the workgroup that has both sums, instead of
+// by every workgroup of the next launch.  Each sum has the bits of the unpaired launch.
+template <class Q, int PRE = kPreNone, int MR = 1, bool PAIR = false>
 __global__ __launch_bounds__(Shape<Q>::kMaxT) __attribute__((amdgpu_waves_per_eu(Shape<Q>::kWavesPerEu, Shape<Q>::kWavesPerEu)))
 void matvec_rowstep_kernel(MatvecArgs a, const float* __restrict__ bias)
 {
     static_assert(MR == 1 || PRE == kPreNone, "row tiling is for plain launches");
+    static_assert(!PAIR || MR == 1, "paired halves are for single input rows");
     constexpr int kDepth = Shape<Q>::kDepth;
     __shared__ float part[2][MR * kMaxWG];
     __shared__ __attribute__((aligned(8))) uint32_t grid[Q::kGridWords ? Q::kGridWords : 2];
@@ -539,11 +567,21 @@ void matvec_rowstep_kernel(MatvecArgs a, const float* __restrict__ bias)
     const float* x = a.x + static_cast<size_t>(row0) * a.in_w;
     float* y = a.y + static_cast<size_t>(row0) * a.out_w;
     const int last_row = a.out_w - 1;
+    const int half = rs >> 1;                                  // PAIR: rows of each half per step
+    // the matrix row of row `r` of step `st` (PAIR: rows 0 .. half - 1 of a step lie in the first half of the matrix)
+    auto row_of = [&](int st, int r) {
+        if constexpr (PAIR) return r < half ? st * half + r : a.pair_rows + st * half + (r - half);
+        else return st * rs + r;
+    };
+    auto row_valid = [&](int st, int r) {
+        if constexpr (PAIR) return st * half + (r < half ? r : r - half) < a.pair_rows;
+        else return st * rs + r < a.out_w;
+    };
 
     // Loads are unconditional: rows past the end re-read the last row, spare lanes re-read row 0 (both stay in L2),
     // and their products are dropped.  That keeps the stream free of branches between loads.
     auto fetch = [&](int step) {
-        const int row = owner ? min(step * rs + rl, last_row) : 0;
+        const int row = owner ? min(row_of(step, rl), last_row) : 0;
         return Q::load(a.w + static_cast<size_t>(row) * a.row_bytes, c);
     };
 
@@ -553,8 +591,9 @@ void matvec_rowstep_kernel(MatvecArgs a, const float* __restrict__ bias)
     const int pieces = a.in_w >> 2;
     const float4* xg = reinterpret_cast<const float4*>(x);
     const int T = blockDim.x;
-    float4 xv0 = tid < pieces ? xg[tid] : make_float4(0.f, 0.f, 0.f, 0.f);
-    float4 xv1 = tid + T < pieces ? xg[tid + T] : make_float4(0.f, 0.f, 0.f, 0.f);
+    // (a vector gathered by heads is shorter than in_w: its pieces are fetched through the index map further down)
+    float4 xv0 = PRE != kPreHeadGather && tid < pieces ? xg[tid] : make_float4(0.f, 0.f, 0.f, 0.f);
+    float4 xv1 = PRE != kPreHeadGather && tid + T < pieces ? xg[tid + T] : make_float4(0.f, 0.f, 0.f, 0.f);
     const float4* x2g = reinterpret_cast<const float4*>(a.x2);
     const float4* gg = reinterpret_cast<const float4*>(a.gamma);
     const bool second = PRE == kPreSiluMultiply || (PRE == kPreRmsNorm && a.x2 != nullptr);
@@ -609,12 +648,25 @@ void matvec_rowstep_kernel(MatvecArgs a, const float* __restrict__ bias)
         // 128 lane-strided partial sums of squares ...
         const float* xs = reinterpret_cast<const float*>(xstage);
         float sq = 0.0f;
-        if (tid < 128)
-            for (int j = tid; j < a.in_w; j += 128) {
+        if (tid < 128) {
+            // (eight reads on their way at a time instead of one dependent read per addition; the additions keep their order)
+            auto at = [&](int j) {
                 const int L = j >> 2;
-                const float v = xs[4 * (L + (L >> 4)) + (j & 3)];
+                return xs[4 * (L + (L >> 4)) + (j & 3)];
+            };
+            int j = tid;
+            for (; j + 7 * 128 < a.in_w; j += 8 * 128) {
+                float v[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) v[u] = at(j + u * 128);
+#pragma unroll
+                for (int u = 0; u < 8; ++u) sq += v[u] * v[u];
+            }
+            for (; j < a.in_w; j += 128) {
+                const float v = at(j);
                 sq += v * v;
             }
+        }
         // ... then the halving tree: 64 through LDS (the two waves that hold the partials), 32 .. 1 inside wave 0
         if (tid >= 64 && tid < 128) part[0][tid - 64] = sq;
         __syncthreads();
@@ -645,6 +697,11 @@ void matvec_rowstep_kernel(MatvecArgs a, const float* __restrict__ bias)
             xstage[L + (L >> 4)] = v;
             if (xo) xo[L] = v;
         }
+    } else if constexpr (PRE == kPreHeadGather) {
+        for (int L = tid; L < pieces; L += T) {
+            const int h = L / a.head4;
+            xstage[L + (L >> 4)] = xg[(h / a.head_group) * a.head4 + (L - h * a.head4)];
+        }
     } else {
         if (tid < pieces) xstage[tid + (tid >> 4)] = xv0;
         if (tid + T < pieces) xstage[tid + T + ((tid + T) >> 4)] = xv1;
@@ -672,6 +729,15 @@ void matvec_rowstep_kernel(MatvecArgs a, const float* __restrict__ bias)
     int first_held = step;        // step number of ybuf[0 .. rs)
     auto flush = [&]() {
         __syncthreads();
+        if constexpr (PAIR) {
+            for (int i = tid; i < held * half; i += T) {
+                const int j = i / half, r = i - j * half;
+                const int row = (first_held + j * stride) * half + r;
+                if (row < a.pair_rows) y[row] = silu_mul1(ybuf[j * rs + r], ybuf[j * rs + half + r]);
+            }
+            held = 0;
+            return;
+        }
         for (int i = tid; i < held * rs * MR; i += T) {
             const int j = i / (rs * MR), rem = i - j * rs * MR;
             const int m = MR == 1 ? 0 : rem / rs;
@@ -704,8 +770,8 @@ void matvec_rowstep_kernel(MatvecArgs a, const float* __restrict__ bias)
         __syncthreads();
         for (int rr = wave; rr < rs * MR; rr += waves) {
             const int m = MR == 1 ? 0 : rr / rs, r0 = rr - m * rs;
-            const int row = st * rs + r0;
-            if (row < a.out_w && (MR == 1 || row0 + m < a.rows)) {
+            const int row = row_of(st, r0);
+            if (row_valid(st, r0) && (MR == 1 || row0 + m < a.rows)) {
                 float t = 0.0f;
                 for (int u = lane; u < upr; u += 64) t += part[buf][m * kMaxWG + r0 * upr + u];
                 t = wave_sum(t);
@@ -977,7 +1043,7 @@ struct Geometry {
 // a workgroup parks the results of a whole turn of the register ring (depth steps of RS rows for each of the MR input
 // rows of the tile) in its result buffer before it can flush, so depth * RS * MR must fit kYBuf.  The cap only binds
 // for rows of one to five units; a row's bits do not depend on RS.
-bool plan(int in_w, int out_w, int compute_units, int max_t, int rs_cap, Geometry* g)
+bool plan(int in_w, int out_w, int compute_units, int max_t, int rs_cap, Geometry* g, bool pair = false)
 {
     const int upr = in_w / kUnitW;
     if (upr < 1 || upr > max_t || rs_cap < 1) return false;
@@ -986,7 +1052,12 @@ bool plan(int in_w, int out_w, int compute_units, int max_t, int rs_cap, Geometr
     const int rs_min = (3 * rs_max + 3) / 4;     // never give up more than a quarter of the lanes
     int best_rs = 0;
     long best_cost = 0;
-    for (int rs = rs_max; rs >= rs_min && rs >= 1; --rs) {
+    if (pair) {
+        // a step is RS / 2 rows of each half of the matrix
+        if (rs_max < 2 || (out_w & 1)) return false;
+        rs_max &= ~1;
+    }
+    for (int rs = rs_max; rs >= rs_min && rs >= 1; rs -= pair ? 2 : 1) {
         const int steps = (out_w + rs - 1) / rs;
         const int rounds = (steps + compute_units - 1) / compute_units;
         const long cost = static_cast<long>(rounds) * rs;
@@ -1022,16 +1093,16 @@ int row_tile_of(int rows, size_t lds_one_row)
 
 // The whole launch shape of matvec_rowstep_kernel<Q, PRE, MR> for one call; false if a row does not fit a workgroup.
 template <class Q, int PRE>
-bool rowstep_shape(int rows, int in_w, int out_w, int compute_units, int* mr, Geometry* g)
+bool rowstep_shape(int rows, int in_w, int out_w, int compute_units, int* mr, Geometry* g, bool pair = false)
 {
     const size_t lds = static_cast<size_t>(kChunkPieces) * (in_w / kUnitW) * sizeof(float4);
-    *mr = row_tile_of<Q, PRE>(rows, lds);
-    if (!plan(in_w, out_w, compute_units, Shape<Q>::kMaxT, kYBuf / (Shape<Q>::kDepth * *mr), g)) return false;
+    *mr = pair ? 1 : row_tile_of<Q, PRE>(rows, lds);
+    if (!plan(in_w, out_w, compute_units, Shape<Q>::kMaxT, kYBuf / (Shape<Q>::kDepth * *mr), g, pair)) return false;
     if (PRE == kPreRmsNorm && g->threads < 128) g->threads = 128;     // the norm's partial sums take 128 lanes
     return true;
 }
 
-template <class Q, int PRE, int MR>
+template <class Q, int PRE, int MR, bool PAIR = false>
 hipError_t launch_rowstep_tiled(Lane* lane, const MatvecArgs& args, const Geometry& g, int rows, size_t lds)
 {
     // what the kernel's result buffer and partial-sum arrays assume (see plan)
@@ -1040,11 +1111,11 @@ hipError_t launch_rowstep_tiled(Lane* lane, const MatvecArgs& args, const Geomet
         return hipErrorInvalidConfiguration;
     static LdsLimit big_lds;
     if (lds > 32 * 1024) {
-        const hipError_t e = big_lds.ensure(lane->device, reinterpret_cast<const void*>(&matvec_rowstep_kernel<Q, PRE, MR>),
+        const hipError_t e = big_lds.ensure(lane->device, reinterpret_cast<const void*>(&matvec_rowstep_kernel<Q, PRE, MR, PAIR>),
                                             max_dynamic_lds(MR));
         if (e != hipSuccess) return e;
     }
-    hipLaunchKernelGGL((matvec_rowstep_kernel<Q, PRE, MR>), dim3(g.groups, (rows + MR - 1) / MR), dim3(g.threads), lds,
+    hipLaunchKernelGGL((matvec_rowstep_kernel<Q, PRE, MR, PAIR>), dim3(g.groups, (rows + MR - 1) / MR), dim3(g.threads), lds,
                        lane->stream, args, args.bias);
     return hipGetLastError();
 }
@@ -1054,11 +1125,17 @@ hipError_t launch_rowstep(Lane* lane, MatvecArgs args, int rows)
 {
     Geometry g;
     int mr = 1;
-    if (!rowstep_shape<Q, PRE>(rows, args.in_w, args.out_w, lane->compute_units, &mr, &g)) return hipErrorInvalidValue;
+    const bool pair = args.pair_rows > 0;
+    if (!rowstep_shape<Q, PRE>(rows, args.in_w, args.out_w, lane->compute_units, &mr, &g, pair)) return hipErrorInvalidValue;
     args.rows_per_step = g.rows_per_step;
     args.steps = g.steps;
     args.rows = rows;
     const size_t lds = static_cast<size_t>(kChunkPieces) * args.units_per_row * sizeof(float4);
+    if constexpr (PRE == kPreNone || PRE == kPreRmsNorm) {
+        if (pair) return launch_rowstep_tiled<Q, PRE, 1, true>(lane, args, g, rows, lds);
+    } else {
+        if (pair) return hipErrorInvalidValue;
+    }
     if constexpr (PRE == kPreNone && (std::is_same<Q, Q8_0Unit>::value || std::is_same<Q, BF16Unit>::value)) {
         if (mr == 4) return launch_rowstep_tiled<Q, PRE, 4>(lane, args, g, rows, 4 * lds);
         if (mr == 2) return launch_rowstep_tiled<Q, PRE, 2>(lane, args, g, rows, 2 * lds);
@@ -1214,18 +1291,6 @@ hipError_t launch_matvec(Lane* lane, uint32_t type, const float* x, const void* 
         hipLaunchKernelGGL(matvec_q8_0_oddrow_kernel, dim3((out_w + 3) / 4, rows), dim3(256), 0, lane->stream, a);
         return hipGetLastError();
     }
-    if (rows == 1 && matvec_stream_takes(type, NNHIP_PRE_NONE, x, w, in_w, out_w)) {
-        nnhip_fused_matvec_desc d{};
-        d.ggml_type = type;
-        d.pre_op = NNHIP_PRE_NONE;
-        d.x = x;
-        d.w = w;
-        d.bias = bias;
-        d.y = y;
-        d.in_w = in_w;
-        d.out_w = out_w;
-        return launch_matvec_stream(lane, d);
-    }
 
     a.units_per_row = in_w / kUnitW;
     a.magic = static_cast<uint32_t>((0x100000000ull + a.units_per_row - 1) / a.units_per_row);
@@ -1264,9 +1329,6 @@ bool matvec_fused_supported(uint32_t type, int in_w)
 
 hipError_t launch_matvec_fused(Lane* lane, const nnhip_fused_matvec_desc& d)
 {
-    if (matvec_stream_takes(d.ggml_type, static_cast<int>(d.pre_op), d.x, d.w, d.in_w, d.out_w) &&
-        !(reinterpret_cast<uintptr_t>(d.x2) & 15u) && !(reinterpret_cast<uintptr_t>(d.norm_weight) & 15u))
-        return launch_matvec_stream(lane, d);
     int elems = 0, bytes = 0;
     type_block(d.ggml_type, &elems, &bytes);
     MatvecArgs a{};
@@ -1289,6 +1351,10 @@ hipError_t launch_matvec_fused(Lane* lane, const nnhip_fused_matvec_desc& d)
     a.lora_b = d.lora_b;
     a.lora_rank = d.lora_rank;
     a.lora_scale = d.lora_scale;
+    a.head4 = d.x_head_width >> 2;
+    a.head_group = d.x_head_group;
+    a.pair_rows = d.post_op == NNHIP_POST_SILU_PAIR ? d.out_w / 2 : 0;
+    if (d.x_head_width > 0) return launch_fused_of<kPreHeadGather>(lane, d.ggml_type, a);
     switch (d.pre_op) {
     case NNHIP_PRE_NONE: return launch_fused_of<kPreNone>(lane, d.ggml_type, a);
     case NNHIP_PRE_RMS_NORM: return launch_fused_of<kPreRmsNorm>(lane, d.ggml_type, a);

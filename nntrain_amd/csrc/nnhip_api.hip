@@ -614,27 +614,13 @@ int nnhip_add_in_place(void* handle, float* destination, const float* source, in
     return NNHIP_OK;
 }
 
-// The checks of one fused mat-vec descriptor, shared by the single call and the steps of a chain.
-static int check_fused(uint32_t op, nnhip::Lane* lane, const nnhip_fused_matvec_desc* d, bool chain_step)
+int nnhip_quant_matvec_fused(void* handle, const nnhip_fused_matvec_desc* d)
 {
-    using namespace nnhip;
+    NNHIP_LANE(handle, NNHIP_OP_MATVEC_FUSED)
+    const uint32_t op = NNHIP_OP_MATVEC_FUSED;
     if (!d || d->struct_size != sizeof(nnhip_fused_matvec_desc))
         return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0, "descriptor is null or has the wrong struct_size");
-    if (d->x_head_width < 0 || d->x_head_group < 0 || (d->x_head_width > 0) != (d->x_head_group > 0))
-        return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0, "x_head_width and x_head_group must both be positive or both be zero");
-    if (d->post_op != NNHIP_POST_NONE) {
-        if (!chain_step || d->post_op != NNHIP_POST_SILU_PAIR)
-            return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0, "post_op is NNHIP_POST_SILU_PAIR, and for steps of a chain only");
-        if (d->out_w % 2 != 0 || d->addend || d->lora_rank != 0)
-            return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0, "NNHIP_POST_SILU_PAIR needs an even out_w, no addend and no low-rank branch");
-    }
-    if (d->x_head_width > 0) {
-        if (!chain_step) return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0, "x_head_width is for steps of a chain");
-        if (d->x_head_width % 4 != 0 || d->in_w % (d->x_head_width * d->x_head_group) != 0 || d->pre_op != NNHIP_PRE_NONE)
-            return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0,
-                        "x_head_width must be a multiple of 4, in_w a whole number of head groups, and the step without a pre-op");
-    }
-    const int rc = check_linear(op, lane, d->ggml_type, d->x, d->w, d->y, 1, d->in_w, d->out_w);
+    int rc = check_linear(op, lane, d->ggml_type, d->x, d->w, d->y, 1, d->in_w, d->out_w);
     if (rc != NNHIP_OK) return rc;
     if (d->in_w > matvec_max_in_w(d->ggml_type))
         return fail(NNHIP_ERR_TOO_LARGE, op, lane->device, 0, "in_w %d exceeds the %d values one workgroup can stage", d->in_w, matvec_max_in_w(d->ggml_type));
@@ -662,6 +648,18 @@ static int check_fused(uint32_t op, nnhip::Lane* lane, const nnhip_fused_matvec_
     default:
         return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0, "unknown pre_op %u", d->pre_op);
     }
+    if (d->reserved != 0) return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0, "reserved must be 0");
+    if (d->x_head_width < 0 || d->x_head_group < 0 || (d->x_head_width > 0) != (d->x_head_group > 0))
+        return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0, "x_head_width and x_head_group must both be positive or both be zero");
+    if (d->x_head_width > 0 && (d->x_head_width % 4 != 0 || d->in_w % (d->x_head_width * d->x_head_group) != 0 || d->pre_op != NNHIP_PRE_NONE))
+        return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0,
+                    "x_head_width must be a multiple of 4, in_w a whole number of head groups, and pre_op NNHIP_PRE_NONE");
+    if (d->post_op != NNHIP_POST_NONE) {
+        if (d->post_op != NNHIP_POST_SILU_PAIR) return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0, "unknown post_op %u", d->post_op);
+        if (d->out_w % 2 != 0 || d->addend || d->lora_rank != 0 || d->pre_op == NNHIP_PRE_SILU_MULTIPLY || d->x_head_width > 0)
+            return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0,
+                        "NNHIP_POST_SILU_PAIR needs an even out_w, no addend, no low-rank branch, and pre_op NNHIP_PRE_NONE or NNHIP_PRE_RMS_NORM");
+    }
     if (d->lora_rank < 0 || (d->lora_rank > 0 && (!d->lora_z || !d->lora_b)) || (d->lora_rank == 0 && (d->lora_z || d->lora_b)))
         return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0, "lora_z and lora_b go with a positive lora_rank, and only with one");
     if (d->lora_rank > 0 && !std::isfinite(d->lora_scale))
@@ -676,100 +674,9 @@ static int check_fused(uint32_t op, nnhip::Lane* lane, const nnhip_fused_matvec_
     if (overlaps(d->x_out, d->x) || overlaps(d->x_out, d->x2) || overlaps(d->sum_out, d->x) || overlaps(d->sum_out, d->x2) ||
         overlaps(d->x_out, d->sum_out))
         return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0, "x_out and sum_out must not overlap the inputs or each other");
-    return NNHIP_OK;
-}
-
-int nnhip_quant_matvec_fused(void* handle, const nnhip_fused_matvec_desc* d)
-{
-    NNHIP_LANE(handle, NNHIP_OP_MATVEC_FUSED)
-    const uint32_t op = NNHIP_OP_MATVEC_FUSED;
-    const int rc = check_fused(op, lane, d, false);
-    if (rc != NNHIP_OK) return rc;
     hipError_t e = launch_matvec_fused(lane, *d);
     if (e != hipSuccess) return hip_fail(e, op, lane->device, "fused mat-vec launch");
     lane->counters.kernel_launches += 1;
-    return NNHIP_OK;
-}
-
-namespace {
-constexpr uint32_t kChainMagic = 0x4e43484eu;   // "NCHN"
-struct ChainHandle {
-    uint32_t magic = kChainMagic;
-    nnhip::Lane* lane = nullptr;
-    nnhip::ChainImpl* impl = nullptr;
-};
-}  // namespace
-
-int nnhip_chain_create(void* handle, const nnhip_fused_matvec_desc* steps, int count, void** chain)
-{
-    NNHIP_LANE(handle, NNHIP_OP_CHAIN)
-    const uint32_t op = NNHIP_OP_CHAIN;
-    if (!steps || !chain || count < 1)
-        return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0, "steps and chain must be non-null and count positive");
-    if (lane->capturing)
-        return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0, "a chain cannot be created while a graph is being captured");
-    for (int i = 0; i < count; ++i) {
-        const int rc = check_fused(op, lane, steps + i, true);
-        if (rc != NNHIP_OK) return rc;
-    }
-    ChainImpl* impl = nullptr;
-    hipError_t e = chain_build(lane, steps, count, &impl);
-    if (e == hipErrorNotSupported)
-        return fail(NNHIP_ERR_INVALID_ARGUMENT, op, lane->device, 0, "a step gathers x by heads or pairs its rows but does not run on the matrix cores");
-    if (e != hipSuccess) return hip_fail(e, op, lane->device, "chain table");
-    ChainHandle* h = new ChainHandle();
-    h->lane = lane;
-    h->impl = impl;
-    *chain = h;
-    return NNHIP_OK;
-}
-
-#define NNHIP_CHAIN(ptr) \
-    ChainHandle* ch = static_cast<ChainHandle*>(ptr); \
-    if (!ch || ch->magic != kChainMagic || ch->lane != lane) \
-        return fail(NNHIP_ERR_BAD_HANDLE, NNHIP_OP_CHAIN, lane->device, 0, "chain handle was not created on this lane");
-
-int nnhip_chain_launch(void* handle, void* chain)
-{
-    NNHIP_LANE(handle, NNHIP_OP_CHAIN)
-    NNHIP_CHAIN(chain)
-    hipError_t e = chain_launch(lane, ch->impl);
-    if (e != hipSuccess) return hip_fail(e, NNHIP_OP_CHAIN, lane->device, "chain launch");
-    return NNHIP_OK;
-}
-
-int nnhip_chain_status(void* handle, void* chain, int* gave_up)
-{
-    NNHIP_LANE(handle, NNHIP_OP_CHAIN)
-    NNHIP_CHAIN(chain)
-    if (!gave_up) return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_CHAIN, lane->device, 0, "gave_up is null");
-    if (lane->capturing)
-        return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_CHAIN, lane->device, 0, "the status cannot be read while a graph is being captured");
-    hipError_t e = chain_status(lane, ch->impl, gave_up);
-    if (e != hipSuccess) return hip_fail(e, NNHIP_OP_CHAIN, lane->device, "chain status");
-    return NNHIP_OK;
-}
-
-int nnhip_chain_launches(void* handle, void* chain, int* launches)
-{
-    NNHIP_LANE(handle, NNHIP_OP_CHAIN)
-    NNHIP_CHAIN(chain)
-    if (!launches) return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_CHAIN, lane->device, 0, "launches is null");
-    *launches = chain_launch_count(ch->impl);
-    return NNHIP_OK;
-}
-
-int nnhip_chain_destroy(void* handle, void* chain)
-{
-    NNHIP_LANE(handle, NNHIP_OP_CHAIN)
-    NNHIP_CHAIN(chain)
-    if (lane->capturing)
-        return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_CHAIN, lane->device, 0, "a chain cannot be destroyed while a graph is being captured");
-    hipError_t e = hipStreamSynchronize(lane->stream);      // (a launch may still read the table)
-    ch->magic = 0;
-    chain_free(ch->impl);
-    delete ch;
-    if (e != hipSuccess) return hip_fail(e, NNHIP_OP_CHAIN, lane->device, "chain destroy");
     return NNHIP_OK;
 }
 

@@ -85,17 +85,6 @@ hipError_t launch_matvec(Lane* lane, uint32_t type, const float* x, const void* 
 bool matvec_fused_supported(uint32_t type, int in_w);
 hipError_t launch_matvec_fused(Lane* lane, const nnhip_fused_matvec_desc& d);
 hipError_t launch_matvec_batch(Lane* lane, const nnhip_matvec_desc* descs, int count);
-// One mat-vec per launch on the matrix cores (gemv_mfma_stream.hip): whether it takes a call (storage type, row length,
-// alignment, activation preparation), and the launch; a plain call is a descriptor without preparation or epilogue.
-bool matvec_stream_takes(uint32_t type, int pre_op, const void* x, const void* w, int in_w, int out_w);
-hipError_t launch_matvec_stream(Lane* lane, const nnhip_fused_matvec_desc& d);
-// Chains of dependent fused mat-vecs (gemv_mfma_stream.hip): built once (blocking), launched any number of times.
-struct ChainImpl;
-hipError_t chain_build(Lane* lane, const nnhip_fused_matvec_desc* steps, int count, ChainImpl** out);
-hipError_t chain_launch(Lane* lane, const ChainImpl* chain);
-hipError_t chain_status(Lane* lane, const ChainImpl* chain, int* gave_up);
-int chain_launch_count(const ChainImpl* chain);
-void chain_free(ChainImpl* chain);
 // Matrix-core form of the mat-vec (gemv_mfma_kernels.hip): whether it takes a shape (and with which geometry), and its launch.
 struct MfmaPlan {
     int waves, cols, kchunks, stages, stage_bytes, loads_per_wave, lds_bytes;

@@ -94,24 +94,4 @@ __device__ __forceinline__ void k4_scale_pair(uint32_t s0, uint32_t s1, uint32_t
     mn = j < 2 ? lo_mn : hi_mn;
 }
 
-__device__ __forceinline__ float4 add4(const float4 a, const float4 b) { return make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w); }
-
-// gate * sigmoid(gate) * up with the two-sided sigmoid of the reference (NNtrain.Arc/Kernels/qwen35_attention.cl:9-14,
-// 38-43): exp never sees a positive argument.
-__device__ __forceinline__ float silu_mul1(float g, float u)
-{
-    float sig;
-    if (g >= 0.0f) {
-        sig = 1.0f / (1.0f + expf(-g));
-    } else {
-        const float e = expf(g);
-        sig = e / (1.0f + e);
-    }
-    return g * sig * u;
-}
-__device__ __forceinline__ float4 silu_mul4(const float4 g, const float4 u)
-{
-    return make_float4(silu_mul1(g.x, u.x), silu_mul1(g.y, u.y), silu_mul1(g.z, u.z), silu_mul1(g.w, u.w));
-}
-
 }  // namespace nnhip

@@ -7,7 +7,8 @@ with one launch per operation.  This module runs the same sequence of projection
 (token_embd, blk.N.attn_norm / attn_q / attn_k / attn_v / attn_output / ffn_norm / ffn_gate / ffn_up / ffn_down,
 output_norm, output) on one lane, either that way (`fused=False`) or with the launches this library fuses
 (`fused=True`: q|k|v and gate|up stacked, the norms and the SiLU product folded into the projections that consume them,
-the residual add folded into the down projection): five launches per layer instead of twelve, same bits.
+the residual adds folded into the o and down projections, the value heads read by the o projection itself, SiLU(gate) * up
+left by the stacked gate|up projection): four launches per layer instead of twelve, same bits.
 
 What is NOT here: the attention core and the key/value cache (outside the quantized-linear path).  Every token is
 decoded as the first token of its own sequence, where causal attention is exact without a cache: the single key has
@@ -28,7 +29,6 @@ from . import qwen35_gpu
 from .gguf import GgufReader, InvalidDataError
 from .lane import HipBuffer, HipExecutionLane
 from .loader import GgufTensorDirectory, HipGgufLoader, NotSupportedError
-from .chain import HipMatvecChain
 from .native import POST_SILU_PAIR
 from .quantized_matrix import PRE_RMS_NORM, PRE_SILU_MULTIPLY, HipQuantizedMatrix
 
@@ -183,8 +183,6 @@ class QuantizedDecoder:
                                        self.logits]
         self._graph = None
         self._graph_start = 0
-        self._chains: list | None = None       # build_chains(): the token step as chains of dependent mat-vecs
-        self._chain_start = 0
 
     # ---------------------------------------------------------------------------------------------- one token
     def _layers_and_head(self) -> None:
@@ -196,7 +194,19 @@ class QuantizedDecoder:
         gate_view, up_view = self._gate_up.view(0, 4 * ffn), self._gate_up.view(4 * ffn, 4 * ffn)
         for L in self.layers:
             cur, nxt = self._hidden[self._cur], self._hidden[self._cur ^ 1]
-            if self.fused:
+            if self.fused and L.qkv is not None and L.gate_up is not None:
+                # Four launches.  The o projection reads the value heads itself (what first-token attention would have
+                # copied) and adds the residual stream; the stacked gate | up projection leaves SiLU(gate) * up, so the
+                # down projection reads one vector and nobody forms the product twice.  Every value has the bits of the
+                # one-launch-per-operation sequence.
+                L.qkv.forward_fused(lane, cur, pre_op=PRE_RMS_NORM, norm_weight=L.attn_norm, epsilon=eps, out=self._qkv)
+                L.o.forward_fused(lane, v_view, addend=cur, out=nxt, x_head_width=d.head_width,
+                                  x_head_group=d.head_count // d.kv_head_count)
+                L.gate_up.forward_fused(lane, nxt, pre_op=PRE_RMS_NORM, norm_weight=L.ffn_norm, epsilon=eps, out=self._act,
+                                        post_op=POST_SILU_PAIR)
+                L.down.forward_fused(lane, self._act, addend=nxt, out=nxt)
+                self._cur ^= 1
+            elif self.fused:
                 if L.qkv is not None:
                     L.qkv.forward_fused(lane, cur, pre_op=PRE_RMS_NORM, norm_weight=L.attn_norm, epsilon=eps, out=self._qkv)
                 else:
@@ -234,82 +244,10 @@ class QuantizedDecoder:
             qwen35_gpu.rms_norm(lane, hidden, self.output_norm, 1, d.embedding_length, eps, out=self._norm)
             self.output.forward(lane, self._norm, None, out=self.logits)
 
-    # ---------------------------------------------------------------------------------------------- chained form
-    def build_chains(self, fold_attention: bool = False) -> None:
-        """Hands the fused launches of a token step to the library as chains (HipMatvecChain): per layer one chain
-        [o -> add + RMSNorm + gate|up -> SiLU * up + down + add -> RMSNorm + next q|k|v (or the head)] with the attention
-        launch between chains, or, with fold_attention, the whole token as one chain in which the o projection gathers
-        its input from the value heads itself (what first-token attention computes).  Needs the stacked projections of
-        fused=True.  forward_token then runs the chains; dispose() frees them."""
-        if not self.fused or any(L.qkv is None or L.gate_up is None for L in self.layers):
-            raise NotSupportedError("Chains need fused=True and projections that could be stacked.")
-        if self._chains is not None:
-            return
-        d, lane = self.descriptor, self.lane
-        q_width, kv_width, ffn, eps = d.head_count * d.head_width, d.kv_head_count * d.head_width, d.feed_forward_length, d.rms_epsilon
-        v_view = self._qkv.view(4 * (q_width + kv_width), 4 * kv_width)
-        group = d.head_count // d.kv_head_count
-        plan: list = []                   # ("chain", [steps]) and ("attention",) in launch order
-        steps: list = []
-        cur_i = self._cur
-        for i, L in enumerate(self.layers):
-            cur, nxt = self._hidden[cur_i], self._hidden[cur_i ^ 1]
-            steps.append(L.qkv.fused_descriptor(lane, cur, pre_op=PRE_RMS_NORM, norm_weight=L.attn_norm, epsilon=eps, out=self._qkv))
-            # the o projection adds the residual stream itself (the same single FP32 addition as add + RMSNorm makes), so
-            # the next step normalizes one vector
-            if fold_attention:
-                steps.append(L.o.fused_descriptor(lane, v_view, addend=cur, out=nxt, x_head_width=d.head_width, x_head_group=group))
-            else:
-                plan.append(("chain", steps))
-                plan.append(("attention",))
-                steps = [L.o.fused_descriptor(lane, self._ctx, addend=cur, out=nxt)]
-            # the stacked gate | up projection leaves SiLU(gate) * up itself: the down projection reads one vector, and
-            # no workgroup computes the product for rows it did not multiply
-            steps.append(L.gate_up.fused_descriptor(lane, nxt, pre_op=PRE_RMS_NORM, norm_weight=L.ffn_norm, epsilon=eps,
-                                                    out=self._act, post_op=POST_SILU_PAIR))
-            steps.append(L.down.fused_descriptor(lane, self._act, addend=nxt, out=nxt))
-            cur_i ^= 1
-        steps.append(self.output.fused_descriptor(lane, self._hidden[cur_i], pre_op=PRE_RMS_NORM, norm_weight=self.output_norm,
-                                                  epsilon=eps, out=self.logits))
-        plan.append(("chain", steps))
-        chains = []
-        try:
-            for item in plan:
-                chains.append(HipMatvecChain(lane, item[1]) if item[0] == "chain" else None)
-        except BaseException:
-            for c in chains:
-                if c is not None:
-                    c.dispose()
-            raise
-        self._chains, self._chain_start, self._chain_end = chains, self._cur, cur_i
-        self._v_view = v_view
-
-    def _run_chains(self) -> None:
-        d = self.descriptor
-        for c in self._chains:
-            if c is None:
-                qwen35_gpu.first_token_attention(self.lane, self._v_view, d.head_count, d.kv_head_count, d.head_width, out=self._ctx)
-            else:
-                c.launch()
-
-    @property
-    def chain_launches(self) -> int:
-        """Kernel launches of one token step in the chained form (the embedding lookup not counted)."""
-        return sum(1 if c is None else c.launches for c in self._chains or [])
-
-    def chains_gave_up(self) -> bool:
-        return any(c.gave_up() for c in self._chains or [] if c is not None)
-
     def forward_token(self, token_id: int) -> HipBuffer:
         """Logits of `token_id` decoded as the first token of a sequence; the buffer is reused by the next call."""
         if not 0 <= token_id < self.descriptor.vocabulary:
             raise IndexError(f"Embedding index {token_id} is outside the vocabulary.")
-        if self._graph is None and self._chains is not None:
-            self._cur = self._chain_start
-            self.embedding.dequantize(self.lane, row=token_id, out=self._hidden[self._cur])
-            self._run_chains()
-            self._cur = self._chain_end
-            return self.logits
         if self._graph is not None:
             self._cur = self._graph_start
             self.embedding.dequantize(self.lane, row=token_id, out=self._hidden[self._cur])
@@ -325,15 +263,10 @@ class QuantizedDecoder:
         embedding lookup stays outside: its source row changes with the token).  One eager step must have run."""
         if self._graph is not None:
             return
-        self._graph_start = self._cur if self._chains is None else self._chain_start
-        self._cur = self._graph_start
+        self._graph_start = self._cur
         self.lane.graph_begin()
         try:
-            if self._chains is not None:
-                self._run_chains()
-                self._cur = self._chain_end
-            else:
-                self._layers_and_head()
+            self._layers_and_head()
         finally:
             graph = self.lane.graph_end()
         self._graph, self._graph_end = graph, self._cur
@@ -360,24 +293,10 @@ class QuantizedDecoder:
         rate = (len(tokens) - 1) * 1000.0 / (last - first) if len(tokens) > 1 and last > first else None
         return tokens, GenerationTiming(len(tokens), total, first, rate)
 
-    def release_graph(self) -> None:
-        """Back to eager launches (a later capture_graph records the form in use then)."""
+    def dispose(self) -> None:
         if getattr(self, "_graph", None) is not None and not self.lane.disposed:
             self.lane.graph_destroy(self._graph)
         self._graph = None
-
-    def release_chains(self) -> None:
-        """Back to one launch per fused operation; a graph that replays the chains is released with them."""
-        if getattr(self, "_chains", None) is not None:
-            self.release_graph()
-        for c in getattr(self, "_chains", None) or []:
-            if c is not None:
-                c.dispose()
-        self._chains = None
-
-    def dispose(self) -> None:
-        self.release_graph()
-        self.release_chains()
         for item in reversed(getattr(self, "_owned", [])):
             item.dispose()
         self._owned = []

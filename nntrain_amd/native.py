@@ -98,11 +98,6 @@ PROTOTYPES = {
     "nnhip_quant_matvec_batch": (c_int, [c_void_p, POINTER(MatvecDesc), c_int]),
     "nnhip_quant_matvec_batch_static": (c_int, [c_void_p, POINTER(MatvecDesc), c_int]),
     "nnhip_quant_matvec_fused": (c_int, [c_void_p, POINTER(FusedMatvecDesc)]),
-    "nnhip_chain_create": (c_int, [c_void_p, POINTER(FusedMatvecDesc), c_int, POINTER(c_void_p)]),
-    "nnhip_chain_launch": (c_int, [c_void_p, c_void_p]),
-    "nnhip_chain_status": (c_int, [c_void_p, c_void_p, POINTER(c_int)]),
-    "nnhip_chain_launches": (c_int, [c_void_p, c_void_p, POINTER(c_int)]),
-    "nnhip_chain_destroy": (c_int, [c_void_p, c_void_p]),
     "nnhip_quant_matmul": (c_int, [c_void_p, c_uint32, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int]),
     "nnhip_quant_matmul_bf16": (c_int, [c_void_p, c_uint32, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int]),
     "nnhip_rms_norm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float]),

@@ -163,9 +163,7 @@ class HipQuantizedMatrix:
                          out: HipBuffer, lora_z: HipBuffer | None = None, lora_b: HipBuffer | None = None,
                          lora_rank: int = 0, lora_scale: float = 0.0, x_head_width: int = 0,
                          x_head_group: int = 0, post_op: int = 0) -> FusedMatvecDesc:
-        """The native descriptor of forward_fused with these arguments (also one step of a HipMatvecChain, where
-        x_head_width / x_head_group gather x by heads first: v[h * width + j] = x[(h // group) * width + j], and
-        post_op POST_SILU_PAIR stores SiLU(z[o]) * z[out / 2 + o] for the first half of the rows instead of z)."""
+        """The native descriptor of forward_fused with these arguments."""
         if lora_rank < 0:
             raise ValueError("lora_rank must not be negative.")
         if lora_rank > 0 and (lora_z is None or lora_b is None or lora_z.nbytes < 4 * lora_rank
@@ -191,19 +189,25 @@ class HipQuantizedMatrix:
                       norm_weight: HipBuffer | None = None, epsilon: float = 0.0, x_out: HipBuffer | None = None,
                       sum_out: HipBuffer | None = None, bias: HipBuffer | None = None, addend: HipBuffer | None = None,
                       out: HipBuffer | None = None, lora_z: HipBuffer | None = None, lora_b: HipBuffer | None = None,
-                      lora_rank: int = 0, lora_scale: float = 0.0) -> HipBuffer:
+                      lora_rank: int = 0, lora_scale: float = 0.0, x_head_width: int = 0, x_head_group: int = 0,
+                      post_op: int = 0) -> HipBuffer:
         """One decode mat-vec with its neighbours fused into the launch: v = RMSNorm(x + x2) * norm_weight
         (PRE_RMS_NORM; x2 optional) or SiLU(x) * x2 (PRE_SILU_MULTIPLY) or x, then y = addend + bias + W v.
         x_out / sum_out receive v and x + x2 when given.  `out` may be `addend` (the residual stream updated in place).
         lora_z [rank] and lora_b [out, rank] add the low-rank adapter branch lora_scale * z . b^T before the addend
-        (Matrix.ForwardFusedLora, Qwen35QuantizedModel.cs:1387)."""
-        if out is not None and out.nbytes < 4 * self.output_width:
+        (Matrix.ForwardFusedLora, Qwen35QuantizedModel.cs:1387).  x_head_width / x_head_group: x holds key/value heads and
+        is gathered first, v[h * width + j] = x[(h // group) * width + j] (what first-token attention hands the o
+        projection).  post_op POST_SILU_PAIR: the matrix stacks gate | up and `out` receives output_width / 2 values,
+        SiLU(gate) * up."""
+        n_y = self.output_width // 2 if post_op else self.output_width
+        if out is not None and out.nbytes < 4 * n_y:
             raise ValueError("Quantized linear 'out' width mismatch.")
-        y = out if out is not None else lane.allocate(self.output_width)
+        y = out if out is not None else lane.allocate(n_y)
         try:
             desc = self.fused_descriptor(lane, x, pre_op=pre_op, x2=x2, norm_weight=norm_weight, epsilon=epsilon, x_out=x_out,
                                          sum_out=sum_out, bias=bias, addend=addend, out=y, lora_z=lora_z, lora_b=lora_b,
-                                         lora_rank=lora_rank, lora_scale=lora_scale)
+                                         lora_rank=lora_rank, lora_scale=lora_scale, x_head_width=x_head_width,
+                                         x_head_group=x_head_group, post_op=post_op)
             with lane.kernel("quant_matvec_fused"):
                 check(lane._lib.nnhip_quant_matvec_fused(lane._handle, ctypes.byref(desc)), "quant_matvec_fused")
         except BaseException:

@@ -11,6 +11,7 @@ import pytest
 import oracle
 from nntrain_amd import (GGML_BF16, GGML_IQ2_S, GGML_IQ3_S, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_Q8_0, HipExecutionLane,
                          HipQuantizedMatrix, NnHipError, qwen35_gpu, synth)
+from nntrain_amd.native import POST_SILU_PAIR
 from nntrain_amd.quantized_matrix import PRE_NONE, PRE_RMS_NORM, PRE_SILU_MULTIPLY
 
 pytestmark = pytest.mark.gpu
@@ -86,6 +87,80 @@ def test_silu_down_projection_and_residual_add_equal_the_unfused_sequence_bitwis
     for b in (gate, upv, stream_a, stream_b, act, down, x_out):
         b.dispose()
     m.dispose()
+
+
+@pytest.mark.parametrize("typ", TYPES)
+@pytest.mark.parametrize("in_w,half", [(256, 5), (1024, 67), (5120, 300), (5376, 1031)])
+def test_stacked_gate_up_with_silu_pair_equals_the_unfused_sequence_bitwise(lane, typ, in_w, half):
+    """NNHIP_POST_SILU_PAIR: y[o] = SiLU(z[o]) * z[half + o], against projection -> nnhip_silu_multiply of the two halves;
+    with and without the RMSNorm in front, with a bias, odd halves and halves that do not fill the last row step."""
+    if typ == GGML_Q8_0 and (in_w // 32) % 2:
+        pytest.skip("rows of an odd number of Q8_0 blocks are not covered by the fused entry")
+    out_w = 2 * half
+    v = _vectors(in_w, out_w, in_w + 3 * typ)
+    m = _matrix(typ, out_w, in_w, 6)
+    x, gam, bias = lane.upload_raw(v["hidden"]), lane.upload_raw(v["gamma"]), lane.upload_raw(v["bias"])
+    for pre in (PRE_NONE, PRE_RMS_NORM):
+        vec = x if pre == PRE_NONE else qwen35_gpu.rms_norm(lane, x, gam, 1, in_w, EPS)
+        z = m.forward(lane, vec, bias)
+        ref = qwen35_gpu.silu_multiply(lane, z.view(0, 4 * half), z.view(4 * half, 4 * half), half)
+        y = lane.allocate(half + 3)
+        lane.fill_u32(y, 0x7FC00000, half + 3)
+        m.forward_fused(lane, x, pre_op=pre, norm_weight=gam if pre else None, epsilon=EPS if pre else 0.0, bias=bias,
+                        out=y, post_op=POST_SILU_PAIR)
+        got = lane.read(y, count=half + 3)
+        assert np.array_equal(_bits(got[:half]), _bits(lane.read(ref, count=half))), (typ, in_w, half, pre)
+        assert np.all(np.isnan(got[half:]))                       # nothing is written past the half
+        for b in (z, ref, y) + ((vec,) if pre else ()):
+            b.dispose()
+    for b in (x, gam, bias):
+        b.dispose()
+    m.dispose()
+
+
+@pytest.mark.parametrize("typ", [GGML_Q8_0, GGML_Q4_K, GGML_Q6_K, GGML_IQ3_S, GGML_BF16])
+@pytest.mark.parametrize("heads,kv,width,out_w", [(8, 2, 64, 37), (32, 16, 128, 300), (6, 6, 128, 9)])
+def test_head_gather_equals_first_token_attention_then_projection_bitwise(lane, typ, heads, kv, width, out_w):
+    """x_head_width / x_head_group: the o projection reads the value heads itself; with the residual stream as addend."""
+    in_w = heads * width
+    if typ == GGML_Q8_0 and (in_w // 32) % 2:
+        pytest.skip("rows of an odd number of Q8_0 blocks are not covered by the fused entry")
+    if in_w % 256:
+        pytest.skip("in_w is not a whole number of blocks")
+    rng = np.random.default_rng(heads + kv)
+    values = rng.standard_normal(kv * width).astype(np.float32)
+    stream = rng.standard_normal(out_w).astype(np.float32)
+    m = _matrix(typ, out_w, in_w, 8)
+    vb, sa, sb = lane.upload_raw(values), lane.upload_raw(stream), lane.upload_raw(stream)
+    ctx = qwen35_gpu.first_token_attention(lane, vb, heads, kv, width)
+    attn = m.forward(lane, ctx, None)
+    qwen35_gpu.add_in_place(lane, sa, attn, out_w)
+    out = m.forward_fused(lane, vb, addend=sb, out=sb, x_head_width=width, x_head_group=heads // kv)
+    assert out is sb
+    assert np.array_equal(_bits(lane.read(sb, count=out_w)), _bits(lane.read(sa, count=out_w)))
+    for b in (vb, sa, sb, ctx, attn):
+        b.dispose()
+    m.dispose()
+
+
+def test_new_descriptor_fields_are_checked(lane):
+    m = _matrix(GGML_Q4_K, 64, 1024, 2)
+    x, y, stream = lane.allocate(1024), lane.allocate(64), lane.allocate(64)
+    bad = [dict(post_op=2), dict(post_op=POST_SILU_PAIR, addend=stream), dict(x_head_width=128, x_head_group=0),
+           dict(x_head_width=130, x_head_group=1), dict(x_head_width=128, x_head_group=3),
+           dict(x_head_width=128, x_head_group=2, pre_op=PRE_RMS_NORM, norm_weight=x, epsilon=EPS),
+           dict(post_op=POST_SILU_PAIR, pre_op=PRE_SILU_MULTIPLY, x2=x)]
+    for kw in bad:
+        with pytest.raises(NnHipError) as info:
+            m.forward_fused(lane, x, out=y, **kw)
+        assert info.value.status == 1, kw
+    odd = _matrix(GGML_Q4_K, 65, 1024, 2)
+    with pytest.raises(NnHipError):
+        odd.forward_fused(lane, x, out=y, post_op=POST_SILU_PAIR)
+    for b in (x, y, stream):
+        b.dispose()
+    m.dispose()
+    odd.dispose()
 
 
 @pytest.mark.parametrize("typ", [GGML_Q8_0, GGML_Q4_K, GGML_IQ2_S])
