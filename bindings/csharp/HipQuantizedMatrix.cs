@@ -36,12 +36,17 @@ public sealed class HipQuantizedMatrix : IDisposable
     /// <summary>Rows at or above which Forward uses the matrix-core mat-mul (Qwen35QuantizedModel.cs:1249).</summary>
     public const int PrefillMinRows = 16;
 
+    /// <summary>Opt-in, like Qwen35ExecutionOptions.InferenceXmxPrefill (Qwen35ExecutionOptions.cs:50): rows >= 16 go to
+    /// the bfloat16 matrix-core mat-mul (2e-3 of the exact product) instead of the FP32-grade mat-vec (1e-5).</summary>
+    public bool InferenceMatmulPrefill { get; init; }
+
     /// <summary>Whether Forward sends this many input rows to the matrix-core mat-mul.</summary>
-    public bool UsesPrefill(int rows) => rows >= PrefillMinRows && InputWidth % 256 == 0;
+    public bool UsesPrefill(int rows) => InferenceMatmulPrefill && rows >= PrefillMinRows && InputWidth % 256 == 0;
 
     /// <summary>y[rows, out] = bias + x[rows, in] . W^T, FP32 activations; the caller disposes the result.
-    /// rows >= 16 go to the bf16 matrix-core mat-mul (activations rounded to bfloat16 on the device), fewer rows to the
-    /// dequantization-fused mat-vec, as Matrix.Forward routes them (Qwen35QuantizedModel.cs:1249-1369).  Allocating the
+    /// Every row count goes to the dequantization-fused mat-vec unless InferenceMatmulPrefill is set, in which case rows
+    /// >= 16 go to the bf16 matrix-core mat-mul (activations rounded to bfloat16 on the device), the counterpart of the
+    /// reference's opt-in XMX prefill (Qwen35QuantizedModel.cs:1249-1317).  Allocating the
     /// output per call is cheap: the lane hands out the block a previous Dispose returned.</summary>
     public HipBuffer Forward(HipExecutionLane lane, HipBuffer input, HipBuffer? bias, int rows = 1)
     {

@@ -144,7 +144,8 @@ NNHIP_API int nnhip_lane_destroy(void* lane);
  * all work of a lane is ordered on its one stream - so the reference's pattern of allocating each projection's output
  * and disposing it after use (Qwen35QuantizedModel.cs:488-491) costs no synchronisation.  Larger blocks are returned
  * to the driver after the stream has drained.  While a graph is being captured nnhip_alloc can only hand out kept
- * blocks.  nnhip_lane_trim drains the stream and returns every kept block to the driver; it has no counterpart in the
+ * blocks, and a block freed during the capture stays out of circulation until that graph is destroyed (the recorded
+ * work names it; a replay must not write into memory that has a new owner).  nnhip_lane_trim drains the stream and returns every kept block to the driver; it has no counterpart in the
  * reference, whose OpenCL runtime defers releases itself. */
 NNHIP_API int nnhip_alloc(void* lane, size_t bytes, void** dptr);
 NNHIP_API int nnhip_free(void* lane, void* dptr);
@@ -192,10 +193,11 @@ NNHIP_API int nnhip_dequantize(void* lane, uint32_t ggml_type, const void* w, fl
  * by Qwen35QuantizedModel.Matrix.Forward (Qwen35QuantizedModel.cs:1210-1369) and Tensor.ArcQwenQuantizedLinear
  * (NNtrain.Core/Tensors/Tensor.QwenQuantized.cs:29-96) for decode (rows == 1) and small row counts.  Each
  * output row of y is computed with the same operation order whatever `rows` is, so rows > 1 equals stacked
- * rows == 1 calls bit for bit (Qwen35InferencePrefillLinearTests.cs:64-77), except for calls with 2 - 16 input rows
- * on Q4_K / Q5_K / Q6_K / IQ2_S matrices (3 - 16 on Q8_0) with rows x ceil(out_w / 16) >= 2048: those take the matrix-core path described
- * at nnhip_quant_matvec_batch (up to four input rows per pass over the weights; a row's bits do not depend on the
- * rows it travels with; 1e-6 from the rows == 1 result).  bias may be null (zero).  Asynchronous. */
+ * rows == 1 calls bit for bit (Qwen35InferencePrefillLinearTests.cs:64-77), except for calls with two or more input rows
+ * on Q4_K / Q5_K / Q6_K / IQ2_S matrices (three or more on Q8_0) with rows x ceil(out_w / 16) >= 2048: those take the
+ * matrix-core path described at nnhip_quant_matvec_batch (up to four input rows per pass over the weights, sixteen per
+ * launch; a row's bits do not depend on the rows it travels with; 1e-6 from the rows == 1 result).  bias may be null
+ * (zero).  Asynchronous. */
 NNHIP_API int nnhip_quant_matvec(void* lane, uint32_t ggml_type, const float* x, const void* w, const float* bias,
                                  float* y, int rows, int in_w, int out_w);
 
@@ -235,7 +237,14 @@ NNHIP_API int nnhip_matvec_plan(uint32_t ggml_type, int rows, int in_w, int out_
  * Those results are deterministic,
  * depend on the weights, in_w and the activations of the row only (not on out_w, the other matrices or input rows of
  * the call, or the order), agree with the single launch to FP32 summation accuracy (relative L2 difference below 1e-6)
- * and are closer to the exact product than it.
+ * and are closer to the exact product than it.  The fixed point is relative to the largest magnitude of the input row,
+ * v = rint(x * 2^e) with |v| <= 2^30, products and sums of v and the quants are exact integers, so
+ *     |y[o] - exact[o]| <= 2^-31 * max_k |x[k]| * sum_k |w[o, k]|  +  the rounding of the FP32 accumulation;
+ * for activations of ordinary dynamic range that is below one FP32 rounding per product.  An input row whose largest
+ * magnitude exceeds its other values by a factor of 2^24 or more loses those other values' low bits (by 2^31 or more:
+ * all of them), which FP32 arithmetic would keep in the rows whose weight at the large activation is zero; such rows
+ * belong in nnhip_quant_matvec with rows == 1, which multiplies FP32 activations.  A NaN or an infinity in an input row
+ * makes every output of that row NaN.
  * The descriptors reach the device as a table in lane-owned memory, written by a small kernel on the lane's stream
  * (skipped when the table already holds them), so the call never waits for the device.  Under graph capture the write
  * is recorded with the launch and a replay restores the table it needs; the table cannot grow during a capture

@@ -1652,7 +1652,7 @@ int plan_matvec_batch(const nnhip_matvec_desc* descs, int count, int compute_uni
 
 bool matvec_rows_share_pass(uint32_t type, int rows, int in_w, int out_w, const void* w)
 {
-    return rows >= shared_pass_min_rows(type) && rows <= 16 &&
+    return rows >= shared_pass_min_rows(type) &&
            static_cast<long>(rows) * ((out_w + 15) / 16) >= kMfmaBatchMinTiles && matvec_mfma_wide_geometry(type, in_w, out_w, w, 4);
 }
 

@@ -1913,7 +1913,7 @@ bool describe_matvec_rows_shared(uint32_t type, int rows, int in_w, int out_w, i
 {
     WideGeom g;
     if (!plan_wide(type, in_w, 4, &g)) return false;
-    const int tiles = (out_w + kTileRows - 1) / kTileRows * ((rows + 3) / 4);
+    const int tiles = (out_w + kTileRows - 1) / kTileRows * (((rows < 16 ? rows : 16) + 3) / 4);      // (of one launch: sixteen input rows)
     info->kernel = NNHIP_MATVEC_KERNEL_MATRIX_CORE;
     info->threads = 64 * g.waves;
     info->rows_per_step = kTileRows;
@@ -1960,20 +1960,29 @@ hipError_t launch_matvec_mfma_wide_table(Lane* lane, uint32_t type, int in_w, in
 }
 
 hipError_t launch_matvec_rows_shared(Lane* lane, uint32_t type, const float* x, const void* w, const float* bias, float* y,
-                                     int rows, int in_w, int out_w)
+                                     int rows, int in_w, int out_w, int* launches)
 {
-    if (rows < 2 || rows > 16) return hipErrorInvalidValue;
-    WideArgs a{};
-    a.table = nullptr;
-    for (int r = 0; r < rows; r += 4) {
-        MfmaTableEntry e = matvec_mfma_entry(type, x + static_cast<size_t>(r) * in_w, w, bias, y + static_cast<size_t>(r) * out_w,
-                                             in_w, out_w, a.total_tiles);
-        e.rows = rows - r < 4 ? rows - r : 4;
-        a.inline_entries[a.entries++] = e;
-        a.total_tiles += e.tiles;
+    if (rows < 2) return hipErrorInvalidValue;
+    // sixteen input rows per launch (four table entries of four rows travel in the kernel arguments); a row's bits do not
+    // depend on the rows it shares a pass or a launch with
+    *launches = 0;
+    for (int r0 = 0; r0 < rows; r0 += 16) {
+        const int n = rows - r0 < 16 ? rows - r0 : 16;
+        WideArgs a{};
+        a.table = nullptr;
+        for (int r = r0; r < r0 + n; r += 4) {
+            MfmaTableEntry e = matvec_mfma_entry(type, x + static_cast<size_t>(r) * in_w, w, bias, y + static_cast<size_t>(r) * out_w,
+                                                 in_w, out_w, a.total_tiles);
+            e.rows = r0 + n - r < 4 ? r0 + n - r : 4;
+            a.inline_entries[a.entries++] = e;
+            a.total_tiles += e.tiles;
+        }
+        a.chunked = a.entries >= 3 ? 1 : 0;         // (9 - 16 input rows: three or four groups of rows, each with planes of its own)
+        const hipError_t e = launch_wide_args(lane, type, in_w, 4, a);
+        if (e != hipSuccess) return e;
+        ++*launches;
     }
-    a.chunked = a.entries >= 3 ? 1 : 0;         // (9 - 16 input rows: three or four groups of rows, each with planes of its own)
-    return launch_wide_args(lane, type, in_w, 4, a);
+    return hipSuccess;
 }
 
 }  // namespace nnhip

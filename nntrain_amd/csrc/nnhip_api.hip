@@ -287,6 +287,13 @@ int nnhip_lane_destroy(void* handle)
             if (first == hipSuccess) first = e;
         }
     lane->free_blocks.clear();
+    for (const auto& b : lane->capture_pinned) (void)hipFree(b.first);
+    lane->capture_pinned.clear();
+    for (Graph* gr : lane->graphs) {            // graphs the caller never destroyed: their scratch blocks go with the lane
+        for (const auto& b : gr->pinned) (void)hipFree(b.first);
+        gr->pinned.clear();
+    }
+    lane->graphs.clear();
     if (lane->batch_table) (void)hipFree(lane->batch_table);
     for (void* t : lane->retired_tables) (void)hipFree(t);
     for (int i = 0; i < 2; ++i) {
@@ -359,6 +366,11 @@ int nnhip_free(void* handle, void* dptr)
             return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_FREE, lane->device, 0, "a block this large cannot be freed while a graph is being captured");
         lane->counters.allocated_bytes -= it->second.bytes;
         lane->buffers.erase(it);
+        if (keep && lane->capturing) {
+            // the work being recorded names this block: it stays out of circulation until the graph is destroyed
+            lane->capture_pinned.emplace_back(dptr, capacity);
+            return NNHIP_OK;
+        }
         if (keep) {
             lane->free_blocks[capacity].push_back(dptr);
             lane->cached_bytes += capacity;
@@ -524,11 +536,13 @@ int nnhip_quant_matvec(void* handle, uint32_t ggml_type, const float* x, const v
         return fail(NNHIP_ERR_TOO_LARGE, NNHIP_OP_MATVEC, lane->device, 0, "in_w %d exceeds the %d values one workgroup can stage", in_w, matvec_max_in_w(ggml_type));
     if (rows > 65535) return fail(NNHIP_ERR_TOO_LARGE, NNHIP_OP_MATVEC, lane->device, 0, "rows %d exceeds 65535", rows);
     if (matvec_rows_share_pass(ggml_type, rows, in_w, out_w, w)) {
-        // 2 - 15 input rows of a K-quant matrix: up to four rows share a pass over the weights on the matrix cores
-        // (the reference routes such calls to row-tiled kernels, Qwen35QuantizedModel.cs:1335-1344)
-        const hipError_t e = launch_matvec_rows_shared(lane, ggml_type, x, w, bias, y, rows, in_w, out_w);
+        // two or more input rows of a large matrix: up to four rows share a pass over the weights on the matrix cores,
+        // sixteen rows go into a launch (the reference routes such calls to row-tiled kernels,
+        // Qwen35QuantizedModel.cs:1335-1344)
+        int launches = 0;
+        const hipError_t e = launch_matvec_rows_shared(lane, ggml_type, x, w, bias, y, rows, in_w, out_w, &launches);
+        lane->counters.kernel_launches += static_cast<uint64_t>(launches);
         if (e != hipSuccess) return hip_fail(e, NNHIP_OP_MATVEC, lane->device, "mat-vec launch");
-        lane->counters.kernel_launches += 1;
         return NNHIP_OK;
     }
     hipError_t e = launch_matvec(lane, ggml_type, x, w, bias, y, rows, in_w, out_w);
@@ -895,6 +909,21 @@ int nnhip_event_elapsed_ms(void* handle, void* start, void* stop, float* ms)
     return NNHIP_OK;
 }
 
+// Blocks that were pinned to a capture or a graph go back into circulation (or to the driver when the cache is full).
+static void release_pinned(nnhip::Lane* lane, std::vector<std::pair<void*, size_t>>& blocks)
+{
+    std::lock_guard<std::mutex> guard(lane->mutex);
+    for (const auto& b : blocks) {
+        if (lane->cached_bytes + b.second <= nnhip::kCacheTotalMax) {
+            lane->free_blocks[b.second].push_back(b.first);
+            lane->cached_bytes += b.second;
+        } else {
+            (void)hipFree(b.first);
+        }
+    }
+    blocks.clear();
+}
+
 int nnhip_graph_begin(void* handle)
 {
     NNHIP_LANE(handle, NNHIP_OP_GRAPH)
@@ -913,14 +942,19 @@ int nnhip_graph_end(void* handle, void** graph)
     lane->batch_shadow.clear();
     hipGraph_t g = nullptr;
     hipError_t e = hipStreamEndCapture(lane->stream, &g);
-    if (e != hipSuccess) return hip_fail(e, NNHIP_OP_GRAPH, lane->device, "hipStreamEndCapture");
+    if (e != hipSuccess) {
+        release_pinned(lane, lane->capture_pinned);      // (nothing was recorded that could be replayed)
+        return hip_fail(e, NNHIP_OP_GRAPH, lane->device, "hipStreamEndCapture");
+    }
     if (!graph) {
         (void)hipGraphDestroy(g);
+        release_pinned(lane, lane->capture_pinned);
         return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_GRAPH, lane->device, 0, "graph output pointer is null");
     }
     Graph* gr = new (std::nothrow) Graph();
     if (!gr) {
         (void)hipGraphDestroy(g);
+        release_pinned(lane, lane->capture_pinned);
         return fail(NNHIP_ERR_OUT_OF_MEMORY, NNHIP_OP_GRAPH, lane->device, 0, "host allocation failed");
     }
     gr->graph = g;
@@ -928,8 +962,12 @@ int nnhip_graph_end(void* handle, void** graph)
     if (e != hipSuccess) {
         (void)hipGraphDestroy(g);
         delete gr;
+        release_pinned(lane, lane->capture_pinned);
         return hip_fail(e, NNHIP_OP_GRAPH, lane->device, "hipGraphInstantiate");
     }
+    // the blocks freed during the capture belong to the graph from here on
+    gr->pinned.swap(lane->capture_pinned);
+    lane->graphs.push_back(gr);
     *graph = gr;
     return NNHIP_OK;
 }
@@ -953,6 +991,12 @@ int nnhip_graph_destroy(void* handle, void* graph)
     hipError_t e = hipStreamSynchronize(lane->stream);
     hipError_t e2 = hipGraphExecDestroy(gr->exec);
     hipError_t e3 = hipGraphDestroy(gr->graph);
+    release_pinned(lane, gr->pinned);
+    for (size_t i = 0; i < lane->graphs.size(); ++i)
+        if (lane->graphs[i] == gr) {
+            lane->graphs.erase(lane->graphs.begin() + static_cast<long>(i));
+            break;
+        }
     gr->magic = 0;
     delete gr;
     if (e == hipSuccess) e = e2;

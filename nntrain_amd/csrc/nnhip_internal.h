@@ -34,6 +34,11 @@ struct Lane {
     // a block can be reused at once: whatever still reads it was enqueued before whatever the next owner enqueues.
     std::unordered_map<size_t, std::vector<void*>> free_blocks;
     size_t cached_bytes = 0;
+    // Blocks freed while a graph is being captured: the recorded work names them, so they must not be handed out again
+    // while that graph can still be replayed.  They pass to the graph when the capture ends and come back to free_blocks
+    // when it is destroyed.
+    std::vector<std::pair<void*, size_t>> capture_pinned;
+    std::vector<struct Graph*> graphs;          // graphs captured on this lane and not destroyed yet
     std::mutex mutex;                           // guards buffers + counters (uploads may come from loader threads)
     void* batch_table = nullptr;                // device table of the batched mat-vec (written by a kernel on the stream)
     size_t batch_table_bytes = 0;               // its capacity
@@ -55,6 +60,7 @@ struct Graph {
     uint32_t magic = kGraphMagic;
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
+    std::vector<std::pair<void*, size_t>> pinned;      // lane blocks (pointer, capacity) the recorded work uses as scratch
 };
 
 // Raises the dynamic-LDS limit of one kernel, once per device (the attribute belongs to a function on a device).  Lanes
@@ -117,10 +123,11 @@ bool matvec_mfma_wide_geometry(uint32_t type, int in_w, int out_w, const void* w
 // True when a single call with `rows` input rows is served by that form (as a one-descriptor batch) rather than by one
 // row-step pass per input row.
 bool matvec_rows_share_pass(uint32_t type, int rows, int in_w, int out_w, const void* w);
-// That call: 2 - 16 input rows, up to four per pass, the descriptors travelling in the kernel arguments.
+// That call: two or more input rows, up to four per pass and sixteen per launch (the descriptors travel in the kernel
+// arguments); *launches receives the number of launches made.
 bool describe_matvec_rows_shared(uint32_t type, int rows, int in_w, int out_w, int compute_units, nnhip_matvec_plan_info* info);
 hipError_t launch_matvec_rows_shared(Lane* lane, uint32_t type, const float* x, const void* w, const float* bias, float* y,
-                                     int rows, int in_w, int out_w);
+                                     int rows, int in_w, int out_w, int* launches);
 hipError_t launch_matvec_mfma_wide_table(Lane* lane, uint32_t type, int in_w, int inputs, const MfmaTableEntry* device_entries,
                                          int entries, int total_tiles, bool runs);
 // Geometry of one matrix-core launch of a batch (`form` 1: operand A in registers, 2: the wide form, 3: the wide form

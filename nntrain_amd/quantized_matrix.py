@@ -28,7 +28,7 @@ PREFILL_MIN_ROWS = 16
 
 
 class HipQuantizedMatrix:
-    def __init__(self, payload, ggml_type: int, output_width: int, input_width: int):
+    def __init__(self, payload, ggml_type: int, output_width: int, input_width: int, inference_matmul_prefill: bool = False):
         if payload is None:
             raise TypeError("payload is null")
         if ggml_type not in BLOCK_ELEMS:
@@ -49,6 +49,9 @@ class HipQuantizedMatrix:
         self.ggml_type = ggml_type
         self.output_width = output_width
         self.input_width = input_width
+        # Matrix takes inferenceXmxPrefill from the execution options (Qwen35QuantizedModel.cs:252); off unless asked for
+        # (Qwen35ExecutionOptions.InferenceXmxPrefill, Qwen35ExecutionOptions.cs:50), because that route rounds to bfloat16.
+        self.inference_matmul_prefill = bool(inference_matmul_prefill)
         self._lane: HipExecutionLane | None = None
         self._device_payload: HipBuffer | None = None
 
@@ -73,6 +76,7 @@ class HipQuantizedMatrix:
         self.ggml_type = ggml_type
         self.output_width = output_width
         self.input_width = input_width
+        self.inference_matmul_prefill = False
         self._lane = lane
         self._device_payload = buffer
         return self
@@ -125,15 +129,19 @@ class HipQuantizedMatrix:
         self._payload = None
 
     def uses_prefill(self, rows: int) -> bool:
-        """Whether forward() sends `rows` input rows to the matrix-core mat-mul: rows >= 16 as in Matrix.Forward
-        (Qwen35QuantizedModel.cs:1249), when the rows are whole 256-weight blocks; the mat-vec kernels otherwise."""
-        return rows >= PREFILL_MIN_ROWS and self.input_width % 256 == 0
+        """Whether forward() sends `rows` input rows to the bfloat16 matrix-core mat-mul: only when the matrix was
+        given inference_matmul_prefill (the reference's opt-in InferenceXmxPrefill), for rows >= 16 as in Matrix.Forward
+        (Qwen35QuantizedModel.cs:1249) and rows of whole 256-weight blocks; the FP32-grade mat-vec kernels otherwise."""
+        return self.inference_matmul_prefill and rows >= PREFILL_MIN_ROWS and self.input_width % 256 == 0
 
     def forward(self, lane: HipExecutionLane, x: HipBuffer, bias: HipBuffer | None, rows: int = 1,
                 out: HipBuffer | None = None) -> HipBuffer:
         """y[rows, out] = bias + x[rows, in] . W^T on the device; x is FP32.  The caller disposes the result.
-        rows >= 16 go to the bf16 matrix-core mat-mul (the activations are rounded to bfloat16 on the device), fewer
-        rows to the dequantization-fused mat-vec, as Matrix.Forward routes them (Qwen35QuantizedModel.cs:1249-1369)."""
+        Every row count goes to the dequantization-fused mat-vec (FP32 accumulation, 1e-5 of the float64 product; up to
+        four input rows share a pass over the weights on the large matrices).  With inference_matmul_prefill set, rows
+        >= 16 go to the bfloat16 matrix-core mat-mul instead (activations and weights rounded to bfloat16 once: 2e-3),
+        the counterpart of the reference's opt-in XMX prefill (Qwen35QuantizedModel.cs:1249-1317), whose own bound is
+        5e-5 because it splits its operands into two f16 parts; this route does not."""
         if rows < 1:
             raise ValueError("rows must be positive.")
         if x.nbytes < 4 * rows * self.input_width:

@@ -135,15 +135,15 @@ def test_matvec_plan_keeps_a_ring_turn_inside_the_result_buffer():
                         (22, (256, 17408))):
         for in_w in widths:
             for out_w in (1, 2, 63, 300, 1000, 5000, 200_000, 1_000_000):
-                for rows in (1, 2, 3, 4, 7, 16):
+                for rows in (1, 2, 3, 4, 7, 16, 37):
                     assert lib.nnhip_matvec_plan(typ, rows, in_w, out_w, 256, byref(info)) == 0, (typ, in_w, out_w, rows)
                     if info.kernel == 2:
                         # several input rows of a K-quant / IQ2_S / Q8_0 matrix on the matrix cores: 16-row tiles, four rows
-                        # a pass (Q8_0 from three rows on: two stay with its row-tiled kernel)
-                        assert (3 if typ == 8 else 2) <= rows <= 16 and typ in (8, 12, 13, 14, 22) and rows * -(-out_w // 16) >= 2048
+                        # a pass and sixteen a launch (Q8_0 from three rows on: two stay with its row-tiled kernel)
+                        assert (3 if typ == 8 else 2) <= rows and typ in (8, 12, 13, 14, 22) and rows * -(-out_w // 16) >= 2048
                         assert typ != 8 or in_w in (1024, 5376)         # (21504-wide planes of four rows do not fit LDS)
                         assert info.rows_per_step == 16 and info.row_tile == min(rows, 4) and info.threads % 128 == 0
-                        assert info.steps == -(-out_w // 16) * -(-rows // 4) and info.groups == min(info.steps, 256)
+                        assert info.steps == -(-out_w // 16) * -(-min(rows, 16) // 4) and info.groups == min(info.steps, 256)
                         assert info.dynamic_lds_bytes + 8192 <= 160 * 1024
                         seen_tiles.add((typ, "matrix core"))
                         continue
