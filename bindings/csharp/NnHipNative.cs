@@ -24,7 +24,7 @@ internal static unsafe partial class NnHipNative
     [StructLayout(LayoutKind.Sequential)]
     internal struct LaneCounters
     {
-        internal uint StructSize; internal uint Reserved; internal ulong H2DBytes; internal ulong D2HBytes;
+        internal uint StructSize; internal uint DriverAllocations; internal ulong H2DBytes; internal ulong D2HBytes;
         internal ulong AllocatedBytes; internal ulong PeakAllocatedBytes; internal ulong KernelLaunches;
     }
 

@@ -85,7 +85,8 @@ typedef struct nnhip_error_info {
 /* Lane byte counters, the quantities ArcExecutionLane exposes (ArcExecutionLane.cs:71-91). */
 typedef struct nnhip_lane_counters {
     uint32_t struct_size;
-    uint32_t reserved;
+    uint32_t driver_allocations;   /* device and pinned-host allocations the library has asked the driver for on behalf of
+                                    * the lane (buffers, descriptor tables, staging): a call that must not allocate leaves it alone */
     uint64_t h2d_bytes;
     uint64_t d2h_bytes;
     uint64_t allocated_bytes;
@@ -204,7 +205,10 @@ NNHIP_API int nnhip_quant_matvec(void* lane, uint32_t ggml_type, const float* x,
 /* The launch shape nnhip_quant_matvec picks for a call, computed on the host without touching a device: for
  * reporting (the reference prints its kernel choice per matrix, Qwen35QuantizedModel.cs:1335-1344 selects by rows) and
  * for checking the kernels' capacity assumptions in tests.  compute_units is the workgroup count to plan for (256 on
- * MI355X).  Returns NNHIP_ERR_TOO_LARGE when no kernel takes the shape.  struct_size = sizeof of the structure. */
+ * MI355X).  The plan assumes a weight pointer on a 16-byte boundary, which every buffer from nnhip_alloc has: a call
+ * whose w is less aligned (a view at an odd offset into a stacked payload) always takes the row-step kernels, also where
+ * this reports NNHIP_MATVEC_KERNEL_MATRIX_CORE.  Returns NNHIP_ERR_TOO_LARGE when no kernel takes the shape.
+ * struct_size = sizeof of the structure. */
 enum { NNHIP_MATVEC_KERNEL_ROWSTEP = 0, NNHIP_MATVEC_KERNEL_Q8_0_ODD_BLOCKS = 1,
        NNHIP_MATVEC_KERNEL_MATRIX_CORE = 2 /* 16-row tiles over the workgroups, up to four input rows per pass */ };
 
@@ -282,12 +286,15 @@ NNHIP_API int nnhip_matvec_batch_plan(const nnhip_matvec_desc* descs, int count,
 /* nnhip_quant_matvec_batch for callers that cannot allocate device memory: code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same arguments and bit-identical
  * results to nnhip_quant_matvec_batch; the descriptor table lives in a fixed array inside the library's device image (80 bytes per mat-vec row,
- * NNHIP_STATIC_BATCH_MAX_ENTRIES rows = 80 KiB, held on every device the library is loaded on until the process ends)
+ * NNHIP_STATIC_BATCH_MAX_ENTRIES rows = 80 KiB per lane slice, held on every device the library is loaded on until the process ends)
  * instead of lane-owned memory, and the call makes no device or host allocation.  A batch with more rows (the sum of
- * `rows` over the descriptors) is rejected with NNHIP_ERR_TOO_LARGE.  All lanes of a device share the one array: a
- * call rewrites the entries it uses, and calls whose work overlaps on one device (two lanes, or one lane whose earlier
- * static batch is still running while another lane issues one) race on it - serialise them.  Asynchronous. */
+ * `rows` over the descriptors) is rejected with NNHIP_ERR_TOO_LARGE.  The array has NNHIP_STATIC_BATCH_LANES slices of that
+ * size (640 KiB in all); a lane takes one when it is created, in rotation per device, so up to that many lanes of a
+ * device issue static batches (and replay graphs that contain them) independently of each other.  A call rewrites the
+ * entries it uses; lanes that share a slice (the ninth lane of a device shares the first one's) must not have static
+ * batches in flight at the same time.  Asynchronous. */
 #define NNHIP_STATIC_BATCH_MAX_ENTRIES 1024
+#define NNHIP_STATIC_BATCH_LANES 8
 NNHIP_API int nnhip_quant_matvec_batch_static(void* lane, const nnhip_matvec_desc* descs, int count);
 
 /* Prefill: y[r, o] = bias[o] + sum_k x[r, k] * w[o, k] with x given as bfloat16 bit patterns [rows, in_w];

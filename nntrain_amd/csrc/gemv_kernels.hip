@@ -1197,7 +1197,8 @@ hipError_t write_table(Lane* lane, void* device_table, const BatchEntry* entries
 // array so that the entry point never allocates.  Every device holds its own copy at its own address; host code uses
 // the address hipGetSymbolAddress returns for the current device (kept in the lane), never the array's name.
 constexpr int kStaticTableEntries = NNHIP_STATIC_BATCH_MAX_ENTRIES;
-static __device__ __align__(256) unsigned char scratch[kStaticTableEntries * sizeof(BatchEntry)];
+constexpr int kStaticLaneSlices = NNHIP_STATIC_BATCH_LANES;
+static __device__ __align__(256) unsigned char scratch[kStaticLaneSlices * kStaticTableEntries * sizeof(BatchEntry)];
 
 void shape_of(uint32_t type, int* max_t, int* depth)
 {
@@ -1560,6 +1561,7 @@ hipError_t launch_matvec_batch(Lane* lane, const nnhip_matvec_desc* descs, int c
             const size_t want = bytes * 2 < 65536 ? 65536 : bytes * 2;
             void* fresh = nullptr;
             const hipError_t e = hipMalloc(&fresh, want);
+            if (e == hipSuccess) ++lane->counters.driver_allocations;
             if (e != hipSuccess) return e;
             if (lane->batch_table) lane->retired_tables.push_back(lane->batch_table);
             lane->batch_table = fresh;
@@ -1656,9 +1658,14 @@ bool matvec_rows_share_pass(uint32_t type, int rows, int in_w, int out_w, const 
            static_cast<long>(rows) * ((out_w + 15) / 16) >= kMfmaBatchMinTiles && matvec_mfma_wide_geometry(type, in_w, out_w, w, 4);
 }
 
-hipError_t static_table_address(void** address)
+// The slice of the fixed workspace for the `serial`-th lane created on the current device.
+hipError_t static_table_address(void** address, unsigned serial)
 {
-    return hipGetSymbolAddress(address, HIP_SYMBOL(scratch));
+    void* base = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&base, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !base) return e != hipSuccess ? e : hipErrorInvalidSymbol;
+    *address = static_cast<unsigned char*>(base) + static_cast<size_t>(serial % kStaticLaneSlices) * kStaticTableEntries * sizeof(BatchEntry);
+    return hipSuccess;
 }
 
 // As launch_matvec_batch with the table in the device's fixed workspace: no device or host allocation on this path.

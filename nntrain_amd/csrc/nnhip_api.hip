@@ -71,6 +71,7 @@ int staged_upload(nnhip::Lane* lane, void* dptr, size_t offset, size_t bytes, Fi
     for (int i = 0; i < 2; ++i) {
         if (!lane->staging[i]) {
             const hipError_t e = hipHostMalloc(&lane->staging[i], kStagingBytes, hipHostMallocDefault);
+            if (e == hipSuccess) ++lane->counters.driver_allocations;
             if (e != hipSuccess) {
                 lane->staging[i] = nullptr;
                 return hip_fail(e, NNHIP_OP_UPLOAD, lane->device, "pinned staging buffer");
@@ -252,8 +253,10 @@ int nnhip_lane_create(int device, void** out)
         delete lane;
         return hip_fail(e, NNHIP_OP_LANE_CREATE, device, "hipStreamCreateWithFlags");
     }
-    // the fixed batch workspace: every device has its own copy of the array, at its own address
-    e = static_table_address(&lane->static_table);
+    // the fixed batch workspace: every device has its own copy of the array, at its own address; the lanes of a device
+    // take its slices in rotation
+    static std::atomic<unsigned> lane_serial[64];
+    e = static_table_address(&lane->static_table, lane_serial[device & 63].fetch_add(1u));
     if (e != hipSuccess || !lane->static_table) {
         (void)hipStreamDestroy(lane->stream);
         delete lane;
@@ -262,6 +265,7 @@ int nnhip_lane_create(int device, void** out)
     // the descriptor table of batched launches starts with room for 819 mat-vec rows, so that small batches (and calls
     // with a few input rows, which use it) never have to grow it inside a graph capture
     e = hipMalloc(&lane->batch_table, 65536);
+    if (e == hipSuccess) ++lane->counters.driver_allocations;
     if (e != hipSuccess) {
         (void)hipStreamDestroy(lane->stream);
         delete lane;
@@ -340,6 +344,8 @@ int nnhip_alloc(void* handle, size_t bytes, void** dptr)
             }
         }
         if (e != hipSuccess) return hip_fail(e, NNHIP_OP_ALLOC, lane->device, "hipMalloc");
+        std::lock_guard<std::mutex> guard(lane->mutex);
+        ++lane->counters.driver_allocations;
     }
     std::lock_guard<std::mutex> guard(lane->mutex);
     lane->buffers.emplace(p, Lane::Block{bytes, capacity});

@@ -137,7 +137,7 @@ bool describe_matvec_mfma_launch(uint32_t type, int in_w, int form, bool runs, n
 int plan_matvec_batch(const nnhip_matvec_desc* descs, int count, int compute_units, nnhip_batch_launch_info* launches,
                       int capacity);
 // The fixed device workspace: its address on the current device, and the batched launch that uses it.
-hipError_t static_table_address(void** address);
+hipError_t static_table_address(void** address, unsigned serial);
 hipError_t launch_matvec_batch_static(Lane* lane, const nnhip_matvec_desc* descs, int count);
 hipError_t launch_matmul_bf16(Lane* lane, uint32_t type, const uint16_t* x, const void* w, const float* bias,
                               float* y, int rows, int in_w, int out_w);

@@ -225,7 +225,8 @@ class HipExecutionLane:
         c = native.LaneCounters()
         check(self._lib.nnhip_lane_get_counters(self._handle, byref(c), ctypes.sizeof(c)), "counters")
         return {"h2d_bytes": c.h2d_bytes, "d2h_bytes": c.d2h_bytes, "allocated_bytes": c.allocated_bytes,
-                "peak_allocated_bytes": c.peak_allocated_bytes, "kernel_launches": c.kernel_launches}
+                "peak_allocated_bytes": c.peak_allocated_bytes, "kernel_launches": c.kernel_launches,
+                "driver_allocations": c.driver_allocations}
 
     # ---- timing / replay ----
     def event(self) -> HipEvent:

@@ -34,7 +34,7 @@ class ErrorInfo(Structure):
 
 
 class LaneCounters(Structure):
-    _fields_ = [("struct_size", c_uint32), ("reserved", c_uint32), ("h2d_bytes", c_uint64), ("d2h_bytes", c_uint64),
+    _fields_ = [("struct_size", c_uint32), ("driver_allocations", c_uint32), ("h2d_bytes", c_uint64), ("d2h_bytes", c_uint64),
                 ("allocated_bytes", c_uint64), ("peak_allocated_bytes", c_uint64), ("kernel_launches", c_uint64)]
 
 

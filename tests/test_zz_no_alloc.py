@@ -74,7 +74,9 @@ def test_static_workspace_batch_matches_the_allocating_entry_point():
             check(lib.nnhip_quant_matvec_batch_static(h, _descs(items, "y_new"), len(items)), "quant_matvec_batch_static")
             lane.synchronize()
             after = lane.counters()
-            for key in ("h2d_bytes", "d2h_bytes", "allocated_bytes", "peak_allocated_bytes"):
+            # driver_allocations counts every device or pinned-host allocation the library makes for the lane (buffers,
+            # descriptor tables, staging): the static entry point must leave it alone
+            for key in ("h2d_bytes", "d2h_bytes", "allocated_bytes", "peak_allocated_bytes", "driver_allocations"):
                 assert after[key] == before[key], key
             _compare(lane, items)
         # exactly the workspace's capacity is accepted, one row more is refused and nothing is enqueued
@@ -113,8 +115,10 @@ def test_static_workspace_batch_inside_a_captured_graph():
         other = _batch(lane, [(GGML_Q6_K, 256, 31, 1)], seed=700)
         check(lib.nnhip_quant_matvec_batch(h, _descs(items, "y_ref"), len(items)), "quant_matvec_batch")
         lane.synchronize()
+        before = lane.counters()["driver_allocations"]
         lane.graph_begin()
         check(lib.nnhip_quant_matvec_batch_static(h, _descs(items, "y_new"), len(items)), "quant_matvec_batch_static")
+        assert lane.counters()["driver_allocations"] == before
         graph = lane.graph_end()
         for _ in range(3):
             for it in items:
@@ -127,3 +131,25 @@ def test_static_workspace_batch_inside_a_captured_graph():
                 n = it["rows"] * it["out_w"]
                 assert np.array_equal(_bits(lane.read(it["y_ref"])[:n]), _bits(lane.read(it["y_new"])[:n]))
         lane.graph_destroy(graph)
+
+
+def test_two_lanes_of_a_device_use_their_own_slices_of_the_workspace():
+    """Each lane takes one slice of the device's fixed workspace at creation, so two lanes may run this entry point at
+    the same time: both are left unsynchronized here while the other one enqueues."""
+    with HipExecutionLane(0) as one, HipExecutionLane(0) as two:
+        a = _batch(one, [(GGML_Q8_0, 5376, 3000, 1), (GGML_Q4_K, 5120, 2600, 1), (GGML_Q6_K, 1024, 130, 3)], seed=800)
+        b = _batch(two, [(GGML_Q5_K, 2560, 2100, 1), (GGML_Q8_0, 512, 64, 2), (GGML_IQ2_S, 2048, 400, 1)], seed=900)
+        for lane, items in ((one, a), (two, b)):
+            for it in items:
+                for key in ("y_ref", "y_new"):
+                    lane.fill_u32(it[key], NAN_BITS, it["rows"] * it["out_w"] + 2)
+            check(lane._lib.nnhip_quant_matvec_batch(lane._handle, _descs(items, "y_ref"), len(items)), "quant_matvec_batch")
+            lane.synchronize()
+        for _ in range(8):
+            for lane, items in ((one, a), (two, b)):
+                check(lane._lib.nnhip_quant_matvec_batch_static(lane._handle, _descs(items, "y_new"), len(items)),
+                      "quant_matvec_batch_static")
+        one.synchronize()
+        two.synchronize()
+        _compare(one, a)
+        _compare(two, b)
