@@ -594,6 +594,15 @@ void matvec_rowstep_kernel(MatvecArgs a, const float* __restrict__ bias)
     // (a vector gathered by heads is shorter than in_w: its pieces are fetched through the index map further down)
     float4 xv0 = PRE != kPreHeadGather && tid < pieces ? xg[tid] : make_float4(0.f, 0.f, 0.f, 0.f);
     float4 xv1 = PRE != kPreHeadGather && tid + T < pieces ? xg[tid + T] : make_float4(0.f, 0.f, 0.f, 0.f);
+    // A plain launch with a long input (a down projection) asks for up to six more pieces per lane here, ahead of the
+    // weights: whatever is requested after the weight prefetch comes back behind it, one round trip per piece.
+    constexpr int kMorePieces = PRE == kPreNone && MR == 1 ? 6 : 0;
+    float4 xw[kMorePieces ? kMorePieces : 1];
+    if constexpr (kMorePieces > 0) {
+#pragma unroll
+        for (int i = 0; i < kMorePieces; ++i)
+            xw[i] = tid + (2 + i) * T < pieces ? xg[tid + (2 + i) * T] : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
     const float4* x2g = reinterpret_cast<const float4*>(a.x2);
     const float4* gg = reinterpret_cast<const float4*>(a.gamma);
     const bool second = PRE == kPreSiluMultiply || (PRE == kPreRmsNorm && a.x2 != nullptr);
@@ -705,7 +714,14 @@ void matvec_rowstep_kernel(MatvecArgs a, const float* __restrict__ bias)
     } else {
         if (tid < pieces) xstage[tid + (tid >> 4)] = xv0;
         if (tid + T < pieces) xstage[tid + T + ((tid + T) >> 4)] = xv1;
-        for (int L = tid + 2 * T; L < pieces; L += T) xstage[L + (L >> 4)] = xg[L];
+        if constexpr (kMorePieces > 0) {
+#pragma unroll
+            for (int i = 0; i < kMorePieces; ++i) {
+                const int L = tid + (2 + i) * T;
+                if (L < pieces) xstage[L + (L >> 4)] = xw[i];
+            }
+        }
+        for (int L = tid + (2 + kMorePieces) * T; L < pieces; L += T) xstage[L + (L >> 4)] = xg[L];
         // the other input rows of the tile, each in a staging area of its own (rows past the last one: zeros)
         for (int m = 1; m < MR; ++m) {
             float4* xm = xstage + m * kChunkPieces * upr;
