@@ -73,6 +73,30 @@ def q8_bytes(out_w, in_w):
     return out_w * (in_w // 32) * 34
 
 
+def stats(samples, digits=4):
+    """Mean, standard deviation (n - 1), extremes and count of a list of timings, beside the median the text quotes."""
+    a = np.asarray(samples, dtype=np.float64)
+    return {"median": round(float(np.median(a)), digits), "mean": round(float(a.mean()), digits),
+            "sd": round(float(a.std(ddof=1)) if a.size > 1 else 0.0, digits), "min": round(float(a.min()), digits),
+            "max": round(float(a.max()), digits), "n": int(a.size)}
+
+
+def timed_each(lane, fn, reps):
+    """Device time of each of `reps` consecutive calls of fn (an event after every call), and of all of them."""
+    events = [lane.event() for _ in range(reps + 1)]
+    lane.synchronize()
+    events[0].record()
+    for i in range(reps):
+        fn()
+        events[i + 1].record()
+    lane.synchronize()
+    each = [lane.elapsed_ms(events[i], events[i + 1]) for i in range(reps)]
+    total = lane.elapsed_ms(events[0], events[reps])
+    for e in events:
+        e.dispose()
+    return each, total
+
+
 def timed(lane, fn, reps):
     """Device time of `reps` calls of fn on the lane's stream (HIP events), plus host wall time around a sync."""
     e0, e1 = lane.event(), lane.event()
@@ -174,6 +198,9 @@ def run_decode27b(args, lane, nn, oracle):
     launches_before = lane.counters()["kernel_launches"]
     ms, wall = timed(lane, token, args.steps)
     launches_per_token = (lane.counters()["kernel_launches"] - launches_before) // args.steps
+    # the same number of steps once more with an event after every step, for their spread (the figure above stays the
+    # one pair of events around all of them)
+    each_ms, _ = timed_each(lane, token, args.steps)
     rel = max(rel, verify("after timing"))
     # The dominant kernel on its own: in batch mode the library launches once per row length; the 5376-wide matrices
     # (q, k, v, gate, up of every layer and the head: 68 % of the bytes) are one launch of the matrix-core mat-vec.
@@ -190,9 +217,9 @@ def run_decode27b(args, lane, nn, oracle):
             sub_batch()
         lane.synchronize()
         before = lane.counters()["kernel_launches"]
-        sub_ms, _ = timed(lane, sub_batch, args.steps)
+        sub_each, sub_ms = timed_each(lane, sub_batch, args.steps)
         assert (lane.counters()["kernel_launches"] - before) == args.steps, "the 5376-wide group is one launch"
-        dominant = {"ms": sub_ms / args.steps, "bytes": sub_bytes}
+        dominant = {"ms": sub_ms / args.steps, "bytes": sub_bytes, "stats": stats(sub_each)}
         log(f"[decode27b] dominant launch (311 matrices of row length 5376, {sub_bytes} bytes): "
             f"{dominant['ms']:.3f} ms, {sub_bytes / dominant['ms'] / 1e6:.0f} GB/s")
         token()             # (the full table again, for whatever runs next)
@@ -223,7 +250,7 @@ def run_decode27b(args, lane, nn, oracle):
         log(f"[decode27b] HBM traffic per launch of the dominant kernel from counters: {traffic} bytes ({detail})")
     if dominant:
         roof_gbs, roof_bytes = dominant["bytes"] / dominant["ms"] / 1e6, dominant["bytes"]
-        roof_extra = {"launch_ms": round(dominant["ms"], 4),
+        roof_extra = {"launch_ms": round(dominant["ms"], 4), "launch_ms_stats": dominant["stats"],
                       "note": "the launch for the 311 matrices of row length 5376 (68 % of the token's bytes), timed on its own "
                               "with HIP events; the 4096- and 21504-wide groups are launches of <Q8_0Task, 1, 5, 1, false>",
                       "whole_token_gb_per_s": round(gbs, 1)}
@@ -232,6 +259,7 @@ def run_decode27b(args, lane, nn, oracle):
     return {
         "metric": "27B-shape Q8_0 decode tokens/sec", "value": round(tok_s, 2), "unit": "tokens/s",
         "ms_per_step": round(ms_per_step, 4),
+        "ms_per_step_stats": stats(each_ms),
         "config": {"workload": "decode27b: 435 Q8_0 mat-vecs of a Gemma-3-27B-shaped stack (BASELINE configs[2]), "
                                "28,695,625,728 weight bytes/token resident in HBM, batch 1, fp32 activations",
                    "launch": args.mode, "launches_per_token": n_launch},
@@ -298,9 +326,10 @@ GEMV_CONFIGS = [
     ("cfg2 Q5_K 17408x5120", "GGML_Q5_K", 5120, 17408, 2002, 2000),
     ("cfg2 Q6_K 17408x5120", "GGML_Q6_K", 5120, 17408, 2003, 2000),
     ("cfg5 IQ2_S 5120x17408", "GGML_IQ2_S", 17408, 5120, 5001, 5002),
+    ("cfg5 shape in IQ3_S 5120x17408", "GGML_IQ3_S", 17408, 5120, 5003, 5002),
     ("down projection Q4_K 5120x17408", "GGML_Q4_K", 17408, 5120, 2004, 2005),
 ]
-MATRIX_CORE_TYPES = ("GGML_Q8_0", "GGML_Q4_K", "GGML_Q5_K", "GGML_Q6_K", "GGML_IQ2_S")
+MATRIX_CORE_TYPES = ("GGML_Q8_0", "GGML_Q4_K", "GGML_Q5_K", "GGML_Q6_K", "GGML_IQ2_S", "GGML_IQ3_S")
 
 
 def run_gemv(args, lane, nn, oracle):
@@ -345,6 +374,11 @@ def run_gemv(args, lane, nn, oracle):
             ms, _ = timed(lane, lambda: [launch(w0) for _ in ring], 1)
             samples_same.append(ms * 1e3 / len(ring))
         us_ring, us_same = float(np.median(samples_ring)), float(np.median(samples_same))
+        launch(w0)
+        rel_after = oracle.rel_l2(lane.read(y, np.float32), ref[0])
+        if not rel_after <= 1e-5:
+            raise SystemExit(f"{name}: parity failure after timing, rel-L2 {rel_after:.3e}")
+        rel = max(rel, rel_after)
         algo = nbytes + 4 * in_w + 4 * out_w
         # sustained rate: the same mat-vec over every rotated copy as ONE batched launch (no per-launch start-up)
         ys = [lane.allocate(out_w) for _ in ring]
@@ -366,7 +400,13 @@ def run_gemv(args, lane, nn, oracle):
             ms, _ = timed(lane, lambda: nn.native.check(lib.nnhip_quant_matvec_batch(h, descs, len(ring)), "batch"), 1)
             samples_batch.append(ms * 1e3 / len(ring))
         us_batch = float(np.median(samples_batch))
-        out[name] = {"us_per_launch_hbm": round(us_ring, 2), "gb_per_s_hbm": round(algo / us_ring / 1e3, 1),
+        rel_batch_after = oracle.rel_l2(lane.read(ys[0], np.float32), ref[0])
+        if not rel_batch_after <= 1e-5:
+            raise SystemExit(f"{name}: batched launch parity failure after timing, rel-L2 {rel_batch_after:.3e}")
+        rel_batch = max(rel_batch, rel_batch_after)
+        out[name] = {"us_per_launch_hbm": round(us_ring, 2), "us_per_launch_hbm_stats": stats(samples_ring, 2),
+                     "us_per_launch_cache_resident_stats": stats(samples_same, 2),
+                     "sustained_us_per_matvec_batched_stats": stats(samples_batch, 2), "gb_per_s_hbm": round(algo / us_ring / 1e3, 1),
                      "frac_of_8TBs": round(algo / us_ring / 1e3 / HBM_PEAK_GBS, 4),
                      "us_per_launch_cache_resident": round(us_same, 2),
                      "sustained_us_per_matvec_batched": round(us_batch, 2),
@@ -382,7 +422,7 @@ def run_gemv(args, lane, nn, oracle):
             out[name]["cpu_baseline"] = {"gb_per_s": round(nbytes / per_pass / 1e9, 2), "us_per_matvec": round(per_pass * 1e6, 1),
                                          "cores": threads, "one_thread_gb_per_s": round(nbytes / one / 1e9, 3), "kind": "port"}
             log(f"[gemv] {name}: CPU port {nbytes / per_pass / 1e9:.1f} GB/s on {threads} threads, {nbytes / one / 1e9:.2f} GB/s on one")
-        if tname == "GGML_Q8_0" or name.startswith("cfg2"):
+        if tname == "GGML_Q8_0" or name.startswith("cfg2") or name.startswith("cfg5") or name.startswith("down"):
             # several input rows in one call (weights rotated as above): microseconds per call, up to four rows sharing a
             # pass over the weights (Q8_0 with two rows: its row-tiled lane-per-unit kernel; otherwise the matrix cores)
             per_rows = {}
@@ -401,10 +441,17 @@ def run_gemv(args, lane, nn, oracle):
                     ms, _ = timed(lane, lambda: [launch_rows(w) for w in ring], 1)
                     samples.append(ms * 1e3 / len(ring))
                 per_rows[f"rows={rows}"] = round(float(np.median(samples)), 2)
+                per_rows[f"rows={rows} stats"] = stats(samples, 2)
+                # every input row against the oracle, after the timing
+                xr_host = synth.activations(rows, in_w, xseed + rows)
+                ref_rows, _ = oracle.linear_f64(typ, payload, xr_host, None, rows, in_w, out_w)
+                rel_rows = oracle.rel_l2(lane.read(yr, np.float32).reshape(rows, out_w), ref_rows)
+                if not rel_rows <= 1e-5:
+                    raise SystemExit(f"{name}: parity failure with {rows} input rows, rel-L2 {rel_rows:.3e}")
                 xr.dispose()
                 yr.dispose()
             out[name]["us_per_call_with_several_input_rows"] = per_rows
-            log(f"[gemv] {name}: " + ", ".join(f"{k} {v:.1f} us" for k, v in per_rows.items()))
+            log(f"[gemv] {name}: " + ", ".join(f"{k} {v:.1f} us" for k, v in per_rows.items() if not k.endswith("stats")))
         for b in ring + ys + [x, y]:
             b.dispose()
     return out
@@ -478,6 +525,7 @@ def run_ffn(args, lane, nn, oracle):
         state["cur"], state["nxt"] = nxt, cur
 
     results = {}
+    spread = {}
     finals = {}
     for name, fn in (("unfused_6_launches", layer_unfused), ("fused_3_launches", layer_fused), ("fused_2_launches_gate_up_stacked", None)):
         lane.write(hid, hidden0)
@@ -494,10 +542,11 @@ def run_ffn(args, lane, nn, oracle):
             ms, _ = timed(lane, lambda: [fn(w) for w in seq], 1)
             samples.append(ms * 1e3 / layers)
         results[name] = round(float(np.median(samples)), 2)
+        spread[name] = stats(samples, 2)
     if any(not np.array_equal(finals["unfused_6_launches"], f) for f in finals.values()):
         raise SystemExit("ffn: fused and unfused layers differ bitwise")
     wbytes = sum(b.nbytes for b in base.values())
-    out = {"config": "Q4_K, hidden 5120, feed-forward 17408, 8 layers' weights rotated", "us_per_layer": results,
+    out = {"config": "Q4_K, hidden 5120, feed-forward 17408, 8 layers' weights rotated", "us_per_layer": results, "us_per_layer_stats": spread,
            "weight_bytes_per_layer": wbytes,
            "gb_per_s_fused": round(wbytes / results["fused_2_launches_gate_up_stacked"] / 1e3, 1),
            "gb_per_s_unfused": round(wbytes / results["unfused_6_launches"] / 1e3, 1), "bitwise_equal": True}
@@ -590,24 +639,29 @@ def run_decode_loop(args, lane, nn, oracle):
         if not np.array_equal(lane.read(fused.forward_token(t), np.uint32, count=vocab), r):
             raise SystemExit("decode loop: fused and unfused logits differ bitwise")
 
-    def per_token(dec):
+    def per_token(dec, label):
         samples = []
         for _ in range(5):
             ms, _ = timed(lane, lambda: [dec.forward_token(t) for t in tokens], 1)
             samples.append(ms / len(tokens))
+        spread[label] = stats(samples)
         return float(np.median(samples))
 
-    ms_plain, ms_fused = per_token(plain), per_token(fused)
+    spread = {}
+    ms_plain, ms_fused = per_token(plain, "one_launch_per_operation"), per_token(fused, "fused_launches")
     fused.capture_graph()
     if not np.array_equal(lane.read(fused.forward_token(tokens[0]), np.uint32, count=vocab), ref[0]):
         raise SystemExit("decode loop: graph replay differs bitwise")
-    ms_graph = per_token(fused)
+    ms_graph = per_token(fused, "fused_launches_hip_graph")
+    if not np.array_equal(lane.read(fused.forward_token(tokens[1]), np.uint32, count=vocab), ref[1]):
+        raise SystemExit("decode loop: graph replay differs bitwise after timing")
     toks, timing = fused.generate(5, 16)
     out = {"config": f"llama-style, {layers} layers, hidden {emb}, feed-forward {ffn}, heads {heads}/{kv} x {hw}, vocabulary {vocab}, Q4_K",
            "gguf_file_bytes": file_bytes, "load_seconds_file_to_hbm": round(load_s, 2),
            "weight_bytes_streamed_per_token": weight_bytes,
            "ms_per_token": {"one_launch_per_operation": round(ms_plain, 4), "fused_launches": round(ms_fused, 4),
                             "fused_launches_hip_graph": round(ms_graph, 4)},
+           "ms_per_token_stats": spread,
            "launches_per_token": {"one_launch_per_operation": 1 + 12 * layers + 2, "fused_launches": 1 + 4 * layers + 1},
            "gb_per_s_fused_graph": round(weight_bytes / ms_graph / 1e6, 1),
            "frac_of_8TBs_fused_graph": round(weight_bytes / ms_graph / 1e6 / HBM_PEAK_GBS, 4),
@@ -674,19 +728,24 @@ def run_decode27b_chained(args, lane, nn, oracle):
     if not (np.all(np.isfinite(logits)) and rel <= 1e-4):       # the norm is recomputed here in float64: looser than 1e-5
         raise SystemExit(f"decode27b_chained: parity failure, rel-L2 {rel:.3e}")
 
-    def per_token(dec):
+    def per_token(dec, label):
         samples = []
         for _ in range(5):
             ms, _ = timed(lane, lambda: [dec.forward_token(t) for t in tokens], 1)
             samples.append(ms / len(tokens))
+        spread[label] = stats(samples)
         return float(np.median(samples))
 
-    ms_plain, ms_fused = per_token(plain), per_token(fused)
+    spread = {}
+    ms_plain, ms_fused = per_token(plain, "one_launch_per_operation"), per_token(fused, "fused_launches")
     fused.capture_graph()
     if not np.array_equal(lane.read(fused.forward_token(tokens[1]), np.uint32, count=vocab),
                           lane.read(plain.forward_token(tokens[1]), np.uint32, count=vocab)):
         raise SystemExit("decode27b_chained: graph replay differs bitwise")
-    ms_graph = per_token(fused)
+    ms_graph = per_token(fused, "fused_launches_hip_graph")
+    if not np.array_equal(lane.read(fused.forward_token(tokens[2]), np.uint32, count=vocab),
+                          lane.read(plain.forward_token(tokens[2]), np.uint32, count=vocab)):
+        raise SystemExit("decode27b_chained: graph replay differs bitwise after timing")
 
     def entry(ms):
         return {"ms_per_token": round(ms, 4), "tokens_per_s": round(1e3 / ms, 2), "gb_per_s": round(weight_bytes / ms / 1e6, 1),
@@ -697,7 +756,7 @@ def run_decode27b_chained(args, lane, nn, oracle):
                      "embedding), Q8_0, first-token attention (no cache)",
            "weight_bytes_streamed_per_token": weight_bytes,
            "one_launch_per_operation": entry(ms_plain), "fused_launches": entry(ms_fused),
-           "fused_launches_hip_graph": entry(ms_graph),
+           "fused_launches_hip_graph": entry(ms_graph), "ms_per_token_stats": spread,
            "launches_per_token": {"one_launch_per_operation": 1 + 12 * layers + 2, "fused_launches": 1 + 4 * layers + 1},
            "rel_l2_head_vs_f64_oracle": rel, "bitwise_equal": True}
     log(f"[decode27b_chained] per token: {ms_plain:.3f} ms one launch per operation, {ms_fused:.3f} ms fused, "
@@ -741,21 +800,28 @@ def _prefill_of(lane, nn, oracle, typ, tname, ms_list):
             mat.dispose()
             return None
         lane.synchronize()
-        rows = min(m, 16)
-        got = lane.read(y, np.float32, rows * out_w)
-        ref, _ = oracle.linear_f64(typ, payload, xb[:rows], None, rows, in_w, out_w, x_is_bf16=True)
-        rel = oracle.rel_l2(got, ref)
-        if not rel <= 2e-3:
-            raise SystemExit(f"prefill {tname} M={m}: parity failure, rel-L2 {rel:.3e} > 2e-3")
+        # every 16th input row (every 64th at M = 2048: at most 32 rows) against the float64 oracle, before and after timing
+        picked = np.arange(0, m, max(16, m // 32))
+        ref, _ = oracle.linear_f64(typ, payload, np.ascontiguousarray(xb[picked]), None, len(picked), in_w, out_w, x_is_bf16=True)
+
+        def check(tag):
+            got = lane.read(y, np.float32, m * out_w).reshape(m, out_w)[picked]
+            r = oracle.rel_l2(got, ref)
+            if not (np.all(np.isfinite(got)) and r <= 2e-3):
+                raise SystemExit(f"prefill {tname} M={m}: parity failure {tag}, rel-L2 {r:.3e} > 2e-3")
+            return r
+
+        rel = check("before timing")
         samples = []
         for _ in range(7):
             ms, _ = timed(lane, lambda: mat.forward_bf16(lane, x, None, m, out=y), 3)
             samples.append(ms / 3)
         ms = float(np.median(samples))
+        rel = max(rel, check("after timing"))
         flops = 2.0 * m * in_w * out_w
-        out[f"M={m}"] = {"ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 1),
+        out[f"M={m}"] = {"ms": round(ms, 4), "ms_stats": stats(samples), "tflops": round(flops / ms / 1e9, 1),
                          "mfma_util_vs_2500_TFLOPs_bf16": round(flops / ms / 1e9 / BF16_PEAK_TFLOPS, 4),
-                         "rel_l2_vs_f64_oracle": rel}
+                         "rel_l2_vs_f64_oracle": rel, "rows_checked": int(len(picked))}
         log(f"[prefill] {tname} M={m}: {ms:.3f} ms, {flops / ms / 1e9:.0f} TFLOP/s, rel-L2 {rel:.2e}")
         x.dispose()
         y.dispose()
@@ -857,6 +923,8 @@ def main():
         "vs_baseline": None, "dtype": "f32", "data": "synthetic", "config": res["config"],
         "roofline": res["roofline"], "cpu_baseline": res["cpu_baseline"],
     }
+    if "ms_per_step_stats" in res:
+        line["ms_per_step_stats"] = res["ms_per_step_stats"]
     if "parity" in res:
         line["parity"] = res["parity"]
     if also:

@@ -195,10 +195,12 @@ NNHIP_API int nnhip_dequantize(void* lane, uint32_t ggml_type, const void* w, fl
  * (NNtrain.Core/Tensors/Tensor.QwenQuantized.cs:29-96) for decode (rows == 1) and small row counts.  Each
  * output row of y is computed with the same operation order whatever `rows` is, so rows > 1 equals stacked
  * rows == 1 calls bit for bit (Qwen35InferencePrefillLinearTests.cs:64-77), except for calls with two or more input rows
- * on Q4_K / Q5_K / Q6_K / IQ2_S matrices (three or more on Q8_0) with rows x ceil(out_w / 16) >= 2048: those take the
- * matrix-core path described at nnhip_quant_matvec_batch (up to four input rows per pass over the weights, sixteen per
- * launch; a row's bits do not depend on the rows it travels with; 1e-6 from the rows == 1 result).  bias may be null
- * (zero).  Asynchronous. */
+ * on Q4_K / Q5_K / Q6_K / IQ2_S / IQ3_S matrices (three or more on Q8_0) with rows x ceil(out_w / 16) >= 2048, or >= 768
+ * from three rows on (Q8_0: 2048): those take the matrix-core path described at nnhip_quant_matvec_batch (up to four
+ * input rows per pass over the weights, sixteen per launch; a row's bits do not depend on the rows it travels with; 1e-6
+ * from the rows == 1 result).  Rows too long for four sets of activation planes in LDS (in_w above about 8700) get one
+ * matrix-core pass per input row instead, four rows a launch, from rows x ceil(out_w / 16) >= 1024 on (IQ3_S 768, IQ2_S
+ * 512; never Q8_0).  nnhip_matvec_plan reports which form a call takes.  bias may be null (zero).  Asynchronous. */
 NNHIP_API int nnhip_quant_matvec(void* lane, uint32_t ggml_type, const float* x, const void* w, const float* bias,
                                  float* y, int rows, int in_w, int out_w);
 
@@ -234,8 +236,8 @@ NNHIP_API int nnhip_matvec_plan(uint32_t ggml_type, int rows, int in_w, int out_
 /* `count` independent mat-vecs enqueued as one unit of work (a single launch per group of equal type), for the
  * per-token projection sets that ForwardTokenDevice issues back to back (Qwen35QuantizedModel.cs:451-513).
  * `descs` is a host array, read before the call returns.  Results are identical to `count` nnhip_quant_matvec calls,
- * with one exception: Q8_0, Q4_K, Q5_K, Q6_K and IQ2_S matrices of one in_w (at least 1024, a multiple of 256; an even
- * number of 256-blocks for Q6_K and IQ2_S) whose 16-row tiles, counted once per input row, add up to 2048 or more
+ * with one exception: Q8_0, Q4_K, Q5_K, Q6_K, IQ2_S and IQ3_S matrices of one in_w (at least 1024, a multiple of 256; an
+ * even number of 256-blocks for Q6_K, IQ2_S and IQ3_S) whose 16-row tiles, counted once per input row, add up to 2048 or more
  * within a call are multiplied on the matrix cores with the activations in 32-bit fixed point; descriptors with two or
  * more input rows (Q8_0: three or more) share one pass over the weights between up to four rows there.
  * Those results are deterministic,

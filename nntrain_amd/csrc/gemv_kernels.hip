@@ -1264,8 +1264,8 @@ bool describe_rowstep(int rows, int in_w, int out_w, int compute_units, nnhip_ma
 bool describe_matvec(uint32_t type, int rows, int in_w, int out_w, int compute_units, nnhip_matvec_plan_info* info)
 {
     // (the plan is made without the weight pointer: the matrix-core path also needs it 16-byte aligned)
-    if (matvec_rows_share_pass(type, rows, in_w, out_w, nullptr))
-        return describe_matvec_rows_shared(type, rows, in_w, out_w, compute_units, info);
+    if (const int per_pass = matvec_rows_per_pass(type, rows, in_w, out_w, nullptr))
+        return describe_matvec_rows_shared(type, rows, in_w, out_w, per_pass, compute_units, info);
     if (type == NNHIP_TYPE_Q8_0 && ((in_w / 32) & 1)) {
         info->kernel = NNHIP_MATVEC_KERNEL_Q8_0_ODD_BLOCKS;
         info->threads = 256;
@@ -1395,6 +1395,16 @@ constexpr int kBatchGroupsMax = kBatchTypes + 8;      // row-step groups plus ma
 // 8.4 us per matrix against 10.8 us in a launch of twenty, 12.4 against 13.8 in a launch of two) but takes longer to
 // start, so a single matrix of that size stays with the row-step kernel.
 constexpr int kMfmaBatchMinTiles = 2048;
+// The same floor for a single call whose three or more input rows share a pass over a super-block format (measured:
+// 4096 x 5120 with rows = 3 / 4, 13 / 14 us against 15 - 18 / 19 - 23 us for one row-step pass per row; 1024 x 5120 breaks
+// even at eight rows, 2048 x 2048 between four and six).  Q8_0 keeps the higher floor: its row-step kernel already
+// multiplies four input rows per pass.
+constexpr int kSharedPassMinTiles = 768;
+// ... and for a pass per input row on the matrix cores (rows too long for shared passes): the codebook formats, whose
+// row-step kernels are bound by their arithmetic, from fewer tiles on than the K-quants (measured on 5120 x 17408, us per
+// call with 2 / 3 / 4 input rows: IQ2_S 34 / 38 / 45 against 38 / 55 / 70 with row-step passes, IQ3_S 45 / 52 / 62 against
+// 41 / 59 / 75, Q4_K 35 at four rows against 36 at three).
+constexpr int kSeparatePassMinTiles = 1024, kSeparatePassMinTilesIQ3S = 768, kSeparatePassMinTilesIQ2S = 512;
 const uint32_t kBatchTypeOrder[kBatchTypes] = {NNHIP_TYPE_Q8_0, NNHIP_TYPE_Q4_K, NNHIP_TYPE_Q5_K, NNHIP_TYPE_Q6_K,
                                                NNHIP_TYPE_IQ3_S, NNHIP_TYPE_IQ2_S, NNHIP_TYPE_BF16};
 
@@ -1668,10 +1678,22 @@ int plan_matvec_batch(const nnhip_matvec_desc* descs, int count, int compute_uni
     return n;
 }
 
-bool matvec_rows_share_pass(uint32_t type, int rows, int in_w, int out_w, const void* w)
+int matvec_rows_per_pass(uint32_t type, int rows, int in_w, int out_w, const void* w)
 {
-    return rows >= shared_pass_min_rows(type) &&
-           static_cast<long>(rows) * ((out_w + 15) / 16) >= kMfmaBatchMinTiles && matvec_mfma_wide_geometry(type, in_w, out_w, w, 4);
+    if (rows < shared_pass_min_rows(type)) return 0;
+    const long work = static_cast<long>(rows) * ((out_w + 15) / 16);
+    const long floor = rows >= 3 && type != NNHIP_TYPE_Q8_0 ? kSharedPassMinTiles : kMfmaBatchMinTiles;
+    if (work >= floor && matvec_mfma_wide_geometry(type, in_w, out_w, w, 4)) return 4;
+    // Rows too long for four sets of activation planes in LDS (more than about 8700 values): the super-block formats
+    // still stream faster on the matrix cores, one pass per input row (Q8_0's row-step kernel multiplies four input rows
+    // per pass and stays).
+    const long separate_floor = type == NNHIP_TYPE_IQ2_S ? kSeparatePassMinTilesIQ2S
+                              : type == NNHIP_TYPE_IQ3_S ? kSeparatePassMinTilesIQ3S : kSeparatePassMinTiles;
+    if (type != NNHIP_TYPE_Q8_0 && work >= separate_floor &&
+        !matvec_mfma_wide_geometry(type, in_w, out_w, w, 4) &&
+        matvec_mfma_wide_geometry(type, in_w, out_w, w, 1))
+        return 1;
+    return 0;
 }
 
 // The slice of the fixed workspace for the `serial`-th lane created on the current device.

@@ -1,5 +1,5 @@
 // Decode mat-vec on the matrix cores: for the super-block formats whose unpacking is too much vector-ALU work for the
-// lane-per-unit kernels (gemv_kernels.hip), Q4_K, Q5_K, Q6_K and IQ2_S, and for Q8_0, whose signed bytes are operand B
+// lane-per-unit kernels (gemv_kernels.hip), Q4_K, Q5_K, Q6_K, IQ2_S and IQ3_S, and for Q8_0, whose signed bytes are operand B
 // as they lie in memory and whose lane-per-unit kernel is held back by its cached, strided loads.  Used for the large
 // groups of a batched launch and for calls with 2 - 16 input rows, where it streams faster than the row-step kernels;
 // it takes longer to start, so single-row launches stay with those.  Two kernels share the tasks of the formats: matvec_mfma_kernel keeps
@@ -780,6 +780,124 @@ struct IQ2STask {
     {
         // every lookup of the task is requested before the first result is used (the scheduling barrier keeps the
         // compiler from folding the reads back into a chain of eight round trips to LDS)
+        Looked lk;
+        float unused = 0.0f;
+        lookup(r, 0, tables, lk);
+        __builtin_amdgcn_sched_barrier(0);
+        finish(r, lk, xs, accq, unused);
+    }
+};
+
+// IQ3_S (NNtrain.Arc/Kernels/qwen35_iq.cl:421-429): 110 bytes = d (fp16), 64 index bytes, 8 bytes of ninth index bits (one
+// per four weights), 32 sign bytes, 4 bytes of 4-bit scales (one per 32 weights).  Four weights are one entry of a
+// 512-entry codebook of magnitude bytes (odd, 1 .. 15); w = d * (1 + 2 scale) * magnitude * sign.  Two entries are the
+// eight bytes of operand B that a lane supplies for one MFMA, and one sign byte covers them: the signs go in as for IQ2_S
+// (IQ2STask), with the same 256-entry selector table.  Both tables sit in LDS (4 KB).  Quarter P = 32-weight groups 2P and
+// 2P + 1: sixteen index bytes, two bytes of ninth bits, eight sign bytes, one scale byte.  Blocks are 2-byte aligned and
+// fetched like IQ2_S blocks, from the dword boundary at or below their start, into seven pieces.
+__device__ const uint32_t g_iq3s_grid_mv[512] = { NNHIP_IQ3S_GRID_VALUES };
+
+struct IQ3STask {
+    static constexpr int kBlockBytes = 110;
+    static constexpr bool kStacked = false;
+    static constexpr int kPieces = 7;
+    static constexpr int kSumRun = 32;
+    static constexpr int kWideM = 2;
+    static constexpr int kWideLpw = 4;
+    static constexpr int kSharedM = 1;
+    static constexpr int kSharedLpw = 2;
+    static constexpr bool kNeedsSums = false;         // no minimum or offset
+    static constexpr bool kTightStage = true;
+    static constexpr int kGridBytes = 2048;
+    static constexpr int kTableBytes = kGridBytes + 2048;     // the codebook and 256 selector pairs
+    static constexpr int kLdsTableBytes = kTableBytes;
+    using X = XSet<1>;
+    struct Raw { uint32_t q[4], s[2], tops, scales, d; };
+
+    static __device__ __forceinline__ uint32_t piece_src(uint32_t q, bool odd) { return 16u * q - (odd ? 2u : 0u); }
+
+    static __device__ __forceinline__ void init_tables(uint8_t* t, int tid, int threads)
+    {
+        for (int i = tid; i < 512; i += threads) reinterpret_cast<uint32_t*>(t)[i] = g_iq3s_grid_mv[i];
+        for (int i = tid; i < 256; i += threads) {
+            const uint32_t lo = ((static_cast<uint32_t>(i) & 15u) * 0x00204081u) & 0x01010101u;
+            const uint32_t hi = ((static_cast<uint32_t>(i) >> 4) * 0x00204081u) & 0x01010101u;
+            reinterpret_cast<u32x2*>(t + kGridBytes)[i] = u32x2{0x03020100u + (lo << 2), 0x03020100u + (hi << 2)};
+        }
+    }
+
+    static __device__ __forceinline__ void load_x(X& xs, const uint8_t* plane, const float*, int b, int quarter, const uint8_t* zeros)
+    {
+        const uint8_t* src = zeros ? zeros : plane + 256 * b + 64 * quarter;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) xs.a[u] = lds128(src + 16 * u);
+        xs.sx[0] = 0.0f;
+    }
+
+    static __device__ __forceinline__ Raw load(const uint8_t* blk, int quarter, bool odd)
+    {
+        // the block's byte k is at blk + k (+ 2 when odd); its index bytes 16P .. 16P + 15 start at 2 + 16P, the sign bytes
+        // 8P .. 8P + 7 at 74 + 8P: on dword boundaries in an odd block, two bytes past one in an even block
+        const uint32_t* qi = reinterpret_cast<const uint32_t*>(blk + 16 * quarter + (odd ? 4 : 0));
+        const uint32_t* si = reinterpret_cast<const uint32_t*>(blk + 8 * quarter + (odd ? 76 : 72));
+        const uint32_t sh = odd ? 0u : 2u;
+        const uint8_t* b0 = blk + (odd ? 2 : 0);
+        Raw r;
+        const uint32_t q0 = qi[0], q1 = qi[1], q2 = qi[2], q3 = qi[3], q4 = qi[4];
+        const uint32_t s0 = si[0], s1 = si[1], s2 = si[2];
+        r.q[0] = __builtin_amdgcn_alignbyte(q1, q0, sh);
+        r.q[1] = __builtin_amdgcn_alignbyte(q2, q1, sh);
+        r.q[2] = __builtin_amdgcn_alignbyte(q3, q2, sh);
+        r.q[3] = __builtin_amdgcn_alignbyte(q4, q3, sh);
+        r.s[0] = __builtin_amdgcn_alignbyte(s1, s0, sh);
+        r.s[1] = __builtin_amdgcn_alignbyte(s2, s1, sh);
+        r.tops = *reinterpret_cast<const uint16_t*>(b0 + 66 + 2 * quarter);
+        r.scales = b0[106 + quarter];
+        r.d = *reinterpret_cast<const uint16_t*>(b0);
+        return r;
+    }
+
+    // As for IQ2_S: the lookups of a task are made once and every input row of a shared pass multiplies with them.
+    static constexpr bool kSplitLookups = true;
+    struct Looked { u32x2 mag[8], sel[8]; };
+
+    static __device__ __forceinline__ void lookup(const Raw& r, int, const uint8_t* tables, Looked& lk)
+    {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            // MFMA e of the quarter: codebook entries 2e and 2e + 1 (index byte + its ninth bit, bit 2e / 2e + 1 of the tops)
+            const uint32_t word = r.q[e >> 1];
+            const uint32_t i0 = ((word >> (16 * (e & 1))) & 0xffu) | (((r.tops >> (2 * e)) & 1u) << 8);
+            const uint32_t i1 = ((word >> (16 * (e & 1) + 8)) & 0xffu) | (((r.tops >> (2 * e + 1)) & 1u) << 8);
+            const uint32_t sign = (r.s[e >> 2] >> (8 * (e & 3))) & 0xffu;
+            lk.mag[e] = u32x2{*reinterpret_cast<const uint32_t*>(tables + 4u * i0), *reinterpret_cast<const uint32_t*>(tables + 4u * i1)};
+            lk.sel[e] = *reinterpret_cast<const u32x2*>(tables + kGridBytes + 8u * sign);
+        }
+    }
+
+    static __device__ __forceinline__ void finish(const Raw& r, const Looked& lk, const X& xs, float& accq, float&)
+    {
+        i32x4 acc[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            // -m per byte = (m ^ 0xff) + 1: no carry leaves a byte because no magnitude is zero
+            const uint32_t neg0 = (lk.mag[e][0] ^ 0xffffffffu) + 0x01010101u, neg1 = (lk.mag[e][1] ^ 0xffffffffu) + 0x01010101u;
+            const uint32_t b0 = __builtin_amdgcn_perm(neg0, lk.mag[e][0], lk.sel[e][0]);
+            const uint32_t b1 = __builtin_amdgcn_perm(neg1, lk.mag[e][1], lk.sel[e][1]);
+            const u32x4 av = xs.a[e >> 1];
+            acc[e >> 2] = mfma_i8(av[2 * (e & 1)], av[2 * (e & 1) + 1], b0, b1, acc[e >> 2]);
+        }
+        // the plane sums of the two scale groups are added up with the integer factors 1 + 2 s (|sum| < 2 * 31 * 32 * 15 *
+        // 128 < 2^22: exact) and recombined once
+        const int f0 = static_cast<int>(1u + 2u * (r.scales & 15u)), f1 = static_cast<int>(1u + 2u * ((r.scales >> 4) & 15u));
+        i32x4 total;
+#pragma unroll
+        for (int p = 0; p < 4; ++p) total[p] = mul24(f0, acc[0][p]) + mul24(f1, acc[1][p]);
+        accq = fmaf(half_bits_to_float(r.d), recombine_wide(total), accq);
+    }
+
+    static __device__ __forceinline__ void run(const Raw& r, const X& xs, int, const uint8_t* tables, float& accq, float&)
+    {
         Looked lk;
         float unused = 0.0f;
         lookup(r, 0, tables, lk);
@@ -1659,6 +1777,7 @@ int block_bytes_of(uint32_t type)
     case NNHIP_TYPE_Q5_K: return Q5KTask::kBlockBytes;
     case NNHIP_TYPE_Q6_K: return Q6KTask::kBlockBytes;
     case NNHIP_TYPE_IQ2_S: return IQ2STask::kBlockBytes;
+    case NNHIP_TYPE_IQ3_S: return IQ3STask::kBlockBytes;
     case NNHIP_TYPE_Q8_0: return Q8_0Task::kBlockBytes;
     default: return 0;
     }
@@ -1671,6 +1790,7 @@ int block_pieces_of(uint32_t type)
     case NNHIP_TYPE_Q5_K: return Q5KTask::kPieces;
     case NNHIP_TYPE_Q6_K: return Q6KTask::kPieces;
     case NNHIP_TYPE_IQ2_S: return IQ2STask::kPieces;
+    case NNHIP_TYPE_IQ3_S: return IQ3STask::kPieces;
     case NNHIP_TYPE_Q8_0: return Q8_0Task::kPieces;
     default: return 0;
     }
@@ -1694,6 +1814,11 @@ WideTraits wide_traits(uint32_t type, bool shared)
     case NNHIP_TYPE_IQ2_S: {
         WideTraits t = wide_traits_of<IQ2STask>(shared);
         t.table_bytes = IQ2STask::kTableBytes;
+        return t;
+    }
+    case NNHIP_TYPE_IQ3_S: {
+        WideTraits t = wide_traits_of<IQ3STask>(shared);
+        t.table_bytes = IQ3STask::kTableBytes;
         return t;
     }
     case NNHIP_TYPE_Q8_0: {
@@ -1833,7 +1958,7 @@ MfmaTableEntry matvec_mfma_entry(uint32_t type, const float* x, const void* w, c
 
 bool matvec_mfma_geometry(uint32_t type, int in_w, int out_w, const void* w, MfmaPlan* plan)
 {
-    if (type == NNHIP_TYPE_IQ2_S || type == NNHIP_TYPE_Q8_0) return false;       // (these have the wide form only)
+    if (type == NNHIP_TYPE_IQ2_S || type == NNHIP_TYPE_IQ3_S || type == NNHIP_TYPE_Q8_0) return false;       // (these have the wide form only)
 
     if (!entry_ok(type, in_w, out_w, w)) return false;
     MfmaGeom g;
@@ -1889,6 +2014,7 @@ hipError_t launch_wide_args(Lane* lane, uint32_t type, int in_w, int inputs, Wid
     case NNHIP_TYPE_Q5_K: return launch_wide<Q5KTask>(lane, a, inputs);
     case NNHIP_TYPE_Q6_K: return launch_wide<Q6KTask>(lane, a, inputs);
     case NNHIP_TYPE_IQ2_S: return launch_wide<IQ2STask>(lane, a, inputs);
+    case NNHIP_TYPE_IQ3_S: return launch_wide<IQ3STask>(lane, a, inputs);
     case NNHIP_TYPE_Q8_0:
         if (inputs != 1) return launch_wide_of<Q8_0Task, 4>(lane, a);
         a.chunked = 1;          // (always for Q8_0, whose batches are whole models; measured level with every-G-th at one vector)
@@ -1909,17 +2035,19 @@ hipError_t launch_wide_args(Lane* lane, uint32_t type, int in_w, int inputs, Wid
 
 }  // namespace
 
-bool describe_matvec_rows_shared(uint32_t type, int rows, int in_w, int out_w, int compute_units, nnhip_matvec_plan_info* info)
+bool describe_matvec_rows_shared(uint32_t type, int rows, int in_w, int out_w, int per_pass, int compute_units,
+                                 nnhip_matvec_plan_info* info)
 {
     WideGeom g;
-    if (!plan_wide(type, in_w, 4, &g)) return false;
-    const int tiles = (out_w + kTileRows - 1) / kTileRows * (((rows < 16 ? rows : 16) + 3) / 4);      // (of one launch: sixteen input rows)
+    if (!plan_wide(type, in_w, per_pass, &g)) return false;
+    const int launch_rows = rows < 4 * per_pass ? rows : 4 * per_pass;                 // (four table entries per launch)
+    const int tiles = (out_w + kTileRows - 1) / kTileRows * ((launch_rows + per_pass - 1) / per_pass);
     info->kernel = NNHIP_MATVEC_KERNEL_MATRIX_CORE;
     info->threads = 64 * g.waves;
     info->rows_per_step = kTileRows;
     info->steps = tiles;
     info->groups = tiles < compute_units ? tiles : compute_units;
-    info->row_tile = rows < 4 ? rows : 4;
+    info->row_tile = rows < per_pass ? rows : per_pass;
     info->ring_depth = 2;                                   // stage buffers
     info->result_buffer_floats = 2 * 4 * kMaxWaves * kTileRows;
     info->dynamic_lds_bytes = static_cast<int32_t>(g.lds_bytes);
@@ -1960,25 +2088,27 @@ hipError_t launch_matvec_mfma_wide_table(Lane* lane, uint32_t type, int in_w, in
 }
 
 hipError_t launch_matvec_rows_shared(Lane* lane, uint32_t type, const float* x, const void* w, const float* bias, float* y,
-                                     int rows, int in_w, int out_w, int* launches)
+                                     int rows, int in_w, int out_w, int per_pass, int* launches)
 {
-    if (rows < 2) return hipErrorInvalidValue;
-    // sixteen input rows per launch (four table entries of four rows travel in the kernel arguments); a row's bits do not
+    if (rows < 2 || (per_pass != 1 && per_pass != 4)) return hipErrorInvalidValue;
+    // four table entries of `per_pass` input rows per launch (they travel in the kernel arguments); a row's bits do not
     // depend on the rows it shares a pass or a launch with
     *launches = 0;
-    for (int r0 = 0; r0 < rows; r0 += 16) {
-        const int n = rows - r0 < 16 ? rows - r0 : 16;
+    const int per_launch = 4 * per_pass;
+    for (int r0 = 0; r0 < rows; r0 += per_launch) {
+        const int n = rows - r0 < per_launch ? rows - r0 : per_launch;
         WideArgs a{};
         a.table = nullptr;
-        for (int r = r0; r < r0 + n; r += 4) {
+        for (int r = r0; r < r0 + n; r += per_pass) {
             MfmaTableEntry e = matvec_mfma_entry(type, x + static_cast<size_t>(r) * in_w, w, bias, y + static_cast<size_t>(r) * out_w,
                                                  in_w, out_w, a.total_tiles);
-            e.rows = r0 + n - r < 4 ? r0 + n - r : 4;
+            e.rows = r0 + n - r < per_pass ? r0 + n - r : per_pass;
             a.inline_entries[a.entries++] = e;
             a.total_tiles += e.tiles;
         }
-        a.chunked = a.entries >= 3 ? 1 : 0;         // (9 - 16 input rows: three or four groups of rows, each with planes of its own)
-        const hipError_t e = launch_wide_args(lane, type, in_w, 4, a);
+        // (three or four entries, each with planes of its own: runs of consecutive tiles, so that a workgroup converts few vectors)
+        a.chunked = a.entries >= 3 || per_pass == 1 ? 1 : 0;
+        const hipError_t e = launch_wide_args(lane, type, in_w, per_pass, a);
         if (e != hipSuccess) return e;
         ++*launches;
     }

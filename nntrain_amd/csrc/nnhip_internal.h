@@ -120,14 +120,16 @@ hipError_t launch_matvec_mfma_table(Lane* lane, uint32_t type, int in_w, const M
 // The wide form of the matrix-core mat-vec (activation planes in LDS): any in_w of at least four super-blocks, and
 // entries of up to four input rows that share a pass over the weights (`inputs` = 1: every entry has one row).
 bool matvec_mfma_wide_geometry(uint32_t type, int in_w, int out_w, const void* w, int inputs);
-// True when a single call with `rows` input rows is served by that form (as a one-descriptor batch) rather than by one
-// row-step pass per input row.
-bool matvec_rows_share_pass(uint32_t type, int rows, int in_w, int out_w, const void* w);
-// That call: two or more input rows, up to four per pass and sixteen per launch (the descriptors travel in the kernel
-// arguments); *launches receives the number of launches made.
-bool describe_matvec_rows_shared(uint32_t type, int rows, int in_w, int out_w, int compute_units, nnhip_matvec_plan_info* info);
+// Whether a single call with `rows` input rows is served by that form rather than by row-step passes: 0 (it is not), 4
+// (up to four input rows share a pass over the weights) or 1 (a pass per input row, for rows whose four sets of planes do
+// not fit LDS).
+int matvec_rows_per_pass(uint32_t type, int rows, int in_w, int out_w, const void* w);
+// That call: two or more input rows, `per_pass` of them per table entry and four entries per launch (the descriptors
+// travel in the kernel arguments); *launches receives the number of launches made.
+bool describe_matvec_rows_shared(uint32_t type, int rows, int in_w, int out_w, int per_pass, int compute_units,
+                                 nnhip_matvec_plan_info* info);
 hipError_t launch_matvec_rows_shared(Lane* lane, uint32_t type, const float* x, const void* w, const float* bias, float* y,
-                                     int rows, int in_w, int out_w, int* launches);
+                                     int rows, int in_w, int out_w, int per_pass, int* launches);
 hipError_t launch_matvec_mfma_wide_table(Lane* lane, uint32_t type, int in_w, int inputs, const MfmaTableEntry* device_entries,
                                          int entries, int total_tiles, bool runs);
 // Geometry of one matrix-core launch of a batch (`form` 1: operand A in registers, 2: the wide form, 3: the wide form

@@ -11,7 +11,7 @@ import numpy as np
 import pytest
 
 import oracle
-from nntrain_amd import GGML_IQ2_S, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_Q8_0, HipExecutionLane, HipQuantizedMatrix, synth
+from nntrain_amd import GGML_IQ2_S, GGML_IQ3_S, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_Q8_0, HipExecutionLane, HipQuantizedMatrix, synth
 from nntrain_amd.native import BatchLaunchInfo, MatvecDesc, check
 
 pytestmark = pytest.mark.gpu
@@ -589,7 +589,7 @@ def test_q8_0_model_sized_groups_on_the_matrix_cores(lane):
     lane.trim()
 
 
-@pytest.mark.parametrize("typ", [GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_IQ2_S])
+@pytest.mark.parametrize("typ", [GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_IQ2_S, GGML_IQ3_S])
 def test_matrix_core_groups_with_long_rows_and_shared_passes(lane, typ):
     """Rows that do not split into whole stages (17408 = 68 super-blocks, 3072 = 12, 1024 = 4) and descriptors with
     2 - 5 input rows (up to four share a pass over the weights) take the form of the matrix-core mat-vec that keeps the
@@ -638,12 +638,58 @@ def test_matrix_core_groups_with_long_rows_and_shared_passes(lane, typ):
     lane.trim()
 
 
-@pytest.mark.parametrize("typ", [GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_Q8_0, GGML_IQ2_S])
+@pytest.mark.parametrize("typ", [GGML_Q4_K, GGML_IQ2_S, GGML_IQ3_S])
+def test_long_rows_take_a_pass_per_input_row_on_the_matrix_cores(lane, typ):
+    """17408-wide rows: four sets of activation planes do not fit LDS, so a call with several input rows gets one pass per
+    row on the matrix cores (four rows a launch) once rows x tiles reach the format's floor, and row-step passes below
+    it.  Both bars against the oracle, guard elements, the plan reports the form, and a row's bits do not depend on the
+    rows it is issued with."""
+    from ctypes import byref, sizeof
+    from nntrain_amd import native
+    in_w, out_w = 17408, 5120
+    payload = synth.matrix(typ, out_w, in_w, seed=1300 + typ)
+    mat = HipQuantizedMatrix(payload, typ, out_w, in_w)
+    mat.device_payload(lane)
+    bias = np.random.default_rng(4).standard_normal(out_w).astype(np.float32)
+    bd = lane.upload_raw(bias)
+    x = synth.activations(6, in_w, seed=41)
+    x[1] *= 2e-3
+    x[4] *= 7e2
+    xd = lane.upload_raw(x)
+    info = native.MatvecPlanInfo(struct_size=sizeof(native.MatvecPlanInfo))
+    results = {}
+    for rows in (2, 4, 6):
+        assert lane._lib.nnhip_matvec_plan(typ, rows, in_w, out_w, 256, byref(info)) == 0
+        floor = {GGML_Q4_K: 1024, GGML_IQ3_S: 768, GGML_IQ2_S: 512}[typ]
+        assert (info.kernel == 2) == (rows * 320 >= floor), (rows, info.kernel)
+        if info.kernel == 2:
+            assert info.row_tile == 1 and info.steps == 320 * min(rows, 4)
+        yd = lane.allocate(rows * out_w + 2)
+        lane.fill_u32(yd, NAN_BITS, rows * out_w + 2)
+        mat.forward(lane, xd, bd, rows, out=yd)
+        lane.synchronize()
+        y = lane.read(yd)
+        assert np.isnan(y[-1]) and np.isnan(y[-2])
+        y = y[:-2].reshape(rows, out_w)
+        ref, asum = oracle.linear_f64(typ, payload, x[:rows], bias, rows, in_w, out_w)
+        assert oracle.rel_l2(y, ref) <= MATVEC_BAR
+        assert np.all(np.abs(y.astype(np.float64) - ref) <= 2e-6 + 3e-6 * asum)
+        results[rows] = (y, info.kernel)
+        yd.dispose()
+    assert results[4][1] == results[6][1] == 2
+    assert np.array_equal(_bits(results[6][0][:4]), _bits(results[4][0]))
+    for b in (xd, bd):
+        b.dispose()
+    mat.dispose()
+    lane.trim()
+
+
+@pytest.mark.parametrize("typ", [GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_Q8_0, GGML_IQ2_S, GGML_IQ3_S])
 def test_several_input_rows_share_a_pass_in_a_single_call(lane, typ):
     """nnhip_quant_matvec with 2 - 9 input rows (Q8_0: 3 - 9, two rows stay with its row-tiled kernel) on a matrix large
     enough for the matrix cores (rows x 16-row tiles >= 2048): up to four rows share a pass over the weights (Q4_K, Q5_K
-    and Q8_0 with the rows stacked in operand A, Q6_K one row after the other on the unpacked quants, IQ2_S one row after
-    the other on one set of codebook lookups).  Both bars against the oracle, the guard elements,
+    and Q8_0 with the rows stacked in operand A, Q6_K one row after the other on the unpacked quants, IQ2_S and IQ3_S one row
+    after the other on one set of codebook lookups).  Both bars against the oracle, the guard elements,
     no transfers, and a row's bits do not depend on the rows it travels with; the same call inside a captured graph
     gives the same bits on every replay."""
     in_w, out_w = 5120, 17408

@@ -44,7 +44,7 @@ def test_random_batches(lane):
         tname = str(rng.choice(list(TYPES)))
         typ = TYPES[tname]
         in_w = int(rng.choice(widths))
-        if tname in ("Q6_K", "IQ2_S") and (in_w // 256) % 2:
+        if tname in ("Q6_K", "IQ2_S", "IQ3_S") and (in_w // 256) % 2:
             in_w += 256
         n = int(rng.integers(1, 9))
         share = bool(rng.integers(0, 2))
@@ -85,7 +85,7 @@ def test_random_batches(lane):
 
 
 def test_random_single_calls_with_one_to_sixteen_rows(lane):
-    """nnhip_quant_matvec over heights on both sides of the 2048-tile rule and every row count up to sixteen (row-step
+    """nnhip_quant_matvec over heights on both sides of the tile-count rules and every row count up to sixteen (row-step
     passes, row-tiled passes and shared passes on the matrix cores), rows scaled differently from each other."""
     rng = np.random.default_rng(20240612)
     widths = [1024, 2048, 2560, 4096, 5120, 5376]
@@ -93,7 +93,7 @@ def test_random_single_calls_with_one_to_sixteen_rows(lane):
         tname = str(rng.choice(list(TYPES)))
         typ = TYPES[tname]
         in_w = int(rng.choice(widths))
-        if tname in ("Q6_K", "IQ2_S") and (in_w // 256) % 2:
+        if tname in ("Q6_K", "IQ2_S", "IQ3_S") and (in_w // 256) % 2:
             in_w += 256
         rows = int(rng.integers(1, 17))
         out_w = int(rng.choice([100, 2049, 4100, 9000, 17408, 33000]))

@@ -138,13 +138,23 @@ def test_matvec_plan_keeps_a_ring_turn_inside_the_result_buffer():
                 for rows in (1, 2, 3, 4, 7, 16, 37):
                     assert lib.nnhip_matvec_plan(typ, rows, in_w, out_w, 256, byref(info)) == 0, (typ, in_w, out_w, rows)
                     if info.kernel == 2:
-                        # several input rows of a K-quant / IQ2_S / Q8_0 matrix on the matrix cores: 16-row tiles, four rows
-                        # a pass and sixteen a launch (Q8_0 from three rows on: two stay with its row-tiled kernel)
-                        assert (3 if typ == 8 else 2) <= rows and typ in (8, 12, 13, 14, 22) and rows * -(-out_w // 16) >= 2048
+                        # several input rows of a K-quant / IQ2_S / IQ3_S / Q8_0 matrix on the matrix cores: 16-row tiles, four
+                        # rows a pass and sixteen a launch (Q8_0 from three rows on: two stay with its row-tiled kernel); the
+                        # floor is 2048 tiles x rows, 768 from three rows on except for Q8_0
+                        assert (3 if typ == 8 else 2) <= rows and typ in (8, 12, 13, 14, 21, 22)
                         assert typ != 8 or in_w in (1024, 5376)         # (21504-wide planes of four rows do not fit LDS)
-                        assert info.rows_per_step == 16 and info.row_tile == min(rows, 4) and info.threads % 128 == 0
-                        assert info.steps == -(-out_w // 16) * -(-min(rows, 16) // 4) and info.groups == min(info.steps, 256)
-                        assert info.dynamic_lds_bytes + 8192 <= 160 * 1024
+                        assert info.rows_per_step == 16 and info.threads % 128 == 0
+                        if in_w == 17408:
+                            # four sets of planes do not fit LDS: a pass per input row, four rows a launch, from 1024 tiles x rows (IQ2_S: 512)
+                            assert typ in (12, 22) and info.row_tile == 1 and rows * -(-out_w // 16) >= (512 if typ == 22 else 1024)
+                            assert info.steps == -(-out_w // 16) * min(rows, 4)
+                            assert info.dynamic_lds_bytes + 2048 + (10240 if typ == 22 else 0) <= 160 * 1024
+                        else:
+                            assert rows * -(-out_w // 16) >= (768 if rows >= 3 and typ != 8 else 2048)
+                            assert info.row_tile == min(rows, 4)
+                            assert info.steps == -(-out_w // 16) * -(-min(rows, 16) // 4)
+                            assert info.dynamic_lds_bytes + 8192 <= 160 * 1024
+                        assert info.groups == min(info.steps, 256)
                         seen_tiles.add((typ, "matrix core"))
                         continue
                     if info.kernel != 0:
@@ -156,7 +166,13 @@ def test_matvec_plan_keeps_a_ring_turn_inside_the_result_buffer():
                     assert info.steps == -(-out_w // info.rows_per_step) and info.groups == min(info.steps, 256)
                     assert info.dynamic_lds_bytes <= 140 * 1024
                     seen_tiles.add((typ, info.row_tile))
-    assert {(8, 1), (8, 2), (8, 4), (30, 4), (12, 1), (8, "matrix core"), (12, "matrix core"), (14, "matrix core")} <= seen_tiles
+    assert {(8, 1), (8, 2), (8, 4), (30, 4), (12, 1), (8, "matrix core"), (12, "matrix core"), (14, "matrix core"),
+            (21, "matrix core")} <= seen_tiles
+    # three rows reach the matrix cores at 768 tiles x rows, two rows at 2048
+    assert lib.nnhip_matvec_plan(12, 3, 5120, 4096, 256, byref(info)) == 0 and info.kernel == 2
+    assert lib.nnhip_matvec_plan(12, 3, 5120, 4000, 256, byref(info)) == 0 and info.kernel == 0
+    assert lib.nnhip_matvec_plan(12, 2, 5120, 4096, 256, byref(info)) == 0 and info.kernel == 0
+    assert lib.nnhip_matvec_plan(8, 4, 5376, 4096, 256, byref(info)) == 0 and info.kernel == 0
     assert lib.nnhip_matvec_plan(8, 1, 32 * 5, 19, 256, byref(info)) == 0 and info.kernel == 1   # odd block count
     assert lib.nnhip_matvec_plan(12, 1, 255, 19, 256, byref(info)) == 3
     assert lib.nnhip_matvec_plan(12, 1, 256 * 300, 19, 256, byref(info)) == 8
@@ -225,8 +241,8 @@ def test_batch_plan_threshold_counts_tiles_once_per_input_row():
     # a weight pointer the 16-byte loads cannot take keeps a Q6_K matrix with the row-step kernel (4-byte alignment is its rule)
     launches, n = _batch_plan(lib, [_desc(14, 1, 4096, 16 * 3000, w=0x100004)])
     assert n == 1 and launches[0].kernel == 0
-    # Q6_K and IQ2_S rows must hold an even number of 256-blocks for the matrix cores
-    for typ in (14, 22):
+    # Q6_K, IQ2_S and IQ3_S rows must hold an even number of 256-blocks for the matrix cores
+    for typ in (14, 22, 21):
         assert _batch_plan(lib, [_desc(typ, 1, 256 * 17, 16 * 3000)])[0][0].kernel == 0
         assert _batch_plan(lib, [_desc(typ, 1, 256 * 18, 16 * 3000)])[0][0].kernel == 2
     # below 1024 weights a row: never
@@ -245,14 +261,14 @@ def test_batch_plan_shared_passes_and_tile_order():
     two, _ = _batch_plan(lib, [_desc(12, 1, 5120, 17408)] * 10 + [_desc(12, 1, 5120, 17408, x=0x9000)] * 10)
     assert two[0].consecutive_runs == 0
     # input rows of a descriptor share passes four at a time; K-quants from two rows on, Q8_0 from three
-    for typ, rows, entries, per_pass in ((12, 2, 1, 2), (12, 4, 1, 4), (12, 6, 2, 4), (13, 9, 3, 4), (14, 16, 4, 4), (22, 5, 2, 4),
+    for typ, rows, entries, per_pass in ((12, 2, 1, 2), (12, 4, 1, 4), (12, 6, 2, 4), (13, 9, 3, 4), (14, 16, 4, 4), (22, 5, 2, 4), (21, 5, 2, 4),
                                          (8, 2, 2, 1), (8, 3, 1, 3), (8, 7, 2, 4)):
         in_w = 5376 if typ == 8 else 5120 if typ != 22 else 4096
         launches, n = _batch_plan(lib, [_desc(typ, rows, in_w, 17408)])
         l = launches[0]
         assert n == 1 and l.kernel == 2 and (l.entries, l.rows_per_pass) == (entries, per_pass), (typ, rows, l.entries, l.rows_per_pass)
         assert l.units == entries * 1088 and l.activations_in_lds == 1
-        assert l.dynamic_lds_bytes + (8192 if per_pass > 1 else 2048) + (2048 if typ == 22 else 0) <= 160 * 1024
+        assert l.dynamic_lds_bytes + (8192 if per_pass > 1 else 2048) + (2048 if typ in (21, 22) else 0) <= 160 * 1024
     # 21504-wide planes of four rows do not fit LDS: those rows get an entry each
     launches, _ = _batch_plan(lib, [_desc(8, 4, 21504, 16384)])
     assert launches[0].kernel == 2 and (launches[0].entries, launches[0].rows_per_pass) == (4, 1)
