@@ -772,11 +772,52 @@ def run_prefill(args, lane, nn, oracle):
     the kernel decodes (Q5_K, Q6_K, Q8_0, IQ2_S, IQ3_S) at M = 512 under "other_formats"."""
     out = _prefill_of(lane, nn, oracle, nn.GGML_Q4_K, "Q4_K", (128, 256, 512, 2048))
     if out is not None:
+        out["fp32_activations_three_products"] = _prefill_split(lane, nn, oracle, (128, 512))
         out["other_formats"] = {}
         for tname in ("Q5_K", "Q6_K", "Q8_0", "IQ2_S", "IQ3_S"):
             res = _prefill_of(lane, nn, oracle, getattr(nn, "GGML_" + tname), tname, (512,))
             if res is not None:
                 out["other_formats"][tname] = res["M=512"]
+    return out
+
+
+def _prefill_split(lane, nn, oracle, ms_list):
+    """The FP32-activation prefill at the reference's own accuracy gate (both operands as two bfloat16 parts, three
+    products, nnhip_quant_matmul_split) beside the one-product entry with FP32 activations (nnhip_quant_matmul) and the
+    FP32 mat-vec route the operator takes by default, on the Q4_K 17408 x 5120 matrix."""
+    from nntrain_amd import synth
+    typ, in_w, out_w = nn.GGML_Q4_K, 5120, 17408
+    payload = synth.matrix(typ, out_w, in_w, 2001)
+    out = {}
+    for m in ms_list:
+        x_host = synth.activations(m, in_w, 4100 + m)
+        x = lane.upload_raw(x_host)
+        y = lane.allocate(m * out_w)
+        picked = np.arange(0, m, max(16, m // 32))
+        ref, _ = oracle.linear_f64(typ, payload, np.ascontiguousarray(x_host[picked]), None, len(picked), in_w, out_w)
+        # (against the product of the FP32 activations: the one-product entry rounds them too, which the 2e-3 of the
+        # bfloat16-input figures above does not include)
+        entry = {}
+        for label, mode, bar in (("three_products", "split", 5e-5), ("one_product", True, 4e-3), ("mat_vec_passes", False, 1e-5)):
+            mat = nn.HipQuantizedMatrix(payload, typ, out_w, in_w, inference_matmul_prefill=mode)
+            mat.forward(lane, x, None, m, out=y)
+            lane.synchronize()
+            samples = []
+            for _ in range(5 if mode is not False else 3):
+                ms, _ = timed(lane, lambda: mat.forward(lane, x, None, m, out=y), 1)
+                samples.append(ms)
+            rel = oracle.rel_l2(lane.read(y, np.float32, m * out_w).reshape(m, out_w)[picked], ref)
+            if not rel <= bar:
+                raise SystemExit(f"prefill {label} M={m}: parity failure after timing, rel-L2 {rel:.3e} > {bar}")
+            entry[label] = {"ms": round(float(np.median(samples)), 4), "ms_stats": stats(samples), "rel_l2_vs_f64_oracle": rel, "bar": bar}
+            mat.dispose()
+        out[f"M={m}"] = entry
+        log(f"[prefill] FP32 activations M={m}: three products {entry['three_products']['ms']:.3f} ms (rel-L2 "
+            f"{entry['three_products']['rel_l2_vs_f64_oracle']:.1e}), one product {entry['one_product']['ms']:.3f} ms "
+            f"({entry['one_product']['rel_l2_vs_f64_oracle']:.1e}), mat-vec passes {entry['mat_vec_passes']['ms']:.3f} ms "
+            f"({entry['mat_vec_passes']['rel_l2_vs_f64_oracle']:.1e})")
+        x.dispose()
+        y.dispose()
     return out
 
 

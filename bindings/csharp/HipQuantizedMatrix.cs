@@ -40,6 +40,11 @@ public sealed class HipQuantizedMatrix : IDisposable
     /// the bfloat16 matrix-core mat-mul (2e-3 of the exact product) instead of the FP32-grade mat-vec (1e-5).</summary>
     public bool InferenceMatmulPrefill { get; init; }
 
+    /// <summary>With InferenceMatmulPrefill: both operands as two bfloat16 parts and three products (about 3e-6 of the
+    /// exact product, inside the 5e-5 the reference tests its XMX prefill at, Qwen35XmxPrefillLinearTests.cs:87-89) at
+    /// three times the cost.</summary>
+    public bool InferenceMatmulPrefillSplit { get; init; }
+
     /// <summary>Whether Forward sends this many input rows to the matrix-core mat-mul.</summary>
     public bool UsesPrefill(int rows) => InferenceMatmulPrefill && rows >= PrefillMinRows && InputWidth % 256 == 0;
 
@@ -61,8 +66,11 @@ public sealed class HipQuantizedMatrix : IDisposable
         HipBuffer output = lane.Allocate(checked(rows * OutputWidth));
         bool prefill = UsesPrefill(rows);
         int status = lane.Locked(h => prefill
-            ? NnHipNative.nnhip_quant_matmul(h, GgmlType, input.Pointer, encoded.Pointer, bias?.Pointer ?? 0, output.Pointer,
-                rows, InputWidth, OutputWidth)
+            ? (InferenceMatmulPrefillSplit
+                ? NnHipNative.nnhip_quant_matmul_split(h, GgmlType, input.Pointer, encoded.Pointer, bias?.Pointer ?? 0, output.Pointer,
+                    rows, InputWidth, OutputWidth)
+                : NnHipNative.nnhip_quant_matmul(h, GgmlType, input.Pointer, encoded.Pointer, bias?.Pointer ?? 0, output.Pointer,
+                    rows, InputWidth, OutputWidth))
             : NnHipNative.nnhip_quant_matvec(h, GgmlType, input.Pointer, encoded.Pointer, bias?.Pointer ?? 0, output.Pointer,
                 rows, InputWidth, OutputWidth));
         if (status != 0) { output.Dispose(); NnHipNative.Check(status, prefill ? "quantized mat-mul" : "quantized mat-vec"); }

@@ -94,6 +94,7 @@ internal static unsafe partial class NnHipNative
     [LibraryImport(Library)] internal static partial int nnhip_quant_matvec_batch_static(nint lane, MatvecDesc* descs, int count);
     [LibraryImport(Library)] internal static partial int nnhip_quant_matvec_fused(nint lane, FusedMatvecDesc* desc);
     [LibraryImport(Library)] internal static partial int nnhip_quant_matmul(nint lane, uint ggmlType, nint x, nint w, nint bias, nint y, int rows, int inW, int outW);
+    [LibraryImport(Library)] internal static partial int nnhip_quant_matmul_split(nint lane, uint ggmlType, nint x, nint w, nint bias, nint y, int rows, int inW, int outW);
     [LibraryImport(Library)] internal static partial int nnhip_quant_matmul_bf16(nint lane, uint ggmlType, nint xBf16, nint w, nint bias, nint y, int rows, int inW, int outW);
     [LibraryImport(Library)] internal static partial int nnhip_rms_norm(nint lane, nint input, nint weight, nint output, int rows, int width, int inputStride, float epsilon);
     [LibraryImport(Library)] internal static partial int nnhip_add_rms_norm(nint lane, nint destination, nint residual, nint weight, nint output, int rows, int width, int inputStride, float epsilon);

@@ -318,6 +318,19 @@ NNHIP_API int nnhip_quant_matmul_bf16(void* lane, uint32_t ggml_type, const uint
 NNHIP_API int nnhip_quant_matmul(void* lane, uint32_t ggml_type, const float* x, const void* w, const float* bias,
                                  float* y, int rows, int in_w, int out_w);
 
+/* Prefill at the accuracy the reference holds its XMX path to: that path splits the activations into a high and a low
+ * half-precision part and multiplies both (q35l_prefill_xmx_input_f16x2 and the two-panel loop of
+ * q35l_prefill_xmx_<format>_f16x2, NNtrain.Arc/Kernels/qwen35_prefill_xmx.cl:35-47,145-165), and is tested at relative
+ * L2 < 5e-5 against the FP32 mat-vec (NNtrain.Core.Tests/Qwen35XmxPrefillLinearTests.cs:87-89).  Here both operands are
+ * taken as hi + lo bfloat16 parts (hi = bf16(v), lo = bf16(v - hi): what is left is below 2^-17 of v) and three of the
+ * four products are formed on the matrix cores with FP32 accumulation, x_hi w_hi + x_lo w_hi + x_hi w_lo (the fourth is
+ * below 2^-16 of the first): three launches of the kernel of nnhip_quant_matmul_bf16 (two for unquantized bfloat16
+ * weights, which have no low part), the second and third adding to y.  Relative L2 against the exact product: about
+ * 3e-6.  Same type and width rules and the same staging-block behaviour as nnhip_quant_matmul (the block holds both
+ * parts).  Asynchronous. */
+NNHIP_API int nnhip_quant_matmul_split(void* lane, uint32_t ggml_type, const float* x, const void* w, const float* bias,
+                                       float* y, int rows, int in_w, int out_w);
+
 /* --- FP32 row operations around the mat-vec ------------------------------------------------------------------ */
 
 /* output[r, j] = input[r * input_stride + j] * inverse_r * weight[j], inverse_r = 1 / sqrt(sum_j x^2 / width + epsilon),

@@ -55,6 +55,7 @@ struct GemmArgs {
     int M, K, N;
     int cols;              // strip width actually used, <= 16 * CT
     int strips;            // ceil(N / cols)
+    int accumulate;        // 1: the products are added to what y holds (bias is not)
 };
 
 __device__ __forceinline__ uint32_t pack_bf16(float a, float b)
@@ -63,6 +64,20 @@ __device__ __forceinline__ uint32_t pack_bf16(float a, float b)
     typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
     bf16x2 v = {static_cast<__bf16>(a), static_cast<__bf16>(b)};
     return __builtin_bit_cast(uint32_t, v);
+}
+
+// Two weights as bf16: their values rounded (LO = false), or what that rounding left over, w - bf16(w), rounded in turn
+// (LO = true).  A launch with the second form supplies the low-order part of the weights to the three-product form of
+// the mat-mul (x_hi w_hi + x_lo w_hi + x_hi w_lo).
+template <bool LO>
+__device__ __forceinline__ uint32_t pack_w(float a, float b)
+{
+    if constexpr (LO) {
+        const uint32_t hi = pack_bf16(a, b);
+        a -= __uint_as_float(hi << 16);
+        b -= __uint_as_float(hi & 0xffff0000u);
+    }
+    return pack_bf16(a, b);
 }
 
 // 6-bit scale and min of sub-block g from the three dwords holding the 12 packed bytes (GgufQ4K.cs:51-60).
@@ -78,6 +93,7 @@ __device__ __forceinline__ void q4k_scale_min(uint32_t s0, uint32_t s1, uint32_t
     }
 }
 
+template <bool LO>
 __device__ __forceinline__ u32x4 q4k_decode8(uint32_t q_lo, uint32_t q_hi, float scale, float mnv)
 {
     // eight weights (d*sc)*q - dmin*m as one fused multiply-add each (the bf16 rounding that follows is 2^16 times
@@ -88,7 +104,7 @@ __device__ __forceinline__ u32x4 q4k_decode8(uint32_t q_lo, uint32_t q_hi, float
     const float w2 = fmaf(scale, ubyte2(q_lo), -mnv), w3 = fmaf(scale, ubyte3(q_lo), -mnv);
     const float w4 = fmaf(scale, ubyte0(q_hi), -mnv), w5 = fmaf(scale, ubyte1(q_hi), -mnv);
     const float w6 = fmaf(scale, ubyte2(q_hi), -mnv), w7 = fmaf(scale, ubyte3(q_hi), -mnv);
-    return u32x4{pack_bf16(w0, w1), pack_bf16(w2, w3), pack_bf16(w4, w5), pack_bf16(w6, w7)};
+    return u32x4{pack_w<LO>(w0, w1), pack_w<LO>(w2, w3), pack_w<LO>(w4, w5), pack_w<LO>(w6, w7)};
 }
 
 // A 64-byte LDS row holds four 16-byte k-groups.  Group g of row r sits in slot g ^ ((r >> 1) & 3): with that
@@ -140,7 +156,8 @@ __device__ __forceinline__ void k4_block_scales(const u32x4 hdr, float sm[16])
 
 // Q4_K: the thread owns bytes [16 dh, 16 dh + 16) of the 32 nibble bytes of a slice: 16 low-nibble weights of sub-block 2J
 // and 16 high-nibble weights of sub-block 2J + 1.
-struct Q4KDecode {
+template <bool LO>
+struct Q4KDecodeT {
     static constexpr int kBlockBytes = 144;
     static constexpr int kAhead = 2;       // (four slices ahead measured the same)
     u32x4 nq[kAhead];           // nibble bytes of K slices t .. t + kAhead - 1
@@ -172,8 +189,8 @@ struct Q4KDecode {
         for (int g = 0; g < 2; ++g) {
             const uint32_t a0 = q[2 * g], a1 = q[2 * g + 1];
             const int slot = lds_slot(c.dc, 2 * c.dh + g) * 16;
-            st128(c, lo + slot, q4k_decode8(a0 & 0x0f0f0f0fu, a1 & 0x0f0f0f0fu, sm[4 * J], sm[4 * J + 1]));
-            st128(c, hi + slot, q4k_decode8((a0 >> 4) & 0x0f0f0f0fu, (a1 >> 4) & 0x0f0f0f0fu, sm[4 * J + 2], sm[4 * J + 3]));
+            st128(c, lo + slot, q4k_decode8<LO>(a0 & 0x0f0f0f0fu, a1 & 0x0f0f0f0fu, sm[4 * J], sm[4 * J + 1]));
+            st128(c, hi + slot, q4k_decode8<LO>((a0 >> 4) & 0x0f0f0f0fu, (a1 >> 4) & 0x0f0f0f0fu, sm[4 * J + 2], sm[4 * J + 3]));
         }
         nq[J % kAhead] = load_q(c, t + kAhead);
         if (J == 0) load_hdr(c, (t >> 2) + 1);
@@ -183,7 +200,8 @@ struct Q4KDecode {
 
 // Q5_K: as Q4_K with one more bit per weight: bit g of qh[i] belongs to element i of sub-block g (qh: 32 bytes after
 // the header, nibbles after that).  The thread keeps bytes [16 dh, 16 dh + 16) of qh for the whole block.
-struct Q5KDecode {
+template <bool LO>
+struct Q5KDecodeT {
     static constexpr int kBlockBytes = 176;
     u32x4 nq[2];
     u32x4 hdr, qh_next;         // of the next block
@@ -218,9 +236,9 @@ struct Q5KDecode {
         for (int g = 0; g < 2; ++g) {
             const uint32_t a0 = q[2 * g], a1 = q[2 * g + 1], h0 = qh[2 * g], h1 = qh[2 * g + 1];
             const int slot = lds_slot(c.dc, 2 * c.dh + g) * 16;
-            st128(c, lo + slot, q4k_decode8((a0 & 0x0f0f0f0fu) | (((h0 >> (2 * J)) & 0x01010101u) << 4),
+            st128(c, lo + slot, q4k_decode8<LO>((a0 & 0x0f0f0f0fu) | (((h0 >> (2 * J)) & 0x01010101u) << 4),
                             (a1 & 0x0f0f0f0fu) | (((h1 >> (2 * J)) & 0x01010101u) << 4), sm[4 * J], sm[4 * J + 1]));
-            st128(c, hi + slot, q4k_decode8(((a0 >> 4) & 0x0f0f0f0fu) | (((h0 >> (2 * J + 1)) & 0x01010101u) << 4),
+            st128(c, hi + slot, q4k_decode8<LO>(((a0 >> 4) & 0x0f0f0f0fu) | (((h0 >> (2 * J + 1)) & 0x01010101u) << 4),
                             ((a1 >> 4) & 0x0f0f0f0fu) | (((h1 >> (2 * J + 1)) & 0x01010101u) << 4), sm[4 * J + 2], sm[4 * J + 3]));
         }
         nq[J & 1] = load_q(c, t + 2);
@@ -236,7 +254,8 @@ struct Q5KDecode {
 // ql[l] / ql[32 + l] with bits 0-1 / 2-3 of qh[l], weights 64-95 / 96-127 the high nibbles with bits 4-5 / 6-7; weight =
 // d * scale[16-group] * (q - 32).  Slice J of a block is half J / 2, nibble J % 2.  The thread keeps bytes
 // [16 dh, 16 dh + 16) of both ql runs and of qh for a half (two slices), and the 16 scales and d for a block.
-struct Q6KDecode {
+template <bool LO>
+struct Q6KDecodeT {
     static constexpr int kBlockBytes = 210;
     u32x4 qa[2], qb[2], qhv[2];     // [half parity]: ql[l], ql[32 + l], qh[l] runs of the current and the next half
     u32x4 sc_next;                  // the 16 scale bytes of the next block
@@ -285,7 +304,7 @@ struct Q6KDecode {
         const float off = 32.0f * dsv;
 #pragma unroll
         for (int g = 0; g < 2; ++g)
-            st128(c, row + lds_slot(c.dc, group0 + g) * 16, q4k_decode8(bytes[2 * g], bytes[2 * g + 1], dsv, off));
+            st128(c, row + lds_slot(c.dc, group0 + g) * 16, q4k_decode8<LO>(bytes[2 * g], bytes[2 * g + 1], dsv, off));
     }
     template <int J>
     __device__ __forceinline__ void make(const DecodeCtx& c, int t, uint8_t* lo, uint8_t* hi)
@@ -308,7 +327,8 @@ struct Q6KDecode {
 
 // Q8_0: a slice is two 34-byte blocks (d, 32 signed bytes); thread dh decodes block dh of the slice, a whole 64-byte
 // row of its sub-tile.
-struct Q8_0Decode {
+template <bool LO>
+struct Q8_0DecodeT {
     static constexpr int kBlockBytes = 34 * 8;     // bytes per 256 weights
     u32x4 q0[2], q1[2];
     uint32_t dbits[2];
@@ -329,8 +349,8 @@ struct Q8_0Decode {
     }
     static __device__ __forceinline__ u32x4 decode8(uint32_t a, uint32_t b, float d)
     {
-        return u32x4{pack_bf16(d * sbyte0(a), d * sbyte1(a)), pack_bf16(d * sbyte2(a), d * sbyte3(a)),
-                     pack_bf16(d * sbyte0(b), d * sbyte1(b)), pack_bf16(d * sbyte2(b), d * sbyte3(b))};
+        return u32x4{pack_w<LO>(d * sbyte0(a), d * sbyte1(a)), pack_w<LO>(d * sbyte2(a), d * sbyte3(a)),
+                     pack_w<LO>(d * sbyte0(b), d * sbyte1(b)), pack_w<LO>(d * sbyte2(b), d * sbyte3(b))};
     }
     template <int J>
     __device__ __forceinline__ void make(const DecodeCtx& c, int t, uint8_t* lo, uint8_t* hi)
@@ -351,16 +371,18 @@ __device__ const uint64_t g_iq2s_grid_mm[1024] = { NNHIP_IQ2S_GRID_VALUES };
 __device__ const uint32_t g_iq3s_grid_mm[512] = { NNHIP_IQ3S_GRID_VALUES };
 
 // bf16 pair of two magnitudes times db with their sign bits (bit 0 of `signs`: first weight, bit 1: second)
+template <bool LO>
 __device__ __forceinline__ uint32_t iq_pair(float db, float m0, float m1, uint32_t signs)
 {
-    return pack_bf16(db * m0, db * m1) ^ (((signs & 1u) << 15) | ((signs & 2u) << 30));
+    return pack_w<LO>(db * m0, db * m1) ^ (((signs & 1u) << 15) | ((signs & 2u) << 30));
 }
 
 // IQ2_S (82 bytes: d, 32 index bytes, 32 sign bytes, qh[8], scales[8]; NNtrain.Arc/Kernels/qwen35_iq.cl:411-419): thread
 // dh decodes 32-weight group 2 (t % 4) + dh of block t / 4, a whole 64-byte row of its sub-tile = four codebook entries
 // of eight magnitudes.  Index and sign bytes are requested three slices ahead, the codebook entries one slice ahead (from
 // indices that arrived two slices earlier), qh / scales / d of a block a block ahead.
-struct IQ2SDecode {
+template <bool LO>
+struct IQ2SDecodeT {
     static constexpr int kBlockBytes = 82;
     uint32_t qs[4], sg[4];      // index and sign bytes of slices t .. t + 3 (set = slice % 4)
     u32x2 grid[2][4];           // codebook entries of slices t, t + 1 (set = slice % 2)
@@ -419,8 +441,8 @@ struct IQ2SDecode {
         for (int o = 0; o < 4; ++o) {
             const uint32_t m0 = grid[J & 1][o][0], m1 = grid[J & 1][o][1], sb = signs >> (8 * o);
             const float db = o < 2 ? db_lo : db_hi;
-            st128(c, row + lds_slot(c.dc, o) * 16, u32x4{iq_pair(db, ubyte0(m0), ubyte1(m0), sb), iq_pair(db, ubyte2(m0), ubyte3(m0), sb >> 2),
-                      iq_pair(db, ubyte0(m1), ubyte1(m1), sb >> 4), iq_pair(db, ubyte2(m1), ubyte3(m1), sb >> 6)});
+            st128(c, row + lds_slot(c.dc, o) * 16, u32x4{iq_pair<LO>(db, ubyte0(m0), ubyte1(m0), sb), iq_pair<LO>(db, ubyte2(m0), ubyte3(m0), sb >> 2),
+                      iq_pair<LO>(db, ubyte0(m1), ubyte1(m1), sb >> 4), iq_pair<LO>(db, ubyte2(m1), ubyte3(m1), sb >> 6)});
         }
         // slice t + 1 belongs to the next block when J == 3
         load_grid<(J + 1) & 3>(c, qs[(J + 1) & 3], J == 3 ? tail_next : tail, grid[(J + 1) & 1]);
@@ -435,7 +457,8 @@ struct IQ2SDecode {
 
 // IQ3_S (110 bytes: d, 64 index bytes, qh[8], 32 sign bytes, scales[4]; qwen35_iq.cl:421-429): as IQ2_S with eight
 // codebook entries of four magnitudes per 32-weight group and w = (d * (1 + 2 s)) * magnitude * sign.
-struct IQ3SDecode {
+template <bool LO>
+struct IQ3SDecodeT {
     static constexpr int kBlockBytes = 110;
     u32x2 qs[4];                // eight index bytes of slices t .. t + 3
     uint32_t sg[4];
@@ -496,8 +519,8 @@ struct IQ3SDecode {
 #pragma unroll
         for (int o = 0; o < 4; ++o) {
             const uint32_t m0 = grid[J & 1][2 * o], m1 = grid[J & 1][2 * o + 1], sb = signs >> (8 * o);
-            st128(c, row + lds_slot(c.dc, o) * 16, u32x4{iq_pair(db, ubyte0(m0), ubyte1(m0), sb), iq_pair(db, ubyte2(m0), ubyte3(m0), sb >> 2),
-                      iq_pair(db, ubyte0(m1), ubyte1(m1), sb >> 4), iq_pair(db, ubyte2(m1), ubyte3(m1), sb >> 6)});
+            st128(c, row + lds_slot(c.dc, o) * 16, u32x4{iq_pair<LO>(db, ubyte0(m0), ubyte1(m0), sb), iq_pair<LO>(db, ubyte2(m0), ubyte3(m0), sb >> 2),
+                      iq_pair<LO>(db, ubyte0(m1), ubyte1(m1), sb >> 4), iq_pair<LO>(db, ubyte2(m1), ubyte3(m1), sb >> 6)});
         }
         load_grid<(J + 1) & 3>(c, qs[(J + 1) & 3], J == 3 ? qh_next : qh, grid[(J + 1) & 1]);
         load_raw(c, t + 3, (J + 3) & 3);
@@ -509,6 +532,13 @@ struct IQ3SDecode {
         if (J == 0) load_hdr(c, (t >> 2) + 1);
     }
 };
+
+using Q4KDecode = Q4KDecodeT<false>;
+using Q5KDecode = Q5KDecodeT<false>;
+using Q6KDecode = Q6KDecodeT<false>;
+using Q8_0Decode = Q8_0DecodeT<false>;
+using IQ2SDecode = IQ2SDecodeT<false>;
+using IQ3SDecode = IQ3SDecodeT<false>;
 
 // Unquantized bfloat16 weights (matrix storage type 30, and the scratch copy the two-pass path decodes into): thread dh
 // copies weights [32 dh, 32 dh + 32) of the slice, a whole 64-byte row of its sub-tile.
@@ -756,7 +786,10 @@ __global__ __launch_bounds__(kGemmAll) void matmul_bf16_kernel(GemmArgs a)
 #pragma unroll
                     for (int v = 0; v < 4; ++v) {
                         const int m = m0 + wm * RW + i * 16 + (lane >> 4) * 4 + v;
-                        if (m < a.M) a.y[static_cast<size_t>(m) * a.N + n] = acc[i][j][v] + b;
+                        if (m < a.M) {
+                            float* out = a.y + static_cast<size_t>(m) * a.N + n;
+                            *out = a.accumulate ? *out + acc[i][j][v] : acc[i][j][v] + b;
+                        }
                     }
                 }
             }
@@ -784,9 +817,10 @@ hipError_t launch_gemm(Lane* lane, const GemmArgs& a, dim3 grid)
 
 template <class F>
 hipError_t launch_matmul_of(Lane* lane, const uint16_t* x, const void* w, const float* bias, float* y, int rows, int in_w,
-                            int out_w)
+                            int out_w, bool accumulate)
 {
     GemmArgs a{};
+    a.accumulate = accumulate ? 1 : 0;
     a.x = x;
     a.w = static_cast<const uint8_t*>(w);
     a.bias = bias;
@@ -829,6 +863,35 @@ __global__ __launch_bounds__(256) void to_bf16_kernel(const float* __restrict__ 
 
 }  // namespace
 
+namespace {
+
+// FP32 -> the two bfloat16 parts of the three-product mat-mul: hi = bf16(x), lo = bf16(x - hi); x - hi - lo is below
+// 2^-17 of x.  Eight values per thread.
+__global__ __launch_bounds__(256) void to_bf16_parts_kernel(const float* __restrict__ x, uint16_t* __restrict__ hi,
+                                                            uint16_t* __restrict__ lo, size_t count)
+{
+    const size_t i = (static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x) * 8;
+    if (i + 8 <= count) {
+        const float4 a = *reinterpret_cast<const float4*>(x + i), b = *reinterpret_cast<const float4*>(x + i + 4);
+        *reinterpret_cast<u32x4*>(hi + i) = u32x4{pack_w<false>(a.x, a.y), pack_w<false>(a.z, a.w), pack_w<false>(b.x, b.y), pack_w<false>(b.z, b.w)};
+        *reinterpret_cast<u32x4*>(lo + i) = u32x4{pack_w<true>(a.x, a.y), pack_w<true>(a.z, a.w), pack_w<true>(b.x, b.y), pack_w<true>(b.z, b.w)};
+    } else {
+        for (size_t j = i; j < count; ++j) {
+            hi[j] = static_cast<uint16_t>(pack_w<false>(x[j], 0.0f) & 0xffffu);
+            lo[j] = static_cast<uint16_t>(pack_w<true>(x[j], 0.0f) & 0xffffu);
+        }
+    }
+}
+
+}  // namespace
+
+hipError_t launch_to_bf16_parts(Lane* lane, const float* x, uint16_t* hi, uint16_t* lo, size_t count)
+{
+    const size_t groups = (count + 2047) / 2048;
+    hipLaunchKernelGGL(to_bf16_parts_kernel, dim3(static_cast<unsigned>(groups)), dim3(256), 0, lane->stream, x, hi, lo, count);
+    return hipGetLastError();
+}
+
 hipError_t launch_to_bf16(Lane* lane, const float* x, uint16_t* out, size_t count)
 {
     const size_t groups = (count + 2047) / 2048;
@@ -846,18 +909,47 @@ bool matmul_bf16_supported(uint32_t type, int in_w)
 }
 
 hipError_t launch_matmul_bf16(Lane* lane, uint32_t type, const uint16_t* x, const void* w, const float* bias, float* y,
-                              int rows, int in_w, int out_w)
+                              int rows, int in_w, int out_w, bool low_weight_part, bool accumulate)
 {
+    if (low_weight_part) {
+        switch (type) {
+        case NNHIP_TYPE_Q4_K: return launch_matmul_of<Q4KDecodeT<true>>(lane, x, w, bias, y, rows, in_w, out_w, accumulate);
+        case NNHIP_TYPE_Q5_K: return launch_matmul_of<Q5KDecodeT<true>>(lane, x, w, bias, y, rows, in_w, out_w, accumulate);
+        case NNHIP_TYPE_Q6_K: return launch_matmul_of<Q6KDecodeT<true>>(lane, x, w, bias, y, rows, in_w, out_w, accumulate);
+        case NNHIP_TYPE_Q8_0: return launch_matmul_of<Q8_0DecodeT<true>>(lane, x, w, bias, y, rows, in_w, out_w, accumulate);
+        case NNHIP_TYPE_IQ2_S: return launch_matmul_of<IQ2SDecodeT<true>>(lane, x, w, bias, y, rows, in_w, out_w, accumulate);
+        case NNHIP_TYPE_IQ3_S: return launch_matmul_of<IQ3SDecodeT<true>>(lane, x, w, bias, y, rows, in_w, out_w, accumulate);
+        default: return hipErrorNotSupported;        // (bfloat16 weights have no low-order part)
+        }
+    }
     switch (type) {
-    case NNHIP_TYPE_Q4_K: return launch_matmul_of<Q4KDecode>(lane, x, w, bias, y, rows, in_w, out_w);
-    case NNHIP_TYPE_Q5_K: return launch_matmul_of<Q5KDecode>(lane, x, w, bias, y, rows, in_w, out_w);
-    case NNHIP_TYPE_Q6_K: return launch_matmul_of<Q6KDecode>(lane, x, w, bias, y, rows, in_w, out_w);
-    case NNHIP_TYPE_Q8_0: return launch_matmul_of<Q8_0Decode>(lane, x, w, bias, y, rows, in_w, out_w);
-    case NNHIP_TYPE_IQ2_S: return launch_matmul_of<IQ2SDecode>(lane, x, w, bias, y, rows, in_w, out_w);
-    case NNHIP_TYPE_IQ3_S: return launch_matmul_of<IQ3SDecode>(lane, x, w, bias, y, rows, in_w, out_w);
-    case NNHIP_TYPE_BF16: return launch_matmul_of<BF16Decode>(lane, x, w, bias, y, rows, in_w, out_w);
+    case NNHIP_TYPE_Q4_K: return launch_matmul_of<Q4KDecode>(lane, x, w, bias, y, rows, in_w, out_w, accumulate);
+    case NNHIP_TYPE_Q5_K: return launch_matmul_of<Q5KDecode>(lane, x, w, bias, y, rows, in_w, out_w, accumulate);
+    case NNHIP_TYPE_Q6_K: return launch_matmul_of<Q6KDecode>(lane, x, w, bias, y, rows, in_w, out_w, accumulate);
+    case NNHIP_TYPE_Q8_0: return launch_matmul_of<Q8_0Decode>(lane, x, w, bias, y, rows, in_w, out_w, accumulate);
+    case NNHIP_TYPE_IQ2_S: return launch_matmul_of<IQ2SDecode>(lane, x, w, bias, y, rows, in_w, out_w, accumulate);
+    case NNHIP_TYPE_IQ3_S: return launch_matmul_of<IQ3SDecode>(lane, x, w, bias, y, rows, in_w, out_w, accumulate);
+    case NNHIP_TYPE_BF16: return launch_matmul_of<BF16Decode>(lane, x, w, bias, y, rows, in_w, out_w, accumulate);
     default: return hipErrorNotSupported;
     }
+}
+
+// y = bias + x w^T with both operands as the sum of two bfloat16 parts: three launches, x_hi w_hi (+ bias), then
+// x_lo w_hi and x_hi w_lo added to it (the fourth product, x_lo w_lo, is below 2^-16 of the first and left out).
+hipError_t launch_matmul_parts(Lane* lane, uint32_t type, const uint16_t* x_hi, const uint16_t* x_lo, const void* w, const float* bias,
+                               float* y, int rows, int in_w, int out_w, int* launches)
+{
+    *launches = 0;
+    hipError_t e = launch_matmul_bf16(lane, type, x_hi, w, bias, y, rows, in_w, out_w, false, false);
+    if (e != hipSuccess) return e;
+    ++*launches;
+    e = launch_matmul_bf16(lane, type, x_lo, w, nullptr, y, rows, in_w, out_w, false, true);
+    if (e != hipSuccess) return e;
+    ++*launches;
+    if (type == NNHIP_TYPE_BF16) return hipSuccess;
+    e = launch_matmul_bf16(lane, type, x_hi, w, nullptr, y, rows, in_w, out_w, true, true);
+    if (e == hipSuccess) ++*launches;
+    return e;
 }
 
 }  // namespace nnhip

@@ -865,6 +865,34 @@ int nnhip_quant_matmul(void* handle, uint32_t ggml_type, const float* x, const v
     return NNHIP_OK;
 }
 
+int nnhip_quant_matmul_split(void* handle, uint32_t ggml_type, const float* x, const void* w, const float* bias, float* y,
+                             int rows, int in_w, int out_w)
+{
+    NNHIP_LANE(handle, NNHIP_OP_MATMUL)
+    int rc = check_linear(NNHIP_OP_MATMUL, lane, ggml_type, x, w, y, rows, in_w, out_w);
+    if (rc != NNHIP_OK) return rc;
+    if (in_w % 256 != 0 && matmul_bf16_supported(ggml_type, 256))
+        return fail(NNHIP_ERR_INCOMPLETE_BLOCKS, NNHIP_OP_MATMUL, lane->device, 0, "the prefill mat-mul needs in_w to be a multiple of 256 (got %d)", in_w);
+    if (!matmul_bf16_supported(ggml_type, in_w))
+        return fail(NNHIP_ERR_UNSUPPORTED_TYPE, NNHIP_OP_MATMUL, lane->device, 0, "the prefill mat-mul does not support GGML type %u", ggml_type);
+    // both bfloat16 parts of the activations share one lane block for the duration of the launches
+    const size_t count = static_cast<size_t>(rows) * static_cast<size_t>(in_w);
+    const size_t part_bytes = (count * sizeof(uint16_t) + 255u) & ~static_cast<size_t>(255u);
+    void* staged = nullptr;
+    rc = nnhip_alloc(handle, 2 * part_bytes, &staged);
+    if (rc != NNHIP_OK) return rc;
+    uint16_t* hi = static_cast<uint16_t*>(staged);
+    uint16_t* lo = reinterpret_cast<uint16_t*>(static_cast<char*>(staged) + part_bytes);
+    int launches = 0;
+    hipError_t e = launch_to_bf16_parts(lane, x, hi, lo, count);
+    if (e == hipSuccess) e = launch_matmul_parts(lane, ggml_type, hi, lo, w, bias, y, rows, in_w, out_w, &launches);
+    const int freed = nnhip_free(handle, staged);
+    lane->counters.kernel_launches += static_cast<uint64_t>(launches) + 1;
+    if (e != hipSuccess) return hip_fail(e, NNHIP_OP_MATMUL, lane->device, "mat-mul launch");
+    if (freed != NNHIP_OK) return freed;
+    return NNHIP_OK;
+}
+
 int nnhip_event_create(void* handle, void** event)
 {
     NNHIP_LANE(handle, NNHIP_OP_EVENT)

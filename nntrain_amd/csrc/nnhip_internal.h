@@ -141,8 +141,12 @@ int plan_matvec_batch(const nnhip_matvec_desc* descs, int count, int compute_uni
 // The fixed device workspace: its address on the current device, and the batched launch that uses it.
 hipError_t static_table_address(void** address, unsigned serial);
 hipError_t launch_matvec_batch_static(Lane* lane, const nnhip_matvec_desc* descs, int count);
-hipError_t launch_matmul_bf16(Lane* lane, uint32_t type, const uint16_t* x, const void* w, const float* bias,
-                              float* y, int rows, int in_w, int out_w);
+hipError_t launch_matmul_bf16(Lane* lane, uint32_t type, const uint16_t* x, const void* w, const float* bias, float* y,
+                              int rows, int in_w, int out_w, bool low_weight_part = false, bool accumulate = false);
+// The three-product form: both operands as two bfloat16 parts each (see gemm_kernels.hip).
+hipError_t launch_to_bf16_parts(Lane* lane, const float* x, uint16_t* hi, uint16_t* lo, size_t count);
+hipError_t launch_matmul_parts(Lane* lane, uint32_t type, const uint16_t* x_hi, const uint16_t* x_lo, const void* w, const float* bias,
+                               float* y, int rows, int in_w, int out_w, int* launches);
 hipError_t launch_to_bf16(Lane* lane, const float* x, uint16_t* out, size_t count);
 // FP32 row operations (rowop_kernels.hip).  residual == nullptr: plain RMSNorm of io (not modified).
 hipError_t launch_rms_norm(Lane* lane, float* io, const float* residual, const float* weight, float* output, int rows,

@@ -99,6 +99,7 @@ PROTOTYPES = {
     "nnhip_quant_matvec_batch_static": (c_int, [c_void_p, POINTER(MatvecDesc), c_int]),
     "nnhip_quant_matvec_fused": (c_int, [c_void_p, POINTER(FusedMatvecDesc)]),
     "nnhip_quant_matmul": (c_int, [c_void_p, c_uint32, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int]),
+    "nnhip_quant_matmul_split": (c_int, [c_void_p, c_uint32, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int]),
     "nnhip_quant_matmul_bf16": (c_int, [c_void_p, c_uint32, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int]),
     "nnhip_rms_norm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float]),
     "nnhip_add_rms_norm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float]),

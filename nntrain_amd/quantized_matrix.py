@@ -28,7 +28,8 @@ PREFILL_MIN_ROWS = 16
 
 
 class HipQuantizedMatrix:
-    def __init__(self, payload, ggml_type: int, output_width: int, input_width: int, inference_matmul_prefill: bool = False):
+    def __init__(self, payload, ggml_type: int, output_width: int, input_width: int,
+                 inference_matmul_prefill: "bool | str" = False):
         if payload is None:
             raise TypeError("payload is null")
         if ggml_type not in BLOCK_ELEMS:
@@ -51,7 +52,12 @@ class HipQuantizedMatrix:
         self.input_width = input_width
         # Matrix takes inferenceXmxPrefill from the execution options (Qwen35QuantizedModel.cs:252); off unless asked for
         # (Qwen35ExecutionOptions.InferenceXmxPrefill, Qwen35ExecutionOptions.cs:50), because that route rounds to bfloat16.
-        self.inference_matmul_prefill = bool(inference_matmul_prefill)
+        # "split": the three-product form (both operands as two bfloat16 parts), which meets the 5e-5 the reference tests its
+        # XMX prefill at (Qwen35XmxPrefillLinearTests.cs:87-89); True: one bfloat16 rounding of each operand (2e-3), a third
+        # of the cost.
+        if inference_matmul_prefill not in (False, True, "split"):
+            raise ValueError("inference_matmul_prefill must be False, True or 'split'.")
+        self.inference_matmul_prefill = inference_matmul_prefill
         self._lane: HipExecutionLane | None = None
         self._device_payload: HipBuffer | None = None
 
@@ -132,7 +138,7 @@ class HipQuantizedMatrix:
         """Whether forward() sends `rows` input rows to the bfloat16 matrix-core mat-mul: only when the matrix was
         given inference_matmul_prefill (the reference's opt-in InferenceXmxPrefill), for rows >= 16 as in Matrix.Forward
         (Qwen35QuantizedModel.cs:1249) and rows of whole 256-weight blocks; the FP32-grade mat-vec kernels otherwise."""
-        return self.inference_matmul_prefill and rows >= PREFILL_MIN_ROWS and self.input_width % 256 == 0
+        return bool(self.inference_matmul_prefill) and rows >= PREFILL_MIN_ROWS and self.input_width % 256 == 0
 
     def forward(self, lane: HipExecutionLane, x: HipBuffer, bias: HipBuffer | None, rows: int = 1,
                 out: HipBuffer | None = None) -> HipBuffer:
@@ -140,8 +146,9 @@ class HipQuantizedMatrix:
         Every row count goes to the dequantization-fused mat-vec (FP32 accumulation, 1e-5 of the float64 product; up to
         four input rows share a pass over the weights on the large matrices).  With inference_matmul_prefill set, rows
         >= 16 go to the bfloat16 matrix-core mat-mul instead (activations and weights rounded to bfloat16 once: 2e-3),
-        the counterpart of the reference's opt-in XMX prefill (Qwen35QuantizedModel.cs:1249-1317), whose own bound is
-        5e-5 because it splits its operands into two f16 parts; this route does not."""
+        the counterpart of the reference's opt-in XMX prefill (Qwen35QuantizedModel.cs:1249-1317); that path's own bound is
+        5e-5 because it splits its operands into two f16 parts, which inference_matmul_prefill="split" does with bfloat16
+        parts (three products, about 3e-6)."""
         if rows < 1:
             raise ValueError("rows must be positive.")
         if x.nbytes < 4 * rows * self.input_width:
@@ -152,8 +159,12 @@ class HipQuantizedMatrix:
         if out is not None and out.nbytes < 4 * rows * self.output_width:
             raise ValueError("output buffer too small")
         y = out if out is not None else lane.allocate(rows * self.output_width)
-        entry, fn = (("quant_matmul", lane._lib.nnhip_quant_matmul) if self.uses_prefill(rows)
-                     else ("quant_matvec", lane._lib.nnhip_quant_matvec))
+        if not self.uses_prefill(rows):
+            entry, fn = "quant_matvec", lane._lib.nnhip_quant_matvec
+        elif self.inference_matmul_prefill == "split":
+            entry, fn = "quant_matmul_split", lane._lib.nnhip_quant_matmul_split
+        else:
+            entry, fn = "quant_matmul", lane._lib.nnhip_quant_matmul
         try:
             with lane.kernel(entry):
                 check(fn(lane._handle, self.ggml_type, c_void_p(x._require()), c_void_p(w._require()),

@@ -192,6 +192,73 @@ def test_forward_routes_sixteen_rows_and_more_to_the_matrix_cores(lane, typ):
     narrow.dispose()
 
 
+SPLIT_BAR = 5e-5           # what the reference holds its XMX prefill to (Qwen35XmxPrefillLinearTests.cs:87-89)
+
+
+@pytest.mark.parametrize("shape", [(17, 512, 65), (129, 5120, 129), (256, 17408, 65)])
+def test_split_prefill_meets_the_bar_of_the_reference_on_its_shapes(lane, shape):
+    """The three-product mat-mul (both operands as two bfloat16 parts) on the shapes the reference tests its XMX prefill
+    with (rows x input x output, Qwen35XmxPrefillLinearTests.cs:20-29), every storage format the mat-mul takes: relative
+    L2 below 5e-5 against the float64 product and against the FP32 mat-vec, as the reference asserts; in practice about
+    3e-6.  The operator reaches it through inference_matmul_prefill="split"."""
+    from nntrain_amd import GGML_BF16
+    rows, in_w, out_w = shape
+    types = [GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_Q8_0, GGML_IQ2_S, GGML_IQ3_S, GGML_BF16]
+    x = synth.activations(rows, in_w, seed=rows + in_w)
+    x[1] *= 250.0
+    x[3] *= 4e-3
+    xd = lane.upload_raw(x)
+    bias = np.random.default_rng(rows).standard_normal(out_w).astype(np.float32)
+    bd = lane.upload_raw(bias)
+    for typ in types if in_w <= 5120 else [GGML_Q4_K, GGML_Q8_0, GGML_IQ2_S]:
+        payload = synth.matrix(typ, out_w, in_w, seed=60 + typ)
+        mat = HipQuantizedMatrix(payload, typ, out_w, in_w, inference_matmul_prefill="split")
+        assert mat.uses_prefill(rows)
+        yd = lane.allocate(rows * out_w + 2)
+        lane.fill_u32(yd, NAN_BITS, rows * out_w + 2)
+        launches = lane.counters()["kernel_launches"]
+        mat.forward(lane, xd, bd, rows, out=yd)
+        assert lane.counters()["kernel_launches"] - launches == (3 if typ == GGML_BF16 else 4)     # conversion + products
+        y = lane.read(yd)
+        assert np.isnan(y[-1]) and np.isnan(y[-2])
+        y = y[:-2].reshape(rows, out_w)
+        assert np.all(np.isfinite(y))
+        ref, _ = oracle.linear_f64(typ, payload, x, bias, rows, in_w, out_w)
+        rel = oracle.rel_l2(y, ref)
+        assert rel <= SPLIT_BAR, (typ, rel)
+        assert rel <= 1e-5, (typ, rel)                # what the three products leave in practice
+        for r in range(rows):                         # every input row on its own: none hides behind a large one
+            assert oracle.rel_l2(y[r], ref[r]) <= SPLIT_BAR, (typ, r)
+        exact = HipQuantizedMatrix(payload, typ, out_w, in_w)
+        y32 = lane.read(exact.forward(lane, xd, bd, rows)).reshape(rows, out_w)
+        assert oracle.rel_l2(y, y32.astype(np.float64)) <= SPLIT_BAR
+        # the one-product route on the same call, for scale: three orders of magnitude coarser
+        fast = HipQuantizedMatrix(payload, typ, out_w, in_w, inference_matmul_prefill=True)
+        yf = lane.read(fast.forward(lane, xd, bd, rows)).reshape(rows, out_w)
+        assert oracle.rel_l2(yf, ref) > 20 * rel or typ == GGML_BF16
+        for m in (mat, exact, fast):
+            m.dispose()
+        yd.dispose()
+    for b in (xd, bd):
+        b.dispose()
+    lane.trim()
+
+
+def test_split_prefill_rejects_what_the_mat_mul_rejects(lane):
+    lib, h = lane._lib, lane._handle
+    x = lane.allocate(16 * 320)
+    w = lane.upload_raw(synth.matrix(GGML_Q8_0, 8, 320, seed=1))
+    y = lane.allocate(16 * 8)
+    from ctypes import c_void_p
+    assert lib.nnhip_quant_matmul_split(h, GGML_Q8_0, c_void_p(x.ptr), c_void_p(w.ptr), None, c_void_p(y.ptr), 16, 320, 8) == 3
+    assert lib.nnhip_quant_matmul_split(h, 99, c_void_p(x.ptr), c_void_p(w.ptr), None, c_void_p(y.ptr), 16, 256, 8) == 2
+    assert lib.nnhip_quant_matmul_split(h, GGML_Q8_0, None, c_void_p(w.ptr), None, c_void_p(y.ptr), 16, 256, 8) == 1
+    with pytest.raises(ValueError):
+        HipQuantizedMatrix(synth.matrix(GGML_Q8_0, 8, 320, seed=1), GGML_Q8_0, 8, 320, inference_matmul_prefill="fast")
+    for b in (x, w, y):
+        b.dispose()
+
+
 def test_forward_with_many_rows_beats_one_weight_pass_per_row(lane):
     in_w, out_w, rows = 5120, 4096, 128
     mat = HipQuantizedMatrix(synth.matrix(GGML_Q5_K, out_w, in_w, seed=9), GGML_Q5_K, out_w, in_w, inference_matmul_prefill=True)
