@@ -28,6 +28,19 @@ public sealed unsafe class HipExecutionLane : IDisposable
     public long AllocatedBytes => (long)Counters().AllocatedBytes;
     public long PeakAllocatedBytes => (long)Counters().PeakAllocatedBytes;
 
+    /// <summary>Keeps every mat-vec of the lane on the FP32 row-step kernels: calls with several input rows then equal
+    /// stacked single-row calls bit for bit (Qwen35InferencePrefillLinearTests.cs:64-77), without the shared
+    /// matrix-core passes.</summary>
+    public bool RowStepOnly
+    {
+        get
+        {
+            NnHipNative.Check(NnHipNative.nnhip_lane_get_option(Handle, NnHipNative.OptionRowStepOnly, out long value), "lane option");
+            return value != 0;
+        }
+        set => NnHipNative.Check(NnHipNative.nnhip_lane_set_option(Handle, NnHipNative.OptionRowStepOnly, value ? 1 : 0), "lane option");
+    }
+
     public HipBuffer Allocate(int elements) => AllocateBytes(checked(elements * sizeof(float)));
 
     public HipBuffer AllocateBytes(long bytes)

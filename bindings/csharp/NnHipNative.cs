@@ -86,6 +86,9 @@ internal static unsafe partial class NnHipNative
     [LibraryImport(Library)] internal static partial int nnhip_synchronize(nint lane);
     [LibraryImport(Library)] internal static partial int nnhip_lane_get_counters(nint lane, out LaneCounters counters, nuint size);
     [LibraryImport(Library)] internal static partial int nnhip_lane_stream(nint lane, out nint stream);
+    internal const uint OptionRowStepOnly = 1;
+    [LibraryImport(Library)] internal static partial int nnhip_lane_set_option(nint lane, uint option, long value);
+    [LibraryImport(Library)] internal static partial int nnhip_lane_get_option(nint lane, uint option, out long value);
     [LibraryImport(Library)] internal static partial int nnhip_dequantize(nint lane, uint ggmlType, nint w, nint output, long elements);
     [LibraryImport(Library)] internal static partial int nnhip_quant_matvec(nint lane, uint ggmlType, nint x, nint w, nint bias, nint y, int rows, int inW, int outW);
     [LibraryImport(Library)] internal static partial int nnhip_matvec_plan(uint ggmlType, int rows, int inW, int outW, int computeUnits, MatvecPlanInfo* info);

@@ -179,6 +179,17 @@ NNHIP_API int nnhip_lane_get_counters(void* lane, nnhip_lane_counters* out, size
 /* The lane's hipStream_t, for callers that interoperate with other HIP code. */
 NNHIP_API int nnhip_lane_stream(void* lane, void** stream);
 
+/* Lane options (all 0 when a lane is created).
+ * NNHIP_OPTION_ROW_STEP_ONLY = 1: nnhip_quant_matvec, nnhip_quant_matvec_batch and nnhip_quant_matvec_batch_static keep
+ * every product on the FP32 row-step kernels, whatever the number of input rows or the size of the batch.  With it the
+ * property the reference tests for its row-tiled kernels holds without exception: a call with rows > 1 equals stacked
+ * rows == 1 calls bit for bit (Qwen35InferencePrefillLinearTests.cs:64-77), and a batch equals its single calls.  The
+ * price is the shared matrix-core passes (a call with four input rows on 17408 x 5120 Q4_K: about twice the time).
+ * Unknown options: NNHIP_ERR_INVALID_ARGUMENT. */
+enum { NNHIP_OPTION_ROW_STEP_ONLY = 1 };
+NNHIP_API int nnhip_lane_set_option(void* lane, uint32_t option, int64_t value);
+NNHIP_API int nnhip_lane_get_option(void* lane, uint32_t option, int64_t* value);
+
 /* --- compute ------------------------------------------------------------------------------------------------ */
 
 /* out[i] = decoded weight i, FP32, bit-identical to the managed decoders GgufQ4K.Dequantize / GgufQ6K.Dequantize
@@ -200,7 +211,8 @@ NNHIP_API int nnhip_dequantize(void* lane, uint32_t ggml_type, const void* w, fl
  * input rows per pass over the weights, sixteen per launch; a row's bits do not depend on the rows it travels with; 1e-6
  * from the rows == 1 result).  Rows too long for four sets of activation planes in LDS (in_w above about 8700) get one
  * matrix-core pass per input row instead, four rows a launch, from rows x ceil(out_w / 16) >= 1024 on (IQ3_S 768, IQ2_S
- * 512; never Q8_0).  nnhip_matvec_plan reports which form a call takes.  bias may be null (zero).  Asynchronous. */
+ * 512; never Q8_0).  nnhip_matvec_plan reports which form a call takes; a lane with NNHIP_OPTION_ROW_STEP_ONLY set takes
+ * none of these forms and keeps the bit-for-bit property for every call.  bias may be null (zero).  Asynchronous. */
 NNHIP_API int nnhip_quant_matvec(void* lane, uint32_t ggml_type, const float* x, const void* w, const float* bias,
                                  float* y, int rows, int in_w, int out_w);
 

@@ -1419,7 +1419,7 @@ static_assert(sizeof(MfmaTableEntry) == sizeof(BatchEntry), "both kinds of entry
 int shared_pass_min_rows(uint32_t type) { return type == NNHIP_TYPE_Q8_0 ? 3 : 2; }
 
 long build_batch(const nnhip_matvec_desc* descs, int count, BatchEntry* out, size_t cap, BatchGroup* groups, int* ngroups,
-                 uint8_t* forms)
+                 uint8_t* forms, bool row_step_only = false)
 {
     size_t n = 0;
     *ngroups = 0;
@@ -1430,7 +1430,8 @@ long build_batch(const nnhip_matvec_desc* descs, int count, BatchEntry* out, siz
     for (int i = 0; i < count; ++i) {
         const nnhip_matvec_desc& d = descs[i];
         int form = 0;
-        if (d.rows >= shared_pass_min_rows(d.ggml_type) && matvec_mfma_wide_geometry(d.ggml_type, d.in_w, d.out_w, d.w, 4)) form = 3;
+        if (row_step_only) form = 0;
+        else if (d.rows >= shared_pass_min_rows(d.ggml_type) && matvec_mfma_wide_geometry(d.ggml_type, d.in_w, d.out_w, d.w, 4)) form = 3;
         else if (matvec_mfma_geometry(d.ggml_type, d.in_w, d.out_w, d.w, nullptr)) form = 1;
         else if (matvec_mfma_wide_geometry(d.ggml_type, d.in_w, d.out_w, d.w, 1)) form = 2;
         forms[i] = static_cast<uint8_t>(form);
@@ -1578,7 +1579,7 @@ hipError_t launch_matvec_batch(Lane* lane, const nnhip_matvec_desc* descs, int c
     std::vector<uint8_t> forms(static_cast<size_t>(count > 0 ? count : 1));
     BatchGroup groups[kBatchGroupsMax];
     int ngroups = 0;
-    const long n = build_batch(descs, count, all.data(), cap, groups, &ngroups, forms.data());
+    const long n = build_batch(descs, count, all.data(), cap, groups, &ngroups, forms.data(), lane->row_step_only);
     if (n < 0) return hipErrorInvalidValue;
     const size_t bytes = static_cast<size_t>(n) * sizeof(BatchEntry);
     if (bytes) {
@@ -1716,7 +1717,7 @@ hipError_t launch_matvec_batch_static(Lane* lane, const nnhip_matvec_desc* descs
     uint8_t forms[kStaticTableEntries];
     BatchGroup groups[kBatchGroupsMax];
     int ngroups = 0;
-    const long n = build_batch(descs, count, entries, kStaticTableEntries, groups, &ngroups, forms);
+    const long n = build_batch(descs, count, entries, kStaticTableEntries, groups, &ngroups, forms, lane->row_step_only);
     if (n < 0) return hipErrorInvalidValue;
     if (n > 0) {
         const hipError_t e = write_table(lane, lane->static_table, entries, static_cast<size_t>(n));

@@ -1700,14 +1700,17 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
 
 // The (KC, M, LPW) combinations the kernel is instantiated for.
 struct Variant { int kc, m, lpw; };
-constexpr Variant kVariants[] = {{1, 2, 5}, {1, 2, 6}, {2, 1, 3}, {1, 1, 3}, {2, 2, 5}, {2, 2, 6}, {1, 1, 2}, {2, 1, 2},
-                                 {1, 1, 4}, {2, 1, 4}};
+constexpr Variant kVariants[] = {{1, 2, 5}, {1, 2, 6}, {2, 1, 3}, {1, 1, 3}, {1, 1, 2}, {2, 1, 2}, {1, 1, 4}, {2, 1, 4}};
 
 // Picks W and C for (block bytes, in_w).  C = W * M columns per stage must divide the row's super-blocks into KC whole
 // stages, two stage buffers must fit LDS (one of them doubles as scratch for the digit planes when the activations
-// change), (KC, M, LPW) must be an instantiated variant, and among those the choice maximises the bytes a stage holds,
-// then the waves.
-bool plan_mfma(int block_pieces, int in_w, bool even_waves, MfmaGeom* out)
+// change), (KC, M, LPW) must be an instantiated variant.  Two columns per wave are for Q4_K only (`two_columns`): the
+// other formats' unpacking does not leave the registers for a second set of operand A, and their spills cost more than
+// the wide form does.  Among the candidates a stage of whole rows comes first (a tile is then one run of whole 128-byte
+// lines, where two half-row stages request the line they meet in twice: 3 % of the traffic; Q4_K at 4096 / 5120 / 6144
+// wide streams at 82 / 85 / 81 % of the HBM peak so, against 74 / 83 / 79 % in half rows), then one column per wave, the
+// larger stage, the waves.
+bool plan_mfma(int block_pieces, int in_w, bool even_waves, bool two_columns, MfmaGeom* out)
 {
     const int nblocks = in_w / 256;
     const int bp = block_pieces;
@@ -1716,7 +1719,7 @@ bool plan_mfma(int block_pieces, int in_w, bool even_waves, MfmaGeom* out)
     double best_score = -1.0;
     MfmaGeom best{};
     for (int W = 6; W <= kMaxWaves; ++W) {
-        for (int m = 1; m <= 2; ++m) {
+        for (int m = 1; m <= (two_columns ? 2 : 1); ++m) {
             MfmaGeom g{};
             if (even_waves && (W & 1)) continue;       // block parity must be wave parity (Q6_K)
             g.waves = W;
@@ -1734,8 +1737,8 @@ bool plan_mfma(int block_pieces, int in_w, bool even_waves, MfmaGeom* out)
             if (!ok) continue;
             g.stages = 2;
             g.lds_bytes = 2 * static_cast<size_t>(g.stage_bytes);
-            // one column per wave keeps the register sets small (no spills); then the larger stage, then the waves
-            const double score = (m == 1 ? 1.0 : 0.0) + static_cast<double>(g.stage_bytes) / (256.0 * 1024) + 1e-3 * W;
+            const double score = (g.kchunks == 1 ? 2.0 : 0.0) + (m == 1 ? 1.0 : 0.0) +
+                                 static_cast<double>(g.stage_bytes) / (256.0 * 1024) + 1e-3 * W;
             if (score > best_score) {
                 best_score = score;
                 best = g;
@@ -1764,8 +1767,11 @@ hipError_t launch_mfma(Lane* lane, const MfmaArgs& a)
     const dim3 grid(groups);
     const int kc = a.g.kchunks, m = a.g.tasks, lpw = a.g.loads_per_wave;
 #define NNHIP_VARIANT(K, MM, L) if (kc == K && m == MM && lpw == L) return launch_mfma_variant<F, K, MM, L>(lane, a, grid);
-    NNHIP_VARIANT(1, 2, 5) NNHIP_VARIANT(1, 2, 6) NNHIP_VARIANT(2, 1, 3) NNHIP_VARIANT(1, 1, 3) NNHIP_VARIANT(2, 2, 5)
-    NNHIP_VARIANT(2, 2, 6) NNHIP_VARIANT(1, 1, 2) NNHIP_VARIANT(2, 1, 2) NNHIP_VARIANT(1, 1, 4) NNHIP_VARIANT(2, 1, 4)
+    if constexpr (std::is_same_v<F, Q4KTask>) {
+        NNHIP_VARIANT(1, 2, 5) NNHIP_VARIANT(1, 2, 6)
+    }
+    NNHIP_VARIANT(2, 1, 3) NNHIP_VARIANT(1, 1, 3) NNHIP_VARIANT(1, 1, 2) NNHIP_VARIANT(2, 1, 2) NNHIP_VARIANT(1, 1, 4)
+    NNHIP_VARIANT(2, 1, 4)
 #undef NNHIP_VARIANT
     return hipErrorInvalidConfiguration;
 }
@@ -1962,7 +1968,7 @@ bool matvec_mfma_geometry(uint32_t type, int in_w, int out_w, const void* w, Mfm
 
     if (!entry_ok(type, in_w, out_w, w)) return false;
     MfmaGeom g;
-    if (!plan_mfma(block_pieces_of(type), in_w, block_bytes_of(type) % 16 != 0, &g)) return false;
+    if (!plan_mfma(block_pieces_of(type), in_w, block_bytes_of(type) % 16 != 0, type == NNHIP_TYPE_Q4_K, &g)) return false;
     if (plan) {
         plan->waves = g.waves;
         plan->cols = g.cols;
@@ -1980,7 +1986,7 @@ hipError_t launch_matvec_mfma_table(Lane* lane, uint32_t type, int in_w, const M
 {
     MfmaArgs a{};
     MfmaGeom g;
-    if (!plan_mfma(block_pieces_of(type), in_w, block_bytes_of(type) % 16 != 0, &g)) return hipErrorInvalidValue;
+    if (!plan_mfma(block_pieces_of(type), in_w, block_bytes_of(type) % 16 != 0, type == NNHIP_TYPE_Q4_K, &g)) return hipErrorInvalidValue;
     fill_args(type, in_w, g, &a);
     a.table = device_entries;
     a.entries = entries;
@@ -2058,7 +2064,7 @@ bool describe_matvec_mfma_launch(uint32_t type, int in_w, int form, bool runs, n
 {
     if (form == 1) {
         MfmaGeom g;
-        if (!plan_mfma(block_pieces_of(type), in_w, block_bytes_of(type) % 16 != 0, &g)) return false;
+        if (!plan_mfma(block_pieces_of(type), in_w, block_bytes_of(type) % 16 != 0, type == NNHIP_TYPE_Q4_K, &g)) return false;
         info->threads = 64 * g.waves;
         info->stage_buffers = g.stages;
         info->dynamic_lds_bytes = static_cast<int32_t>(g.lds_bytes);

@@ -511,6 +511,25 @@ int nnhip_lane_stream(void* handle, void** stream)
     return NNHIP_OK;
 }
 
+int nnhip_lane_set_option(void* handle, uint32_t option, int64_t value)
+{
+    NNHIP_LANE(handle, NNHIP_OP_NONE)
+    if (option != NNHIP_OPTION_ROW_STEP_ONLY)
+        return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_NONE, lane->device, 0, "unknown lane option %u", option);
+    std::lock_guard<std::mutex> guard(lane->mutex);
+    lane->row_step_only = value != 0;
+    return NNHIP_OK;
+}
+
+int nnhip_lane_get_option(void* handle, uint32_t option, int64_t* value)
+{
+    NNHIP_LANE(handle, NNHIP_OP_NONE)
+    if (option != NNHIP_OPTION_ROW_STEP_ONLY || !value)
+        return fail(NNHIP_ERR_INVALID_ARGUMENT, NNHIP_OP_NONE, lane->device, 0, "unknown lane option %u, or value is null", option);
+    *value = lane->row_step_only ? 1 : 0;
+    return NNHIP_OK;
+}
+
 int nnhip_dequantize(void* handle, uint32_t ggml_type, const void* w, float* out, int64_t elements)
 {
     NNHIP_LANE(handle, NNHIP_OP_DEQUANTIZE)
@@ -541,7 +560,7 @@ int nnhip_quant_matvec(void* handle, uint32_t ggml_type, const float* x, const v
     if (in_w > matvec_max_in_w(ggml_type))
         return fail(NNHIP_ERR_TOO_LARGE, NNHIP_OP_MATVEC, lane->device, 0, "in_w %d exceeds the %d values one workgroup can stage", in_w, matvec_max_in_w(ggml_type));
     if (rows > 65535) return fail(NNHIP_ERR_TOO_LARGE, NNHIP_OP_MATVEC, lane->device, 0, "rows %d exceeds 65535", rows);
-    if (const int per_pass = matvec_rows_per_pass(ggml_type, rows, in_w, out_w, w)) {
+    if (const int per_pass = lane->row_step_only ? 0 : matvec_rows_per_pass(ggml_type, rows, in_w, out_w, w)) {
         // two or more input rows of a large matrix: up to four rows share a pass over the weights on the matrix cores,
         // sixteen rows go into a launch (the reference routes such calls to row-tiled kernels,
         // Qwen35QuantizedModel.cs:1335-1344)

@@ -27,6 +27,7 @@ struct Lane {
     int compute_units = 0;
     hipStream_t stream = nullptr;
     bool capturing = false;
+    bool row_step_only = false;                 // NNHIP_OPTION_ROW_STEP_ONLY
     nnhip_lane_counters counters{};
     struct Block { size_t bytes, capacity; };   // bytes asked for; bytes the allocation really has
     std::unordered_map<void*, Block> buffers;   // device allocations handed out and still owned by the lane

@@ -228,6 +228,20 @@ class HipExecutionLane:
                 "peak_allocated_bytes": c.peak_allocated_bytes, "kernel_launches": c.kernel_launches,
                 "driver_allocations": c.driver_allocations}
 
+    # ---- options ----
+    @property
+    def row_step_only(self) -> bool:
+        """Whether every mat-vec of this lane stays on the FP32 row-step kernels, so that a call with several input rows
+        equals stacked single-row calls bit for bit (the property of Qwen35InferencePrefillLinearTests.cs:64-77), at the
+        price of the shared matrix-core passes.  Off when a lane is created."""
+        v = ctypes.c_int64()
+        check(self._lib.nnhip_lane_get_option(self._handle, native.OPTION_ROW_STEP_ONLY, byref(v)), "lane_get_option")
+        return bool(v.value)
+
+    @row_step_only.setter
+    def row_step_only(self, on: bool) -> None:
+        check(self._lib.nnhip_lane_set_option(self._handle, native.OPTION_ROW_STEP_ONLY, 1 if on else 0), "lane_set_option")
+
     # ---- timing / replay ----
     def event(self) -> HipEvent:
         return HipEvent(self)

@@ -13,6 +13,7 @@ from ctypes import POINTER, Structure, byref, c_char_p, c_float, c_int, c_int32,
 from pathlib import Path
 
 ABI_MAJOR = 1
+OPTION_ROW_STEP_ONLY = 1   # nnhip_lane_set_option: every mat-vec on the FP32 row-step kernels
 
 STATUS_NAMES = {
     0: "OK", 1: "INVALID_ARGUMENT", 2: "UNSUPPORTED_TYPE", 3: "INCOMPLETE_BLOCKS", 4: "OUT_OF_MEMORY", 5: "HIP",
@@ -91,6 +92,8 @@ PROTOTYPES = {
     "nnhip_synchronize": (c_int, [c_void_p]),
     "nnhip_lane_get_counters": (c_int, [c_void_p, POINTER(LaneCounters), c_size_t]),
     "nnhip_lane_stream": (c_int, [c_void_p, POINTER(c_void_p)]),
+    "nnhip_lane_set_option": (c_int, [c_void_p, c_uint32, c_int64]),
+    "nnhip_lane_get_option": (c_int, [c_void_p, c_uint32, POINTER(c_int64)]),
     "nnhip_dequantize": (c_int, [c_void_p, c_uint32, c_void_p, c_void_p, c_int64]),
     "nnhip_quant_matvec": (c_int, [c_void_p, c_uint32, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int]),
     "nnhip_matvec_plan": (c_int, [c_uint32, c_int, c_int, c_int, c_int, POINTER(MatvecPlanInfo)]),

@@ -806,3 +806,64 @@ def test_several_input_rows_share_a_pass_in_a_single_call(lane, typ):
         b.dispose()
     mat.dispose()
     lane.trim()
+
+
+@pytest.mark.parametrize("typ", [GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_Q8_0, GGML_IQ2_S, GGML_IQ3_S])
+@pytest.mark.parametrize("in_w,out_w", [(5120, 17408), (17408, 5120)])
+def test_row_step_only_lane_keeps_rows_equal_to_stacked_single_rows_bitwise(typ, in_w, out_w):
+    """The property NNtrain.Core.Tests/Qwen35InferencePrefillLinearTests.cs:64-77 asserts for the reference's row-tiled
+    kernels, on the two large shapes where a lane otherwise shares matrix-core passes between input rows: with
+    NNHIP_OPTION_ROW_STEP_ONLY set, rows in {2, 4, 9, 16} give, row for row, the bits of the rows == 1 call, through the
+    single entry point and through a batch; the same lane with the option cleared goes back to the shared passes (other
+    bits, same bars).  Oracle bars on the sixteen-row result."""
+    payload = synth.matrix(typ, out_w, in_w, seed=1300 + typ)
+    x = synth.activations(16, in_w, seed=77)
+    x[3] *= 2e3
+    bias = np.random.default_rng(4).standard_normal(out_w).astype(np.float32)
+    with HipExecutionLane(0) as lane:
+        assert lane.row_step_only is False
+        lane.row_step_only = True
+        assert lane.row_step_only is True
+        mat = HipQuantizedMatrix(payload, typ, out_w, in_w)
+        mat.device_payload(lane)
+        bd = lane.upload_raw(bias)
+        xd = lane.upload_raw(x)
+        yd = lane.allocate(16 * out_w)
+        singles = np.empty((16, out_w), np.float32)
+        for r in range(16):
+            check(lane._lib.nnhip_quant_matvec(lane._handle, typ, c_void_p(xd.ptr + 4 * r * in_w), c_void_p(mat.device_payload(lane).ptr),
+                                               c_void_p(bd.ptr), c_void_p(yd.ptr), 1, in_w, out_w), "quant_matvec")
+            singles[r] = lane.read(yd, np.float32, out_w)
+        for rows in (2, 4, 9, 16):
+            lane.fill_u32(yd, NAN_BITS, 16 * out_w)
+            launches = lane.counters()["kernel_launches"]
+            mat.forward(lane, xd, bd, rows, out=yd)
+            y = lane.read(yd, np.float32, rows * out_w).reshape(rows, out_w)
+            assert lane.counters()["kernel_launches"] - launches == 1
+            assert np.array_equal(_bits(y), _bits(singles[:rows])), rows
+        ref, asum = oracle.linear_f64(typ, payload, x, bias, 16, in_w, out_w)
+        assert oracle.rel_l2(singles, ref) <= MATVEC_BAR
+        assert np.all(np.abs(singles.astype(np.float64) - ref) <= 2e-6 + 3e-6 * asum)
+        # a batch of three descriptors (1, 4 and 9 input rows of the same matrix) has the same bits as well
+        outs = [lane.allocate(n * out_w) for n in (1, 4, 9)]
+        descs = (MatvecDesc * 3)()
+        for i, n in enumerate((1, 4, 9)):
+            descs[i] = MatvecDesc(xd.ptr, mat.device_payload(lane).ptr, bd.ptr, outs[i].ptr, typ, n, in_w, out_w)
+        check(lane._lib.nnhip_quant_matvec_batch(lane._handle, descs, 3), "quant_matvec_batch")
+        for i, n in enumerate((1, 4, 9)):
+            assert np.array_equal(_bits(lane.read(outs[i], np.float32).reshape(n, out_w)), _bits(singles[:n])), n
+        # option cleared: the shared passes are back
+        lane.row_step_only = False
+        mat.forward(lane, xd, bd, 16, out=yd)
+        y = lane.read(yd, np.float32).reshape(16, out_w)
+        assert oracle.rel_l2(y, ref) <= MATVEC_BAR
+        from nntrain_amd import native
+        info = native.MatvecPlanInfo(struct_size=ctypes.sizeof(native.MatvecPlanInfo))
+        assert lane._lib.nnhip_matvec_plan(typ, 16, in_w, out_w, 256, ctypes.byref(info)) == 0
+        # (Q8_0 rows of 17408 values stay with the row-tiled kernel either way)
+        assert np.array_equal(_bits(y), _bits(singles)) == (info.kernel != 2)
+        with pytest.raises(Exception):
+            check(lane._lib.nnhip_lane_set_option(lane._handle, 99, 1), "lane_set_option")
+        for b in outs + [bd, xd, yd]:
+            b.dispose()
+        mat.dispose()
