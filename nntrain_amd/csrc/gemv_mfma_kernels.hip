@@ -76,6 +76,7 @@ struct MfmaGeom {
     int loads_per_wave;   // ceil(stage_loads / W)
     int stages;           // LDS stage buffers (2)
     int tasks;            // M: super-block columns a wave owns per stage
+    int one_set;          // 1: one register set on its way instead of two (stages of whole rows, see the kernel)
     size_t lds_bytes;     // the stage buffers
 };
 
@@ -89,6 +90,7 @@ struct MfmaArgs {
     int nblocks;                   // super-blocks per row
     uint32_t row_bytes;
     uint32_t row_pieces_magic;     // ceil(2^32 / row_pieces)
+    uint32_t used_pieces_magic;    // ceil(2^32 / (cols * pieces per block)): the pieces of a stage row that are blocks
     int chunked;                   // 1: a workgroup takes a run of consecutive tiles, 0: every G-th tile
     MfmaGeom g;
 };
@@ -189,6 +191,7 @@ struct Q4KTask {
     static constexpr int kBlockBytes = kQ4KBytes;     // 144 = 9 pieces; blocks and rows are 16-byte aligned
     static constexpr int kLdsTableBytes = 0;          // no lookup tables in LDS
     static constexpr int kPieces = 9;                 // 16-byte pieces a block takes in a stage
+    static constexpr bool kWholePieces = true;        // a row of blocks is a row of pieces, nothing else
     static constexpr int kSumRun = 32;                // activations per FP32 sum (one sub-block)
     static constexpr int kWideM = 1;                  // wide form: block columns per wave and stage,
     static constexpr int kWideLpw = 3;                // and 1 KB pieces per wave and stage (W <= 12)
@@ -308,6 +311,7 @@ struct Q5KTask {
     static constexpr int kBlockBytes = kQ5KBytes;
     static constexpr int kLdsTableBytes = 0;          // no lookup tables in LDS
     static constexpr int kPieces = 11;
+    static constexpr bool kWholePieces = true;
     static constexpr int kSumRun = 32;
     static constexpr int kWideM = 1;
     static constexpr int kWideLpw = 3;
@@ -906,6 +910,9 @@ struct IQ3STask {
     }
 };
 
+template <class F, class = void> struct WholePieces { static constexpr bool value = false; };
+template <class F> struct WholePieces<F, std::enable_if_t<F::kWholePieces>> { static constexpr bool value = true; };
+
 // Loads of the weight stream: 16 bytes per lane through a buffer descriptor that spans the matrix, non-temporal.  An
 // offset beyond the buffer returns zeros without touching memory.
 __device__ __forceinline__ u32x4 stream16(__amdgpu_buffer_rsrc_t matrix, uint32_t off)
@@ -916,10 +923,19 @@ __device__ __forceinline__ u32x4 stream16(__amdgpu_buffer_rsrc_t matrix, uint32_
 // grid.x = workgroups striding over the launch's 16-row tiles, blockDim.x = 64 * W.  KC = stages per tile (1 or 2),
 // M = super-block columns a wave owns per stage, LPW = 1 KB pieces of a stage a wave moves.  A lane keeps operand A of its KC * M columns in registers for as long as the activations stay
 // the same.
-template <class F, int KC, int M, int LPW>
+// ONESET (stages of whole rows, two columns per wave, for the formats whose unpacking leaves no registers for two sets):
+// a wave has one set of pieces on its way.  It parks the set at the end of a stage and asks for the stage after next
+// into the same registers, so one stage (as many bytes as two half-row stages) travels while one is multiplied.
+template <class F, int KC, int M, int LPW, bool ONESET = false>
 __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_kernel(MfmaArgs a)
 {
     static_assert(KC == 1 || KC == 2, "a turn of the two register sets is one or two tiles");
+    static_assert(!ONESET || KC == 1, "one register set is for stages of whole rows");
+    // A stage of whole rows of whole pieces is one run of memory: the wave's 1 KB requests are then cut on 1 KB
+    // boundaries of the tile (whole 128-byte lines, each asked for once; cut by the padded LDS rows instead, one request
+    // in ten shares a line with its neighbour's and 1 % of the lines came in twice), and each lane parks its piece at
+    // the padded place.
+    constexpr bool kLinear = KC == 1 && WholePieces<F>::value;
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
     __shared__ float part[2][kMaxWaves][kTileRows];
     __shared__ uint32_t red[kMaxWaves];
@@ -954,14 +970,23 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_kernel(MfmaArgs a)
     // not exist get an offset beyond any matrix and read as zeros.
     const int pieces_used = g.cols * F::kPieces;
     uint32_t rel[LPW];
+    uint32_t lds_at[kLinear ? LPW : 1];      // kLinear: where the piece is parked (kNoPiece: nowhere)
 #pragma unroll
     for (int i = 0; i < LPW; ++i) {
         const uint32_t slot = static_cast<uint32_t>(64 * (wave + W * i) + lane);
-        const uint32_t r = __umulhi(slot, a.row_pieces_magic);
-        const uint32_t q = slot - r * static_cast<uint32_t>(g.row_pieces);
-        const uint32_t c = q / static_cast<uint32_t>(F::kPieces);
-        const bool real = r < static_cast<uint32_t>(kTileRows) && q < static_cast<uint32_t>(pieces_used);
-        rel[i] = real ? r * a.row_bytes + c * F::kBlockBytes + F::piece_src(q - c * F::kPieces, c & 1u) : kNoPiece;
+        if constexpr (kLinear) {
+            const uint32_t r = __umulhi(slot, a.used_pieces_magic);
+            const uint32_t q = slot - r * static_cast<uint32_t>(pieces_used);
+            const bool real = r < static_cast<uint32_t>(kTileRows);
+            rel[i] = real ? 16u * slot : kNoPiece;
+            lds_at[i] = real ? 16u * (r * static_cast<uint32_t>(g.row_pieces) + q) : kNoPiece;
+        } else {
+            const uint32_t r = __umulhi(slot, a.row_pieces_magic);
+            const uint32_t q = slot - r * static_cast<uint32_t>(g.row_pieces);
+            const uint32_t c = q / static_cast<uint32_t>(F::kPieces);
+            const bool real = r < static_cast<uint32_t>(kTileRows) && q < static_cast<uint32_t>(pieces_used);
+            rel[i] = real ? r * a.row_bytes + c * F::kBlockBytes + F::piece_src(q - c * F::kPieces, c & 1u) : kNoPiece;
+        }
     }
 
     // ---- the stage sequence of this workgroup: tiles blockIdx.x, blockIdx.x + G, ... of the launch's tile sequence,
@@ -1039,7 +1064,14 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_kernel(MfmaArgs a)
         // (a buffer has room for all W * LPW pieces; those past the stage's last are zeros nobody reads)
         uint8_t* dst = buf + wave * 1024 + lane * 16;
 #pragma unroll
-        for (int i = 0; i < LPW; ++i) *reinterpret_cast<u32x4*>(dst + W * i * 1024) = set[i];
+        for (int i = 0; i < LPW; ++i) {
+            if constexpr (kLinear) {
+                if (lds_at[i] != kNoPiece) *reinterpret_cast<u32x4*>(buf + lds_at[i]) = set[i];
+            } else {
+                // (ONESET: the buffers end with the stage's last piece)
+                if (!ONESET || wave + W * i < g.stage_loads) *reinterpret_cast<u32x4*>(dst + W * i * 1024) = set[i];
+            }
+        }
     };
 
     // ---- consume side
@@ -1126,10 +1158,10 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_kernel(MfmaArgs a)
     uint8_t* const buf0 = smem;
     uint8_t* const buf1 = smem + g.stage_bytes;
     // (a third register set, three stages on their way, was measured without gain)
-    u32x4 regs[2][LPW];
+    u32x4 regs[ONESET ? 1 : 2][LPW];
     fetch_enter();
     fetch(regs[0]);
-    fetch(regs[1]);
+    if constexpr (!ONESET) fetch(regs[1]);
 
     const uint32_t row_off = static_cast<uint32_t>(row_l) * (static_cast<uint32_t>(g.row_pieces) * 16u) +
                              static_cast<uint32_t>(wave) * (16u * F::kPieces);
@@ -1171,7 +1203,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_kernel(MfmaArgs a)
                 new_x = ce.x != regs_x;
             }
         }
-        fetch(refill);                  // (before the activations are dealt with: the stream must not pause for them)
+        if constexpr (!ONESET) fetch(refill);      // (before the activations are dealt with: the stream must not pause for them)
         if (k == 0 && new_x) prepare_x(nxt);
         if (done) finalize();
         const uint8_t* stage = cur + row_off;
@@ -1195,15 +1227,17 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_kernel(MfmaArgs a)
             c_t += t_step;
         }
         park(nxt, landing);
+        if constexpr (ONESET) fetch(refill);
         __syncthreads();                // publishes `nxt`, frees `cur`
     };
 
     park(buf0, regs[0]);
+    if constexpr (ONESET) fetch(regs[0]);
     __syncthreads();
     using std::integral_constant;
     for (int n = 0; n < total; n += 2) {
-        stage_step(integral_constant<int, 0>{}, buf0, buf1, regs[0], regs[1]);
-        if (n + 1 < total) stage_step(integral_constant<int, KC - 1>{}, buf1, buf0, regs[1], regs[0]);
+        stage_step(integral_constant<int, 0>{}, buf0, buf1, regs[0], regs[ONESET ? 0 : 1]);
+        if (n + 1 < total) stage_step(integral_constant<int, KC - 1>{}, buf1, buf0, regs[ONESET ? 0 : 1], regs[0]);
     }
     if (done) finalize();
 }
@@ -1701,16 +1735,19 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
 // The (KC, M, LPW) combinations the kernel is instantiated for.
 struct Variant { int kc, m, lpw; };
 constexpr Variant kVariants[] = {{1, 2, 5}, {1, 2, 6}, {2, 1, 3}, {1, 1, 3}, {1, 1, 2}, {2, 1, 2}, {1, 1, 4}, {2, 1, 4}};
+constexpr Variant kOneSetVariants[] = {{1, 2, 6}};
 
 // Picks W and C for (block bytes, in_w).  C = W * M columns per stage must divide the row's super-blocks into KC whole
 // stages, two stage buffers must fit LDS (one of them doubles as scratch for the digit planes when the activations
-// change), (KC, M, LPW) must be an instantiated variant.  Two columns per wave are for Q4_K only (`two_columns`): the
-// other formats' unpacking does not leave the registers for a second set of operand A, and their spills cost more than
-// the wide form does.  Among the candidates a stage of whole rows comes first (a tile is then one run of whole 128-byte
+// change), (KC, M, LPW) must be an instantiated variant.  Two columns per wave (`two_columns`) are for stages of whole
+// rows only: with two register sets on their way for Q4_K (1), with one set for Q5_K (2), whose unpacking does not leave
+// the registers for both a second set of operand A and a second set of pieces (spills cost more than the wide form
+// does; Q5_K at 5120 wide streams at 83 - 84 % of the HBM peak so, against 80 % in half rows; Q6_K gained nothing from
+// either and stays with one column).  Among the candidates a stage of whole rows comes first (a tile is then one run of whole 128-byte
 // lines, where two half-row stages request the line they meet in twice: 3 % of the traffic; Q4_K at 4096 / 5120 / 6144
 // wide streams at 82 / 85 / 81 % of the HBM peak so, against 74 / 83 / 79 % in half rows), then one column per wave, the
 // larger stage, the waves.
-bool plan_mfma(int block_pieces, int in_w, bool even_waves, bool two_columns, MfmaGeom* out)
+bool plan_mfma(int block_pieces, int in_w, bool even_waves, int two_columns, bool whole_pieces, MfmaGeom* out)
 {
     const int nblocks = in_w / 256;
     const int bp = block_pieces;
@@ -1728,12 +1765,23 @@ bool plan_mfma(int block_pieces, int in_w, bool even_waves, bool two_columns, Mf
             g.kchunks = nblocks / g.cols;
             g.tasks = m;
             g.row_pieces = (g.cols * bp) | 1;
-            g.stage_loads = (kTileRows * g.row_pieces + 63) / 64;
+            // (stages of whole rows of whole pieces are requested as the run of memory they are, without the padding)
+            const bool linear = whole_pieces && g.kchunks == 1;
+            g.stage_loads = (kTileRows * (linear ? g.cols * bp : g.row_pieces) + 63) / 64;
             g.loads_per_wave = (g.stage_loads + W - 1) / W;
-            g.stage_bytes = g.loads_per_wave * W * 1024;          // every wave parks loads_per_wave pieces
+            g.one_set = m == 2 && two_columns == 2 ? 1 : 0;
+            if (m == 2 && g.kchunks != 1) continue;
+            if (g.one_set && W > 10) continue;          // (measured: twelve waves stream faster in half rows with two sets)
+            // every wave parks loads_per_wave pieces (one set: only those the stage has)
+            g.stage_bytes = linear ? (kTileRows * g.row_pieces * 16 + 1023) / 1024 * 1024
+                                   : (g.one_set ? g.stage_loads : g.loads_per_wave * W) * 1024;
             if (g.stage_bytes < planes_bytes || 2 * g.stage_bytes > kLdsBudget) continue;
             bool ok = false;
-            for (const Variant& v : kVariants) ok = ok || (v.kc == g.kchunks && v.m == m && v.lpw == g.loads_per_wave);
+            if (g.one_set) {
+                for (const Variant& v : kOneSetVariants) ok = ok || (v.kc == g.kchunks && v.m == m && v.lpw == g.loads_per_wave);
+            } else {
+                for (const Variant& v : kVariants) ok = ok || (v.kc == g.kchunks && v.m == m && v.lpw == g.loads_per_wave);
+            }
             if (!ok) continue;
             g.stages = 2;
             g.lds_bytes = 2 * static_cast<size_t>(g.stage_bytes);
@@ -1750,13 +1798,13 @@ bool plan_mfma(int block_pieces, int in_w, bool even_waves, bool two_columns, Mf
     return true;
 }
 
-template <class F, int KC, int M, int LPW>
+template <class F, int KC, int M, int LPW, bool ONESET = false>
 hipError_t launch_mfma_variant(Lane* lane, const MfmaArgs& a, dim3 grid)
 {
     static LdsLimit big_lds;
-    const hipError_t e = big_lds.ensure(lane->device, reinterpret_cast<const void*>(&matvec_mfma_kernel<F, KC, M, LPW>), kLdsBudget);
+    const hipError_t e = big_lds.ensure(lane->device, reinterpret_cast<const void*>(&matvec_mfma_kernel<F, KC, M, LPW, ONESET>), kLdsBudget);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((matvec_mfma_kernel<F, KC, M, LPW>), grid, dim3(64 * a.g.waves), a.g.lds_bytes, lane->stream, a);
+    hipLaunchKernelGGL((matvec_mfma_kernel<F, KC, M, LPW, ONESET>), grid, dim3(64 * a.g.waves), a.g.lds_bytes, lane->stream, a);
     return hipGetLastError();
 }
 
@@ -1769,6 +1817,8 @@ hipError_t launch_mfma(Lane* lane, const MfmaArgs& a)
 #define NNHIP_VARIANT(K, MM, L) if (kc == K && m == MM && lpw == L) return launch_mfma_variant<F, K, MM, L>(lane, a, grid);
     if constexpr (std::is_same_v<F, Q4KTask>) {
         NNHIP_VARIANT(1, 2, 5) NNHIP_VARIANT(1, 2, 6)
+    } else if constexpr (std::is_same_v<F, Q5KTask>) {
+        if (a.g.one_set && kc == 1 && m == 2 && lpw == 6) return launch_mfma_variant<F, 1, 2, 6, true>(lane, a, grid);
     }
     NNHIP_VARIANT(2, 1, 3) NNHIP_VARIANT(1, 1, 3) NNHIP_VARIANT(1, 1, 2) NNHIP_VARIANT(2, 1, 2) NNHIP_VARIANT(1, 1, 4)
     NNHIP_VARIANT(2, 1, 4)
@@ -1942,6 +1992,8 @@ void fill_args(uint32_t type, int in_w, const MfmaGeom& g, MfmaArgs* a)
     a->nblocks = in_w / 256;
     a->row_bytes = static_cast<uint32_t>(a->nblocks) * static_cast<uint32_t>(block_bytes_of(type));
     a->row_pieces_magic = static_cast<uint32_t>((0x100000000ull + g.row_pieces - 1) / g.row_pieces);
+    const uint32_t used = static_cast<uint32_t>(g.cols) * static_cast<uint32_t>(block_pieces_of(type));
+    a->used_pieces_magic = static_cast<uint32_t>((0x100000000ull + used - 1) / used);
 }
 
 }  // namespace
@@ -1968,7 +2020,8 @@ bool matvec_mfma_geometry(uint32_t type, int in_w, int out_w, const void* w, Mfm
 
     if (!entry_ok(type, in_w, out_w, w)) return false;
     MfmaGeom g;
-    if (!plan_mfma(block_pieces_of(type), in_w, block_bytes_of(type) % 16 != 0, type == NNHIP_TYPE_Q4_K, &g)) return false;
+    if (!plan_mfma(block_pieces_of(type), in_w, block_bytes_of(type) % 16 != 0, type == NNHIP_TYPE_Q4_K ? 1 : type == NNHIP_TYPE_Q5_K ? 2 : 0,
+                   type == NNHIP_TYPE_Q4_K || type == NNHIP_TYPE_Q5_K, &g)) return false;
     if (plan) {
         plan->waves = g.waves;
         plan->cols = g.cols;
@@ -1986,7 +2039,8 @@ hipError_t launch_matvec_mfma_table(Lane* lane, uint32_t type, int in_w, const M
 {
     MfmaArgs a{};
     MfmaGeom g;
-    if (!plan_mfma(block_pieces_of(type), in_w, block_bytes_of(type) % 16 != 0, type == NNHIP_TYPE_Q4_K, &g)) return hipErrorInvalidValue;
+    if (!plan_mfma(block_pieces_of(type), in_w, block_bytes_of(type) % 16 != 0, type == NNHIP_TYPE_Q4_K ? 1 : type == NNHIP_TYPE_Q5_K ? 2 : 0,
+                   type == NNHIP_TYPE_Q4_K || type == NNHIP_TYPE_Q5_K, &g)) return hipErrorInvalidValue;
     fill_args(type, in_w, g, &a);
     a.table = device_entries;
     a.entries = entries;
@@ -2064,7 +2118,8 @@ bool describe_matvec_mfma_launch(uint32_t type, int in_w, int form, bool runs, n
 {
     if (form == 1) {
         MfmaGeom g;
-        if (!plan_mfma(block_pieces_of(type), in_w, block_bytes_of(type) % 16 != 0, type == NNHIP_TYPE_Q4_K, &g)) return false;
+        if (!plan_mfma(block_pieces_of(type), in_w, block_bytes_of(type) % 16 != 0, type == NNHIP_TYPE_Q4_K ? 1 : type == NNHIP_TYPE_Q5_K ? 2 : 0,
+                   type == NNHIP_TYPE_Q4_K || type == NNHIP_TYPE_Q5_K, &g)) return false;
         info->threads = 64 * g.waves;
         info->stage_buffers = g.stages;
         info->dynamic_lds_bytes = static_cast<int32_t>(g.lds_bytes);
