@@ -867,3 +867,53 @@ def test_row_step_only_lane_keeps_rows_equal_to_stacked_single_rows_bitwise(typ,
         for b in outs + [bd, xd, yd]:
             b.dispose()
         mat.dispose()
+
+
+@pytest.mark.parametrize("typ", [GGML_Q4_K, GGML_Q5_K])
+@pytest.mark.parametrize("in_w", [1536, 2048, 3072, 3584, 4096, 4608, 5632, 6144, 7168, 8192])
+def test_matrix_core_stage_geometries_over_row_lengths(lane, typ, in_w):
+    """Every row length picks its own stage geometry on the matrix cores: whole rows per stage with one or two block
+    columns per wave (requested as 1 KB runs of whole memory lines and parked at padded LDS rows), half rows, or the
+    wide form for rows that are neither.  A group large enough for the matrix cores at each of them, with a ragged last
+    tile, bias and a second matrix of another height: first and last rows of the big matrix and the whole small one
+    against the float64 oracle at both bars, guard words behind the outputs, and the big matrix' bits do not depend on
+    the company."""
+    out_w = 33000 + 7
+    small_w = 16 * 3 + 5
+    payload = synth.matrix(typ, out_w, in_w, seed=4000 + in_w + typ)
+    small = synth.matrix(typ, small_w, in_w, seed=4001 + in_w + typ)
+    rng = np.random.default_rng(in_w + typ)
+    x = rng.standard_normal((1, in_w)).astype(np.float32)
+    bias = rng.standard_normal(out_w).astype(np.float32)
+    xd, bd = lane.upload_raw(x), lane.upload_raw(bias)
+    items = [dict(typ=typ, in_w=in_w, out_w=out_w, rows=1, payload=payload, x=x, xd=xd, bias=bias, wd=lane.upload_raw(payload), bd=bd,
+                  yd=lane.allocate(out_w + 2)),
+             dict(typ=typ, in_w=in_w, out_w=small_w, rows=1, payload=small, x=x, xd=xd, bias=None, wd=lane.upload_raw(small), bd=None,
+                  yd=lane.allocate(small_w + 2))]
+    info = (BatchLaunchInfo * 4)()
+    for i in range(4):
+        info[i].struct_size = ctypes.sizeof(BatchLaunchInfo)
+    descs = (MatvecDesc * 2)()
+    for i, it in enumerate(items):
+        descs[i] = MatvecDesc(it["xd"].ptr, it["wd"].ptr, it["bd"].ptr if it["bd"] else None, it["yd"].ptr, typ, 1, in_w, it["out_w"])
+    n = ctypes.c_int()
+    check(lane._lib.nnhip_matvec_batch_plan(descs, 2, 256, info, 4, ctypes.byref(n)), "matvec_batch_plan")
+    assert n.value == 1 and info[0].kernel == 2, "the group was meant for the matrix cores"
+    got = _batch_run(lane, items)
+    row_bytes = payload.size // out_w
+    y = got[0][0]
+    for r0, cnt in ((0, 80), (out_w - 87, 87)):
+        ref, asum = oracle.linear_f64(typ, payload[r0 * row_bytes:(r0 + cnt) * row_bytes], x, bias[r0:r0 + cnt], 1, in_w, cnt)
+        assert oracle.rel_l2(y[r0:r0 + cnt], ref[0]) <= MATVEC_BAR, (in_w, r0)
+        assert np.all(np.abs(y[r0:r0 + cnt].astype(np.float64) - ref[0]) <= 2e-6 + 3e-6 * asum[0]), (in_w, r0)
+    ref, asum = oracle.linear_f64(typ, small, x, None, 1, in_w, small_w)
+    assert np.all(np.abs(got[1][0].astype(np.float64) - ref[0]) <= 2e-6 + 3e-6 * asum[0])
+    assert np.all(np.isfinite(y))
+    alone = _batch_run(lane, items[:1])
+    assert np.array_equal(_bits(alone[0]), _bits(got[0]))
+    for it in items:
+        it["wd"].dispose()
+        it["yd"].dispose()
+    xd.dispose()
+    bd.dispose()
+    lane.trim()
