@@ -426,7 +426,7 @@ def run_gemv(args, lane, nn, oracle):
             # several input rows in one call (weights rotated as above): microseconds per call, up to four rows sharing a
             # pass over the weights (Q8_0 with two rows: its row-tiled lane-per-unit kernel; otherwise the matrix cores)
             per_rows = {}
-            for rows in (2, 4, 8):
+            for rows in (2, 4, 8, 16):
                 xr = lane.upload_raw(synth.activations(rows, in_w, xseed + rows))
                 yr = lane.allocate(rows * out_w)
 

@@ -1264,7 +1264,7 @@ bool describe_rowstep(int rows, int in_w, int out_w, int compute_units, nnhip_ma
 bool describe_matvec(uint32_t type, int rows, int in_w, int out_w, int compute_units, nnhip_matvec_plan_info* info)
 {
     // (the plan is made without the weight pointer: the matrix-core path also needs it 16-byte aligned)
-    if (const int per_pass = matvec_rows_per_pass(type, rows, in_w, out_w, nullptr))
+    if (const int per_pass = matvec_rows_per_pass(type, rows, in_w, out_w, nullptr, compute_units))
         return describe_matvec_rows_shared(type, rows, in_w, out_w, per_pass, compute_units, info);
     if (type == NNHIP_TYPE_Q8_0 && ((in_w / 32) & 1)) {
         info->kernel = NNHIP_MATVEC_KERNEL_Q8_0_ODD_BLOCKS;
@@ -1679,12 +1679,24 @@ int plan_matvec_batch(const nnhip_matvec_desc* descs, int count, int compute_uni
     return n;
 }
 
-int matvec_rows_per_pass(uint32_t type, int rows, int in_w, int out_w, const void* w)
+int matvec_rows_per_pass(uint32_t type, int rows, int in_w, int out_w, const void* w, int compute_units)
 {
     if (rows < shared_pass_min_rows(type)) return 0;
     const long work = static_cast<long>(rows) * ((out_w + 15) / 16);
     const long floor = rows >= 3 && type != NNHIP_TYPE_Q8_0 ? kSharedPassMinTiles : kMfmaBatchMinTiles;
     if (work >= floor && matvec_mfma_wide_geometry(type, in_w, out_w, w, 4)) return 4;
+    // Rows too long for four sets of activation planes in LDS (more than about 8700 values): shared passes in the split
+    // form, the planes of one group of block columns at a time.
+    // It pays from three and a half rounds of (16 matrix rows x 4 input rows) over the workgroups on (IQ2_S: two and a
+    // half): fewer leave compute units idle in the last round, and every change of entry costs a workgroup a conversion
+    // per part, while a pass per input row deals four times as many tiles.  IQ3_S, whose codebook lookups a shared
+    // pass makes once for four rows, gains from three rows on.  Measured on 5120 x 17408, us per call, shared against a
+    // pass per row: Q4_K 8 rows 85 / 68, 9 rows 69 / 89, 16 rows 77 / 136; IQ2_S 4 rows 49 / 46, 8 rows 77 / 89, 16 rows
+    // 91 / 173; IQ3_S 4 rows 53 / 64, 16 rows 98 / 242; on 17408 x 14336 Q4_K 4 rows 67 / 82, 16 rows 233 / 332.
+    const long shared_units = static_cast<long>((rows + 3) / 4) * ((out_w + 15) / 16);
+    const long shared_floor = type == NNHIP_TYPE_IQ3_S ? 0 : type == NNHIP_TYPE_IQ2_S ? 5L * compute_units : 7L * compute_units;
+    if (work >= floor && 2 * shared_units >= shared_floor && matvec_mfma_split_geometry(type, in_w, out_w, w, compute_units))
+        return 4;
     // Rows too long for four sets of activation planes in LDS (more than about 8700 values): the super-block formats
     // still stream faster on the matrix cores, one pass per input row (Q8_0's row-step kernel multiplies four input rows
     // per pass and stays).

@@ -1275,14 +1275,27 @@ struct WideArgs {
     uint32_t row_bytes;
     uint32_t row_pieces_magic;
     int chunked;                   // 1: a workgroup takes consecutive tiles (few changes of activations), 0: every G-th
+    int parts, part_stages;        // SPLIT: a row's stages are taken in `parts` groups of `part_stages` (see the kernel)
     WideGeom g;
     MfmaEntry inline_entries[4];   // a call with up to 16 input rows needs no table in device memory
 };
 
-template <class F, int M, int LPW, int R, bool ONE = false>
+// SPLIT: most tiles of one table entry that a workgroup may meet (their sums wait in LDS from part to part)
+constexpr int kSplitUnits = 8;
+
+// SPLIT (shared passes over rows too long for R full sets of planes in LDS): the stages of a tile are taken in `parts`
+// groups of `part_stages`, and LDS holds the planes of one group of block columns at a time.  A workgroup works through
+// its tiles of a table entry once per part: planes of part 0 (with a fixed-point scale of their own), that part of
+// every tile, planes of part 1, ...; the sums of a tile wait in LDS (bias + part 0, + part 1, ...: one order, so the
+// bits of a row depend on its weights, its activations and the launch geometry only) and are stored after the last part.
+// Every stage of every tile is still requested and multiplied once; what is paid is a conversion of the activations
+// per entry and workgroup, as before, now in `parts` pieces.
+template <class F, int M, int LPW, int R, bool ONE = false, bool SPLIT = false>
 __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideArgs a)
 {
+    static_assert(!SPLIT || (!ONE && R > 1), "parts are for shared passes with two stage buffers");
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+    __shared__ float split_sums[SPLIT ? kSplitUnits : 1][R][kTileRows];   // SPLIT: a tile's sums between its parts
     __shared__ float part[2][R][kMaxWaves][kTileRows];
     __shared__ uint32_t red[R][kMaxWaves];
     __shared__ float inv_of_row[R];                                       // 2^-e of each input row's fixed-point scale
@@ -1349,10 +1362,10 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
     const int t_end = a.chunked ? t_first + my_tiles : a.total_tiles;       // no requests from here on
     const int total = my_tiles * KC;
     const uint32_t chunk_bytes = static_cast<uint32_t>(g.cols) * F::kBlockBytes;
-    const int n4 = a.in_w >> 2;
 
     // ---- prefetch side
     int f_t = t_first, f_k = 0, f_m = 0;
+    int f_p = 0, f_first = t_first, f_end = 0;           // SPLIT: part, first tile and end of the run of tiles of one entry
     if (a.chunked && my_tiles > 0) {
         // the entry that holds this workgroup's first tile: the last one whose first_tile is not beyond it (a run may
         // start hundreds of entries into the table, and walking there costs a trip to memory per entry)
@@ -1378,7 +1391,27 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
         const bool tail = f_k == KC - 1;
 #pragma unroll
         for (int i = 0; i < LPW; ++i) set[i] = stream16(f_matrix, tail && !((in_tail >> i) & 1u) ? kNoPiece : base + rel[i]);
-        if (++f_k == KC) {
+        if constexpr (SPLIT) {
+            const int part_end = (f_p + 1) * a.part_stages < KC ? (f_p + 1) * a.part_stages : KC;
+            if (++f_k == part_end) {
+                f_t += t_step;
+                if (f_t < f_end) {                       // the same part of the entry's next tile
+                    f_k = f_p * a.part_stages;
+                } else if (f_p + 1 < a.parts) {          // the next part, from the run's first tile again
+                    ++f_p;
+                    f_t = f_first;
+                    f_k = f_p * a.part_stages;
+                } else {                                 // the next entry
+                    f_p = 0;
+                    f_first = f_t;
+                    f_k = 0;
+                    if (f_t < t_end) {
+                        fetch_enter();
+                        f_end = fe.first_tile + fe.tiles < t_end ? fe.first_tile + fe.tiles : t_end;
+                    }
+                }
+            }
+        } else if (++f_k == KC) {
             f_k = 0;
             f_t += t_step;
             if (f_t < t_end && f_t >= fe.first_tile + fe.tiles) fetch_enter();
@@ -1402,6 +1435,10 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
     uint8_t* const planes = smem + (ONE ? 1 : 2) * g.stage_bytes;
     F::init_tables(tables, tid, T);
     int c_t = t_first, c_k = 0, c_m = m_first - 1;      // (ce.tiles == 0: the first stage enters entry m_first)
+    // SPLIT: part, first tile and end of the run of this workgroup's tiles of one entry, the tile's number in the run,
+    // whether the stage about to be multiplied is the first of a part (its planes have to be made)
+    int c_p = 0, c_first = t_first, c_end = 0, c_u = 0;
+    bool c_part_start = true;
     MfmaEntry ce{};
     float inv[R] = {};
     const float* planes_x = nullptr;       // the vector(s) the planes in LDS were made from
@@ -1414,7 +1451,11 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
     // Every wave has left the stage that last read the planes when this runs.  (Requesting the whole vector at once into
     // registers, one trip to memory instead of two, made the compiler wait for every outstanding load before each
     // parking write of the main loop in the one-row form: 12.6 instead of 8.6 us per 17408-wide Q4_K mat-vec.)
+    // (SPLIT: of the block columns of part c_p only, x_first values into every input row)
+    const int part_values = SPLIT ? a.part_stages * g.cols * 256 : 0;
     auto prepare_x = [&]() {
+        const int x_first = SPLIT ? c_p * part_values : 0;
+        const int n4 = SPLIT ? ((a.in_w - x_first < part_values ? a.in_w - x_first : part_values) >> 2) : (a.in_w >> 2);
         auto umax4 = [](uint32_t m, const float4& v) {
             m = umax_u(m, __float_as_uint(v.x) & 0x7fffffffu);
             m = umax_u(m, __float_as_uint(v.y) & 0x7fffffffu);
@@ -1425,7 +1466,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
         // With shared passes the rows are requested together when they fit kPrep float4 per lane (one trip to memory
         // instead of two per row: 1.5 us of a 30 us call); the one-row form keeps the loops (see above).
         // (Not with four tiles in flight per wave: the registers do not hold both.)
-        constexpr int kPrep = R > 1 && LPW <= 3 ? 8 : 0;
+        constexpr int kPrep = R > 1 && LPW <= 3 && !SPLIT ? 8 : 0;      // (SPLIT: measured 8 % slower with it)
         if (kPrep > 0 && rows * n4 <= kPrep * T) {
             float4 xr[kPrep > 0 ? kPrep : 1];
             const float4* x4 = reinterpret_cast<const float4*>(ce.x);      // the rows are consecutive: x4[r * n4 + i]
@@ -1501,7 +1542,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             if (r < rows) {
-                const float4* x4 = reinterpret_cast<const float4*>(ce.x + static_cast<size_t>(r) * a.in_w);
+                const float4* x4 = reinterpret_cast<const float4*>(ce.x + static_cast<size_t>(r) * a.in_w + x_first);
                 uint32_t mx = 0;
                 for (int i = tid; i < n4; i += T) mx = umax4(mx, x4[i]);
                 mx = wave_umax(mx);
@@ -1524,7 +1565,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
                 if (tid == 0) inv_of_row[r] = inv[r];
                 uint8_t* set = planes + r * g.set_bytes;
                 float* sumx = reinterpret_cast<float*>(set + 4 * g.plane_stride);
-                const float4* x4 = reinterpret_cast<const float4*>(ce.x + static_cast<size_t>(r) * a.in_w);
+                const float4* x4 = reinterpret_cast<const float4*>(ce.x + static_cast<size_t>(r) * a.in_w + x_first);
                 for (int i = tid; i < n4; i += T) {       // (whole groups of eight lanes are in or out: n4 % 64 == 0)
                     const float4 v = x4[i];
                     uint32_t pl[4];
@@ -1553,6 +1594,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
 
     u32x4 regs[2][LPW];
     fetch_enter();
+    if constexpr (SPLIT) f_end = fe.first_tile + fe.tiles < t_end ? fe.first_tile + fe.tiles : t_end;
     fetch(regs[0]);
     fetch(regs[1]);
 
@@ -1561,6 +1603,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
     int pbuf = 0;
     bool done = false;
     int done_row0 = 0;
+    int done_u = 0, done_p = 0;            // SPLIT: the finished tile's number in its run, and the part that was finished
     // Adds up and stores the tile whose wave partials sit in part[pbuf ^ 1].  It runs before the next stage enters its
     // matrix, so the tile's matrix is still `ce` (no copies of its fields: the kernel is short of scalar registers).
     auto finalize = [&]() {
@@ -1573,7 +1616,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
             if (r < done_inputs) {
                 float t = 0.0f;
                 for (int w2 = 0; w2 < W; ++w2) t += part[pbuf ^ 1][r][w2][j0];
-                if (done_bias) {
+                if (done_bias && (!SPLIT || done_p == 0)) {
                     const NNHIP_CONST_PTR float* cb = (const NNHIP_CONST_PTR float*)done_bias + done_row0;
                     float bv = 0.0f;
 #pragma unroll
@@ -1583,10 +1626,39 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
                     }
                     t += bv;
                 }
-                if (j0 < done_rows) done_y[static_cast<size_t>(r) * done_out_w + done_row0 + j0] = t;
+                if constexpr (SPLIT) {
+                    // (written and read by this lane only: no barrier between the parts)
+                    if (done_p > 0) t = split_sums[done_u][r][j0] + t;
+                    if (done_p + 1 < a.parts) split_sums[done_u][r][j0] = t;
+                    else if (j0 < done_rows) done_y[static_cast<size_t>(r) * done_out_w + done_row0 + j0] = t;
+                } else {
+                    if (j0 < done_rows) done_y[static_cast<size_t>(r) * done_out_w + done_row0 + j0] = t;
+                }
             }
         }
         done = false;
+    };
+    // SPLIT: the stage just multiplied was the last of its part of tile c_t: where the next stage lies
+    auto next_of_part = [&]() {
+        done_u = c_u;
+        done_p = c_p;
+        c_t += t_step;
+        ++c_u;
+        if (c_t < c_end) {
+            c_k = c_p * a.part_stages;
+        } else if (c_p + 1 < a.parts) {
+            ++c_p;
+            c_t = c_first;
+            c_u = 0;
+            c_k = c_p * a.part_stages;
+            c_part_start = true;
+        } else {
+            c_p = 0;
+            c_first = c_t;
+            c_u = 0;
+            c_k = 0;
+            c_part_start = true;
+        }
     };
 
     float accq[R], accm[R];
@@ -1594,6 +1666,13 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
     for (int r = 0; r < R; ++r) accq[r] = accm[r] = 0.0f;
     // The matrix of the stage about to be multiplied; true when its activations are not the ones in LDS.
     auto enter = [&]() {
+        if constexpr (SPLIT) {
+            if (!c_part_start) return false;
+            c_part_start = false;
+            while (c_t >= ce.first_tile + ce.tiles) ce = entry_at(++c_m);      // (only where a run begins)
+            c_end = ce.first_tile + ce.tiles < t_end ? ce.first_tile + ce.tiles : t_end;
+            return true;
+        }
         bool new_x = false;
         if (c_k == 0 && c_t >= ce.first_tile + ce.tiles) {
             while (c_t >= ce.first_tile + ce.tiles) ce = entry_at(++c_m);
@@ -1610,17 +1689,18 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
             const uint8_t* a_plane = planes + (row_l >> 2) * g.set_bytes + (row_l & 3) * g.plane_stride + 8 * quarter;
             const float* d_sums = reinterpret_cast<const float*>(planes + quarter * g.set_bytes + 4 * g.plane_stride);
             const int b0 = c_k * g.cols + wave;
+            const int pb = SPLIT ? c_p * a.part_stages * g.cols : 0;        // the first block column the planes in LDS hold
             const uint8_t* stage = cur + row_off;
             constexpr int kSumsPerBlock = 256 / F::kSumRun;
 #pragma unroll
             for (int t = 0; t < M; ++t) {
                 const int b = b0 + t * W;
                 if (b < a.nblocks)
-                    F::run_stacked(F::load_stacked(stage + t * W * (16 * F::kPieces), quarter, (wave & 1) != 0), a_plane + 256 * b,
-                                   d_sums + kSumsPerBlock * b, tables, acc_sq, acc_sm);
+                    F::run_stacked(F::load_stacked(stage + t * W * (16 * F::kPieces), quarter, (wave & 1) != 0), a_plane + 256 * (b - pb),
+                                   d_sums + kSumsPerBlock * (b - pb), tables, acc_sq, acc_sm);
             }
-            if (++c_k == KC) {
-                c_k = 0;
+            const int k_end = SPLIT && (c_p + 1) * a.part_stages < KC ? (c_p + 1) * a.part_stages : KC;
+            if (++c_k == k_end) {
                 const float p = fmaf(acc_sq, inv_of_row[quarter], -acc_sm);     // (from LDS: a register array indexed by the lane would go to scratch memory)
                 if (quarter < ce.rows) part[pbuf][quarter][wave][row_l] = p;
                 acc_sq = 0.0f;
@@ -1628,13 +1708,20 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
                 done = true;
                 done_row0 = (c_t - ce.first_tile) * kTileRows;
                 pbuf ^= 1;
-                c_t += t_step;
+                if constexpr (SPLIT) {
+                    next_of_part();
+                } else {
+                    c_k = 0;
+                    c_t += t_step;
+                }
             }
         } else {
         // task t of this wave: block column c_k * cols + t * W + wave of the row (W is even: the block's parity is the
         // wave's).  Stages whose tasks all exist run them as one straight piece of code, so that the lookups and products
         // of one task overlap the other's; a tile's last stage may hold fewer.
-        auto task = [&](const typename F::Raw& raw, int b) {
+        const int pb = SPLIT ? c_p * a.part_stages * g.cols : 0;            // the first block column the planes in LDS hold
+        auto task = [&](const typename F::Raw& raw, int b_of_row) {
+            const int b = b_of_row - pb;
             if constexpr (SplitLookups<F>::value && R > 1) {
                 // what the block's lookups return does not depend on the input row: made once, used by every row
                 typename F::Looked lk;
@@ -1676,8 +1763,8 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
             for (int t = 0; t < M - 1; ++t)
                 if (b0 + t * W < a.nblocks) task(F::load(stage + t * W * (16 * F::kPieces), quarter, (wave & 1) != 0), b0 + t * W);
         }
-        if (++c_k == KC) {
-            c_k = 0;
+        const int k_end = SPLIT && (c_p + 1) * a.part_stages < KC ? (c_p + 1) * a.part_stages : KC;
+        if (++c_k == k_end) {
 #pragma unroll
             for (int r = 0; r < R; ++r) {
                 float p = fmaf(accq[r], inv[r], -accm[r]);
@@ -1689,7 +1776,12 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
             done = true;
             done_row0 = (c_t - ce.first_tile) * kTileRows;
             pbuf ^= 1;
-            c_t += t_step;
+            if constexpr (SPLIT) {
+                next_of_part();
+            } else {
+                c_k = 0;
+                c_t += t_step;
+            }
         }
         }
     };
@@ -1957,6 +2049,62 @@ bool plan_wide(uint32_t type, int in_w, int inputs, WideGeom* out)
     return true;
 }
 
+// The split form of the shared pass (four input rows per entry) for rows whose four sets of planes do not fit LDS: W as
+// above, and the fewest parts (groups of whole stages) whose planes do.  Not for Q8_0, whose row-tiled row-step kernel
+// serves such calls.
+bool plan_wide_split(uint32_t type, int in_w, WideGeom* out, int* parts, int* part_stages)
+{
+    const WideTraits tr = wide_traits(type, true);
+    const int nblocks = in_w / 256;
+    if (!tr.pieces || nblocks < 4 || type == NNHIP_TYPE_Q8_0) return false;
+    double best_score = -1.0;
+    for (int W = 12; W >= 6; W -= 2) {
+        WideGeom g{};
+        g.waves = W;
+        g.cols = W * tr.m;
+        if (g.cols > nblocks + tr.m) continue;
+        g.kchunks = (nblocks + g.cols - 1) / g.cols;
+        g.tail_cols = nblocks - (g.kchunks - 1) * g.cols;
+        g.row_pieces = (g.cols * tr.pieces) | 1;
+        const int loads = (kTileRows * g.row_pieces + 63) / 64;
+        if ((loads + W - 1) / W > tr.lpw) continue;
+        g.stage_bytes = (tr.tight ? loads : tr.lpw * W) * 1024;
+        for (int P = 2; P <= 6; ++P) {
+            const int SP = (g.kchunks + P - 1) / P;
+            if ((P - 1) * SP >= g.kchunks) continue;            // (every part holds a stage)
+            const int part_w = SP * g.cols * 256;
+            g.plane_stride = part_w + 16;
+            g.set_bytes = (4 * g.plane_stride + (tr.sums ? (part_w / 16) * 4 : 0) + 15) / 16 * 16;
+            g.lds_bytes = 2 * static_cast<size_t>(g.stage_bytes) + 4 * static_cast<size_t>(g.set_bytes);
+            if (g.lds_bytes + wide_static_lds(4) + 2048 + tr.table_bytes > static_cast<size_t>(160 * 1024)) continue;
+            const double fill = static_cast<double>(nblocks) / (g.kchunks * g.cols);
+            const double score = fill * W / 12.0 * (W % 4 == 0 ? 1.0 : 0.95) * (0.9 + 0.1 * fill) * (1.0 - 0.02 * (P - 2));
+            if (score > best_score) {
+                best_score = score;
+                *out = g;
+                *parts = P;
+                *part_stages = SP;
+            }
+            break;
+        }
+    }
+    return best_score >= 0;
+}
+
+template <class F>
+hipError_t launch_wide_split_of(Lane* lane, const WideArgs& a)
+{
+    constexpr int M = F::kSharedM, LPW = F::kSharedLpw;
+    static LdsLimit big_lds;
+    const void* fn = reinterpret_cast<const void*>(&matvec_mfma_wide_kernel<F, M, LPW, 4, false, true>);
+    const hipError_t e = big_lds.ensure(lane->device, fn, 160 * 1024 - wide_static_lds(4) - 2048 - F::kLdsTableBytes);
+    if (e != hipSuccess) return e;
+    const int groups = a.total_tiles < lane->compute_units ? a.total_tiles : lane->compute_units;
+    hipLaunchKernelGGL((matvec_mfma_wide_kernel<F, M, LPW, 4, false, true>), dim3(groups), dim3(64 * a.g.waves), a.g.lds_bytes,
+                       lane->stream, a);
+    return hipGetLastError();
+}
+
 template <class F, int R>
 hipError_t launch_wide_of(Lane* lane, const WideArgs& a)
 {
@@ -2060,15 +2208,44 @@ bool matvec_mfma_wide_geometry(uint32_t type, int in_w, int out_w, const void* w
     return inputs >= 1 && inputs <= 4 && entry_ok(type, in_w, out_w, w) && plan_wide(type, in_w, inputs == 1 ? 1 : 4, &g);
 }
 
+bool matvec_mfma_split_geometry(uint32_t type, int in_w, int out_w, const void* w, int compute_units)
+{
+    WideGeom g;
+    int parts = 0, part_stages = 0;
+    if (!entry_ok(type, in_w, out_w, w) || plan_wide(type, in_w, 4, &g) || !plan_wide_split(type, in_w, &g, &parts, &part_stages)) return false;
+    // a workgroup's tiles of one entry (every G-th tile of the launch) wait in LDS between the parts
+    const int tiles = (out_w + kTileRows - 1) / kTileRows;
+    return compute_units > 0 && (tiles + compute_units - 1) / compute_units <= kSplitUnits;
+}
+
 namespace {
 
 hipError_t launch_wide_args(Lane* lane, uint32_t type, int in_w, int inputs, WideArgs& a)
 {
-    if (!plan_wide(type, in_w, inputs == 1 ? 1 : 4, &a.g)) return hipErrorInvalidValue;
+    bool split = false;
+    if (!plan_wide(type, in_w, inputs == 1 ? 1 : 4, &a.g)) {
+        // four input rows per entry on rows too long for their planes: the split form (entries in the kernel arguments)
+        if (inputs == 1 || a.table || !plan_wide_split(type, in_w, &a.g, &a.parts, &a.part_stages)) return hipErrorInvalidValue;
+        split = true;
+        // runs of consecutive tiles (a workgroup then meets one or two entries, i.e. converts few vectors) where the
+        // tiles of a run fit the sums kept in LDS between the parts
+        const int groups = a.total_tiles < lane->compute_units ? a.total_tiles : lane->compute_units;
+        a.chunked = (a.total_tiles + groups - 1) / groups <= kSplitUnits ? 1 : 0;
+    }
     a.in_w = in_w;
     a.nblocks = in_w / 256;
     a.row_bytes = static_cast<uint32_t>(a.nblocks) * static_cast<uint32_t>(block_bytes_of(type));
     a.row_pieces_magic = static_cast<uint32_t>((0x100000000ull + a.g.row_pieces - 1) / a.g.row_pieces);
+    if (split) {
+        switch (type) {
+        case NNHIP_TYPE_Q4_K: return launch_wide_split_of<Q4KTask>(lane, a);
+        case NNHIP_TYPE_Q5_K: return launch_wide_split_of<Q5KTask>(lane, a);
+        case NNHIP_TYPE_Q6_K: return launch_wide_split_of<Q6KTask>(lane, a);
+        case NNHIP_TYPE_IQ2_S: return launch_wide_split_of<IQ2STask>(lane, a);
+        case NNHIP_TYPE_IQ3_S: return launch_wide_split_of<IQ3STask>(lane, a);
+        default: return hipErrorInvalidValue;
+        }
+    }
     switch (type) {
     case NNHIP_TYPE_Q4_K: return launch_wide<Q4KTask>(lane, a, inputs);
     case NNHIP_TYPE_Q5_K: return launch_wide<Q5KTask>(lane, a, inputs);
@@ -2099,7 +2276,8 @@ bool describe_matvec_rows_shared(uint32_t type, int rows, int in_w, int out_w, i
                                  nnhip_matvec_plan_info* info)
 {
     WideGeom g;
-    if (!plan_wide(type, in_w, per_pass, &g)) return false;
+    int parts = 0, part_stages = 0;
+    if (!plan_wide(type, in_w, per_pass, &g) && (per_pass != 4 || !plan_wide_split(type, in_w, &g, &parts, &part_stages))) return false;
     const int launch_rows = rows < 4 * per_pass ? rows : 4 * per_pass;                 // (four table entries per launch)
     const int tiles = (out_w + kTileRows - 1) / kTileRows * ((launch_rows + per_pass - 1) / per_pass);
     info->kernel = NNHIP_MATVEC_KERNEL_MATRIX_CORE;

@@ -560,7 +560,7 @@ int nnhip_quant_matvec(void* handle, uint32_t ggml_type, const float* x, const v
     if (in_w > matvec_max_in_w(ggml_type))
         return fail(NNHIP_ERR_TOO_LARGE, NNHIP_OP_MATVEC, lane->device, 0, "in_w %d exceeds the %d values one workgroup can stage", in_w, matvec_max_in_w(ggml_type));
     if (rows > 65535) return fail(NNHIP_ERR_TOO_LARGE, NNHIP_OP_MATVEC, lane->device, 0, "rows %d exceeds 65535", rows);
-    if (const int per_pass = lane->row_step_only ? 0 : matvec_rows_per_pass(ggml_type, rows, in_w, out_w, w)) {
+    if (const int per_pass = lane->row_step_only ? 0 : matvec_rows_per_pass(ggml_type, rows, in_w, out_w, w, lane->compute_units)) {
         // two or more input rows of a large matrix: up to four rows share a pass over the weights on the matrix cores,
         // sixteen rows go into a launch (the reference routes such calls to row-tiled kernels,
         // Qwen35QuantizedModel.cs:1335-1344)

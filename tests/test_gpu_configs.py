@@ -706,11 +706,12 @@ def test_matrix_core_groups_with_long_rows_and_shared_passes(lane, typ):
 
 
 @pytest.mark.parametrize("typ", [GGML_Q4_K, GGML_IQ2_S, GGML_IQ3_S])
-def test_long_rows_take_a_pass_per_input_row_on_the_matrix_cores(lane, typ):
-    """17408-wide rows: four sets of activation planes do not fit LDS, so a call with several input rows gets one pass per
-    row on the matrix cores (four rows a launch) once rows x tiles reach the format's floor, and row-step passes below
-    it.  Both bars against the oracle, guard elements, the plan reports the form, and a row's bits do not depend on the
-    rows it is issued with."""
+def test_long_rows_with_few_input_rows_on_the_matrix_cores(lane, typ):
+    """17408-wide rows: four full sets of activation planes do not fit LDS.  A call with a few input rows gets one pass
+    per row on the matrix cores (four rows a launch) once rows x tiles reach the format's floor and row-step passes
+    below it, or, where the groups of four rows make enough tiles (IQ3_S: always), shared passes in the split form.
+    Both bars against the oracle, guard elements, the plan reports the form, and a row's bits do not depend on the rows
+    it is issued with as long as the form is the same."""
     from ctypes import byref, sizeof
     from nntrain_amd import native
     in_w, out_w = 17408, 5120
@@ -730,7 +731,9 @@ def test_long_rows_take_a_pass_per_input_row_on_the_matrix_cores(lane, typ):
         floor = {GGML_Q4_K: 1024, GGML_IQ3_S: 768, GGML_IQ2_S: 512}[typ]
         assert (info.kernel == 2) == (rows * 320 >= floor), (rows, info.kernel)
         if info.kernel == 2:
-            assert info.row_tile == 1 and info.steps == 320 * min(rows, 4)
+            split = typ == GGML_IQ3_S or (typ == GGML_IQ2_S and rows > 4)
+            assert info.row_tile == (min(rows, 4) if split else 1)
+            assert info.steps == 320 * (-(-rows // 4) if split else min(rows, 4))
         yd = lane.allocate(rows * out_w + 2)
         lane.fill_u32(yd, NAN_BITS, rows * out_w + 2)
         mat.forward(lane, xd, bd, rows, out=yd)
@@ -741,11 +744,75 @@ def test_long_rows_take_a_pass_per_input_row_on_the_matrix_cores(lane, typ):
         ref, asum = oracle.linear_f64(typ, payload, x[:rows], bias, rows, in_w, out_w)
         assert oracle.rel_l2(y, ref) <= MATVEC_BAR
         assert np.all(np.abs(y.astype(np.float64) - ref) <= 2e-6 + 3e-6 * asum)
-        results[rows] = (y, info.kernel)
+        results[rows] = (y, info.kernel, info.row_tile)
         yd.dispose()
     assert results[4][1] == results[6][1] == 2
-    assert np.array_equal(_bits(results[6][0][:4]), _bits(results[4][0]))
+    if (results[4][2] == 1) == (results[6][2] == 1):
+        assert np.array_equal(_bits(results[6][0][:4]), _bits(results[4][0]))
     for b in (xd, bd):
+        b.dispose()
+    mat.dispose()
+    lane.trim()
+
+
+@pytest.mark.parametrize("typ", [GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_IQ2_S, GGML_IQ3_S])
+def test_long_rows_share_passes_in_the_split_form(lane, typ):
+    """Many input rows on 17408-wide rows: up to four of them share a pass over the weights with the planes of one
+    group of block columns in LDS at a time (the split form: a workgroup takes its tiles of an entry once per group and
+    keeps their sums in LDS in between).  9, 13 and 16 rows (three or four entries per launch, the last one ragged) and
+    21 rows (two launches) against the oracle at both bars, with bias and rows of very different magnitudes, guard
+    words, no transfers; a row's bits do not depend on the rows it travels with; a captured call replays to the same
+    bits with eager calls of other shapes in between."""
+    from ctypes import byref, sizeof
+    from nntrain_amd import native
+    in_w, out_w = 17408, 5120 + 16 * 3 + 5
+    payload = synth.matrix(typ, out_w, in_w, seed=1700 + typ)
+    mat = HipQuantizedMatrix(payload, typ, out_w, in_w)
+    mat.device_payload(lane)
+    bias = np.random.default_rng(6).standard_normal(out_w).astype(np.float32)
+    bd = lane.upload_raw(bias)
+    x = synth.activations(21, in_w, seed=43)
+    x[2] *= 3e-3
+    x[10] *= 9e2
+    x[12, 5000:9000] = 0.0
+    xd = lane.upload_raw(x)
+    info = native.MatvecPlanInfo(struct_size=sizeof(native.MatvecPlanInfo))
+    results = {}
+    for rows in (9, 13, 16, 21):
+        assert lane._lib.nnhip_matvec_plan(typ, rows, in_w, out_w, 256, byref(info)) == 0
+        assert info.kernel == 2 and info.row_tile == 4 and info.steps == 324 * -(-min(rows, 16) // 4)
+        yd = lane.allocate(rows * out_w + 2)
+        lane.fill_u32(yd, NAN_BITS, rows * out_w + 2)
+        before = lane.counters()
+        mat.forward(lane, xd, bd, rows, out=yd)
+        lane.synchronize()
+        after = lane.counters()
+        assert after["h2d_bytes"] == before["h2d_bytes"] and after["allocated_bytes"] == before["allocated_bytes"]
+        assert after["kernel_launches"] - before["kernel_launches"] == -(-rows // 16)
+        y = lane.read(yd)
+        assert np.isnan(y[-1]) and np.isnan(y[-2])
+        results[rows] = y[:-2].reshape(rows, out_w)
+        yd.dispose()
+    ref, asum = oracle.linear_f64(typ, payload, x, bias, 21, in_w, out_w)
+    for rows, y in results.items():
+        assert oracle.rel_l2(y, ref[:rows]) <= MATVEC_BAR, rows
+        assert np.all(np.abs(y.astype(np.float64) - ref[:rows]) <= 2e-6 + 3e-6 * asum[:rows]), rows
+    assert np.array_equal(_bits(results[21][:16]), _bits(results[16]))
+    assert np.array_equal(_bits(results[16][:13]), _bits(results[13]))
+    assert np.array_equal(_bits(results[13][:9]), _bits(results[9]))
+    yd = lane.allocate(13 * out_w)
+    lane.graph_begin()
+    mat.forward(lane, xd, bd, 13, out=yd)
+    graph = lane.graph_end()
+    for _ in range(3):
+        lane.fill_u32(yd, NAN_BITS, 13 * out_w)
+        mat.forward(lane, xd, None, 9)
+        lane.synchronize()
+        lane.graph_launch(graph)
+        lane.synchronize()
+        assert np.array_equal(_bits(lane.read(yd).reshape(13, out_w)), _bits(results[13]))
+    lane.graph_destroy(graph)
+    for b in (xd, bd, yd):
         b.dispose()
     mat.dispose()
     lane.trim()

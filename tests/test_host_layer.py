@@ -144,11 +144,21 @@ def test_matvec_plan_keeps_a_ring_turn_inside_the_result_buffer():
                         assert (3 if typ == 8 else 2) <= rows and typ in (8, 12, 13, 14, 21, 22)
                         assert typ != 8 or in_w in (1024, 5376)         # (21504-wide planes of four rows do not fit LDS)
                         assert info.rows_per_step == 16 and info.threads % 128 == 0
-                        if in_w == 17408:
+                        if in_w == 17408 and info.row_tile == 1:
                             # four sets of planes do not fit LDS: a pass per input row, four rows a launch, from 1024 tiles x rows (IQ2_S: 512)
-                            assert typ in (12, 22) and info.row_tile == 1 and rows * -(-out_w // 16) >= (512 if typ == 22 else 1024)
+                            assert typ in (12, 22) and rows * -(-out_w // 16) >= (512 if typ == 22 else 1024)
                             assert info.steps == -(-out_w // 16) * min(rows, 4)
                             assert info.dynamic_lds_bytes + 2048 + (10240 if typ == 22 else 0) <= 160 * 1024
+                        elif in_w == 17408:
+                            # ... or shared passes in the split form (the planes of one group of block columns at a time) where
+                            # the groups of four input rows make 3.5 rounds of tiles over the workgroups (IQ2_S: 2.5) and a
+                            # workgroup's tiles of one group fit the sums kept in LDS
+                            tiles = -(-out_w // 16)
+                            assert typ in (12, 22) and info.row_tile == min(rows, 4)
+                            assert 2 * -(-rows // 4) * tiles >= (5 if typ == 22 else 7) * 256 and -(-tiles // 256) <= 8
+                            assert info.steps == tiles * -(-min(rows, 16) // 4)
+                            assert info.dynamic_lds_bytes + 10240 + (10240 if typ == 22 else 0) <= 160 * 1024
+                            seen_tiles.add((typ, "split"))
                         else:
                             assert rows * -(-out_w // 16) >= (768 if rows >= 3 and typ != 8 else 2048)
                             assert info.row_tile == min(rows, 4)
@@ -167,7 +177,7 @@ def test_matvec_plan_keeps_a_ring_turn_inside_the_result_buffer():
                     assert info.dynamic_lds_bytes <= 140 * 1024
                     seen_tiles.add((typ, info.row_tile))
     assert {(8, 1), (8, 2), (8, 4), (30, 4), (12, 1), (8, "matrix core"), (12, "matrix core"), (14, "matrix core"),
-            (21, "matrix core")} <= seen_tiles
+            (21, "matrix core"), (12, "split"), (22, "split")} <= seen_tiles
     # three rows reach the matrix cores at 768 tiles x rows, two rows at 2048
     assert lib.nnhip_matvec_plan(12, 3, 5120, 4096, 256, byref(info)) == 0 and info.kernel == 2
     assert lib.nnhip_matvec_plan(12, 3, 5120, 4000, 256, byref(info)) == 0 and info.kernel == 0

@@ -53,25 +53,29 @@ def _short(name):
 
 
 # (task, stages per tile or tasks per wave, ...) of the variants the planners pick for the shapes of the benchmark and
-# the tests: register form <Task, KC, M, LPW, one register set>, wide form <Task, M, LPW, R, one stage buffer>
+# the tests: register form <Task, KC, M, LPW, one register set>, wide form <Task, M, LPW, R, one stage buffer, split>
 USED = ["matvec_mfma_kernelINS0_7Q4KTaskELi1ELi2ELi5ELb0", "matvec_mfma_kernelINS0_7Q4KTaskELi2ELi1ELi3ELb0",
         "matvec_mfma_kernelINS0_7Q5KTaskELi2ELi1ELi3ELb0",
         "matvec_mfma_kernelINS0_7Q6KTaskELi2ELi1ELi4ELb0", "matvec_mfma_kernelINS0_7Q4KTaskELi1ELi1ELi3ELb0",
-        "matvec_mfma_wide_kernelINS0_7Q4KTaskELi1ELi3ELi1ELb0", "matvec_mfma_wide_kernelINS0_7Q4KTaskELi1ELi3ELi4ELb0",
-        "matvec_mfma_wide_kernelINS0_7Q5KTaskELi1ELi3ELi1ELb0", "matvec_mfma_wide_kernelINS0_7Q5KTaskELi1ELi3ELi4ELb0",
-        "matvec_mfma_wide_kernelINS0_7Q6KTaskELi1ELi4ELi1ELb0", "matvec_mfma_wide_kernelINS0_7Q6KTaskELi1ELi4ELi4ELb0",
-        "matvec_mfma_wide_kernelINS0_8IQ2STaskELi2ELi4ELi1ELb0", "matvec_mfma_wide_kernelINS0_8IQ2STaskELi1ELi2ELi4ELb0",
-        "matvec_mfma_wide_kernelINS0_8Q8_0TaskELi1ELi5ELi1ELb0",
-        "matvec_mfma_wide_kernelINS0_8Q8_0TaskELi2ELi8ELi1ELb1",
-        "matvec_mfma_wide_kernelINS0_8Q8_0TaskELi1ELi5ELi4ELb0"]
+        "matvec_mfma_wide_kernelINS0_7Q4KTaskELi1ELi3ELi1ELb0ELb0", "matvec_mfma_wide_kernelINS0_7Q4KTaskELi1ELi3ELi4ELb0ELb0",
+        "matvec_mfma_wide_kernelINS0_7Q5KTaskELi1ELi3ELi1ELb0ELb0", "matvec_mfma_wide_kernelINS0_7Q5KTaskELi1ELi3ELi4ELb0ELb0",
+        "matvec_mfma_wide_kernelINS0_7Q6KTaskELi1ELi4ELi1ELb0ELb0", "matvec_mfma_wide_kernelINS0_7Q6KTaskELi1ELi4ELi4ELb0ELb0",
+        "matvec_mfma_wide_kernelINS0_8IQ2STaskELi2ELi4ELi1ELb0ELb0", "matvec_mfma_wide_kernelINS0_8IQ2STaskELi1ELi2ELi4ELb0ELb0",
+        "matvec_mfma_wide_kernelINS0_8Q8_0TaskELi1ELi5ELi1ELb0ELb0",
+        "matvec_mfma_wide_kernelINS0_8Q8_0TaskELi2ELi8ELi1ELb1ELb0",
+        "matvec_mfma_wide_kernelINS0_8Q8_0TaskELi1ELi5ELi4ELb0ELb0"]
 # With one register set the last parking write of a stage rightly waits for everything: nothing else is on its way.
 USED_ONE_SET = ["matvec_mfma_kernelINS0_7Q5KTaskELi1ELi2ELi6ELb1"]
+# the split form of the shared pass (rows too long for four sets of planes in LDS)
+USED_SPLIT = ["matvec_mfma_wide_kernelINS0_7Q4KTaskELi1ELi3ELi4ELb0ELb1", "matvec_mfma_wide_kernelINS0_7Q5KTaskELi1ELi3ELi4ELb0ELb1",
+              "matvec_mfma_wide_kernelINS0_7Q6KTaskELi1ELi4ELi4ELb0ELb1", "matvec_mfma_wide_kernelINS0_8IQ2STaskELi1ELi2ELi4ELb0ELb1",
+              "matvec_mfma_wide_kernelINS0_8IQ3STaskELi1ELi2ELi4ELb0ELb1"]
 
 
 def test_parking_writes_wait_only_for_their_own_register_set(isa):
     bodies, _ = _kernels(isa)
     by_short = {_short(k): v for k, v in bodies.items()}
-    for name in USED:
+    for name in USED + USED_SPLIT:
         assert name in by_short, f"{name} is no longer generated"
         last_wait, parks = None, []
         for line in by_short[name]:
@@ -88,6 +92,6 @@ def test_parking_writes_wait_only_for_their_own_register_set(isa):
 def test_variants_in_use_do_not_spill(isa):
     _, meta = _kernels(isa)
     by_short = {_short(k): v for k, v in meta.items()}
-    for name in USED + USED_ONE_SET:
+    for name in USED + USED_ONE_SET + USED_SPLIT:
         assert name in by_short, f"{name} has no metadata"
         assert by_short[name] == {"private": 0, "vgpr_spills": 0}, (name, by_short[name])
