@@ -211,8 +211,8 @@ NNHIP_API int nnhip_dequantize(void* lane, uint32_t ggml_type, const void* w, fl
  * input rows per pass over the weights, sixteen per launch; a row's bits do not depend on the rows it travels with; 1e-6
  * from the rows == 1 result).  Rows too long for four sets of activation planes in LDS (in_w above about 8700; never
  * Q8_0) share passes in a split form, with the planes of one group of block columns in LDS at a time, where the groups
- * of four input rows make at least 3.5 rounds of 16-row tiles over the compute units (IQ2_S 2.5; IQ3_S always) and
- * out_w is at most 32768; otherwise they get one matrix-core pass per input row, four rows a launch, from
+ * of four input rows make at least 3.5 rounds of 16-row tiles over the compute units (IQ2_S 2.5; IQ3_S always);
+ * otherwise they get one matrix-core pass per input row, four rows a launch, from
  * rows x ceil(out_w / 16) >= 1024 on (IQ3_S 768, IQ2_S 512).  A row's bits depend on which of these forms the call
  * takes, not on the rows it travels with.  nnhip_matvec_plan reports which form a call takes; a lane with NNHIP_OPTION_ROW_STEP_ONLY set takes
  * none of these forms and keeps the bit-for-bit property for every call.  bias may be null (zero).  Asynchronous. */

@@ -1684,7 +1684,9 @@ int matvec_rows_per_pass(uint32_t type, int rows, int in_w, int out_w, const voi
     if (rows < shared_pass_min_rows(type)) return 0;
     const long work = static_cast<long>(rows) * ((out_w + 15) / 16);
     const long floor = rows >= 3 && type != NNHIP_TYPE_Q8_0 ? kSharedPassMinTiles : kMfmaBatchMinTiles;
-    if (work >= floor && matvec_mfma_wide_geometry(type, in_w, out_w, w, 4)) return 4;
+    bool split = false;
+    const bool shared = matvec_mfma_wide_geometry(type, in_w, out_w, w, 4, &split);
+    if (work >= floor && shared && !split) return 4;
     // Rows too long for four sets of activation planes in LDS (more than about 8700 values): shared passes in the split
     // form, the planes of one group of block columns at a time.
     // It pays from three and a half rounds of (16 matrix rows x 4 input rows) over the workgroups on (IQ2_S: two and a
@@ -1695,16 +1697,13 @@ int matvec_rows_per_pass(uint32_t type, int rows, int in_w, int out_w, const voi
     // 91 / 173; IQ3_S 4 rows 53 / 64, 16 rows 98 / 242; on 17408 x 14336 Q4_K 4 rows 67 / 82, 16 rows 233 / 332.
     const long shared_units = static_cast<long>((rows + 3) / 4) * ((out_w + 15) / 16);
     const long shared_floor = type == NNHIP_TYPE_IQ3_S ? 0 : type == NNHIP_TYPE_IQ2_S ? 5L * compute_units : 7L * compute_units;
-    if (work >= floor && 2 * shared_units >= shared_floor && matvec_mfma_split_geometry(type, in_w, out_w, w, compute_units))
-        return 4;
+    if (work >= floor && shared && split && 2 * shared_units >= shared_floor) return 4;
     // Rows too long for four sets of activation planes in LDS (more than about 8700 values): the super-block formats
     // still stream faster on the matrix cores, one pass per input row (Q8_0's row-step kernel multiplies four input rows
     // per pass and stays).
     const long separate_floor = type == NNHIP_TYPE_IQ2_S ? kSeparatePassMinTilesIQ2S
                               : type == NNHIP_TYPE_IQ3_S ? kSeparatePassMinTilesIQ3S : kSeparatePassMinTiles;
-    if (type != NNHIP_TYPE_Q8_0 && work >= separate_floor &&
-        !matvec_mfma_wide_geometry(type, in_w, out_w, w, 4) &&
-        matvec_mfma_wide_geometry(type, in_w, out_w, w, 1))
+    if (type != NNHIP_TYPE_Q8_0 && work >= separate_floor && (!shared || split) && matvec_mfma_wide_geometry(type, in_w, out_w, w, 1))
         return 1;
     return 0;
 }

@@ -1276,16 +1276,17 @@ struct WideArgs {
     uint32_t row_pieces_magic;
     int chunked;                   // 1: a workgroup takes consecutive tiles (few changes of activations), 0: every G-th
     int parts, part_stages;        // SPLIT: a row's stages are taken in `parts` groups of `part_stages` (see the kernel)
+    int run_tiles;                 // SPLIT: most tiles of a run (their sums wait in LDS from part to part, behind the planes)
     WideGeom g;
     MfmaEntry inline_entries[4];   // a call with up to 16 input rows needs no table in device memory
 };
 
-// SPLIT: most tiles of one table entry that a workgroup may meet (their sums wait in LDS from part to part)
-constexpr int kSplitUnits = 8;
+// SPLIT: a run is as long as the LDS the geometry leaves over holds sums for, up to this many tiles
+constexpr int kSplitRunMax = 64;
 
-// SPLIT (shared passes over rows too long for R full sets of planes in LDS): the stages of a tile are taken in `parts`
+// SPLIT (rows too long for R full sets of planes in LDS): the stages of a tile are taken in `parts`
 // groups of `part_stages`, and LDS holds the planes of one group of block columns at a time.  A workgroup works through
-// its tiles of a table entry once per part: planes of part 0 (with a fixed-point scale of their own), that part of
+// a run of its tiles of a table entry (at most run_tiles of them) once per part: planes of part 0 (with a fixed-point scale of their own), that part of
 // every tile, planes of part 1, ...; the sums of a tile wait in LDS (bias + part 0, + part 1, ...: one order, so the
 // bits of a row depend on its weights, its activations and the launch geometry only) and are stored after the last part.
 // Every stage of every tile is still requested and multiplied once; what is paid is a conversion of the activations
@@ -1293,9 +1294,8 @@ constexpr int kSplitUnits = 8;
 template <class F, int M, int LPW, int R, bool ONE = false, bool SPLIT = false>
 __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideArgs a)
 {
-    static_assert(!SPLIT || (!ONE && R > 1), "parts are for shared passes with two stage buffers");
+    static_assert(!SPLIT || !ONE, "parts are for the form with two stage buffers");
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
-    __shared__ float split_sums[SPLIT ? kSplitUnits : 1][R][kTileRows];   // SPLIT: a tile's sums between its parts
     __shared__ float part[2][R][kMaxWaves][kTileRows];
     __shared__ uint32_t red[R][kMaxWaves];
     __shared__ float inv_of_row[R];                                       // 2^-e of each input row's fixed-point scale
@@ -1363,9 +1363,16 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
     const int total = my_tiles * KC;
     const uint32_t chunk_bytes = static_cast<uint32_t>(g.cols) * F::kBlockBytes;
 
+    // SPLIT: a run of this workgroup's tiles that starts at tile `first` ends with the entry, with the workgroup's tiles,
+    // or after run_tiles tiles
+    auto run_end = [&](int first, int entry_end) {
+        int e = entry_end < t_end ? entry_end : t_end;
+        const int cap = first + a.run_tiles * t_step;
+        return e < cap ? e : cap;
+    };
     // ---- prefetch side
     int f_t = t_first, f_k = 0, f_m = 0;
-    int f_p = 0, f_first = t_first, f_end = 0;           // SPLIT: part, first tile and end of the run of tiles of one entry
+    int f_p = 0, f_first = t_first;                      // SPLIT: part and first tile of the run of tiles of one entry
     if (a.chunked && my_tiles > 0) {
         // the entry that holds this workgroup's first tile: the last one whose first_tile is not beyond it (a run may
         // start hundreds of entries into the table, and walking there costs a trip to memory per entry)
@@ -1395,7 +1402,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
             const int part_end = (f_p + 1) * a.part_stages < KC ? (f_p + 1) * a.part_stages : KC;
             if (++f_k == part_end) {
                 f_t += t_step;
-                if (f_t < f_end) {                       // the same part of the entry's next tile
+                if (f_t < run_end(f_first, fe.first_tile + fe.tiles)) {      // the same part of the entry's next tile
                     f_k = f_p * a.part_stages;
                 } else if (f_p + 1 < a.parts) {          // the next part, from the run's first tile again
                     ++f_p;
@@ -1405,10 +1412,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
                     f_p = 0;
                     f_first = f_t;
                     f_k = 0;
-                    if (f_t < t_end) {
-                        fetch_enter();
-                        f_end = fe.first_tile + fe.tiles < t_end ? fe.first_tile + fe.tiles : t_end;
-                    }
+                    if (f_t < t_end) fetch_enter();
                 }
             }
         } else if (++f_k == KC) {
@@ -1435,10 +1439,9 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
     uint8_t* const planes = smem + (ONE ? 1 : 2) * g.stage_bytes;
     F::init_tables(tables, tid, T);
     int c_t = t_first, c_k = 0, c_m = m_first - 1;      // (ce.tiles == 0: the first stage enters entry m_first)
-    // SPLIT: part, first tile and end of the run of this workgroup's tiles of one entry, the tile's number in the run,
-    // whether the stage about to be multiplied is the first of a part (its planes have to be made)
-    int c_p = 0, c_first = t_first, c_end = 0, c_u = 0;
-    bool c_part_start = true;
+    // SPLIT: part, first tile and end of the run of this workgroup's tiles of one entry, the tile's number in the run
+    // (the first stage of tile 0 of a part is where the part's planes have to be made)
+    int c_p = 0, c_first = t_first, c_u = 0;
     MfmaEntry ce{};
     float inv[R] = {};
     const float* planes_x = nullptr;       // the vector(s) the planes in LDS were made from
@@ -1594,7 +1597,6 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
 
     u32x4 regs[2][LPW];
     fetch_enter();
-    if constexpr (SPLIT) f_end = fe.first_tile + fe.tiles < t_end ? fe.first_tile + fe.tiles : t_end;
     fetch(regs[0]);
     fetch(regs[1]);
 
@@ -1603,7 +1605,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
     int pbuf = 0;
     bool done = false;
     int done_row0 = 0;
-    int done_u = 0, done_p = 0;            // SPLIT: the finished tile's number in its run, and the part that was finished
+    int done_up = 0;                       // SPLIT: the finished tile's number in its run times 8, plus the part that was finished
     // Adds up and stores the tile whose wave partials sit in part[pbuf ^ 1].  It runs before the next stage enters its
     // matrix, so the tile's matrix is still `ce` (no copies of its fields: the kernel is short of scalar registers).
     auto finalize = [&]() {
@@ -1616,6 +1618,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
             if (r < done_inputs) {
                 float t = 0.0f;
                 for (int w2 = 0; w2 < W; ++w2) t += part[pbuf ^ 1][r][w2][j0];
+                const int done_p = SPLIT ? done_up & 7 : 0;
                 if (done_bias && (!SPLIT || done_p == 0)) {
                     const NNHIP_CONST_PTR float* cb = (const NNHIP_CONST_PTR float*)done_bias + done_row0;
                     float bv = 0.0f;
@@ -1628,8 +1631,10 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
                 }
                 if constexpr (SPLIT) {
                     // (written and read by this lane only: no barrier between the parts)
-                    if (done_p > 0) t = split_sums[done_u][r][j0] + t;
-                    if (done_p + 1 < a.parts) split_sums[done_u][r][j0] = t;
+                    // the sums of the run's tiles between their parts lie behind the planes: [tile of the run][input row][row]
+                    float* const kept = reinterpret_cast<float*>(smem + 2 * g.stage_bytes + R * g.set_bytes) + ((done_up >> 3) * R + r) * kTileRows + j0;
+                    if (done_p > 0) t = *kept + t;
+                    if (done_p + 1 < a.parts) *kept = t;
                     else if (j0 < done_rows) done_y[static_cast<size_t>(r) * done_out_w + done_row0 + j0] = t;
                 } else {
                     if (j0 < done_rows) done_y[static_cast<size_t>(r) * done_out_w + done_row0 + j0] = t;
@@ -1640,24 +1645,21 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
     };
     // SPLIT: the stage just multiplied was the last of its part of tile c_t: where the next stage lies
     auto next_of_part = [&]() {
-        done_u = c_u;
-        done_p = c_p;
+        done_up = c_u * 8 + c_p;
         c_t += t_step;
         ++c_u;
-        if (c_t < c_end) {
+        if (c_t < run_end(c_first, ce.first_tile + ce.tiles)) {
             c_k = c_p * a.part_stages;
         } else if (c_p + 1 < a.parts) {
             ++c_p;
             c_t = c_first;
             c_u = 0;
             c_k = c_p * a.part_stages;
-            c_part_start = true;
         } else {
             c_p = 0;
             c_first = c_t;
             c_u = 0;
             c_k = 0;
-            c_part_start = true;
         }
     };
 
@@ -1667,10 +1669,8 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
     // The matrix of the stage about to be multiplied; true when its activations are not the ones in LDS.
     auto enter = [&]() {
         if constexpr (SPLIT) {
-            if (!c_part_start) return false;
-            c_part_start = false;
+            if (c_u != 0 || c_k != c_p * a.part_stages) return false;
             while (c_t >= ce.first_tile + ce.tiles) ce = entry_at(++c_m);      // (only where a run begins)
-            c_end = ce.first_tile + ce.tiles < t_end ? ce.first_tile + ce.tiles : t_end;
             return true;
         }
         bool new_x = false;
@@ -2049,14 +2049,14 @@ bool plan_wide(uint32_t type, int in_w, int inputs, WideGeom* out)
     return true;
 }
 
-// The split form of the shared pass (four input rows per entry) for rows whose four sets of planes do not fit LDS: W as
-// above, and the fewest parts (groups of whole stages) whose planes do.  Not for Q8_0, whose row-tiled row-step kernel
-// serves such calls.
-bool plan_wide_split(uint32_t type, int in_w, WideGeom* out, int* parts, int* part_stages)
+// The split form for rows whose sets of planes (one, or four with shared passes) do not fit LDS beside two stage
+// buffers of a useful size: W as above, and the fewest parts (groups of whole stages) whose planes do.  Q8_0 has it with
+// one input row per entry only: its row-tiled row-step kernel serves calls with several input rows.
+bool plan_wide_split(uint32_t type, int in_w, int inputs, WideGeom* out, int* parts, int* part_stages, int* run_tiles)
 {
-    const WideTraits tr = wide_traits(type, true);
+    const WideTraits tr = wide_traits(type, inputs > 1);
     const int nblocks = in_w / 256;
-    if (!tr.pieces || nblocks < 4 || type == NNHIP_TYPE_Q8_0) return false;
+    if (!tr.pieces || nblocks < 4 || (type == NNHIP_TYPE_Q8_0 && inputs > 1)) return false;
     double best_score = -1.0;
     for (int W = 12; W >= 6; W -= 2) {
         WideGeom g{};
@@ -2075,8 +2075,14 @@ bool plan_wide_split(uint32_t type, int in_w, WideGeom* out, int* parts, int* pa
             const int part_w = SP * g.cols * 256;
             g.plane_stride = part_w + 16;
             g.set_bytes = (4 * g.plane_stride + (tr.sums ? (part_w / 16) * 4 : 0) + 15) / 16 * 16;
-            g.lds_bytes = 2 * static_cast<size_t>(g.stage_bytes) + 4 * static_cast<size_t>(g.set_bytes);
-            if (g.lds_bytes + wide_static_lds(4) + 2048 + tr.table_bytes > static_cast<size_t>(160 * 1024)) continue;
+            g.lds_bytes = 2 * static_cast<size_t>(g.stage_bytes) + static_cast<size_t>(inputs) * g.set_bytes;
+            // what is left holds the sums of a run's tiles: at least eight tiles
+            const size_t per_tile = static_cast<size_t>(inputs) * kTileRows * sizeof(float);
+            const size_t fixed = g.lds_bytes + wide_static_lds(inputs) + tr.table_bytes;
+            if (fixed + 8 * per_tile > static_cast<size_t>(160 * 1024)) continue;
+            size_t run = (static_cast<size_t>(160 * 1024) - fixed) / per_tile;
+            if (run > static_cast<size_t>(kSplitRunMax)) run = kSplitRunMax;
+            g.lds_bytes += run * per_tile;
             const double fill = static_cast<double>(nblocks) / (g.kchunks * g.cols);
             const double score = fill * W / 12.0 * (W % 4 == 0 ? 1.0 : 0.95) * (0.9 + 0.1 * fill) * (1.0 - 0.02 * (P - 2));
             if (score > best_score) {
@@ -2084,6 +2090,7 @@ bool plan_wide_split(uint32_t type, int in_w, WideGeom* out, int* parts, int* pa
                 *out = g;
                 *parts = P;
                 *part_stages = SP;
+                *run_tiles = static_cast<int>(run);
             }
             break;
         }
@@ -2091,16 +2098,38 @@ bool plan_wide_split(uint32_t type, int in_w, WideGeom* out, int* parts, int* pa
     return best_score >= 0;
 }
 
-template <class F>
+// The geometry a launch of the wide form takes: the plain form where it gets at least eight waves, else the split form
+// where that exists (rows of 28672 values leave the plain one-row form four waves), else whatever the plain form gets.
+// *parts = 0: the plain form.
+bool plan_wide_any(uint32_t type, int in_w, int inputs, WideGeom* out, int* parts, int* part_stages, int* run_tiles = nullptr)
+{
+    int run_unused = 0;
+    if (!run_tiles) run_tiles = &run_unused;
+    WideGeom plain{};
+    const bool have_plain = plan_wide(type, in_w, inputs, &plain);
+    *parts = 0;
+    *part_stages = 0;
+    if (have_plain && (plain.waves >= 8 || plain.single)) {
+        *out = plain;
+        return true;
+    }
+    if (plan_wide_split(type, in_w, inputs, out, parts, part_stages, run_tiles)) return true;
+    *parts = 0;
+    *part_stages = 0;
+    if (have_plain) *out = plain;
+    return have_plain;
+}
+
+template <class F, int R>
 hipError_t launch_wide_split_of(Lane* lane, const WideArgs& a)
 {
-    constexpr int M = F::kSharedM, LPW = F::kSharedLpw;
+    constexpr int M = R == 1 ? F::kWideM : F::kSharedM, LPW = R == 1 ? F::kWideLpw : F::kSharedLpw;
     static LdsLimit big_lds;
-    const void* fn = reinterpret_cast<const void*>(&matvec_mfma_wide_kernel<F, M, LPW, 4, false, true>);
-    const hipError_t e = big_lds.ensure(lane->device, fn, 160 * 1024 - wide_static_lds(4) - 2048 - F::kLdsTableBytes);
+    const void* fn = reinterpret_cast<const void*>(&matvec_mfma_wide_kernel<F, M, LPW, R, false, true>);
+    const hipError_t e = big_lds.ensure(lane->device, fn, 160 * 1024 - wide_static_lds(R) - F::kLdsTableBytes);
     if (e != hipSuccess) return e;
     const int groups = a.total_tiles < lane->compute_units ? a.total_tiles : lane->compute_units;
-    hipLaunchKernelGGL((matvec_mfma_wide_kernel<F, M, LPW, 4, false, true>), dim3(groups), dim3(64 * a.g.waves), a.g.lds_bytes,
+    hipLaunchKernelGGL((matvec_mfma_wide_kernel<F, M, LPW, R, false, true>), dim3(groups), dim3(64 * a.g.waves), a.g.lds_bytes,
                        lane->stream, a);
     return hipGetLastError();
 }
@@ -2202,47 +2231,36 @@ hipError_t launch_matvec_mfma_table(Lane* lane, uint32_t type, int in_w, const M
     }
 }
 
-bool matvec_mfma_wide_geometry(uint32_t type, int in_w, int out_w, const void* w, int inputs)
-{
-    WideGeom g;
-    return inputs >= 1 && inputs <= 4 && entry_ok(type, in_w, out_w, w) && plan_wide(type, in_w, inputs == 1 ? 1 : 4, &g);
-}
-
-bool matvec_mfma_split_geometry(uint32_t type, int in_w, int out_w, const void* w, int compute_units)
+bool matvec_mfma_wide_geometry(uint32_t type, int in_w, int out_w, const void* w, int inputs, bool* split)
 {
     WideGeom g;
     int parts = 0, part_stages = 0;
-    if (!entry_ok(type, in_w, out_w, w) || plan_wide(type, in_w, 4, &g) || !plan_wide_split(type, in_w, &g, &parts, &part_stages)) return false;
-    // a workgroup's tiles of one entry (every G-th tile of the launch) wait in LDS between the parts
-    const int tiles = (out_w + kTileRows - 1) / kTileRows;
-    return compute_units > 0 && (tiles + compute_units - 1) / compute_units <= kSplitUnits;
+    const bool ok = inputs >= 1 && inputs <= 4 && entry_ok(type, in_w, out_w, w) &&
+                    plan_wide_any(type, in_w, inputs == 1 ? 1 : 4, &g, &parts, &part_stages);
+    if (split) *split = ok && parts > 0;
+    return ok;
 }
 
 namespace {
 
 hipError_t launch_wide_args(Lane* lane, uint32_t type, int in_w, int inputs, WideArgs& a)
 {
-    bool split = false;
-    if (!plan_wide(type, in_w, inputs == 1 ? 1 : 4, &a.g)) {
-        // four input rows per entry on rows too long for their planes: the split form (entries in the kernel arguments)
-        if (inputs == 1 || a.table || !plan_wide_split(type, in_w, &a.g, &a.parts, &a.part_stages)) return hipErrorInvalidValue;
-        split = true;
-        // runs of consecutive tiles (a workgroup then meets one or two entries, i.e. converts few vectors) where the
-        // tiles of a run fit the sums kept in LDS between the parts
-        const int groups = a.total_tiles < lane->compute_units ? a.total_tiles : lane->compute_units;
-        a.chunked = (a.total_tiles + groups - 1) / groups <= kSplitUnits ? 1 : 0;
-    }
+    if (!plan_wide_any(type, in_w, inputs == 1 ? 1 : 4, &a.g, &a.parts, &a.part_stages, &a.run_tiles)) return hipErrorInvalidValue;
+    const bool split = a.parts > 0;
+    // (the split form: runs of consecutive tiles, so that a workgroup meets few entries, i.e. converts few vectors)
+    if (split) a.chunked = 1;
     a.in_w = in_w;
     a.nblocks = in_w / 256;
     a.row_bytes = static_cast<uint32_t>(a.nblocks) * static_cast<uint32_t>(block_bytes_of(type));
     a.row_pieces_magic = static_cast<uint32_t>((0x100000000ull + a.g.row_pieces - 1) / a.g.row_pieces);
     if (split) {
         switch (type) {
-        case NNHIP_TYPE_Q4_K: return launch_wide_split_of<Q4KTask>(lane, a);
-        case NNHIP_TYPE_Q5_K: return launch_wide_split_of<Q5KTask>(lane, a);
-        case NNHIP_TYPE_Q6_K: return launch_wide_split_of<Q6KTask>(lane, a);
-        case NNHIP_TYPE_IQ2_S: return launch_wide_split_of<IQ2STask>(lane, a);
-        case NNHIP_TYPE_IQ3_S: return launch_wide_split_of<IQ3STask>(lane, a);
+        case NNHIP_TYPE_Q4_K: return inputs == 1 ? launch_wide_split_of<Q4KTask, 1>(lane, a) : launch_wide_split_of<Q4KTask, 4>(lane, a);
+        case NNHIP_TYPE_Q5_K: return inputs == 1 ? launch_wide_split_of<Q5KTask, 1>(lane, a) : launch_wide_split_of<Q5KTask, 4>(lane, a);
+        case NNHIP_TYPE_Q6_K: return inputs == 1 ? launch_wide_split_of<Q6KTask, 1>(lane, a) : launch_wide_split_of<Q6KTask, 4>(lane, a);
+        case NNHIP_TYPE_IQ2_S: return inputs == 1 ? launch_wide_split_of<IQ2STask, 1>(lane, a) : launch_wide_split_of<IQ2STask, 4>(lane, a);
+        case NNHIP_TYPE_IQ3_S: return inputs == 1 ? launch_wide_split_of<IQ3STask, 1>(lane, a) : launch_wide_split_of<IQ3STask, 4>(lane, a);
+        case NNHIP_TYPE_Q8_0: return inputs == 1 ? launch_wide_split_of<Q8_0Task, 1>(lane, a) : hipErrorInvalidValue;
         default: return hipErrorInvalidValue;
         }
     }
@@ -2277,7 +2295,7 @@ bool describe_matvec_rows_shared(uint32_t type, int rows, int in_w, int out_w, i
 {
     WideGeom g;
     int parts = 0, part_stages = 0;
-    if (!plan_wide(type, in_w, per_pass, &g) && (per_pass != 4 || !plan_wide_split(type, in_w, &g, &parts, &part_stages))) return false;
+    if (!plan_wide_any(type, in_w, per_pass, &g, &parts, &part_stages)) return false;
     const int launch_rows = rows < 4 * per_pass ? rows : 4 * per_pass;                 // (four table entries per launch)
     const int tiles = (out_w + kTileRows - 1) / kTileRows * ((launch_rows + per_pass - 1) / per_pass);
     info->kernel = NNHIP_MATVEC_KERNEL_MATRIX_CORE;
@@ -2306,7 +2324,9 @@ bool describe_matvec_mfma_launch(uint32_t type, int in_w, int form, bool runs, n
         return true;
     }
     WideGeom g;
-    if (!plan_wide(type, in_w, form == 3 ? 4 : 1, &g)) return false;
+    int parts = 0, part_stages = 0;
+    if (!plan_wide_any(type, in_w, form == 3 ? 4 : 1, &g, &parts, &part_stages)) return false;
+    if (parts > 0) runs = true;
     info->threads = 64 * g.waves;
     info->stage_buffers = g.single ? 1 : 2;
     info->dynamic_lds_bytes = static_cast<int32_t>(g.lds_bytes);

@@ -120,14 +120,13 @@ hipError_t launch_matvec_mfma_table(Lane* lane, uint32_t type, int in_w, const M
                                     int total_tiles, bool runs);
 // The wide form of the matrix-core mat-vec (activation planes in LDS): any in_w of at least four super-blocks, and
 // entries of up to four input rows that share a pass over the weights (`inputs` = 1: every entry has one row).
-bool matvec_mfma_wide_geometry(uint32_t type, int in_w, int out_w, const void* w, int inputs);
+// *split (optional) receives whether the launch would take the split form (planes of one group of block columns in LDS
+// at a time: rows too long for `inputs` full sets of planes beside useful stage buffers).
+bool matvec_mfma_wide_geometry(uint32_t type, int in_w, int out_w, const void* w, int inputs, bool* split = nullptr);
 // Whether a single call with `rows` input rows is served by that form rather than by row-step passes: 0 (it is not), 4
 // (up to four input rows share a pass over the weights) or 1 (a pass per input row, for rows whose four sets of planes do
 // not fit LDS).
 int matvec_rows_per_pass(uint32_t type, int rows, int in_w, int out_w, const void* w, int compute_units);
-// Whether four input rows can share a pass in the split form (rows too long for four sets of planes in LDS: the planes of
-// one group of block columns at a time).
-bool matvec_mfma_split_geometry(uint32_t type, int in_w, int out_w, const void* w, int compute_units);
 // That call: two or more input rows, `per_pass` of them per table entry and four entries per launch (the descriptors
 // travel in the kernel arguments); *launches receives the number of launches made.
 bool describe_matvec_rows_shared(uint32_t type, int rows, int in_w, int out_w, int per_pass, int compute_units,

@@ -984,3 +984,49 @@ def test_matrix_core_stage_geometries_over_row_lengths(lane, typ, in_w):
     xd.dispose()
     bd.dispose()
     lane.trim()
+
+
+@pytest.mark.parametrize("typ", [GGML_Q8_0, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_IQ2_S, GGML_IQ3_S])
+def test_batched_groups_with_very_long_rows_take_the_split_form(lane, typ):
+    """Rows of 28672 values (the down projection of a 70B-class model): one set of activation planes and two useful stage
+    buffers do not fit LDS together, so a batched group on the matrix cores takes the split form with one input row per
+    entry (planes of half the block columns at a time, runs of consecutive tiles).  Eight descriptors of one matrix, each
+    with activations of its own, against the float64 oracle at both bars, guard words, and the bits of a row do not
+    depend on its place in the batch."""
+    in_w, out_w = 28672, 4133
+    payload = synth.matrix(typ, out_w, in_w, seed=2100 + typ)
+    wd = lane.upload_raw(payload)
+    rng = np.random.default_rng(typ + 5)
+    bias = rng.standard_normal(out_w).astype(np.float32)
+    bd = lane.upload_raw(bias)
+    items = []
+    for i in range(8):
+        rows = 1
+        x = rng.standard_normal((rows, in_w)).astype(np.float32) * np.float32([1.0, 3e-3, 40.0][i % 3])
+        items.append(dict(typ=typ, in_w=in_w, out_w=out_w, rows=rows, payload=payload, x=x, xd=lane.upload_raw(x),
+                          bias=bias if i % 2 else None, wd=wd, bd=bd if i % 2 else None, yd=lane.allocate(rows * out_w + 2)))
+    info = (BatchLaunchInfo * 4)()
+    for i in range(4):
+        info[i].struct_size = ctypes.sizeof(BatchLaunchInfo)
+    descs = (MatvecDesc * 8)()
+    for i, it in enumerate(items):
+        descs[i] = MatvecDesc(it["xd"].ptr, wd.ptr, it["bd"].ptr if it["bd"] else None, it["yd"].ptr, typ, it["rows"], in_w, out_w)
+    n = ctypes.c_int()
+    check(lane._lib.nnhip_matvec_batch_plan(descs, 8, 256, info, 4, ctypes.byref(n)), "matvec_batch_plan")
+    assert n.value == 1 and info[0].kernel == 2 and info[0].consecutive_runs == 1 and info[0].activations_in_lds == 1
+    got = _batch_run(lane, items)
+    for i in (0, 4, 5):
+        it = items[i]
+        ref, asum = oracle.linear_f64(typ, payload, it["x"], it["bias"], it["rows"], in_w, out_w)
+        assert oracle.rel_l2(got[i], ref) <= MATVEC_BAR, i
+        assert np.all(np.abs(got[i].astype(np.float64) - ref) <= 2e-6 + 3e-6 * asum), i
+    order = [4, 0, 7, 1, 5, 2, 3, 6]              # (the same tiles in all: the group stays on the matrix cores)
+    again = _batch_run(lane, [items[i] for i in order])
+    for i, y in zip(order, again):
+        assert np.array_equal(_bits(y), _bits(got[i])), i
+    for it in items:
+        it["xd"].dispose()
+        it["yd"].dispose()
+    wd.dispose()
+    bd.dispose()
+    lane.trim()

@@ -151,13 +151,13 @@ def test_matvec_plan_keeps_a_ring_turn_inside_the_result_buffer():
                             assert info.dynamic_lds_bytes + 2048 + (10240 if typ == 22 else 0) <= 160 * 1024
                         elif in_w == 17408:
                             # ... or shared passes in the split form (the planes of one group of block columns at a time) where
-                            # the groups of four input rows make 3.5 rounds of tiles over the workgroups (IQ2_S: 2.5) and a
-                            # workgroup's tiles of one group fit the sums kept in LDS
+                            # the groups of four input rows make 3.5 rounds of tiles over the workgroups (IQ2_S: 2.5)
                             tiles = -(-out_w // 16)
                             assert typ in (12, 22) and info.row_tile == min(rows, 4)
-                            assert 2 * -(-rows // 4) * tiles >= (5 if typ == 22 else 7) * 256 and -(-tiles // 256) <= 8
+                            assert 2 * -(-rows // 4) * tiles >= (5 if typ == 22 else 7) * 256
                             assert info.steps == tiles * -(-min(rows, 16) // 4)
-                            assert info.dynamic_lds_bytes + 10240 + (10240 if typ == 22 else 0) <= 160 * 1024
+                            # (the sums of a run's tiles take what the planes and the stage buffers leave)
+                            assert info.dynamic_lds_bytes + 8192 + (10240 if typ == 22 else 0) <= 160 * 1024
                             seen_tiles.add((typ, "split"))
                         else:
                             assert rows * -(-out_w // 16) >= (768 if rows >= 3 and typ != 8 else 2048)

@@ -69,7 +69,10 @@ USED_ONE_SET = ["matvec_mfma_kernelINS0_7Q5KTaskELi1ELi2ELi6ELb1"]
 # the split form of the shared pass (rows too long for four sets of planes in LDS)
 USED_SPLIT = ["matvec_mfma_wide_kernelINS0_7Q4KTaskELi1ELi3ELi4ELb0ELb1", "matvec_mfma_wide_kernelINS0_7Q5KTaskELi1ELi3ELi4ELb0ELb1",
               "matvec_mfma_wide_kernelINS0_7Q6KTaskELi1ELi4ELi4ELb0ELb1", "matvec_mfma_wide_kernelINS0_8IQ2STaskELi1ELi2ELi4ELb0ELb1",
-              "matvec_mfma_wide_kernelINS0_8IQ3STaskELi1ELi2ELi4ELb0ELb1"]
+              "matvec_mfma_wide_kernelINS0_8IQ3STaskELi1ELi2ELi4ELb0ELb1",
+              "matvec_mfma_wide_kernelINS0_7Q4KTaskELi1ELi3ELi1ELb0ELb1", "matvec_mfma_wide_kernelINS0_7Q5KTaskELi1ELi3ELi1ELb0ELb1",
+              "matvec_mfma_wide_kernelINS0_7Q6KTaskELi1ELi4ELi1ELb0ELb1", "matvec_mfma_wide_kernelINS0_8IQ2STaskELi2ELi4ELi1ELb0ELb1",
+              "matvec_mfma_wide_kernelINS0_8IQ3STaskELi2ELi4ELi1ELb0ELb1", "matvec_mfma_wide_kernelINS0_8Q8_0TaskELi1ELi5ELi1ELb0ELb1"]
 
 
 def test_parking_writes_wait_only_for_their_own_register_set(isa):
