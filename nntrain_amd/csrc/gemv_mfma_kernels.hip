@@ -1286,7 +1286,7 @@ constexpr int kSplitRunMax = 64;
 
 // SPLIT (rows too long for R full sets of planes in LDS): the stages of a tile are taken in `parts`
 // groups of `part_stages`, and LDS holds the planes of one group of block columns at a time.  A workgroup works through
-// a run of its tiles of a table entry (at most run_tiles of them) once per part: planes of part 0 (with a fixed-point scale of their own), that part of
+// a run of its tiles of a table entry (at most run_tiles of them) once per part: planes of part 0, that part of
 // every tile, planes of part 1, ...; the sums of a tile wait in LDS (bias + part 0, + part 1, ...: one order, so the
 // bits of a row depend on its weights, its activations and the launch geometry only) and are stored after the last part.
 // Every stage of every tile is still requested and multiplied once; what is paid is a conversion of the activations
@@ -1542,17 +1542,22 @@ __global__ __launch_bounds__(64 * kMaxWaves) void matvec_mfma_wide_kernel(WideAr
             __syncthreads();
             return;
         }
+        // (SPLIT: the largest magnitudes are those of the whole rows, taken where a run begins and kept in `red` for its
+        // other parts: one trip to memory per part instead of two, and one fixed-point scale per input row)
+        if (!SPLIT || c_p == 0) {
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-            if (r < rows) {
-                const float4* x4 = reinterpret_cast<const float4*>(ce.x + static_cast<size_t>(r) * a.in_w + x_first);
-                uint32_t mx = 0;
-                for (int i = tid; i < n4; i += T) mx = umax4(mx, x4[i]);
-                mx = wave_umax(mx);
-                if (lane == 0) red[r][wave] = mx;
+            for (int r = 0; r < R; ++r) {
+                if (r < rows) {
+                    const float4* x4 = reinterpret_cast<const float4*>(ce.x + static_cast<size_t>(r) * a.in_w);
+                    const int n4_max = SPLIT ? a.in_w >> 2 : n4;
+                    uint32_t mx = 0;
+                    for (int i = tid; i < n4_max; i += T) mx = umax4(mx, x4[i]);
+                    mx = wave_umax(mx);
+                    if (lane == 0) red[r][wave] = mx;
+                }
             }
+            __syncthreads();
         }
-        __syncthreads();
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             if (r < rows) {
