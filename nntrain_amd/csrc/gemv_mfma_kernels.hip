@@ -35,6 +35,7 @@
 // on the storage type and in_w only, and a launch is a table of matrices that share both, worked through as one sequence
 // of tiles dealt round-robin to the workgroups: a row's bits depend on its weights, in_w and the activation vector, never
 // on out_w, on the other matrices of the launch or on its place in it.
+#include <cmath>
 #include <cstddef>
 #include <cstring>
 #include <type_traits>
@@ -2016,8 +2017,13 @@ bool plan_wide(uint32_t type, int in_w, int inputs, WideGeom* out)
         if (g.lds_bytes + wide_static_lds(inputs) + tr.table_bytes > static_cast<size_t>(160 * 1024)) continue;
         const double fill = static_cast<double>(nblocks) / (g.kchunks * g.cols);
         // (throughput grows with the waves: a stage holds W * M blocks per row and W tasks run side by side)
-        // (and of two equal products the fuller stages win: 16 blocks go as 2 x 8 rather than 12 + 4)
-        const double score = fill * W / 12.0 * (W % 4 == 0 ? 1.0 : 0.95) * (0.9 + 0.1 * fill);
+        // (and of two equal products the fuller stages win: 16 blocks go as 2 x 8 rather than 12 + 4; measured on rows of
+        // 28 blocks: three stages of ten columns stream 3 - 6 % faster than three of twelve, the last a third full)
+        // (one input row per pass of a K-quant: 1 - 9 % on rows of 17 - 50 blocks; the codebook formats lost 3 - 5 % to it
+        // and keep the plain product, as do the shared passes and Q8_0, where it was not measured)
+        const bool k_quant = type == NNHIP_TYPE_Q4_K || type == NNHIP_TYPE_Q5_K || type == NNHIP_TYPE_Q6_K;
+        const double emptiness = inputs == 1 && k_quant ? fill * std::sqrt(fill) : fill;
+        const double score = emptiness * W / 12.0 * (W % 4 == 0 ? 1.0 : 0.95) * (0.9 + 0.1 * fill);
         if (score > best_score) {
             best_score = score;
             best = g;
