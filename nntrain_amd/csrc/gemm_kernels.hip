@@ -828,20 +828,43 @@ hipError_t launch_matmul_of(Lane* lane, const uint16_t* x, const void* w, const 
     a.M = rows;
     a.K = in_w;
     a.N = out_w;
-    // Row tile and strip width: BM = 128 rows for M <= 128, else 256; strips as wide as the column tiles allow, narrowed
-    // so that strips x row tiles is a whole number of rounds over the compute units when that keeps them >= 70 % wide.
-    const int bm = rows <= 128 ? 128 : 256;
-    const int m_tiles = (rows + bm - 1) / bm;
-    const int max_cols = (rows <= 256) ? 80 : 144;
-    int strips = (out_w + max_cols - 1) / max_cols;
+    // Three tilings: 128 rows x 80 columns, 256 x 80 and 256 x 144 per workgroup.  For each, the strips are as wide as the
+    // column tiles allow, narrowed so that strips x row tiles is a whole number of rounds over the compute units when
+    // that keeps them >= 70 % wide; the one with the shortest estimated launch is taken (rounds x time of a K step of
+    // that tiling, measured on 17408 x 5120: 0.64 / 0.99 / 1.33 us, a quarter of it scaled with the strip width; ties go to the larger
+    // tile).  The large tile wins where it fills the device (17408 columns at M >= 512); a matrix with few columns
+    // (a down projection: 5120 x 17408 makes 76 workgroups of 256 x 144) runs on more, smaller tiles: measured at
+    // M = 512, 0.261 -> 0.162 ms; 4096 x 4096 0.074 -> 0.042 ms.
+    struct Tiling { int bm, max_cols; double step_us; };
+    static const Tiling tilings[3] = {{128, 80, 0.64}, {256, 80, 0.99}, {256, 144, 1.33}};
+    int best = -1, best_cols = 0, best_strips = 0, best_m_tiles = 0;
+    double best_cost = 0.0;
     const int per_round = lane->compute_units;
-    const int even = (strips * m_tiles + per_round - 1) / per_round * per_round / m_tiles;
-    if (even > strips && (out_w + even - 1) / even * 10 >= max_cols * 7) strips = even;
-    a.cols = (out_w + strips - 1) / strips;
-    a.strips = (out_w + a.cols - 1) / a.cols;
-    const dim3 grid(a.strips, m_tiles);
-    if (rows <= 128) return launch_gemm<F, 16, 5, 1>(lane, a, grid);
-    if (rows <= 256) return launch_gemm<F, 32, 5, 1>(lane, a, grid);
+    for (int t = 0; t < 3; ++t) {
+        const Tiling& tl = tilings[t];
+        if (t == 0 && rows > 128 && rows <= 256) continue;          // (two row tiles of 128 are never better than one of 256)
+        const int m_tiles = (rows + tl.bm - 1) / tl.bm;
+        int strips = (out_w + tl.max_cols - 1) / tl.max_cols;
+        const int even = (strips * m_tiles + per_round - 1) / per_round * per_round / m_tiles;
+        if (even > strips && (out_w + even - 1) / even * 10 >= tl.max_cols * 7) strips = even;
+        const int cols = (out_w + strips - 1) / strips;
+        strips = (out_w + cols - 1) / cols;
+        const int rounds = (strips * m_tiles + per_round - 1) / per_round;
+        // (rows of a last, ragged row tile cost as much as a full one)
+        const double cost = rounds * tl.step_us * (0.75 + 0.25 * cols / tl.max_cols);
+        if (best < 0 || cost <= best_cost * 1.02) {
+            best = t;
+            best_cost = cost;
+            best_cols = cols;
+            best_strips = strips;
+            best_m_tiles = m_tiles;
+        }
+    }
+    a.cols = best_cols;
+    a.strips = best_strips;
+    const dim3 grid(a.strips, best_m_tiles);
+    if (best == 0) return launch_gemm<F, 16, 5, 1>(lane, a, grid);
+    if (best == 1) return launch_gemm<F, 32, 5, 1>(lane, a, grid);
     return launch_gemm<F, 64, 9, 2>(lane, a, grid);
 }
 
