@@ -115,6 +115,38 @@ def test_random_single_calls_with_one_to_sixteen_rows(lane):
         lane.trim()
 
 
+def test_random_single_calls_on_long_rows(lane):
+    """The same over rows of 6656 - 28672 values, where the planes of four input rows (and, from 24000 values on, of one)
+    do not fit LDS beside the stage buffers: shared passes in the split form, a pass per input row, row-tiled and
+    row-step passes, as the tile counts decide."""
+    rng = np.random.default_rng(20240613)
+    widths = [6656, 7168, 8192, 11264, 14336, 17408, 21504, 24576, 28672]
+    for case in range(36):
+        tname = str(rng.choice(list(TYPES)))
+        typ = TYPES[tname]
+        in_w = int(rng.choice(widths))
+        if tname in ("Q6_K", "IQ2_S", "IQ3_S") and (in_w // 256) % 2:
+            in_w += 256
+        rows = int(rng.choice([1, 2, 3, 4, 5, 8, 9, 12, 13, 16, 19]))
+        out_w = int(rng.choice([37, 1030, 2049, 4100, 5120, 9000]))
+        payload = synth.matrix(typ, out_w, in_w, seed=99000 + case)
+        x = rng.standard_normal((rows, in_w)).astype(np.float32)
+        x *= rng.choice([1e-2, 1.0, 30.0], size=(rows, 1)).astype(np.float32)
+        bias = rng.standard_normal(out_w).astype(np.float32) if rng.integers(0, 2) else None
+        xd, wd = lane.upload_raw(x), lane.upload_raw(payload)
+        bd = lane.upload_raw(bias) if bias is not None else None
+        yd = lane.allocate(rows * out_w + 2)
+        lane.fill_u32(yd, NAN_BITS, rows * out_w + 2)
+        check(lane._lib.nnhip_quant_matvec(lane._handle, typ, c_void_p(xd.ptr), c_void_p(wd.ptr), c_void_p(bd.ptr) if bd else None,
+                                           c_void_p(yd.ptr), rows, in_w, out_w), "matvec")
+        lane.synchronize()
+        _check(f"case {case} {tname} in_w={in_w} out_w={out_w} rows={rows}", lane.read(yd), rows, out_w, typ, payload, x, bias, in_w)
+        for b in (xd, wd, bd, yd):
+            if b is not None:
+                b.dispose()
+        lane.trim()
+
+
 def test_random_prefill_shapes(lane):
     """The bf16 matrix-core mat-mul over row counts around its tile sizes (16 .. 600), heights that do not fill a strip,
     every storage format, with the activations handed over as FP32 (rounded to bfloat16 on the device) or as bfloat16
