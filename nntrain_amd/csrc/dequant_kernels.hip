@@ -41,14 +41,22 @@ __device__ __forceinline__ float4 deq4_q45_k(const uint8_t* w, int64_t e)
 {
     const uint8_t* p = w + (e >> 8) * (FIVE ? 176 : 144);
     const int i = static_cast<int>(e & 255), g = i >> 5, j = i & 31;
-    const float d = half_bits_to_float(ld16(p)), dmin = half_bits_to_float(ld16(p + 2));
-    uint32_t sc, mn;
-    k4_scale_min(p + 4, g, sc, mn);
+    // d, dmin and the twelve bytes of 6-bit scales and minima in one load (blocks are 16-byte aligned); the eight groups
+    // of a block lie in one wave, so the bytes are picked with selects rather than with branches and byte loads
+    const u32x4 h = *reinterpret_cast<const u32x4*>(p);
+    const float d = half_bits_to_float(h[0]), dmin = half_bits_to_float(h[0] >> 16);
+    auto packed = [&](int k) {                       // byte k of the twelve
+        const uint32_t word = k < 4 ? h[1] : (k < 8 ? h[2] : h[3]);
+        return (word >> (8 * (k & 3))) & 0xffu;
+    };
+    const uint32_t a = packed(g & 3), b = packed((g & 3) + 4), c = packed((g & 3) + 8);
+    const uint32_t sc = g < 4 ? a & 63u : (c & 15u) | ((a >> 6) << 4);
+    const uint32_t mn = g < 4 ? b & 63u : (c >> 4) | ((b >> 6) << 4);
     uint32_t q = *reinterpret_cast<const uint32_t*>(p + (FIVE ? 48 : 16) + (g >> 1) * 32 + j);
     q = (g & 1) ? (q >> 4) & 0x0f0f0f0fu : q & 0x0f0f0f0fu;
     if (FIVE) {
-        const uint32_t h = *reinterpret_cast<const uint32_t*>(p + 16 + j);
-        q |= ((h >> g) & 0x01010101u) << 4;
+        const uint32_t hb = *reinterpret_cast<const uint32_t*>(p + 16 + j);
+        q |= ((hb >> g) & 0x01010101u) << 4;
     }
     const float scale = __fmul_rn(d, static_cast<float>(sc));
     const float min = __fmul_rn(dmin, static_cast<float>(mn));
@@ -135,7 +143,11 @@ __global__ __launch_bounds__(256) void dequantize_kernel(const uint8_t* __restri
         else if (TYPE == NNHIP_TYPE_IQ3_S) v = deq4_iq3_s(w, e);
         else if (TYPE == NNHIP_TYPE_BF16) v = deq4_bf16(w, e);
         else v = deq4_iq2_s(w, e);
-        out[t] = v;
+        // (a stream of writes that nothing reads back soon: stored past the caches)
+        __builtin_nontemporal_store(v.x, &out[t].x);
+        __builtin_nontemporal_store(v.y, &out[t].y);
+        __builtin_nontemporal_store(v.z, &out[t].z);
+        __builtin_nontemporal_store(v.w, &out[t].w);
     }
 }
 
