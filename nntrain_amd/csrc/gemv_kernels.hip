@@ -763,7 +763,18 @@ void matvec_rowstep_kernel(MatvecArgs a, const float* __restrict__ bias)
                 if (a.lora_rank > 0) {      // the branch of q35l_*_sg16_lora (NNtrain.Arc/Kernels/qwen35_linear_fast.cl:262-268)
                     const float* br = a.lora_b + static_cast<size_t>(row) * a.lora_rank;
                     float sum = 0.0f;
-                    for (int r = 0; r < a.lora_rank; ++r) sum = fmaf(a.lora_z[r], br[r], sum);
+                    int r = 0;
+                    // (four coefficients a load where the rows of b are 16-byte aligned; the same products in the same order)
+                    if ((a.lora_rank & 3) == 0 && (reinterpret_cast<uintptr_t>(a.lora_b) & 15u) == 0) {
+                        for (; r < a.lora_rank; r += 4) {
+                            const float4 b4 = *reinterpret_cast<const float4*>(br + r);
+                            sum = fmaf(a.lora_z[r], b4.x, sum);
+                            sum = fmaf(a.lora_z[r + 1], b4.y, sum);
+                            sum = fmaf(a.lora_z[r + 2], b4.z, sum);
+                            sum = fmaf(a.lora_z[r + 3], b4.w, sum);
+                        }
+                    }
+                    for (; r < a.lora_rank; ++r) sum = fmaf(a.lora_z[r], br[r], sum);
                     v = v + a.lora_scale * sum;
                 }
                 y[static_cast<size_t>(m) * a.out_w + row] = a.addend ? a.addend[row] + v : v;
