@@ -260,7 +260,7 @@ def run_decode27b(args, lane, nn, oracle):
         "metric": "27B-shape Q8_0 decode tokens/sec", "value": round(tok_s, 2), "unit": "tokens/s",
         "ms_per_step": round(ms_per_step, 4),
         "ms_per_step_stats": stats(each_ms),
-        "config": {"workload": "decode27b: 435 Q8_0 mat-vecs of a Gemma-3-27B-shaped stack (BASELINE configs[2]), "
+        "config": {"workload": "decode27b: 435 Q8_0 mat-vecs of a Gemma-3-27B-shaped stack (the headline configuration), "
                                "28,695,625,728 weight bytes/token resident in HBM, batch 1, fp32 activations",
                    "launch": args.mode, "launches_per_token": n_launch},
         "roofline": {"bound": "hbm", "achieved": round(roof_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
@@ -768,7 +768,7 @@ def run_decode27b_chained(args, lane, nn, oracle):
 
 
 def run_prefill(args, lane, nn, oracle):
-    """Q4_K 17408x5120 bf16-MFMA prefill mat-mul at M = 128, 256, 512, 2048 (BASELINE configs[3]); the other formats
+    """Q4_K 17408x5120 bf16-MFMA prefill mat-mul at M = 128, 256, 512, 2048 (the prefill configuration of the benchmark list); the other formats
     the kernel decodes (Q5_K, Q6_K, Q8_0, IQ2_S, IQ3_S) at M = 512 under "other_formats"."""
     out = _prefill_of(lane, nn, oracle, nn.GGML_Q4_K, "Q4_K", (128, 256, 512, 2048))
     if out is not None:

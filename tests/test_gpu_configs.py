@@ -102,7 +102,7 @@ def q4k_full():
 
 @pytest.mark.parametrize("rows", [256, 512, 2048])
 def test_prefill_full_shape_sampled_rows(lane, q4k_full, rows):
-    """BASELINE's prefill matrix (Q4_K 17408 x 5120) at M = 256, 512 and 2048 (the 32-row and the 64-row wave tiles over
+    """The benchmark's prefill matrix (Q4_K 17408 x 5120) at M = 256, 512 and 2048 (the 32-row and the 64-row wave tiles over
     256 and 128 strips): every output of every 16th input row, both bars, through the FP32-activation entry point."""
     in_w, out_w = 5120, 17408
     payload, w_bf16 = q4k_full

@@ -453,7 +453,7 @@ def test_prefill_matmul_model_width_sample(lane, typ):
 
 
 def test_prefill_matmul_full_width_sample(lane):
-    """BASELINE prefill shape at M = 128: every output of 16 sampled rows against the oracle."""
+    """The benchmark prefill shape (Q4_K 17408 x 5120) at M = 128: every output of 16 sampled rows against the oracle."""
     in_w, out_w, rows = 5120, 17408, 128
     payload = synth.matrix(GGML_Q4_K, out_w, in_w, 2001)
     xb = synth.to_bf16_bits(synth.activations(rows, in_w, 4000))
