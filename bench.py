@@ -240,7 +240,7 @@ def run_decode27b(args, lane, nn, oracle):
     # batch mode: the library groups the 435 matrices by row length (5376, 4096, 21504) and launches the matrix-core
     # mat-vec once per group; the figures below are per launch on average (a third of the token's bytes and time each)
     n_launch = len(tensors) if args.mode != "batch" else launches_per_token
-    batch_kernel = "matvec_mfma_wide_kernel<Q8_0Task, 2, 8, 1, true>"
+    batch_kernel = "matvec_mfma_wide_kernel<Q8_0Task, 2, 8, 1, true, false>"
     traffic = None
     if args.traffic_from:
         if args.mode != "batch":
@@ -252,7 +252,7 @@ def run_decode27b(args, lane, nn, oracle):
         roof_gbs, roof_bytes = dominant["bytes"] / dominant["ms"] / 1e6, dominant["bytes"]
         roof_extra = {"launch_ms": round(dominant["ms"], 4), "launch_ms_stats": dominant["stats"],
                       "note": "the launch for the 311 matrices of row length 5376 (68 % of the token's bytes), timed on its own "
-                              "with HIP events; the 4096- and 21504-wide groups are launches of <Q8_0Task, 1, 5, 1, false>",
+                              "with HIP events; the 4096- and 21504-wide groups are launches of <Q8_0Task, 1, 5, 1, false, false>",
                       "whole_token_gb_per_s": round(gbs, 1)}
     else:
         roof_gbs, roof_bytes, roof_extra = gbs, total_bytes // n_launch, {}
